@@ -1,0 +1,445 @@
+// Atomic fingerprints (2-body, 3-body) and their parameter gradients from the
+// energy branch.  Replaces radialAFs_kernel, angularAFs_kernel,
+// alphagrad_dist_kernel and alphagrad_ang_kernel
+// (STAF/src/fingerprint/{rad,ang}/reforce.cu.cc, STAF/src/grad_finger/{rad,ang}/reforce.cu.cc).
+//
+// One wavefront owns one centre atom.  Sums over an atom's slots/triplets are
+// reduced inside the wave with a fixed butterfly; sums over atoms (the
+// parameter gradients) go through per-workgroup partials and a second,
+// fixed-order pass.  There are no floating-point atomics, so results are
+// bit-reproducible from run to run.
+#include "staf_tile.hpp"
+
+namespace staf {
+
+constexpr int AF_BLOCK = 256;
+constexpr int AF_WAVES = AF_BLOCK / WAVE;
+constexpr int GRAD_MAX_BLOCKS = 1024;
+
+// ---------------------------------------------------------------------------
+// 2-body fingerprints: AF2[b,p,a] = sum_s D_s exp(alpha[t_s,a] D_s) c2[t_s,a]
+// lane <-> channel, sequential over the slots (same order as the slot index).
+// ---------------------------------------------------------------------------
+template <typename real>
+__global__ __launch_bounds__(AF_BLOCK) void af2_kernel(const real* __restrict__ D, const int* __restrict__ im2,
+                                                       const real* __restrict__ alpha2b,
+                                                       const real* __restrict__ emb2b,
+                                                       const int* __restrict__ type_map, real* __restrict__ out,
+                                                       int nf, int Nl, int ld, int nr, int Ar, int nt) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  real* p_al = (real*)smem;          // [nt*Ar]
+  real* p_c2 = p_al + nt * Ar;       // [nt*Ar]
+  real* w_D = p_c2 + nt * Ar;        // [AF_WAVES][nr]
+  int* w_t = (int*)(w_D + AF_WAVES * nr);  // [AF_WAVES][nr]
+  for (int q = threadIdx.x; q < nt * Ar; q += blockDim.x) { p_al[q] = alpha2b[q]; p_c2[q] = emb2b[q]; }
+  const int wave = threadIdx.x / WAVE, lane = lane_id();
+  real* myD = w_D + wave * nr;
+  int* myT = w_t + wave * nr;
+  const int atom = blockIdx.x * AF_WAVES + wave;
+  int cnt = 0;
+  size_t rowAtom = 0;
+  if (atom < nf * Nl) {
+    const int b = atom / Nl, p = atom - b * Nl;
+    rowAtom = (size_t)b * ld + p;
+    const int* im = im2 + rowAtom * (nr + 1);
+    cnt = im[0];
+    if (cnt > nr) cnt = nr;
+    for (int s = lane; s < cnt; s += WAVE) { myD[s] = D[rowAtom * nr + s]; myT[s] = type_map[im[1 + s]]; }
+  }
+  __syncthreads();
+  if (atom >= nf * Nl) return;
+  for (int a = lane; a < Ar; a += WAVE) {
+    real acc = 0;
+    for (int s = 0; s < cnt; s++) {
+      const real d = myD[s];
+      const int t = myT[s];
+      acc += d * (r_exp(p_al[t * Ar + a] * d) * p_c2[t * Ar + a]);
+    }
+    out[(size_t)atom * Ar + a] = acc;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// dL/dalpha2b, dL/demb2b from P = dL/dAF2:
+//   dalpha[t,a] += P c2 D^2 e^{alpha D},  demb[t,a] += P D e^{alpha D}
+// lane <-> channel; per-species accumulators in registers; workgroup partials.
+// ---------------------------------------------------------------------------
+template <typename real>
+__global__ __launch_bounds__(AF_BLOCK) void grad2_kernel(const real* __restrict__ D, const int* __restrict__ im2,
+                                                         const real* __restrict__ alpha2b,
+                                                         const real* __restrict__ emb2b,
+                                                         const int* __restrict__ type_map,
+                                                         const real* __restrict__ P, real* __restrict__ partial,
+                                                         int nf, int Nl, int ld, int nr, int Ar, int nt) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  real* p_al = (real*)smem;                 // [nt*Ar]
+  real* p_c2 = p_al + nt * Ar;              // [nt*Ar]
+  real* w_acc = p_c2 + nt * Ar;             // [AF_WAVES][2*nt*Ar]
+  real* w_D = w_acc + AF_WAVES * 2 * nt * Ar;  // [AF_WAVES][nr]
+  int* w_t = (int*)(w_D + AF_WAVES * nr);   // [AF_WAVES][nr]
+  for (int q = threadIdx.x; q < nt * Ar; q += blockDim.x) { p_al[q] = alpha2b[q]; p_c2[q] = emb2b[q]; }
+  const int wave = threadIdx.x / WAVE, lane = lane_id();
+  real* myD = w_D + wave * nr;
+  int* myT = w_t + wave * nr;
+  real* myAcc = w_acc + wave * 2 * nt * Ar;
+  for (int q = lane; q < 2 * nt * Ar; q += WAVE) myAcc[q] = 0;
+  __syncthreads();
+  const int total = nf * Nl;
+  const int stride = gridDim.x * AF_WAVES;
+  for (int atom = blockIdx.x * AF_WAVES + wave; atom < total; atom += stride) {
+    const int b = atom / Nl, p = atom - b * Nl;
+    const size_t rowAtom = (size_t)b * ld + p;
+    const int* im = im2 + rowAtom * (nr + 1);
+    int cnt = im[0];
+    if (cnt > nr) cnt = nr;
+    for (int s = lane; s < cnt; s += WAVE) { myD[s] = D[rowAtom * nr + s]; myT[s] = type_map[im[1 + s]]; }
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
+    for (int a = lane; a < Ar; a += WAVE) {
+      const real pg = P[(size_t)atom * Ar + a];
+      real ga[NT_MAX], ge[NT_MAX];
+#pragma unroll
+      for (int t = 0; t < NT_MAX; t++) { ga[t] = 0; ge[t] = 0; }
+      for (int s = 0; s < cnt; s++) {
+        const real d = myD[s];
+        const int t = __builtin_amdgcn_readfirstlane(myT[s]);
+        const real e = r_exp(p_al[t * Ar + a] * d) * pg;
+        const real va = d * d * e * p_c2[t * Ar + a];
+        const real ve = d * e;
+#pragma unroll
+        for (int u = 0; u < NT_MAX; u++)
+          if (u == t) { ga[u] += va; ge[u] += ve; }
+      }
+#pragma unroll
+      for (int u = 0; u < NT_MAX; u++)
+        if (u < nt) { myAcc[u * Ar + a] += ga[u]; myAcc[nt * Ar + u * Ar + a] += ge[u]; }
+    }
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
+  }
+  __syncthreads();
+  const int nout = 2 * nt * Ar;
+  for (int q = threadIdx.x; q < nout; q += blockDim.x) {
+    real s = 0;
+#pragma unroll
+    for (int w = 0; w < AF_WAVES; w++) s += w_acc[w * nout + q];
+    partial[(size_t)blockIdx.x * nout + q] = s;
+  }
+}
+
+// Second pass of every parameter-gradient op: out[e] = sum over the blocks'
+// partials in ascending block order.  out0 takes the first n0 elements, out1
+// (may be null) the next n1.
+template <typename real>
+__global__ void reduce_partials_kernel(const real* __restrict__ partial, int nblocks, int nout, real* out0, int n0,
+                                       real* out1, int n1) {
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= nout) return;
+  real s = 0;
+  for (int g = 0; g < nblocks; g++) s += partial[(size_t)g * nout + e];
+  if (e < n0) out0[e] = s;
+  else if (out1 && e - n0 < n1) out1[e - n0] = s;
+}
+
+template <typename real>
+__global__ void fill_zero_kernel(real* p, int n) {
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e < n) p[e] = 0;
+}
+
+// ---------------------------------------------------------------------------
+// 3-body fingerprints and their parameter gradient.
+//   AF3[b,p,a] = sum_{j<k} T/2 (e^{a1 Dj + a2 Dk} + e^{a2 Dj + a1 Dk}) e^{be T} c3[sigma,a]
+// MODE 0: forward.  MODE 1: gradient wrt (a1,a2,be) given P = dL/dAF3.
+// ---------------------------------------------------------------------------
+template <typename real, int MODE>
+__global__ __launch_bounds__(AF_BLOCK) void af3_kernel(const real* __restrict__ Dsup, const real* __restrict__ Tang,
+                                                       const int* __restrict__ im2, const real* __restrict__ alpha3b,
+                                                       const real* __restrict__ emb3b,
+                                                       const int* __restrict__ type_map,
+                                                       const int* __restrict__ numtriplet,
+                                                       const real* __restrict__ P, real* __restrict__ out, int nf,
+                                                       int Nl, int ld, int nr, int na, int Aa, int nt) {
+  constexpr int CH = (MODE == 0) ? 8 : 4;
+  constexpr int NV = (MODE == 0) ? 1 : 3;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int nsig = 2 * nt - 1;
+  ChanTable<real> tab;
+  unsigned char* sp = tab.carve(smem, nsig, Aa);
+  const int nacc = (MODE == 0) ? Aa : nsig * Aa * 3;
+  real* w_acc = (real*)sp;                    // [AF_WAVES][nacc]
+  real* w_D = w_acc + AF_WAVES * nacc;        // [AF_WAVES][nr]
+  real* w_P = w_D + AF_WAVES * nr;            // [AF_WAVES][Aa] (MODE 1)
+  int* w_lst = (int*)(w_P + AF_WAVES * Aa);   // [AF_WAVES][nr]
+  int* w_off = w_lst + AF_WAVES * nr;         // [AF_WAVES][NT_MAX+1]
+  tab.build(alpha3b, emb3b);
+  const int wave = threadIdx.x / WAVE, lane = lane_id();
+  real* acc_l = w_acc + wave * nacc;
+  real* myD = w_D + wave * nr;
+  real* myP = w_P + wave * Aa;
+  int* lst = w_lst + wave * nr;
+  int* off = w_off + wave * (NT_MAX + 1);
+  if (MODE == 1)
+    for (int q = lane; q < nacc; q += WAVE) acc_l[q] = 0;
+  __syncthreads();
+
+  const int total = nf * Nl;
+  const int stride = gridDim.x * AF_WAVES;
+  for (int atom = blockIdx.x * AF_WAVES + wave; atom < total; atom += stride) {
+    const int b = atom / Nl, p = atom - b * Nl;
+    const size_t rowAtom = (size_t)b * ld + p;
+    const int* im = im2 + rowAtom * (nr + 1);
+    int m = numtriplet[rowAtom];
+    if (m > nr) m = nr;
+    m = __builtin_amdgcn_readfirstlane(m);
+    const real* Trow = Tang + rowAtom * na;
+    for (int s = lane; s < m; s += WAVE) myD[s] = Dsup[rowAtom * nr + s];
+    if (MODE == 0)
+      for (int q = lane; q < Aa; q += WAVE) acc_l[q] = 0;
+    else
+      for (int q = lane; q < Aa; q += WAVE) myP[q] = P[(size_t)atom * Aa + q];
+    group_slots_by_type(m, nt, im, type_map, lst, off);
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
+
+    for (int ta = 0; ta < nt; ta++) {
+      const int oa = __builtin_amdgcn_readfirstlane(off[ta]);
+      const int na_ = __builtin_amdgcn_readfirstlane(off[ta + 1]) - oa;
+      if (na_ == 0) continue;
+      for (int tb = ta; tb < nt; tb++) {
+        const int ob = __builtin_amdgcn_readfirstlane(off[tb]);
+        const int nb_ = __builtin_amdgcn_readfirstlane(off[tb + 1]) - ob;
+        const bool same = (ta == tb);
+        const int size = same ? (na_ * (na_ - 1)) / 2 : na_ * nb_;
+        if (size == 0) continue;
+        const int sg = ta + tb;
+        const int nch = __builtin_amdgcn_readfirstlane(tab.nact[sg]);
+        const int pb = sg * Aa;
+        for (int c0 = 0; c0 < nch; c0 += CH) {
+          real acc[CH][NV];
+#pragma unroll
+          for (int u = 0; u < CH; u++)
+#pragma unroll
+            for (int v = 0; v < NV; v++) acc[u][v] = 0;
+          for (int q = lane; q < size; q += WAVE) {
+            int j, k, nn;
+            class_pair(q, same, nb_, lst + oa, lst + ob, m, j, k, nn);
+            if (nn >= na) continue;
+            const real T = Trow[nn];
+            const real Dj = myD[j], Dk = myD[k];
+#pragma unroll
+            for (int u = 0; u < CH; u++) {
+              if (c0 + u < nch) {
+                const real a1 = tab.a1[pb + c0 + u], a2 = tab.a2[pb + c0 + u], be = tab.be[pb + c0 + u];
+                const real e1 = r_exp(a1 * Dj + a2 * Dk);
+                const real e2 = r_exp(a2 * Dj + a1 * Dk);
+                const real eb = r_exp(be * T);
+                if (MODE == 0) {
+                  acc[u][0] += T * (e1 + e2) * eb;
+                } else {
+                  const real w = eb * T;
+                  acc[u][0] += (e1 * Dj + e2 * Dk) * w;
+                  acc[u][1] += (e1 * Dk + e2 * Dj) * w;
+                  acc[u][NV - 1] += (e1 + e2) * w * T;
+                }
+              }
+            }
+          }
+#pragma unroll
+          for (int u = 0; u < CH; u++) {
+            if (c0 + u < nch) {
+              const int a = tab.ch[pb + c0 + u];
+              const real c3h = tab.c3[pb + c0 + u] * real(0.5);
+              if (MODE == 0) {
+                const real tot = wave_sum(acc[u][0]);
+                if (lane == 0) acc_l[a] += tot * c3h;
+              } else {
+                const real f = c3h * myP[a];
+#pragma unroll
+                for (int v = 0; v < NV; v++) {
+                  const real tot = wave_sum(acc[u][v]);
+                  if (lane == 0) acc_l[(sg * Aa + a) * 3 + v] += tot * f;
+                }
+              }
+            }
+          }
+        }
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
+    if (MODE == 0)
+      for (int q = lane; q < Aa; q += WAVE) out[(size_t)atom * Aa + q] = acc_l[q];
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (MODE == 1) {
+    __syncthreads();
+    for (int q = threadIdx.x; q < nacc; q += blockDim.x) {
+      real s = 0;
+#pragma unroll
+      for (int w = 0; w < AF_WAVES; w++) s += w_acc[w * nacc + q];
+      out[(size_t)blockIdx.x * nacc + q] = s;
+    }
+  }
+}
+
+template <typename real, int MODE>
+static size_t af3_lds(int nr, int Aa, int nt) {
+  const int nsig = 2 * nt - 1;
+  const int nacc = (MODE == 0) ? Aa : nsig * Aa * 3;
+  return chan_table_bytes<real>(nsig, Aa) + (size_t)AF_WAVES * (nacc + nr + Aa) * sizeof(real) +
+         (size_t)AF_WAVES * (nr + NT_MAX + 1) * sizeof(int);
+}
+
+// ---- host launchers --------------------------------------------------------
+
+static inline int grad_blocks(int atoms) {
+  int nb = (atoms + AF_WAVES - 1) / AF_WAVES;
+  return nb < GRAD_MAX_BLOCKS ? nb : GRAD_MAX_BLOCKS;
+}
+
+template <typename real>
+static int radial_afs(const real* D, int nr, const real* alpha2b, int Ar, real* out, int nf, int Nl, const int* im2,
+                      const real* emb2b, const int* type_map, int nt, int ld, void* stream_) {
+  if (!D || !alpha2b || !out || !im2 || !emb2b || !type_map || nr <= 0 || Ar <= 0 || nf <= 0 || Nl <= 0 || nt <= 0)
+    return STAF_E_BAD_ARG;
+  if (nt > NT_MAX) return STAF_E_LIMIT;
+  if (ld <= 0) ld = Nl;
+  size_t lds = (size_t)2 * nt * Ar * sizeof(real) + (size_t)AF_WAVES * nr * (sizeof(real) + sizeof(int));
+  if (lds > 64 * 1024) return STAF_E_LIMIT;
+  const int atoms = nf * Nl;
+  hipLaunchKernelGGL(af2_kernel<real>, dim3((atoms + AF_WAVES - 1) / AF_WAVES), dim3(AF_BLOCK), lds,
+                     (hipStream_t)stream_, D, im2, alpha2b, emb2b, type_map, out, nf, Nl, ld, nr, Ar, nt);
+  return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
+}
+
+template <typename real>
+static int alpha_dist_grad(const real* D, int nr, const real* alpha2b, int Ar, real* g_alpha, int nf, int Nl,
+                           const int* im2, const real* P, const real* emb2b, const int* type_map, real* g_emb, int nt,
+                           int ld, void* stream_) {
+  if (!D || !alpha2b || !g_alpha || !g_emb || !im2 || !P || !emb2b || !type_map || nr <= 0 || Ar <= 0 || nf <= 0 ||
+      Nl <= 0 || nt <= 0)
+    return STAF_E_BAD_ARG;
+  if (nt > NT_MAX) return STAF_E_LIMIT;
+  if (ld <= 0) ld = Nl;
+  DeviceState* st = device_state();
+  if (!st) return STAF_E_HIP;
+  hipStream_t stream = (hipStream_t)stream_;
+  const int nout = 2 * nt * Ar;
+  const int nb = grad_blocks(nf * Nl);
+  real* partial = (real*)scratch_reserve(st, (size_t)nb * nout * sizeof(real));
+  if (!partial) return STAF_E_HIP;
+  size_t lds = (size_t)(2 * nt * Ar + AF_WAVES * nout + AF_WAVES * nr) * sizeof(real) + (size_t)AF_WAVES * nr * sizeof(int);
+  if (lds > 64 * 1024) return STAF_E_LIMIT;
+  hipLaunchKernelGGL(grad2_kernel<real>, dim3(nb), dim3(AF_BLOCK), lds, stream, D, im2, alpha2b, emb2b, type_map, P,
+                     partial, nf, Nl, ld, nr, Ar, nt);
+  hipLaunchKernelGGL(reduce_partials_kernel<real>, dim3((nout + 127) / 128), dim3(128), 0, stream, partial, nb, nout,
+                     g_alpha, nt * Ar, g_emb, nt * Ar);
+  return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
+}
+
+template <typename real>
+static int angular_afs(const real* Dsup, const real* Tang, int nr, int na, real* out, int nf, int Nl, const int* im3,
+                       const int* im2, const real* alpha3b, int Aa, const real* emb3b, const int* type_map,
+                       const int* numtriplet, int nt, int ld, void* stream_) {
+  (void)im3;
+  if (!Dsup || !Tang || !out || !im2 || !alpha3b || !emb3b || !type_map || !numtriplet || nr <= 0 || na <= 0 ||
+      Aa <= 0 || nf <= 0 || Nl <= 0 || nt <= 0)
+    return STAF_E_BAD_ARG;
+  if (nt > NT_MAX) return STAF_E_LIMIT;
+  if (ld <= 0) ld = Nl;
+  size_t lds = af3_lds<real, 0>(nr, Aa, nt);
+  if (lds > 64 * 1024) return STAF_E_LIMIT;
+  const int atoms = nf * Nl;
+  hipLaunchKernelGGL((af3_kernel<real, 0>), dim3((atoms + AF_WAVES - 1) / AF_WAVES), dim3(AF_BLOCK), lds,
+                     (hipStream_t)stream_, Dsup, Tang, im2, alpha3b, emb3b, type_map, numtriplet, (const real*)nullptr,
+                     out, nf, Nl, ld, nr, na, Aa, nt);
+  return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
+}
+
+template <typename real>
+static int alphagrad_ang(const real* Dsup, const real* Tang, int nr, int na, const real* P, int nf, int Nl,
+                         const int* im3, const int* im2, const real* alpha3b, int Aa, real* g_alpha,
+                         const real* emb3b, const int* type_map, real* g_emb, const int* numtriplet, int ntc, int nt,
+                         int ld, void* stream_) {
+  (void)im3;
+  if (!Dsup || !Tang || !P || !im2 || !alpha3b || !g_alpha || !g_emb || !emb3b || !type_map || !numtriplet ||
+      nr <= 0 || na <= 0 || Aa <= 0 || nf <= 0 || Nl <= 0 || nt <= 0 || ntc < 2 * nt - 1)
+    return STAF_E_BAD_ARG;
+  if (nt > NT_MAX) return STAF_E_LIMIT;
+  if (ld <= 0) ld = Nl;
+  DeviceState* st = device_state();
+  if (!st) return STAF_E_HIP;
+  hipStream_t stream = (hipStream_t)stream_;
+  const int nsig = 2 * nt - 1;
+  const int nout = nsig * Aa * 3;
+  const int nb = grad_blocks(nf * Nl);
+  real* partial = (real*)scratch_reserve(st, (size_t)nb * nout * sizeof(real));
+  if (!partial) return STAF_E_HIP;
+  size_t lds = af3_lds<real, 1>(nr, Aa, nt);
+  if (lds > 64 * 1024) return STAF_E_LIMIT;
+  // rows sigma >= nsig of the outputs receive no contribution
+  const int nall = ntc * Aa * 3;
+  if (nall > nout)
+    hipLaunchKernelGGL(fill_zero_kernel<real>, dim3((nall - nout + 127) / 128), dim3(128), 0, stream, g_alpha + nout,
+                       nall - nout);
+  hipLaunchKernelGGL(fill_zero_kernel<real>, dim3((ntc * Aa + 127) / 128), dim3(128), 0, stream, g_emb, ntc * Aa);
+  hipLaunchKernelGGL((af3_kernel<real, 1>), dim3(nb), dim3(AF_BLOCK), lds, stream, Dsup, Tang, im2, alpha3b, emb3b,
+                     type_map, numtriplet, P, partial, nf, Nl, ld, nr, na, Aa, nt);
+  hipLaunchKernelGGL(reduce_partials_kernel<real>, dim3((nout + 127) / 128), dim3(128), 0, stream, partial, nb, nout,
+                     g_alpha, nout, (real*)nullptr, 0);
+  return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
+}
+
+}  // namespace staf
+
+extern "C" {
+
+int staf_op_radial_afs_f32(const float* D, int nr, const float* alpha2b, int Ar, float* out, int nf, int Nl,
+                           const int* im2, const float* emb2b, const int* type_map, int nt, int ld, void* stream) {
+  return staf::radial_afs<float>(D, nr, alpha2b, Ar, out, nf, Nl, im2, emb2b, type_map, nt, ld, stream);
+}
+int staf_op_radial_afs_f64(const double* D, int nr, const double* alpha2b, int Ar, double* out, int nf, int Nl,
+                           const int* im2, const double* emb2b, const int* type_map, int nt, int ld, void* stream) {
+  return staf::radial_afs<double>(D, nr, alpha2b, Ar, out, nf, Nl, im2, emb2b, type_map, nt, ld, stream);
+}
+int staf_op_angular_afs_f32(const float* Dsup, const float* Tang, int nr, int na, float* out, int nf, int Nl,
+                            const int* im3, const int* im2, const float* alpha3b, int Aa, const float* emb3b,
+                            const int* type_map, const int* numtriplet, int nt, int ld, void* stream) {
+  return staf::angular_afs<float>(Dsup, Tang, nr, na, out, nf, Nl, im3, im2, alpha3b, Aa, emb3b, type_map, numtriplet,
+                                  nt, ld, stream);
+}
+int staf_op_angular_afs_f64(const double* Dsup, const double* Tang, int nr, int na, double* out, int nf, int Nl,
+                            const int* im3, const int* im2, const double* alpha3b, int Aa, const double* emb3b,
+                            const int* type_map, const int* numtriplet, int nt, int ld, void* stream) {
+  return staf::angular_afs<double>(Dsup, Tang, nr, na, out, nf, Nl, im3, im2, alpha3b, Aa, emb3b, type_map,
+                                   numtriplet, nt, ld, stream);
+}
+int staf_op_alpha_dist_grad_f32(const float* D, int nr, const float* alpha2b, int Ar, float* g_alpha, int nf, int Nl,
+                                const int* im2, const float* P, const float* emb2b, const int* type_map,
+                                float* g_emb, int nt, int ld, void* stream) {
+  return staf::alpha_dist_grad<float>(D, nr, alpha2b, Ar, g_alpha, nf, Nl, im2, P, emb2b, type_map, g_emb, nt, ld,
+                                      stream);
+}
+int staf_op_alpha_dist_grad_f64(const double* D, int nr, const double* alpha2b, int Ar, double* g_alpha, int nf,
+                                int Nl, const int* im2, const double* P, const double* emb2b, const int* type_map,
+                                double* g_emb, int nt, int ld, void* stream) {
+  return staf::alpha_dist_grad<double>(D, nr, alpha2b, Ar, g_alpha, nf, Nl, im2, P, emb2b, type_map, g_emb, nt, ld,
+                                       stream);
+}
+int staf_op_alphagrad_ang_f32(const float* Dsup, const float* Tang, int nr, int na, const float* P, int nf, int Nl,
+                              const int* im3, const int* im2, const float* alpha3b, int Aa, float* g_alpha,
+                              const float* emb3b, const int* type_map, float* g_emb, const int* numtriplet, int ntc,
+                              int nt, int ld, void* stream) {
+  return staf::alphagrad_ang<float>(Dsup, Tang, nr, na, P, nf, Nl, im3, im2, alpha3b, Aa, g_alpha, emb3b, type_map,
+                                    g_emb, numtriplet, ntc, nt, ld, stream);
+}
+int staf_op_alphagrad_ang_f64(const double* Dsup, const double* Tang, int nr, int na, const double* P, int nf, int Nl,
+                              const int* im3, const int* im2, const double* alpha3b, int Aa, double* g_alpha,
+                              const double* emb3b, const int* type_map, double* g_emb, const int* numtriplet, int ntc,
+                              int nt, int ld, void* stream) {
+  return staf::alphagrad_ang<double>(Dsup, Tang, nr, na, P, nf, Nl, im3, im2, alpha3b, Aa, g_alpha, emb3b, type_map,
+                                     g_emb, numtriplet, ntc, nt, ld, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,107 @@
+// Shared device/host helpers of the gfx950 STAF kernels.
+//
+// One templated source serves fp32 and fp64: every kernel is a template on
+// `real` and the extern "C" entry points instantiate it twice (_f32/_f64).
+// Wavefronts are 64 lanes wide; all cross-lane reductions below use a fixed
+// butterfly tree, so a sum's rounding does not depend on scheduling.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/staf_ops.h"
+
+namespace staf {
+
+constexpr int WAVE = 64;
+constexpr int NT_MAX = 8;  // species supported by the per-type bookkeeping
+
+template <typename real> struct Vec2;
+template <> struct Vec2<float> { using type = float2; };
+template <> struct Vec2<double> { using type = double2; };
+
+// The reference's value of pi (STAF/src/descriptor_builder/reforce.cu.cc:15).
+template <typename real> __host__ __device__ inline real pi_ref() { return real(3.141592654); }
+
+__device__ inline float r_exp(float x) { return expf(x); }
+__device__ inline double r_exp(double x) { return exp(x); }
+__device__ inline float r_cos(float x) { return cosf(x); }
+__device__ inline double r_cos(double x) { return cos(x); }
+__device__ inline float r_sin(float x) { return sinf(x); }
+__device__ inline double r_sin(double x) { return sin(x); }
+__device__ inline float r_sqrt(float x) { return sqrtf(x); }
+__device__ inline double r_sqrt(double x) { return sqrt(x); }
+__device__ inline float r_pow(float x, float n) { return powf(x, n); }
+__device__ inline double r_pow(double x, double n) { return pow(x, n); }
+__device__ inline float r_rint(float x) { return rintf(x); }
+__device__ inline double r_rint(double x) { return rint(x); }
+__device__ inline float r_fma(float a, float b, float c) { return fmaf(a, b, c); }
+__device__ inline double r_fma(double a, double b, double c) { return fma(a, b, c); }
+
+__device__ inline int lane_id() { return threadIdx.x & (WAVE - 1); }
+
+// Butterfly all-reduce over the 64 lanes of a wave; every lane returns the sum.
+template <typename T>
+__device__ inline T wave_sum(T v) {
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+  return v;
+}
+__device__ inline int wave_max(int v) {
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) v = max(v, __shfl_xor(v, o, WAVE));
+  return v;
+}
+
+// First flat index of row j in the row-major upper triangle over m items
+// (pairs j<k): the reference's triplet numbering,
+// STAF/src/descriptor_builder/reforce.cu.cc:137-146.
+__device__ inline int tri_rowstart(int j, int m) { return j * m - (j * (j + 1)) / 2; }
+
+// Inverse of the numbering: nn -> (j,k), 0 <= nn < m(m-1)/2.
+__device__ inline void tri_decode(int nn, int m, int& j, int& k) {
+  const int t = 2 * m - 1;
+  int jj = (int)(((float)t - sqrtf((float)(t * t - 8 * nn))) * 0.5f);
+  if (jj < 0) jj = 0;
+  if (jj > m - 2) jj = m - 2;
+  while (jj < m - 2 && tri_rowstart(jj + 1, m) <= nn) ++jj;
+  while (jj > 0 && tri_rowstart(jj, m) > nn) --jj;
+  j = jj;
+  k = nn - tri_rowstart(jj, m) + jj + 1;
+}
+
+// Pair index q inside an n-item triangle (x<y) -> (x,y); same numbering.
+__device__ inline void tri_decode_xy(int q, int n, int& x, int& y) { tri_decode(q, n, x, y); }
+
+// ---- library-owned device state (per device) -------------------------------
+struct Workspace {
+  void* buf = nullptr;
+  size_t bytes = 0;
+};
+
+struct DeviceState {
+  int device = -1;
+  int* status_d = nullptr;   // device word, error bits OR-ed in by kernels
+  int* status_h = nullptr;   // pinned host mirror
+  Workspace scratch;         // per-slot partial forces / partial sums
+  Workspace buckets;         // transpose buckets (counters + entries), kept zeroed between calls
+  size_t bucket_counters = 0;
+};
+
+DeviceState* device_state();                                   // for the current device, created on demand
+void* scratch_reserve(DeviceState* st, size_t bytes);          // grows, never shrinks
+int* bucket_reserve(DeviceState* st, size_t n_counters, size_t n_entries, hipStream_t stream, int** entries);
+int finish_op(DeviceState* st, hipStream_t stream);            // launch check (+ optional sync & status fetch)
+bool sync_errors_enabled();
+
+// Descriptor geometry shared by all devices (set by construct_descriptors_light).
+template <typename real>
+struct DescConfig {
+  bool ready = false;
+  int nr = 0, na = 0, n_max = 0, max_batch = 0;
+  real Rc = 0, Rs = 0, Ra = 0;
+  real cA = 0, cB = 0, cC = 0, pa = 0, pb = 0;
+  int dist2_fma = 0;
+  int zero_padding = 0;
+};
+
+}  // namespace staf

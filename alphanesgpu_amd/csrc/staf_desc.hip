@@ -1,0 +1,413 @@
+// Descriptor op: neighbour list under minimum-image PBC + radial and angular
+// descriptors with their Jacobians, one kernel launch for the whole batch.
+//
+// Replaces the reference chain convert_carte_to_int -> celleBuild -> imeBuild ->
+// sort_neighbors -> DescriptorsRadial -> DescriptorsAngular
+// (STAF/src/descriptor_builder/celle_gpu.cu.cc:11-201, reforce.cu.cc:17-236).
+//
+// Layout of the work: one 256-thread workgroup per (frame, centre atom).
+//   1. all-pairs candidate scan of the frame (positions are a few KB and stay
+//      in L2), accepted neighbours compacted into LDS;
+//   2. rank sort on the key (dist2, index) -> canonical order, independent of
+//      the order candidates arrived in;
+//   3. per-slot radial quantities written coalesced along the slot axis and
+//      kept in LDS as the neighbour tile (unit vector, 1/r, fc, grad fc);
+//   4. the j<k triplets of the tile are enumerated over the lanes, each lane
+//      owning consecutive triplet indices so that angdescr / intmap3b / der3b
+//      rows are written as contiguous vectors.
+// The neighbour list never touches HBM; the only HBM traffic is the position
+// read and the nine op outputs, each written exactly once (padding included).
+#include "staf_common.hpp"
+
+#include <math.h>
+#include <stdio.h>
+#include <mutex>
+
+namespace staf {
+
+template <typename real>
+struct DescArgs {
+  const real* pos;
+  const real* box;
+  int nf, N, nr, na;
+  real Rc, Ra, Rs, cA, cB, cC, pa, pb;
+  int dist2_fma, zero_padding;
+  real* raddescr;
+  real* angdescr;
+  real* des3bsupp;
+  int* intmap2b;
+  int* intmap3b;
+  real* der2b;
+  real* der3b;
+  real* der3bsupp;
+  int* numtriplet;
+  int* status;
+};
+
+// Everything that decides an integer output (which atoms are neighbours, their
+// order, how many fall inside Ra) is computed without FMA contraction, in the
+// operation order of the reference source, so that it matches a plain IEEE
+// evaluation bit for bit.
+template <typename real>
+__device__ inline void inverse_box(const real* b, real* inv) {
+#pragma clang fp contract(off)
+  inv[0] = real(1.) / b[0];
+  inv[1] = -b[1] / (b[0] * b[3]);
+  inv[2] = (b[1] * b[4]) / (b[0] * b[3] * b[5]) - b[2] / (b[0] * b[5]);
+  inv[3] = real(1.) / b[3];
+  inv[4] = -b[4] / (b[3] * b[5]);
+  inv[5] = real(1.) / b[5];
+}
+
+template <typename real>
+__device__ inline void to_frac(const real* inv, real px, real py, real pz, real* s) {
+#pragma clang fp contract(off)
+  s[0] = (inv[0] * px + inv[1] * py + inv[2] * pz);
+  s[1] = (inv[3] * py + inv[4] * pz);
+  s[2] = (inv[5] * pz);
+}
+
+// d = H * ((sa - sb) - rint(sa - sb)), returns |d|^2 as the neighbour test sees it.
+template <typename real>
+__device__ inline real mic_delta(const real* box, const real* sa, const real* sb, int fma_mode, real* d) {
+#pragma clang fp contract(off)
+  real ox = sa[0] - sb[0], oy = sa[1] - sb[1], oz = sa[2] - sb[2];
+  ox -= r_rint(ox);
+  oy -= r_rint(oy);
+  oz -= r_rint(oz);
+  d[0] = box[0] * ox + box[1] * oy + box[2] * oz;
+  d[1] = box[3] * oy + box[4] * oz;
+  d[2] = box[5] * oz;
+  if (fma_mode) return r_fma(d[2], d[2], r_fma(d[1], d[1], d[0] * d[0]));
+  return (d[0] * d[0] + d[1] * d[1]) + d[2] * d[2];
+}
+
+template <typename real>
+__device__ inline real norm_plain(const real* d) {
+#pragma clang fp contract(off)
+  return r_sqrt((d[0] * d[0] + d[1] * d[1]) + d[2] * d[2]);
+}
+
+template <typename real>
+__global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
+  using real2 = typename Vec2<real>::type;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int nr = A.nr, na = A.na, N = A.N;
+  // LDS carve-up
+  real* c_d2 = (real*)smem;            // [nr] candidate dist2
+  real* c_d = c_d2 + nr;               // [3*nr] candidate delta (neighbour - centre)
+  real* s_u = c_d + 3 * nr;            // [3*nr] unit vector centre - neighbour, sorted
+  real* s_g = s_u + 3 * nr;            // [3*nr] grad of fc wrt d, sorted
+  real* s_invr = s_g + 3 * nr;         // [nr]
+  real* s_fc = s_invr + nr;            // [nr]
+  int* c_j = (int*)(s_fc + nr);        // [nr] candidate index
+  int* s_j = c_j + nr;                 // [nr] sorted neighbour index
+  __shared__ int cnt_all, cnt_ang;
+  __shared__ real sbox[6];
+
+  const int tid = threadIdx.x;
+  const int b = blockIdx.x / N;
+  const int i = blockIdx.x - b * N;
+  if (tid == 0) { cnt_all = 0; cnt_ang = 0; }
+  if (tid < 6) sbox[tid] = A.box[b * 6 + tid];
+  __syncthreads();
+
+  real box[6], inv[6];
+#pragma unroll
+  for (int c = 0; c < 6; c++) box[c] = sbox[c];
+  inverse_box(box, inv);
+  const real* pf = A.pos + (size_t)b * N * 3;
+  real si[3];
+  to_frac(inv, pf[3 * i], pf[3 * i + 1], pf[3 * i + 2], si);
+  const real rc2 = A.Rc * A.Rc;
+
+  // 1. candidate scan
+  for (int j = tid; j < N; j += blockDim.x) {
+    real sj[3], d[3];
+    to_frac(inv, pf[3 * j], pf[3 * j + 1], pf[3 * j + 2], sj);
+    real d2 = mic_delta(box, sj, si, A.dist2_fma, d);
+    if (d2 < rc2 && j != i) {
+      int slot = atomicAdd(&cnt_all, 1);
+      if (slot < nr) {
+        c_j[slot] = j;
+        c_d2[slot] = d2;
+        c_d[3 * slot] = d[0];
+        c_d[3 * slot + 1] = d[1];
+        c_d[3 * slot + 2] = d[2];
+      }
+    }
+  }
+  __syncthreads();
+  const int hm = cnt_all;
+  const int n = hm < nr ? hm : nr;
+  if (hm > nr && tid == 0) atomicOr(A.status, 1);
+
+  const size_t atom = (size_t)b * N + i;
+  const size_t row = atom * nr;
+  const size_t row3 = atom * 3 * nr;
+  int* im = A.intmap2b + atom * (nr + 1);
+  const real PI = pi_ref<real>();
+
+  // 2+3. rank sort and radial fill
+  for (int e = tid; e < nr; e += blockDim.x) {
+    if (e < n) {
+      const real d2 = c_d2[e];
+      const int j = c_j[e];
+      int rank = 0;
+      for (int o = 0; o < n; o++) {
+        const real od2 = c_d2[o];
+        const int oj = c_j[o];
+        rank += (od2 < d2 || (od2 == d2 && oj < j)) ? 1 : 0;
+      }
+      // centre - neighbour: exact negation of the scan's neighbour - centre
+      real d[3] = {-c_d[3 * e], -c_d[3 * e + 1], -c_d[3 * e + 2]};
+      const real r = norm_plain(d);
+      const real invr = real(1) / r;
+      real fc = 0, dfc = 0;
+      if (r < A.Ra) {
+        atomicAdd(&cnt_ang, 1);
+        const real x = PI * r / A.Ra;
+        fc = real(0.5) * (r_cos(x) + real(1));
+        dfc = -real(0.5) * r_sin(x) * PI / A.Ra;
+      }
+      real D, dD;
+      if (r < A.Rs) {
+        D = A.cA / r_pow(r, A.pa) + A.cB / r_pow(r, A.pb) + A.cC;
+        dD = -A.pa * A.cA / r_pow(r, A.pa + real(1)) - A.pb * A.cB / r_pow(r, A.pb + real(1));
+      } else {
+        const real x = PI * r / A.Rc;
+        D = real(0.5) * (r_cos(x) + real(1));
+        dD = -real(0.5) * r_sin(x) * PI / A.Rc;
+      }
+      A.raddescr[row + rank] = D;
+      A.des3bsupp[row + rank] = fc;
+      im[1 + rank] = j;
+      s_j[rank] = j;
+      s_invr[rank] = invr;
+      s_fc[rank] = fc;
+#pragma unroll
+      for (int c = 0; c < 3; c++) {
+        const real u = d[c] * invr;
+        A.der2b[row3 + c * nr + rank] = dD * u;
+        A.der3bsupp[row3 + c * nr + rank] = dfc * u;
+        s_u[3 * rank + c] = u;
+        s_g[3 * rank + c] = dfc * u;
+      }
+    } else {
+      A.raddescr[row + e] = 0;
+      A.des3bsupp[row + e] = 0;
+      im[1 + e] = 0;
+#pragma unroll
+      for (int c = 0; c < 3; c++) {
+        A.der2b[row3 + c * nr + e] = 0;
+        A.der3bsupp[row3 + c * nr + e] = 0;
+      }
+    }
+  }
+  __syncthreads();
+  const int m = cnt_ang;
+  if (tid == 0) {
+    im[0] = hm;
+    A.numtriplet[atom] = m;
+  }
+
+  // 4. angular fill: triplet nn <-> (j<k) over the first m sorted neighbours
+  int ntr = (m * (m - 1)) / 2;
+  if (ntr > na) ntr = na;
+  real* ang = A.angdescr + atom * na;
+  int2* im3 = (int2*)A.intmap3b + atom * na;
+  real2* d3 = (real2*)A.der3b + atom * 3 * na;
+  for (int nn = tid; nn < na; nn += blockDim.x) {
+    if (nn < ntr) {
+      int j, k;
+      tri_decode(nn, m, j, k);
+      const real uj0 = s_u[3 * j], uj1 = s_u[3 * j + 1], uj2 = s_u[3 * j + 2];
+      const real uk0 = s_u[3 * k], uk1 = s_u[3 * k + 1], uk2 = s_u[3 * k + 2];
+      const real cs = uj0 * uk0 + uj1 * uk1 + uj2 * uk2;
+      const real fj = s_fc[j], fk = s_fc[k];
+      const real half = real(0.5) * (cs + real(1));
+      const real ff = fj * fk;
+      const real aj = real(0.5) * s_invr[j] * ff, ak = real(0.5) * s_invr[k] * ff;
+      const real hk = half * fk, hj = half * fj;
+      ang[nn] = half * ff;
+      im3[nn] = make_int2(s_j[j], s_j[k]);
+      real2 o;
+      o.x = aj * (uk0 - cs * uj0) + hk * s_g[3 * j];
+      o.y = ak * (uj0 - cs * uk0) + hj * s_g[3 * k];
+      d3[nn] = o;
+      o.x = aj * (uk1 - cs * uj1) + hk * s_g[3 * j + 1];
+      o.y = ak * (uj1 - cs * uk1) + hj * s_g[3 * k + 1];
+      d3[na + nn] = o;
+      o.x = aj * (uk2 - cs * uj2) + hk * s_g[3 * j + 2];
+      o.y = ak * (uj2 - cs * uk2) + hj * s_g[3 * k + 2];
+      d3[2 * na + nn] = o;
+    } else {
+      ang[nn] = 0;
+      im3[nn] = make_int2(0, 0);
+      if (A.zero_padding) {
+        real2 z;
+        z.x = 0;
+        z.y = 0;
+        d3[nn] = z;
+        d3[na + nn] = z;
+        d3[2 * na + nn] = z;
+      }
+    }
+  }
+}
+
+template <typename real>
+size_t desc_lds_bytes(int nr) {
+  return (size_t)nr * (12 * sizeof(real) + 2 * sizeof(int));
+}
+
+// ---- host side -------------------------------------------------------------
+
+static std::mutex g_cfg_mu;
+static DescConfig<float> g_cfg_f;
+static DescConfig<double> g_cfg_d;
+template <typename real> DescConfig<real>& cfg();
+template <> DescConfig<float>& cfg<float>() { return g_cfg_f; }
+template <> DescConfig<double>& cfg<double>() { return g_cfg_d; }
+
+// Short-range coefficients of D(r) = A/r^alpha + B/r^beta + C matching value,
+// slope and curvature of the cosine cutoff at rs; evaluated in `real` like
+// fill_repulsion, STAF/src/descriptor_builder/reforce.cc:101-125.
+template <typename real>
+static void repulsion_coefficients(DescConfig<real>& c) {
+  const real PI = pi_ref<real>();
+  const real al = 1., be = -30.;
+  const real rs = c.Rs, rc = c.Rc;
+  const real cs = std::cos(PI * rs / rc), sn = std::sin(PI * rs / rc);
+  const real f = 0.5 * (cs + 1);
+  const real f1 = -0.5 * PI / rc * sn;
+  const real f2r = -0.5 * (PI / rc) * (PI / rc) * cs * (rs * rs);
+  const real inv = 1. / (al - be);
+  const real gam_r = inv * al - 1;
+  const real del_r = inv * (f * (al - be) - f1 * rs - f * al);
+  const real eta_r = -al / (al - be);
+  const real eps_r = inv * (rs * f1 + al * f);
+  const real c2r = al * (al + 1) * del_r + be * (be + 1) * eps_r;
+  const real c1r = al * (al + 1) * gam_r + be * (be + 1) * eta_r;
+  c.cC = (f2r - c2r) / c1r;
+  const real rsb = std::pow(rs, be), rsa = std::pow(rs, al);
+  const real eta = -al * rsb / (al - be);
+  const real eps = rsb / (al - be) * (rs * f1 + al * f);
+  c.cB = eta * c.cC + eps;
+  const real gam = rsa / (al - be) * al - rsa;
+  const real del = rsa / (al - be) * (f * (al - be) - f1 * rs - f * al);
+  c.cA = gam * c.cC + del;
+  c.pa = al;
+  c.pb = be;
+}
+
+template <typename real>
+static int construct(real Rc, int nr, int na, int numpar, real Rs, real Ra, int max_batch, const char* curve_path) {
+  if (nr <= 0 || na <= 0 || numpar <= 0 || max_batch <= 0 || !(Rc > 0) || !(Ra > 0)) return STAF_E_BAD_ARG;
+  if (nr > 1024) return STAF_E_LIMIT;
+  DescConfig<real> c;
+  c.nr = nr; c.na = na; c.n_max = numpar; c.max_batch = max_batch;
+  c.Rc = Rc; c.Rs = Rs; c.Ra = Ra;
+  repulsion_coefficients(c);
+  c.ready = true;
+  if (curve_path) {
+    FILE* f = fopen(curve_path, "w");
+    if (!f) return STAF_E_BAD_ARG;
+    const real PI = pi_ref<real>();
+    real dx = Rc / 1000., x = 0;
+    for (int k = 0; k < 1000; k++) {
+      x = x + dx;
+      if (x < Rs)
+        fprintf(f, "%g %g\n", x, c.cA / std::pow(x, c.pa) + c.cB / std::pow(x, c.pb) + c.cC);
+      else
+        fprintf(f, "%g %g\n", x, 0.5 * (1 + std::cos(PI * x / Rc)));
+    }
+    fclose(f);
+  }
+  std::lock_guard<std::mutex> lock(g_cfg_mu);
+  c.dist2_fma = cfg<real>().dist2_fma;
+  c.zero_padding = cfg<real>().zero_padding;
+  cfg<real>() = c;
+  return STAF_OK;
+}
+
+template <typename real>
+static int compute(const real* pos, const real* box, int nf, int N, real* raddescr, real* angdescr, real* des3bsupp,
+                   int* intmap2b, int* intmap3b, real* der2b, real* der3b, real* der3bsupp, int* numtriplet,
+                   void* stream_) {
+  DescConfig<real> c;
+  {
+    std::lock_guard<std::mutex> lock(g_cfg_mu);
+    c = cfg<real>();
+  }
+  if (!c.ready) return STAF_E_NOT_CONSTRUCTED;
+  if (!pos || !box || !raddescr || !angdescr || !des3bsupp || !intmap2b || !intmap3b || !der2b || !der3b ||
+      !der3bsupp || !numtriplet || nf <= 0 || N <= 0)
+    return STAF_E_BAD_ARG;
+  DeviceState* st = device_state();
+  if (!st) return STAF_E_HIP;
+  hipStream_t stream = (hipStream_t)stream_;
+  DescArgs<real> A;
+  A.pos = pos; A.box = box; A.nf = nf; A.N = N; A.nr = c.nr; A.na = c.na;
+  A.Rc = c.Rc; A.Ra = c.Ra; A.Rs = c.Rs; A.cA = c.cA; A.cB = c.cB; A.cC = c.cC; A.pa = c.pa; A.pb = c.pb;
+  A.dist2_fma = c.dist2_fma; A.zero_padding = c.zero_padding;
+  A.raddescr = raddescr; A.angdescr = angdescr; A.des3bsupp = des3bsupp; A.intmap2b = intmap2b;
+  A.intmap3b = intmap3b; A.der2b = der2b; A.der3b = der3b; A.der3bsupp = der3bsupp; A.numtriplet = numtriplet;
+  A.status = st->status_d;
+  size_t lds = desc_lds_bytes<real>(c.nr);
+  if (lds > 60 * 1024) return STAF_E_LIMIT;
+  hipLaunchKernelGGL(desc_kernel<real>, dim3((unsigned)(nf * N)), dim3(256), lds, stream, A);
+  return finish_op(st, stream);
+}
+
+}  // namespace staf
+
+extern "C" {
+
+int staf_op_construct_descriptors_light_f32(float rc, int nr, int na, int numpar, float rs, float ra, int max_batch,
+                                            const char* path) {
+  return staf::construct<float>(rc, nr, na, numpar, rs, ra, max_batch, path);
+}
+int staf_op_construct_descriptors_light_f64(double rc, int nr, int na, int numpar, double rs, double ra,
+                                            int max_batch, const char* path) {
+  return staf::construct<double>(rc, nr, na, numpar, rs, ra, max_batch, path);
+}
+
+int staf_op_descriptor_options(int dist2_fma, int zero_padding) {
+  std::lock_guard<std::mutex> lock(staf::g_cfg_mu);
+  staf::g_cfg_f.dist2_fma = staf::g_cfg_d.dist2_fma = dist2_fma ? 1 : 0;
+  staf::g_cfg_f.zero_padding = staf::g_cfg_d.zero_padding = zero_padding ? 1 : 0;
+  return STAF_OK;
+}
+
+int staf_op_descriptor_coefficients_f32(float* o) {
+  std::lock_guard<std::mutex> lock(staf::g_cfg_mu);
+  if (!staf::g_cfg_f.ready) return STAF_E_NOT_CONSTRUCTED;
+  if (!o) return STAF_E_BAD_ARG;
+  o[0] = staf::g_cfg_f.cA; o[1] = staf::g_cfg_f.cB; o[2] = staf::g_cfg_f.cC; o[3] = staf::g_cfg_f.pa; o[4] = staf::g_cfg_f.pb;
+  return STAF_OK;
+}
+int staf_op_descriptor_coefficients_f64(double* o) {
+  std::lock_guard<std::mutex> lock(staf::g_cfg_mu);
+  if (!staf::g_cfg_d.ready) return STAF_E_NOT_CONSTRUCTED;
+  if (!o) return STAF_E_BAD_ARG;
+  o[0] = staf::g_cfg_d.cA; o[1] = staf::g_cfg_d.cB; o[2] = staf::g_cfg_d.cC; o[3] = staf::g_cfg_d.pa; o[4] = staf::g_cfg_d.pb;
+  return STAF_OK;
+}
+
+int staf_op_compute_descriptors_light_f32(const float* pos, const float* box, int nf, int N, float* raddescr,
+                                          float* angdescr, float* des3bsupp, int* intmap2b, int* intmap3b,
+                                          float* der2b, float* der3b, float* der3bsupp, int* numtriplet,
+                                          void* stream) {
+  return staf::compute<float>(pos, box, nf, N, raddescr, angdescr, des3bsupp, intmap2b, intmap3b, der2b, der3b,
+                              der3bsupp, numtriplet, stream);
+}
+int staf_op_compute_descriptors_light_f64(const double* pos, const double* box, int nf, int N, double* raddescr,
+                                          double* angdescr, double* des3bsupp, int* intmap2b, int* intmap3b,
+                                          double* der2b, double* der3b, double* der3bsupp, int* numtriplet,
+                                          void* stream) {
+  return staf::compute<double>(pos, box, nf, N, raddescr, angdescr, des3bsupp, intmap2b, intmap3b, der2b, der3b,
+                               der3bsupp, numtriplet, stream);
+}
+
+}  // extern "C"

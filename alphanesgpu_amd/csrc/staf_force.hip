@@ -1,0 +1,793 @@
+// Forces (2-body, 3-body) and the gradients of the force ops.
+// Replaces computeforce_doublets_kernel, computeforce_tripl_kernel,
+// back_prop_grad_force2b_kernel and gradforce_tripl_kernel
+// (STAF/src/force/{rad,ang}/reforce.cu.cc, STAF/src/grad_force/{rad,ang}/reforce.cu.cc).
+//
+// Force scatter is owner-computes and deterministic:
+//   pass A  (per centre i)   pair force of every neighbour slot -> scratch
+//                            gslot[b,i,s,3], centre's own force -> self[b,i,3];
+//                            each slot is also registered in the bucket of the
+//                            atom that receives it (integer atomics only);
+//   pass B  (per receiver a) the bucket is put in canonical (centre, slot)
+//                            order and summed with a fixed tree.
+// The 120x re-read of der3b by the reference's gradient kernel (one pass per
+// channel and species pair) is gone: der3b is contracted once per triplet with
+// dL/dF into three scalars, and all channels are evaluated from those.
+#include "staf_tile.hpp"
+
+namespace staf {
+
+constexpr int F_BLOCK = 256;
+constexpr int F_WAVES = F_BLOCK / WAVE;
+constexpr int F_PARTS = 4;  // partner split of the per-slot sums in the 3-body force
+constexpr int GRAD_MAX_BLOCKS_F = 1024;
+
+__device__ inline int species_shift(const int* tipos, const int* actual_type) {
+  const int at = actual_type[0];
+  int s = 0;
+  for (int y = 0; y < at; y++) s += tipos[y];
+  return s;
+}
+
+// register slot (key) with the receiving atom `recv` of frame b
+__device__ inline void bucket_push(int* bcnt, int* bent, int cap, size_t recv, int key, int* status) {
+  const int pos = atomicAdd(&bcnt[recv], 1);
+  if (pos < cap) bent[recv * cap + pos] = key;
+  else atomicOr(status, 2);
+}
+
+// ---------------------------------------------------------------------------
+// 2-body force, pass A.  One wave per centre, lane <-> slot.
+//   g_s = 1/2 sum_a G[a] c2[t_s,a] e^{alpha D}(1 + alpha D) * grad D_s
+// ---------------------------------------------------------------------------
+template <typename real>
+__global__ __launch_bounds__(F_BLOCK) void force2_kernel(const real* __restrict__ G, const real* __restrict__ D,
+                                                         const real* __restrict__ dD, const int* __restrict__ im2,
+                                                         const real* __restrict__ alpha2b,
+                                                         const real* __restrict__ emb2b,
+                                                         const int* __restrict__ type_map, real* __restrict__ gslot,
+                                                         real* __restrict__ self, int* bcnt, int* bent, int cap,
+                                                         int* status, int nf, int N, int Nl, int ld, int nr, int Ar,
+                                                         int nt) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  real* p_al = (real*)smem;      // [nt*Ar]
+  real* p_c2 = p_al + nt * Ar;   // [nt*Ar]
+  real* w_G = p_c2 + nt * Ar;    // [F_WAVES][Ar]
+  for (int q = threadIdx.x; q < nt * Ar; q += blockDim.x) { p_al[q] = alpha2b[q]; p_c2[q] = emb2b[q]; }
+  const int wave = threadIdx.x / WAVE, lane = lane_id();
+  real* myG = w_G + wave * Ar;
+  const int atom = blockIdx.x * F_WAVES + wave;
+  const bool live = atom < nf * Nl;
+  int b = 0, p = 0;
+  size_t rowAtom = 0;
+  if (live) {
+    b = atom / Nl; p = atom - b * Nl;
+    rowAtom = (size_t)b * ld + p;
+    for (int a = lane; a < Ar; a += WAVE) myG[a] = G[(size_t)atom * Ar + a];
+  }
+  __syncthreads();
+  if (!live) return;
+  const int* im = im2 + rowAtom * (nr + 1);
+  int cnt = im[0];
+  if (cnt > nr) cnt = nr;
+  real sf[3] = {0, 0, 0};
+  const size_t rowScr = (size_t)atom;
+  for (int s = lane; s < cnt; s += WAVE) {
+    const int nj = im[1 + s];
+    const int t = type_map[nj];
+    const real d = D[rowAtom * nr + s];
+    real w = 0;
+    for (int a = 0; a < Ar; a++) {
+      const real al = p_al[t * Ar + a];
+      w += myG[a] * (p_c2[t * Ar + a] * r_exp(al * d) * (real(1) + al * d));
+    }
+    w *= real(0.5);
+#pragma unroll
+    for (int c = 0; c < 3; c++) {
+      const real g = w * dD[rowAtom * 3 * nr + c * nr + s];
+      gslot[(rowScr * nr + s) * 3 + c] = g;
+      sf[c] -= g;
+    }
+    bucket_push(bcnt, bent, cap, (size_t)b * N + nj, p * nr + s, status);
+  }
+#pragma unroll
+  for (int c = 0; c < 3; c++) {
+    const real tot = wave_sum(sf[c]);
+    if (lane == 0) self[rowScr * 3 + c] = tot;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// 3-body force, pass A.  One 256-thread workgroup per centre.
+// Phase 1 (thread <-> triplet, class-enumerated): channel sums
+//     Sd  = sum_a net_a delta_a,  SBj = sum_a net_a Bp_j,a,  SBk = sum_a net_a Bp_k,a
+//   kept in LDS by storage index nn.
+// Phase 2 (thread <-> slot x component x partner part): force on slot s
+//     F_s = sum_p Sd(s,p) dT/dd_s(s,p) + (sum_p SB_s(s,p)) grad fc_s
+//   summed in a fixed order; der3b is read here, once per element.
+// ---------------------------------------------------------------------------
+template <typename real>
+__global__ __launch_bounds__(F_BLOCK) void force3_kernel(const real* __restrict__ G, const real* __restrict__ Dsup,
+                                                         const real* __restrict__ Tang,
+                                                         const real* __restrict__ dDsup,
+                                                         const real* __restrict__ d3b, const int* __restrict__ im2,
+                                                         const real* __restrict__ alpha3b,
+                                                         const real* __restrict__ emb3b,
+                                                         const int* __restrict__ type_map,
+                                                         const int* __restrict__ numtriplet,
+                                                         real* __restrict__ gslot, real* __restrict__ self, int* bcnt,
+                                                         int* bent, int cap, int* status, int nf, int N, int Nl,
+                                                         int ld, int nr, int na, int Aa, int nt) {
+  using real2 = typename Vec2<real>::type;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int nsig = 2 * nt - 1;
+  ChanTable<real> tab;
+  unsigned char* sp = tab.carve(smem, nsig, Aa);
+  real* scal = (real*)sp;               // [3*na]
+  real* bl_D = scal + 3 * na;           // [nr]
+  real* bl_g = bl_D + nr;               // [3*nr] grad fc rows (der3bsupp)
+  real* bl_G = bl_g + 3 * nr;           // [Aa]
+  real* part = bl_G + Aa;               // [F_PARTS*3*nr]
+  real* fs = part + F_PARTS * 3 * nr;   // [3*nr]
+  int* lst = (int*)(fs + 3 * nr);       // [nr]
+  int* off = lst + nr;                  // [NT_MAX+1]
+  tab.build(alpha3b, emb3b);
+
+  const int tid = threadIdx.x;
+  const int atom = blockIdx.x;
+  const int b = atom / Nl, p = atom - b * Nl;
+  const size_t rowAtom = (size_t)b * ld + p;
+  const int* im = im2 + rowAtom * (nr + 1);
+  int m = numtriplet[rowAtom];
+  if (m > nr) m = nr;
+  for (int s = tid; s < m; s += blockDim.x) {
+    bl_D[s] = Dsup[rowAtom * nr + s];
+#pragma unroll
+    for (int c = 0; c < 3; c++) bl_g[c * nr + s] = dDsup[rowAtom * 3 * nr + c * nr + s];
+  }
+  for (int a = tid; a < Aa; a += blockDim.x) bl_G[a] = G[(size_t)atom * Aa + a];
+  if (tid < WAVE) group_slots_by_type(m, nt, im, type_map, lst, off);
+  __syncthreads();
+
+  const real* Trow = Tang + rowAtom * na;
+  // phase 1
+  for (int ta = 0; ta < nt; ta++) {
+    const int oa = off[ta];
+    const int na_ = off[ta + 1] - oa;
+    if (na_ == 0) continue;
+    for (int tb = ta; tb < nt; tb++) {
+      const int ob = off[tb];
+      const int nb_ = off[tb + 1] - ob;
+      const bool same = (ta == tb);
+      const int size = same ? (na_ * (na_ - 1)) / 2 : na_ * nb_;
+      if (size == 0) continue;
+      const int sg = ta + tb;
+      const int nch = tab.nact[sg];
+      const int pb = sg * Aa;
+      for (int q = tid; q < size; q += blockDim.x) {
+        int j, k, nn;
+        class_pair(q, same, nb_, lst + oa, lst + ob, m, j, k, nn);
+        if (nn >= na) continue;
+        const real T = Trow[nn];
+        const real Dj = bl_D[j], Dk = bl_D[k];
+        real Sd = 0, SBj = 0, SBk = 0;
+        for (int ia = 0; ia < nch; ia++) {
+          const real a1 = tab.a1[pb + ia], a2 = tab.a2[pb + ia], be = tab.be[pb + ia];
+          const real net = real(0.5) * bl_G[tab.ch[pb + ia]] * tab.c3[pb + ia];
+          const real eb = r_exp(be * T);
+          const real sim1 = r_exp(a2 * Dj + a1 * Dk);
+          const real sim2 = r_exp(a1 * Dj + a2 * Dk);
+          const real h = real(0.5) * eb * net;
+          Sd += h * (real(1) + be * T) * (sim1 + sim2);
+          SBj += h * T * (a1 * sim2 + a2 * sim1);
+          SBk += h * T * (a1 * sim1 + a2 * sim2);
+        }
+        scal[3 * nn] = Sd;
+        scal[3 * nn + 1] = SBj;
+        scal[3 * nn + 2] = SBk;
+      }
+    }
+  }
+  __syncthreads();
+
+  // phase 2
+  const real2* d3 = (const real2*)d3b + rowAtom * 3 * na;
+  const int items = m * 3 * F_PARTS;
+  for (int w = tid; w < items; w += blockDim.x) {
+    const int s = w % m;
+    const int c = (w / m) % 3;
+    const int h = w / (3 * m);
+    real acc = 0, accB = 0;
+    for (int pp = h; pp < m; pp += F_PARTS) {
+      if (pp == s) continue;
+      const bool lo = s < pp;
+      const int j = lo ? s : pp, k = lo ? pp : s;
+      const int nn = tri_rowstart(j, m) + k - j - 1;
+      if (nn >= na) continue;
+      const real2 dv = d3[c * na + nn];
+      acc += scal[3 * nn] * (lo ? dv.x : dv.y);
+      accB += scal[3 * nn + (lo ? 1 : 2)];
+    }
+    part[(h * 3 + c) * nr + s] = acc + accB * bl_g[c * nr + s];
+  }
+  __syncthreads();
+  const size_t rowScr = (size_t)atom;
+  for (int w = tid; w < 3 * m; w += blockDim.x) {
+    const int s = w % m, c = w / m;
+    real f = 0;
+#pragma unroll
+    for (int h = 0; h < F_PARTS; h++) f += part[(h * 3 + c) * nr + s];
+    fs[c * nr + s] = f;
+    gslot[(rowScr * nr + s) * 3 + c] = f;
+  }
+  for (int s = tid; s < m; s += blockDim.x)
+    bucket_push(bcnt, bent, cap, (size_t)b * N + im[1 + s], p * nr + s, status);
+  __syncthreads();
+  if (tid < WAVE) {
+#pragma unroll
+    for (int c = 0; c < 3; c++) {
+      real a = 0;
+      for (int s = tid; s < m; s += WAVE) a -= fs[c * nr + s];
+      a = wave_sum(a);
+      if (tid == 0) self[rowScr * 3 + c] = a;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// pass B: one wave per receiving atom.  Bucket entries (keys p*nr+s of the
+// centre slots that point at this atom) are ranked, the slot forces are placed
+// in rank order and summed with a fixed tree; the centre's own force is added
+// when the receiver belongs to the centre species.  Clears the bucket counter.
+// ---------------------------------------------------------------------------
+template <typename real>
+__global__ __launch_bounds__(F_BLOCK) void gather_kernel(const real* __restrict__ gslot,
+                                                         const real* __restrict__ self, int* bcnt,
+                                                         const int* __restrict__ bent, int cap,
+                                                         const int* __restrict__ tipos,
+                                                         const int* __restrict__ actual_type,
+                                                         real* __restrict__ force, int nf, int N, int Nl, int nr) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  real* w_val = (real*)smem;                      // [F_WAVES][3*cap]
+  int* w_key = (int*)(w_val + F_WAVES * 3 * cap);  // [F_WAVES][cap]
+  const int wave = threadIdx.x / WAVE, lane = lane_id();
+  real* val = w_val + wave * 3 * cap;
+  int* key = w_key + wave * cap;
+  const int recv = blockIdx.x * F_WAVES + wave;
+  if (recv >= nf * N) return;
+  const int b = recv / N, a = recv - b * N;
+  const int shift = species_shift(tipos, actual_type);
+  int L = bcnt[recv];
+  L = __builtin_amdgcn_readfirstlane(L);
+  if (L > cap) L = cap;
+  for (int e = lane; e < L; e += WAVE) key[e] = bent[(size_t)recv * cap + e];
+  __builtin_amdgcn_wave_barrier();
+  __threadfence_block();
+  if (lane == 0 && L > 0) bcnt[recv] = 0;
+  for (int e = lane; e < L; e += WAVE) {
+    const int ke = key[e];
+    int rank = 0;
+    for (int o = 0; o < L; o++) rank += (key[o] < ke) ? 1 : 0;
+    const size_t src = ((size_t)b * Nl * nr + ke) * 3;
+    val[3 * rank] = gslot[src];
+    val[3 * rank + 1] = gslot[src + 1];
+    val[3 * rank + 2] = gslot[src + 2];
+  }
+  __builtin_amdgcn_wave_barrier();
+  __threadfence_block();
+  real f[3] = {0, 0, 0};
+  for (int e = lane; e < L; e += WAVE) {
+    f[0] += val[3 * e];
+    f[1] += val[3 * e + 1];
+    f[2] += val[3 * e + 2];
+  }
+#pragma unroll
+  for (int c = 0; c < 3; c++) f[c] = wave_sum(f[c]);
+  if (lane < 3) {
+    real o = lane == 0 ? f[0] : (lane == 1 ? f[1] : f[2]);
+    const int pl = a - shift;
+    if (pl >= 0 && pl < Nl) o += self[((size_t)b * Nl + pl) * 3 + lane];
+    force[((size_t)b * N + a) * 3 + lane] = o;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// gradient of the 2-body force op.  Q = dL/dF.
+//   w_s   = sum_c (Q[j_s,c] - Q[i,c]) * 1/2 dD_s,c
+//   dG[a]      = sum_s w_s c2 e(1+alpha D)
+//   dalpha[t,a]= sum w_s G[a] c2 e D (2+alpha D),  dc2[t,a] = sum w_s G[a] e (1+alpha D)
+// ---------------------------------------------------------------------------
+template <typename real>
+__global__ __launch_bounds__(F_BLOCK) void gradforce2_kernel(
+    const real* __restrict__ Q, const real* __restrict__ G, const real* __restrict__ D, const real* __restrict__ dD,
+    const int* __restrict__ im2, const real* __restrict__ alpha2b, const real* __restrict__ emb2b,
+    const int* __restrict__ type_map, const int* __restrict__ tipos, const int* __restrict__ actual_type,
+    real* __restrict__ gnet, real* __restrict__ partial, int nf, int N, int Nl, int ld, int nr, int Ar, int nt) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  real* p_al = (real*)smem;                     // [nt*Ar]
+  real* p_c2 = p_al + nt * Ar;                  // [nt*Ar]
+  real* w_acc = p_c2 + nt * Ar;                 // [F_WAVES][2*nt*Ar]
+  real* w_D = w_acc + F_WAVES * 2 * nt * Ar;    // [F_WAVES][nr]
+  real* w_w = w_D + F_WAVES * nr;               // [F_WAVES][nr]
+  int* w_t = (int*)(w_w + F_WAVES * nr);        // [F_WAVES][nr]
+  for (int q = threadIdx.x; q < nt * Ar; q += blockDim.x) { p_al[q] = alpha2b[q]; p_c2[q] = emb2b[q]; }
+  const int wave = threadIdx.x / WAVE, lane = lane_id();
+  real* myD = w_D + wave * nr;
+  real* myW = w_w + wave * nr;
+  int* myT = w_t + wave * nr;
+  const int nout = 2 * nt * Ar;
+  real* myAcc = w_acc + wave * nout;
+  for (int q = lane; q < nout; q += WAVE) myAcc[q] = 0;
+  const int shift = species_shift(tipos, actual_type);
+  __syncthreads();
+  const int total = nf * Nl;
+  const int stride = gridDim.x * F_WAVES;
+  for (int atom = blockIdx.x * F_WAVES + wave; atom < total; atom += stride) {
+    const int b = atom / Nl, p = atom - b * Nl;
+    const size_t rowAtom = (size_t)b * ld + p;
+    const int* im = im2 + rowAtom * (nr + 1);
+    int cnt = im[0];
+    if (cnt > nr) cnt = nr;
+    const real* Qi = Q + ((size_t)b * N + p + shift) * 3;
+    const real qi0 = Qi[0], qi1 = Qi[1], qi2 = Qi[2];
+    for (int s = lane; s < cnt; s += WAVE) {
+      const int nj = im[1 + s];
+      const real* Qj = Q + ((size_t)b * N + nj) * 3;
+      const real* dr = dD + rowAtom * 3 * nr + s;
+      myW[s] = real(0.5) * ((Qj[0] - qi0) * dr[0] + (Qj[1] - qi1) * dr[nr] + (Qj[2] - qi2) * dr[2 * nr]);
+      myD[s] = D[rowAtom * nr + s];
+      myT[s] = type_map[nj];
+    }
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
+    for (int a = lane; a < Ar; a += WAVE) {
+      const real g = G[(size_t)atom * Ar + a];
+      real dg = 0;
+      real ga[NT_MAX], ge[NT_MAX];
+#pragma unroll
+      for (int t = 0; t < NT_MAX; t++) { ga[t] = 0; ge[t] = 0; }
+      for (int s = 0; s < cnt; s++) {
+        const real d = myD[s], w = myW[s];
+        const int t = __builtin_amdgcn_readfirstlane(myT[s]);
+        const real al = p_al[t * Ar + a], c2 = p_c2[t * Ar + a];
+        const real e = r_exp(al * d);
+        const real sds = e * (real(1) + al * d);
+        dg += w * c2 * sds;
+        const real va = w * g * c2 * e * d * (real(2) + al * d);
+        const real ve = w * g * sds;
+#pragma unroll
+        for (int u = 0; u < NT_MAX; u++)
+          if (u == t) { ga[u] += va; ge[u] += ve; }
+      }
+      gnet[(size_t)atom * Ar + a] = dg;
+#pragma unroll
+      for (int u = 0; u < NT_MAX; u++)
+        if (u < nt) { myAcc[u * Ar + a] += ga[u]; myAcc[nt * Ar + u * Ar + a] += ge[u]; }
+    }
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
+  }
+  __syncthreads();
+  for (int q = threadIdx.x; q < nout; q += blockDim.x) {
+    real s = 0;
+#pragma unroll
+    for (int w = 0; w < F_WAVES; w++) s += w_acc[w * nout + q];
+    partial[(size_t)blockIdx.x * nout + q] = s;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// gradient of the 3-body force op.  One wave per centre, class-enumerated.
+// Per triplet (j<k), with q_s = Q[atom of slot s] - Q[centre]:
+//   U  = sum_c q_j,c dT/dd_j,c + q_k,c dT/dd_k,c      (der3b contracted once)
+//   V_s = sum_c q_s,c grad fc_s,c                      (per slot)
+// and per channel
+//   dG[a]      += c3/2 (delta U + Bp_j V_j + Bp_k V_k)
+//   dpar[sg,a] += G[a] c3/2 (d delta/dpar U + d Bp_j/dpar V_j + d Bp_k/dpar V_k)
+// ---------------------------------------------------------------------------
+template <typename real>
+__global__ __launch_bounds__(F_BLOCK) void gradforce3_kernel(
+    const real* __restrict__ Q, const real* __restrict__ G, const real* __restrict__ Dsup,
+    const real* __restrict__ Tang, const real* __restrict__ dDsup, const real* __restrict__ d3b,
+    const int* __restrict__ im2, const real* __restrict__ alpha3b, const real* __restrict__ emb3b,
+    const int* __restrict__ type_map, const int* __restrict__ tipos, const int* __restrict__ actual_type,
+    const int* __restrict__ numtriplet, real* __restrict__ gnet, real* __restrict__ partial, int nf, int N, int Nl,
+    int ld, int nr, int na, int Aa, int nt) {
+  using real2 = typename Vec2<real>::type;
+  constexpr int CH = 4;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int nsig = 2 * nt - 1;
+  ChanTable<real> tab;
+  unsigned char* sp = tab.carve(smem, nsig, Aa);
+  const int nacc = nsig * Aa * 3;
+  real* w_acc = (real*)sp;                     // [F_WAVES][nacc]
+  real* w_D = w_acc + F_WAVES * nacc;          // [F_WAVES][nr]
+  real* w_V = w_D + F_WAVES * nr;              // [F_WAVES][nr]
+  real* w_q = w_V + F_WAVES * nr;              // [F_WAVES][3*nr]
+  real* w_G = w_q + F_WAVES * 3 * nr;          // [F_WAVES][Aa]
+  real* w_o = w_G + F_WAVES * Aa;              // [F_WAVES][Aa]
+  int* w_lst = (int*)(w_o + F_WAVES * Aa);     // [F_WAVES][nr]
+  int* w_off = w_lst + F_WAVES * nr;           // [F_WAVES][NT_MAX+1]
+  tab.build(alpha3b, emb3b);
+  const int wave = threadIdx.x / WAVE, lane = lane_id();
+  real* acc_l = w_acc + wave * nacc;
+  real* myD = w_D + wave * nr;
+  real* myV = w_V + wave * nr;
+  real* myQ = w_q + wave * 3 * nr;
+  real* myG = w_G + wave * Aa;
+  real* myO = w_o + wave * Aa;
+  int* lst = w_lst + wave * nr;
+  int* off = w_off + wave * (NT_MAX + 1);
+  for (int q = lane; q < nacc; q += WAVE) acc_l[q] = 0;
+  const int shift = species_shift(tipos, actual_type);
+  __syncthreads();
+
+  const int total = nf * Nl;
+  const int stride = gridDim.x * F_WAVES;
+  for (int atom = blockIdx.x * F_WAVES + wave; atom < total; atom += stride) {
+    const int b = atom / Nl, p = atom - b * Nl;
+    const size_t rowAtom = (size_t)b * ld + p;
+    const int* im = im2 + rowAtom * (nr + 1);
+    int m = numtriplet[rowAtom];
+    if (m > nr) m = nr;
+    m = __builtin_amdgcn_readfirstlane(m);
+    const real* Trow = Tang + rowAtom * na;
+    const real2* d3 = (const real2*)d3b + rowAtom * 3 * na;
+    const real* Qi = Q + ((size_t)b * N + p + shift) * 3;
+    const real qi0 = Qi[0], qi1 = Qi[1], qi2 = Qi[2];
+    for (int s = lane; s < m; s += WAVE) {
+      const int nj = im[1 + s];
+      const real* Qj = Q + ((size_t)b * N + nj) * 3;
+      const real q0 = Qj[0] - qi0, q1 = Qj[1] - qi1, q2 = Qj[2] - qi2;
+      const real* gr = dDsup + rowAtom * 3 * nr + s;
+      myQ[3 * s] = q0; myQ[3 * s + 1] = q1; myQ[3 * s + 2] = q2;
+      myV[s] = q0 * gr[0] + q1 * gr[nr] + q2 * gr[2 * nr];
+      myD[s] = Dsup[rowAtom * nr + s];
+    }
+    for (int a = lane; a < Aa; a += WAVE) { myG[a] = G[(size_t)atom * Aa + a]; myO[a] = 0; }
+    group_slots_by_type(m, nt, im, type_map, lst, off);
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
+
+    for (int ta = 0; ta < nt; ta++) {
+      const int oa = __builtin_amdgcn_readfirstlane(off[ta]);
+      const int na_ = __builtin_amdgcn_readfirstlane(off[ta + 1]) - oa;
+      if (na_ == 0) continue;
+      for (int tb = ta; tb < nt; tb++) {
+        const int ob = __builtin_amdgcn_readfirstlane(off[tb]);
+        const int nb_ = __builtin_amdgcn_readfirstlane(off[tb + 1]) - ob;
+        const bool same = (ta == tb);
+        const int size = same ? (na_ * (na_ - 1)) / 2 : na_ * nb_;
+        if (size == 0) continue;
+        const int sg = ta + tb;
+        const int nch = __builtin_amdgcn_readfirstlane(tab.nact[sg]);
+        const int pb = sg * Aa;
+        for (int c0 = 0; c0 < nch; c0 += CH) {
+          real acc[CH][4];
+#pragma unroll
+          for (int u = 0; u < CH; u++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) acc[u][v] = 0;
+          for (int q = lane; q < size; q += WAVE) {
+            int j, k, nn;
+            class_pair(q, same, nb_, lst + oa, lst + ob, m, j, k, nn);
+            if (nn >= na) continue;
+            const real T = Trow[nn];
+            const real Dj = myD[j], Dk = myD[k];
+            const real Vj = myV[j], Vk = myV[k];
+            real U = 0;
+#pragma unroll
+            for (int c = 0; c < 3; c++) {
+              const real2 dv = d3[c * na + nn];
+              U += myQ[3 * j + c] * dv.x + myQ[3 * k + c] * dv.y;
+            }
+#pragma unroll
+            for (int u = 0; u < CH; u++) {
+              if (c0 + u < nch) {
+                const real a1 = tab.a1[pb + c0 + u], a2 = tab.a2[pb + c0 + u], be = tab.be[pb + c0 + u];
+                const real eb = r_exp(be * T);
+                const real sim1 = r_exp(a2 * Dj + a1 * Dk);
+                const real sim2 = r_exp(a1 * Dj + a2 * Dk);
+                const real ss = sim1 + sim2;
+                const real opb = real(1) + be * T;
+                const real hT = real(0.5) * eb * T;
+                const real suppj = a1 * sim2 + a2 * sim1;
+                const real suppk = a1 * sim1 + a2 * sim2;
+                // value
+                acc[u][0] += real(0.5) * eb * opb * ss * U + hT * (suppj * Vj + suppk * Vk);
+                // d/d alpha1
+                acc[u][1] += real(0.5) * eb * opb * (sim1 * Dk + sim2 * Dj) * U +
+                             hT * ((sim2 + a1 * sim2 * Dj + a2 * sim1 * Dk) * Vj +
+                                   (sim1 + a1 * sim1 * Dk + a2 * sim2 * Dj) * Vk);
+                // d/d alpha2
+                acc[u][2] += real(0.5) * eb * opb * (sim1 * Dj + sim2 * Dk) * U +
+                             hT * ((sim1 + a2 * sim1 * Dj + a1 * sim2 * Dk) * Vj +
+                                   (sim2 + a2 * sim2 * Dk + a1 * sim1 * Dj) * Vk);
+                // d/d beta
+                acc[u][3] += hT * (real(2) + be * T) * ss * U + hT * T * (suppj * Vj + suppk * Vk);
+              }
+            }
+          }
+#pragma unroll
+          for (int u = 0; u < CH; u++) {
+            if (c0 + u < nch) {
+              const int a = tab.ch[pb + c0 + u];
+              const real c3h = tab.c3[pb + c0 + u] * real(0.5);
+              const real t0 = wave_sum(acc[u][0]);
+              const real t1 = wave_sum(acc[u][1]);
+              const real t2 = wave_sum(acc[u][2]);
+              const real t3 = wave_sum(acc[u][3]);
+              if (lane == 0) {
+                myO[a] += t0 * c3h;
+                const real f = c3h * myG[a];
+                acc_l[(sg * Aa + a) * 3] += t1 * f;
+                acc_l[(sg * Aa + a) * 3 + 1] += t2 * f;
+                acc_l[(sg * Aa + a) * 3 + 2] += t3 * f;
+              }
+            }
+          }
+        }
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
+    for (int a = lane; a < Aa; a += WAVE) gnet[(size_t)atom * Aa + a] = myO[a];
+    __builtin_amdgcn_wave_barrier();
+  }
+  __syncthreads();
+  for (int q = threadIdx.x; q < nacc; q += blockDim.x) {
+    real s = 0;
+#pragma unroll
+    for (int w = 0; w < F_WAVES; w++) s += w_acc[w * nacc + q];
+    partial[(size_t)blockIdx.x * nacc + q] = s;
+  }
+}
+
+template <typename real>
+__global__ void reduce_partials_f_kernel(const real* __restrict__ partial, int nblocks, int nout, real* out0, int n0,
+                                         real* out1, int n1) {
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= nout) return;
+  real s = 0;
+  for (int g = 0; g < nblocks; g++) s += partial[(size_t)g * nout + e];
+  if (e < n0) out0[e] = s;
+  else if (out1 && e - n0 < n1) out1[e - n0] = s;
+}
+
+template <typename real>
+__global__ void fill_zero_f_kernel(real* p, int n) {
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e < n) p[e] = 0;
+}
+
+// ---- host launchers --------------------------------------------------------
+
+static inline int grad_blocks_f(int atoms) {
+  int nb = (atoms + F_WAVES - 1) / F_WAVES;
+  return nb < GRAD_MAX_BLOCKS_F ? nb : GRAD_MAX_BLOCKS_F;
+}
+
+struct ForceScratch {
+  void* gslot;
+  void* self;
+  int* bcnt;
+  int* bent;
+  int cap;
+};
+
+template <typename real>
+static int force_scratch(DeviceState* st, int nf, int N, int Nl, int nr, hipStream_t stream, ForceScratch* fs) {
+  const size_t ng = (size_t)nf * Nl * nr * 3, ns = (size_t)nf * Nl * 3;
+  real* base = (real*)scratch_reserve(st, (ng + ns) * sizeof(real));
+  if (!base) return STAF_E_HIP;
+  fs->gslot = base;
+  fs->self = base + ng;
+  fs->cap = 4 * nr;
+  fs->bcnt = bucket_reserve(st, (size_t)nf * N, (size_t)nf * N * fs->cap, stream, &fs->bent);
+  if (!fs->bcnt) return STAF_E_HIP;
+  return STAF_OK;
+}
+
+template <typename real>
+static int launch_gather(DeviceState* st, const ForceScratch& fs, const int* tipos, const int* actual_type,
+                         real* force, int nf, int N, int Nl, int nr, hipStream_t stream) {
+  size_t lds = (size_t)F_WAVES * fs.cap * (3 * sizeof(real) + sizeof(int));
+  if (lds > 64 * 1024) return STAF_E_LIMIT;
+  const int recv = nf * N;
+  hipLaunchKernelGGL(gather_kernel<real>, dim3((recv + F_WAVES - 1) / F_WAVES), dim3(F_BLOCK), lds, stream,
+                     (const real*)fs.gslot, (const real*)fs.self, fs.bcnt, (const int*)fs.bent, fs.cap, tipos,
+                     actual_type, force, nf, N, Nl, nr);
+  return finish_op(st, stream);
+}
+
+template <typename real>
+static int force_doublets(const real* G, const real* D, const real* dD, const int* im2, int nr, int N, int nf, int Ar,
+                          const real* alpha2b, const real* emb2b, int nt, const int* tipos, const int* actual_type,
+                          real* force, const int* type_map, int Nl, real* virial, const real* pos, const real* box,
+                          int ld, void* stream_) {
+  if (!G || !D || !dD || !im2 || !alpha2b || !emb2b || !tipos || !actual_type || !force || !type_map || nr <= 0 ||
+      N <= 0 || nf <= 0 || Ar <= 0 || nt <= 0 || Nl <= 0 || Nl > N)
+    return STAF_E_BAD_ARG;
+  if (virial || pos || box) return STAF_E_LIMIT;  // virial form: not built yet
+  if (nt > NT_MAX) return STAF_E_LIMIT;
+  if (ld <= 0) ld = Nl;
+  DeviceState* st = device_state();
+  if (!st) return STAF_E_HIP;
+  hipStream_t stream = (hipStream_t)stream_;
+  ForceScratch fs;
+  int rc = force_scratch<real>(st, nf, N, Nl, nr, stream, &fs);
+  if (rc) return rc;
+  size_t lds = (size_t)(2 * nt * Ar + F_WAVES * Ar) * sizeof(real);
+  if (lds > 64 * 1024) return STAF_E_LIMIT;
+  const int atoms = nf * Nl;
+  hipLaunchKernelGGL(force2_kernel<real>, dim3((atoms + F_WAVES - 1) / F_WAVES), dim3(F_BLOCK), lds, stream, G, D, dD,
+                     im2, alpha2b, emb2b, type_map, (real*)fs.gslot, (real*)fs.self, fs.bcnt, fs.bent, fs.cap,
+                     st->status_d, nf, N, Nl, ld, nr, Ar, nt);
+  return launch_gather<real>(st, fs, tipos, actual_type, force, nf, N, Nl, nr, stream);
+}
+
+template <typename real>
+static size_t force3_lds(int nr, int na, int Aa, int nt) {
+  return chan_table_bytes<real>(2 * nt - 1, Aa) +
+         (size_t)(3 * na + nr + 3 * nr + Aa + F_PARTS * 3 * nr + 3 * nr) * sizeof(real) +
+         (size_t)(nr + NT_MAX + 1) * sizeof(int);
+}
+
+template <typename real>
+static int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* dDsup, const real* d3b,
+                       const int* im2, const int* im3, int nr, int na, int N, int nf, int Aa, const real* emb3b,
+                       int nt, const int* tipos, const int* actual_type, real* force, const int* numtriplet,
+                       const real* alpha3b, const int* type_map, int Nl, real* virial, const real* pos,
+                       const real* box, int ld, void* stream_) {
+  (void)im3;
+  if (!G || !Dsup || !Tang || !dDsup || !d3b || !im2 || !emb3b || !tipos || !actual_type || !force || !numtriplet ||
+      !alpha3b || !type_map || nr <= 0 || na <= 0 || N <= 0 || nf <= 0 || Aa <= 0 || nt <= 0 || Nl <= 0 || Nl > N)
+    return STAF_E_BAD_ARG;
+  if (virial || pos || box) return STAF_E_LIMIT;  // virial form: not built yet
+  if (nt > NT_MAX) return STAF_E_LIMIT;
+  if (ld <= 0) ld = Nl;
+  DeviceState* st = device_state();
+  if (!st) return STAF_E_HIP;
+  hipStream_t stream = (hipStream_t)stream_;
+  ForceScratch fs;
+  int rc = force_scratch<real>(st, nf, N, Nl, nr, stream, &fs);
+  if (rc) return rc;
+  size_t lds = force3_lds<real>(nr, na, Aa, nt);
+  if (lds > 64 * 1024) {
+    if (lds > 160 * 1024) return STAF_E_LIMIT;
+    if (hipFuncSetAttribute((const void*)force3_kernel<real>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
+        hipSuccess)
+      return STAF_E_LIMIT;
+  }
+  hipLaunchKernelGGL(force3_kernel<real>, dim3(nf * Nl), dim3(F_BLOCK), lds, stream, G, Dsup, Tang, dDsup, d3b, im2,
+                     alpha3b, emb3b, type_map, numtriplet, (real*)fs.gslot, (real*)fs.self, fs.bcnt, fs.bent, fs.cap,
+                     st->status_d, nf, N, Nl, ld, nr, na, Aa, nt);
+  return launch_gather<real>(st, fs, tipos, actual_type, force, nf, N, Nl, nr, stream);
+}
+
+template <typename real>
+static int gradforce_2b(const real* Q, const real* D, int nr, const real* alpha2b, int Ar, const real* dD,
+                        const int* im2, int nf, int N, int Nl, const real* G, const real* emb2b, int nt,
+                        const int* type_map, const int* tipos, const int* actual_type, real* gnet, real* g_alpha,
+                        real* g_emb, const real* Qvir, const real* pos, const real* box, int ld, void* stream_) {
+  if (!Q || !D || !alpha2b || !dD || !im2 || !G || !emb2b || !type_map || !tipos || !actual_type || !gnet ||
+      !g_alpha || !g_emb || nr <= 0 || Ar <= 0 || nf <= 0 || N <= 0 || Nl <= 0 || Nl > N || nt <= 0)
+    return STAF_E_BAD_ARG;
+  if (Qvir || pos || box) return STAF_E_LIMIT;  // virial form: not built yet
+  if (nt > NT_MAX) return STAF_E_LIMIT;
+  if (ld <= 0) ld = Nl;
+  DeviceState* st = device_state();
+  if (!st) return STAF_E_HIP;
+  hipStream_t stream = (hipStream_t)stream_;
+  const int nout = 2 * nt * Ar;
+  const int nb = grad_blocks_f(nf * Nl);
+  real* partial = (real*)scratch_reserve(st, (size_t)nb * nout * sizeof(real));
+  if (!partial) return STAF_E_HIP;
+  size_t lds = (size_t)(2 * nt * Ar + F_WAVES * nout + 2 * F_WAVES * nr) * sizeof(real) +
+               (size_t)F_WAVES * nr * sizeof(int);
+  if (lds > 64 * 1024) return STAF_E_LIMIT;
+  hipLaunchKernelGGL(gradforce2_kernel<real>, dim3(nb), dim3(F_BLOCK), lds, stream, Q, G, D, dD, im2, alpha2b, emb2b,
+                     type_map, tipos, actual_type, gnet, partial, nf, N, Nl, ld, nr, Ar, nt);
+  hipLaunchKernelGGL(reduce_partials_f_kernel<real>, dim3((nout + 127) / 128), dim3(128), 0, stream, partial, nb, nout,
+                     g_alpha, nt * Ar, g_emb, nt * Ar);
+  return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
+}
+
+template <typename real>
+static size_t gradforce3_lds(int nr, int Aa, int nt) {
+  const int nsig = 2 * nt - 1;
+  return chan_table_bytes<real>(nsig, Aa) +
+         (size_t)F_WAVES * (nsig * Aa * 3 + nr + nr + 3 * nr + Aa + Aa) * sizeof(real) +
+         (size_t)F_WAVES * (nr + NT_MAX + 1) * sizeof(int);
+}
+
+template <typename real>
+static int gradforce_tripl(const real* Q, const real* G, const real* Dsup, const real* Tang, const real* dDsup,
+                           const real* d3b, const int* im2, const int* im3, int nr, int na, int N, int nf, int Aa,
+                           const real* emb3b, int nt, const int* tipos, const int* actual_type, const int* numtriplet,
+                           const real* alpha3b, const int* type_map, int Nl, real* gnet, real* g_alpha, real* g_emb,
+                           const real* Qvir, const real* pos, const real* box, int ld, void* stream_) {
+  (void)im3;
+  if (!Q || !G || !Dsup || !Tang || !dDsup || !d3b || !im2 || !emb3b || !tipos || !actual_type || !numtriplet ||
+      !alpha3b || !type_map || !gnet || !g_alpha || !g_emb || nr <= 0 || na <= 0 || N <= 0 || nf <= 0 || Aa <= 0 ||
+      nt <= 0 || Nl <= 0 || Nl > N)
+    return STAF_E_BAD_ARG;
+  if (Qvir || pos || box) return STAF_E_LIMIT;  // virial form: not built yet
+  if (nt > NT_MAX) return STAF_E_LIMIT;
+  if (ld <= 0) ld = Nl;
+  DeviceState* st = device_state();
+  if (!st) return STAF_E_HIP;
+  hipStream_t stream = (hipStream_t)stream_;
+  const int ntc = nt * (nt + 1) / 2;
+  const int nsig = 2 * nt - 1;
+  const int nout = nsig * Aa * 3;
+  const int nb = grad_blocks_f(nf * Nl);
+  real* partial = (real*)scratch_reserve(st, (size_t)nb * nout * sizeof(real));
+  if (!partial) return STAF_E_HIP;
+  size_t lds = gradforce3_lds<real>(nr, Aa, nt);
+  if (lds > 64 * 1024) return STAF_E_LIMIT;
+  const int nall = ntc * Aa * 3;
+  if (nall > nout)
+    hipLaunchKernelGGL(fill_zero_f_kernel<real>, dim3((nall - nout + 127) / 128), dim3(128), 0, stream,
+                       g_alpha + nout, nall - nout);
+  hipLaunchKernelGGL(fill_zero_f_kernel<real>, dim3((ntc * Aa + 127) / 128), dim3(128), 0, stream, g_emb, ntc * Aa);
+  hipLaunchKernelGGL(gradforce3_kernel<real>, dim3(nb), dim3(F_BLOCK), lds, stream, Q, G, Dsup, Tang, dDsup, d3b, im2,
+                     alpha3b, emb3b, type_map, tipos, actual_type, numtriplet, gnet, partial, nf, N, Nl, ld, nr, na,
+                     Aa, nt);
+  hipLaunchKernelGGL(reduce_partials_f_kernel<real>, dim3((nout + 127) / 128), dim3(128), 0, stream, partial, nb, nout,
+                     g_alpha, nout, (real*)nullptr, 0);
+  return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
+}
+
+}  // namespace staf
+
+extern "C" {
+
+#define STAF_FORCE_ENTRY(real, SFX)                                                                                    \
+  int staf_op_force_doublets_##SFX(const real* netderiv, const real* des_r, const real* intderiv_r,                    \
+                                   const int* intmap_r, int nr, int N, int dimbat, int num_alpha_radiale,              \
+                                   const real* alpha_radiale, const real* type_emb2b, int nt, const int* tipos,        \
+                                   const int* actual_type, real* forces2b, const int* type_map, int N_local,           \
+                                   real* virial, const real* pos, const real* box, int ld_atoms, void* stream) {       \
+    return staf::force_doublets<real>(netderiv, des_r, intderiv_r, intmap_r, nr, N, dimbat, num_alpha_radiale,         \
+                                      alpha_radiale, type_emb2b, nt, tipos, actual_type, forces2b, type_map, N_local,  \
+                                      virial, pos, box, ld_atoms, stream);                                             \
+  }                                                                                                                    \
+  int staf_op_force_tripl_##SFX(const real* netderiv, const real* desr, const real* desa, const real* intderiv_r,      \
+                                const real* intderiv_a, const int* intmap_r, const int* intmap_a, int nr, int na,      \
+                                int N, int dimbat, int num_finger, const real* type_emb3b, int nt, const int* tipos,   \
+                                const int* actual_type, real* forces3b, const int* num_triplets, const real* smooth_a, \
+                                const int* type_map, int N_local, real* virial, const real* pos, const real* box,      \
+                                int ld_atoms, void* stream) {                                                          \
+    return staf::force_tripl<real>(netderiv, desr, desa, intderiv_r, intderiv_a, intmap_r, intmap_a, nr, na, N,        \
+                                   dimbat, num_finger, type_emb3b, nt, tipos, actual_type, forces3b, num_triplets,     \
+                                   smooth_a, type_map, N_local, virial, pos, box, ld_atoms, stream);                   \
+  }                                                                                                                    \
+  int staf_op_gradforce_2b_##SFX(const real* prevgrad, const real* radiale, int nr, const real* alpha_radiale,         \
+                                 int num_finger, const real* desder, const int* intmap_r, int dimbat, int N,           \
+                                 int N_local, const real* netderiv, const real* type_emb2b, int nt,                    \
+                                 const int* type_map, const int* tipos, const int* actual_type, real* grad_net,        \
+                                 real* grad_alpha2b, real* grad_emb2b, const real* prevgrad_virial, const real* pos,   \
+                                 const real* box, int ld_atoms, void* stream) {                                        \
+    return staf::gradforce_2b<real>(prevgrad, radiale, nr, alpha_radiale, num_finger, desder, intmap_r, dimbat, N,     \
+                                    N_local, netderiv, type_emb2b, nt, type_map, tipos, actual_type, grad_net,         \
+                                    grad_alpha2b, grad_emb2b, prevgrad_virial, pos, box, ld_atoms, stream);            \
+  }                                                                                                                    \
+  int staf_op_gradforce_tripl_##SFX(const real* prevgrad, const real* netderiv, const real* desr, const real* desa,    \
+                                    const real* intderiv_r, const real* intderiv_a, const int* intmap_r,               \
+                                    const int* intmap_a, int nr, int na, int N, int dimbat, int num_finger,            \
+                                    const real* type_emb3b, int nt, const int* tipos, const int* actual_type,          \
+                                    const int* num_triplets, const real* smooth_a, const int* type_map, int N_local,   \
+                                    real* gradnet_3b, real* grad_alpha3b, real* grad_emb3b,                            \
+                                    const real* prevgrad_virial, const real* pos, const real* box, int ld_atoms,       \
+                                    void* stream) {                                                                    \
+    return staf::gradforce_tripl<real>(prevgrad, netderiv, desr, desa, intderiv_r, intderiv_a, intmap_r, intmap_a, nr, \
+                                       na, N, dimbat, num_finger, type_emb3b, nt, tipos, actual_type, num_triplets,    \
+                                       smooth_a, type_map, N_local, gradnet_3b, grad_alpha3b, grad_emb3b,              \
+                                       prevgrad_virial, pos, box, ld_atoms, stream);                                   \
+  }
+
+STAF_FORCE_ENTRY(float, f32)
+STAF_FORCE_ENTRY(double, f64)
+
+}  // extern "C"

@@ -1,0 +1,129 @@
+// Library-owned per-device state: status word, scratch and scatter buckets.
+#include "staf_common.hpp"
+
+#include <mutex>
+#include <unordered_map>
+#include <memory>
+#include <stdio.h>
+
+namespace staf {
+
+static std::mutex g_mu;
+static std::unordered_map<int, std::unique_ptr<DeviceState>> g_state;
+static int g_sync_errors = 1;
+
+bool sync_errors_enabled() { return g_sync_errors != 0; }
+
+DeviceState* device_state() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+  std::lock_guard<std::mutex> lock(g_mu);
+  auto it = g_state.find(dev);
+  if (it != g_state.end()) return it->second.get();
+  auto st = std::unique_ptr<DeviceState>(new DeviceState());
+  st->device = dev;
+  if (hipMalloc((void**)&st->status_d, sizeof(int)) != hipSuccess) return nullptr;
+  if (hipMemset(st->status_d, 0, sizeof(int)) != hipSuccess) return nullptr;
+  if (hipHostMalloc((void**)&st->status_h, sizeof(int), hipHostMallocDefault) != hipSuccess) return nullptr;
+  *st->status_h = 0;
+  DeviceState* raw = st.get();
+  g_state.emplace(dev, std::move(st));
+  return raw;
+}
+
+void* scratch_reserve(DeviceState* st, size_t bytes) {
+  if (bytes <= st->scratch.bytes) return st->scratch.buf;
+  if (st->scratch.buf) {
+    // hipFree waits for in-flight work that may still read the old block
+    if (hipFree(st->scratch.buf) != hipSuccess) return nullptr;
+    st->scratch.buf = nullptr;
+    st->scratch.bytes = 0;
+  }
+  size_t want = bytes + bytes / 4;
+  if (hipMalloc(&st->scratch.buf, want) != hipSuccess) return nullptr;
+  st->scratch.bytes = want;
+  return st->scratch.buf;
+}
+
+// Scatter buckets: n_counters ints (kept all-zero between calls: the gather
+// kernel clears every counter it consumes) followed by n_entries ints.
+int* bucket_reserve(DeviceState* st, size_t n_counters, size_t n_entries, hipStream_t stream, int** entries) {
+  size_t need = (n_counters + n_entries) * sizeof(int);
+  if (need > st->buckets.bytes || n_counters > st->bucket_counters) {
+    if (st->buckets.buf) {
+      if (hipFree(st->buckets.buf) != hipSuccess) return nullptr;
+      st->buckets.buf = nullptr;
+      st->buckets.bytes = 0;
+    }
+    size_t cnt = n_counters + n_counters / 4;
+    size_t ent = n_entries + n_entries / 4;
+    size_t want = (cnt + ent) * sizeof(int);
+    if (hipMalloc(&st->buckets.buf, want) != hipSuccess) return nullptr;
+    if (hipMemset(st->buckets.buf, 0, cnt * sizeof(int)) != hipSuccess) return nullptr;
+    st->buckets.bytes = want;
+    st->bucket_counters = cnt;
+  }
+  (void)stream;
+  *entries = (int*)st->buckets.buf + st->bucket_counters;
+  return (int*)st->buckets.buf;
+}
+
+static int decode_status(int bits) {
+  if (bits & 1) return STAF_E_RADIAL_OVERFLOW;
+  if (bits & 2) return STAF_E_SCATTER_OVERFLOW;
+  return STAF_OK;
+}
+
+static int fetch_status(DeviceState* st, hipStream_t stream) {
+  if (hipMemcpyAsync(st->status_h, st->status_d, sizeof(int), hipMemcpyDeviceToHost, stream) != hipSuccess)
+    return STAF_E_HIP;
+  if (hipStreamSynchronize(stream) != hipSuccess) return STAF_E_HIP;
+  int bits = *st->status_h;
+  if (bits) {
+    if (hipMemsetAsync(st->status_d, 0, sizeof(int), stream) != hipSuccess) return STAF_E_HIP;
+    if (hipStreamSynchronize(stream) != hipSuccess) return STAF_E_HIP;
+  }
+  return decode_status(bits);
+}
+
+int finish_op(DeviceState* st, hipStream_t stream) {
+  if (hipGetLastError() != hipSuccess) return STAF_E_HIP;
+  if (!g_sync_errors) return STAF_OK;
+  return fetch_status(st, stream);
+}
+
+}  // namespace staf
+
+extern "C" {
+
+const char* staf_ops_version(void) { return "0.1"; }
+
+void staf_ops_set_sync_errors(int mode) { staf::g_sync_errors = mode ? 1 : 0; }
+
+int staf_ops_poll_status(void* stream) {
+  staf::DeviceState* st = staf::device_state();
+  if (!st) return STAF_E_HIP;
+  return staf::fetch_status(st, (hipStream_t)stream);
+}
+
+void staf_ops_release(void) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return;
+  std::lock_guard<std::mutex> lock(staf::g_mu);
+  auto it = staf::g_state.find(dev);
+  if (it == staf::g_state.end()) return;
+  staf::DeviceState* st = it->second.get();
+  (void)hipDeviceSynchronize();
+  if (st->scratch.buf) (void)hipFree(st->scratch.buf);
+  if (st->buckets.buf) (void)hipFree(st->buckets.buf);
+  if (st->status_d) (void)hipFree(st->status_d);
+  if (st->status_h) (void)hipHostFree(st->status_h);
+  staf::g_state.erase(it);
+}
+
+int staf_op_init_force_radial(int buffdim) { return buffdim > 0 ? STAF_OK : STAF_E_BAD_ARG; }
+int staf_op_init_force_tripl(int buffdim) { return buffdim > 0 ? STAF_OK : STAF_E_BAD_ARG; }
+int staf_op_init_grad_force_radial(int buffdim) { return buffdim > 0 ? STAF_OK : STAF_E_BAD_ARG; }
+int staf_op_init_grad_force_tripl(int buffdim) { return buffdim > 0 ? STAF_OK : STAF_E_BAD_ARG; }
+
+}  // extern "C"

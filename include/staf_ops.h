@@ -1,0 +1,243 @@
+/* staf_ops.h -- C ABI of libstaf_hip.so: the STAF fingerprint hot path on MI355X (gfx950).
+ *
+ * One entry point per launcher the reference's TensorFlow op shells call
+ * (device pointers + integer dims + one stream).  Each entry point exists
+ * twice, suffixed _f32 and _f64 (the reference builds one .so per precision
+ * with -DSTAF_REAL_DOUBLE); `real` below stands for float / double.
+ *
+ * Conventions
+ *   - all tensor pointers are DEVICE pointers, row-major, caller-owned;
+ *     outputs are pre-allocated by the caller and fully written by the call
+ *     (no pre-zeroing needed), except where a note says "padding".
+ *   - `stream` is a hipStream_t passed as void* (NULL = default stream).
+ *   - return value: 0 on success, a negative STAF_E_* code otherwise.  No
+ *     entry point ever calls exit().
+ *   - per-species ops take tensors sliced to one centre species, [nf, Nl, ...].
+ *     `ld_atoms` is the distance, in atoms, between consecutive frames of the
+ *     descriptor-derived tensors of the call (raddescr, des3bsupp, angdescr,
+ *     der2b, der3bsupp, der3b, intmap2b, intmap3b, numtriplet): Nl (or 0) for
+ *     the contiguous tensors tf.split produces, N when the pointers are views
+ *     into the descriptor op's [nf, N, ...] outputs (pointer pre-offset to the
+ *     species' first atom).  Channel-width tensors (fingerprints, netderiv,
+ *     prevgrad of the fingerprint ops, gradnet outputs) are always contiguous
+ *     [nf, Nl, channels].
+ *   - type_map [N] int32 species of every atom of a frame; tipos [nt] int32
+ *     atoms per species; actual_type [1] int32 centre species -- device
+ *     pointers, as the reference ops receive them.
+ *   - type-embedding arguments are the SQUARED embeddings (the reference's
+ *     Python layers square them before the op call).
+ *   - state is per device and not re-entrant: calls on one device must be
+ *     ordered on one stream at a time.
+ */
+#ifndef STAF_OPS_H
+#define STAF_OPS_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define STAF_OK 0
+#define STAF_E_NOT_CONSTRUCTED (-1)  /* compute before construct (reference: exit(1), reforce.cc:145-148) */
+#define STAF_E_BAD_ARG (-2)          /* null pointer / non-positive dimension / dims beyond the constructed maxima */
+#define STAF_E_HIP (-3)              /* a HIP runtime call failed */
+#define STAF_E_RADIAL_OVERFLOW (-10) /* an atom has more than radial_buffer neighbours (reference: exit(0), reforce.cc:329-337) */
+#define STAF_E_SCATTER_OVERFLOW (-11)/* an atom is listed by more centres than the force scatter can hold (4*nr) */
+#define STAF_E_LIMIT (-12)           /* nt, channels or buffers beyond the kernels' compile-time limits */
+
+/* ---- library state ------------------------------------------------------ */
+
+/* Version string "major.minor". */
+const char* staf_ops_version(void);
+
+/* Error reporting of conditions only the GPU can detect (neighbour-buffer overflow,
+ * scatter overflow).  mode 1 (default, reference behaviour): the call that can hit
+ * the condition synchronises its stream and returns the code.  mode 0: nothing
+ * synchronises; conditions accumulate in a device word read by staf_ops_poll_status. */
+void staf_ops_set_sync_errors(int mode);
+
+/* Synchronises `stream`, returns the accumulated device-side status (0 or a
+ * negative STAF_E_* code) and clears it. */
+int staf_ops_poll_status(void* stream);
+
+/* Frees all device memory the library holds on the current device. */
+void staf_ops_release(void);
+
+/* ---- descriptor op ------------------------------------------------------ */
+
+/* ConstructDescriptorsLight -- STAF/src/descriptor_builder/reforce.cc:182-238 (+ fill_repulsion :101-141).
+ * Stores the geometry for all later compute calls and derives the short-range coefficients.
+ * cutoff_curve_path: where to write the 1000-row "%g %g" curve the reference writes to
+ * ./cutoff_curve.dat; NULL skips the file. */
+int staf_op_construct_descriptors_light_f32(float radial_cutoff, int radial_buffer, int angular_buffer, int numpar,
+                                            float rs, float ra, int max_batch, const char* cutoff_curve_path);
+int staf_op_construct_descriptors_light_f64(double radial_cutoff, int radial_buffer, int angular_buffer, int numpar,
+                                            double rs, double ra, int max_batch, const char* cutoff_curve_path);
+
+/* Options of the descriptor op (apply to both precisions; call after construct).
+ *   dist2_fma     0: dist2 = (x*x+y*y)+z*z uncontracted (default); 1: fma(z,z,fma(y,y,x*x))
+ *   zero_padding  0: padded slots of der3b are left untouched like the reference (default);
+ *                 1: they are written as 0.  (All other outputs are always fully written.) */
+int staf_op_descriptor_options(int dist2_fma, int zero_padding);
+
+/* Reads back {A, B, C, pow_alpha, pow_beta} computed by construct. */
+int staf_op_descriptor_coefficients_f32(float* out5);
+int staf_op_descriptor_coefficients_f64(double* out5);
+
+/* ComputeDescriptorsLight -- STAF/src/descriptor_builder/reforce.cc:241-444, kernels
+ * celle_gpu.cu.cc:11-201 (cart->frac, cell list, neighbour search, sort) and
+ * reforce.cu.cc:17-236 (radial + angular fill).
+ *   positions [nf, 3N] Cartesian, boxer [nf, 6] = [Lx, xy, xz, Ly, yz, Lz]
+ *   raddescr [nf,N,nr]  angdescr [nf,N,na]  des3bsupp [nf,N,nr]  intmap2b [nf,N,nr+1]
+ *   intmap3b [nf,N,2*na]  der2b [nf,N,3,nr]  der3b [nf,N,3,2*na]  der3bsupp [nf,N,3,nr]  numtriplet [nf,N]
+ * Padded slots are written as 0 (der3b: see staf_op_descriptor_options). */
+int staf_op_compute_descriptors_light_f32(const float* positions, const float* boxer, int nf, int N, float* raddescr,
+                                          float* angdescr, float* des3bsupp, int* intmap2b, int* intmap3b,
+                                          float* der2b, float* der3b, float* der3bsupp, int* numtriplet,
+                                          void* stream);
+int staf_op_compute_descriptors_light_f64(const double* positions, const double* boxer, int nf, int N,
+                                          double* raddescr, double* angdescr, double* des3bsupp, int* intmap2b,
+                                          int* intmap3b, double* der2b, double* der3b, double* der3bsupp,
+                                          int* numtriplet, void* stream);
+
+/* ---- atomic fingerprints (forward) -------------------------------------- */
+
+/* radialAFs_Launcher (ComputeSortProj) -- STAF/src/fingerprint/rad/reforce.cc:13-24, reforce.cu.cc:12-64.
+ *   radial_AFs [nf,Nl,nalpha_r] = sum_k D_k exp(alpha2b[t_k,a] D_k) emb2b[t_k,a];  alpha2b, emb2b [nt,nalpha_r] */
+int staf_op_radial_afs_f32(const float* radial_descriptor, int nr, const float* alpha2b, int nalpha_r,
+                           float* radial_AFs, int dimbat, int N_local, const int* interaction_map_rad,
+                           const float* type_emb2b, const int* type_map, int nt, int ld_atoms, void* stream);
+int staf_op_radial_afs_f64(const double* radial_descriptor, int nr, const double* alpha2b, int nalpha_r,
+                           double* radial_AFs, int dimbat, int N_local, const int* interaction_map_rad,
+                           const double* type_emb2b, const int* type_map, int nt, int ld_atoms, void* stream);
+
+/* angularAFs_Launcher (ComputeSortProj3body) -- STAF/src/fingerprint/ang/reforce.cc:15-30, reforce.cu.cc:13-86.
+ *   radial_descriptor = des3bsupp [nf,Nl,nr]; angular_descriptor [nf,Nl,na]; alpha3b [ntc,3*nsmooth_a]
+ *   (alpha1,alpha2,beta per channel), type_emb3b [ntc,nsmooth_a]; row = t_j + t_k.
+ *   interaction_map_rad [nf,Nl,nr+1] supplies the neighbour species; interaction_map_angular must be the
+ *   one the descriptor op produced with it (it is not re-read). */
+int staf_op_angular_afs_f32(const float* radial_descriptor, const float* angular_descriptor, int nr, int na,
+                            float* three_body_AFs, int dimbat, int N_local, const int* interaction_map_angular,
+                            const int* interaction_map_rad, const float* alpha3b, int nsmooth_a,
+                            const float* type_emb3b, const int* type_map, const int* num_triplets, int nt,
+                            int ld_atoms, void* stream);
+int staf_op_angular_afs_f64(const double* radial_descriptor, const double* angular_descriptor, int nr, int na,
+                            double* three_body_AFs, int dimbat, int N_local, const int* interaction_map_angular,
+                            const int* interaction_map_rad, const double* alpha3b, int nsmooth_a,
+                            const double* type_emb3b, const int* type_map, const int* num_triplets, int nt,
+                            int ld_atoms, void* stream);
+
+/* ---- forces -------------------------------------------------------------- */
+
+/* init_block_dim (InitForceRadial / InitForceTripl / InitGradForceRadial / InitGradForceTripl) --
+ * STAF/src/force/rad/reforce.cc:13-36, force/ang/reforce.cc:14-37, grad_force/rad/reforce.cc:15-38,
+ * grad_force/ang/reforce.cc:14-37.  The reference picks a CUDA block size dividing the buffer; these
+ * kernels need none, so the calls only validate the argument and return the op's output code [0]. */
+int staf_op_init_force_radial(int buffdim);
+int staf_op_init_force_tripl(int buffdim);
+int staf_op_init_grad_force_radial(int buffdim);
+int staf_op_init_grad_force_tripl(int buffdim);
+
+/* computeforce_doublets_Launcher (ComputeForceRadial) -- STAF/src/force/rad/reforce.cc:39-57, reforce.cu.cc:45-172
+ * and computeforce_doublets_virial_Launcher (ComputeForceRadialVirial) -- reforce.cc:124-146, reforce.cu.cc:174-314.
+ *   forces2b [nf,3N] (all atoms; fully written).  virial [nf,9] row-major W_ab -= g_a r_b, pos [nf,3N]
+ *   Cartesian, box [nf,6]; pass virial = pos = box = NULL for the plain op.
+ * Deterministic: per-slot pair forces are reduced by an owner-computes gather, no float atomics. */
+int staf_op_force_doublets_f32(const float* netderiv, const float* des_r, const float* intderiv_r,
+                               const int* intmap_r, int nr, int N, int dimbat, int num_alpha_radiale,
+                               const float* alpha_radiale, const float* type_emb2b, int nt, const int* tipos,
+                               const int* actual_type, float* forces2b, const int* type_map, int N_local,
+                               float* virial, const float* pos, const float* box, int ld_atoms, void* stream);
+int staf_op_force_doublets_f64(const double* netderiv, const double* des_r, const double* intderiv_r,
+                               const int* intmap_r, int nr, int N, int dimbat, int num_alpha_radiale,
+                               const double* alpha_radiale, const double* type_emb2b, int nt, const int* tipos,
+                               const int* actual_type, double* forces2b, const int* type_map, int N_local,
+                               double* virial, const double* pos, const double* box, int ld_atoms, void* stream);
+
+/* computeforce_tripl_Launcher (ComputeForceTripl) -- STAF/src/force/ang/reforce.cc:44-66, reforce.cu.cc:48-248
+ * and computeforce_tripl_virial_Launcher (ComputeForceTriplVirial) -- reforce.cc:151-176, reforce.cu.cc:269-482.
+ *   desr = des3bsupp, desa = angdescr, intderiv_r = der3bsupp, intderiv_a = der3b. */
+int staf_op_force_tripl_f32(const float* netderiv, const float* desr, const float* desa, const float* intderiv_r,
+                            const float* intderiv_a, const int* intmap_r, const int* intmap_a, int nr, int na, int N,
+                            int dimbat, int num_finger, const float* type_emb3b, int nt, const int* tipos,
+                            const int* actual_type, float* forces3b, const int* num_triplets, const float* smooth_a,
+                            const int* type_map, int N_local, float* virial, const float* pos, const float* box,
+                            int ld_atoms, void* stream);
+int staf_op_force_tripl_f64(const double* netderiv, const double* desr, const double* desa,
+                            const double* intderiv_r, const double* intderiv_a, const int* intmap_r,
+                            const int* intmap_a, int nr, int na, int N, int dimbat, int num_finger,
+                            const double* type_emb3b, int nt, const int* tipos, const int* actual_type,
+                            double* forces3b, const int* num_triplets, const double* smooth_a, const int* type_map,
+                            int N_local, double* virial, const double* pos, const double* box, int ld_atoms,
+                            void* stream);
+
+/* ---- parameter gradients from the energy branch ------------------------- */
+
+/* alpha_dist_grad_Launcher (ComputeTwoBodyParGrad) -- STAF/src/grad_finger/rad/reforce.cc:14-29, reforce.cu.cc:12-66.
+ *   prevgrad [nf,Nl,nalpha_r] = dL/dAF2 -> nextgrad_alpha2b, nextgrad_emb2b [nt,nalpha_r] */
+int staf_op_alpha_dist_grad_f32(const float* radial_descriptor, int nr, const float* alpha2b, int nalpha_r,
+                                float* nextgrad_alpha2b, int dimbat, int N_local, const int* interaction_map_rad,
+                                const float* prevgrad, const float* type_emb2b, const int* type_map,
+                                float* nextgrad_emb2b, int nt, int ld_atoms, void* stream);
+int staf_op_alpha_dist_grad_f64(const double* radial_descriptor, int nr, const double* alpha2b, int nalpha_r,
+                                double* nextgrad_alpha2b, int dimbat, int N_local, const int* interaction_map_rad,
+                                const double* prevgrad, const double* type_emb2b, const int* type_map,
+                                double* nextgrad_emb2b, int nt, int ld_atoms, void* stream);
+
+/* alphagrad_ang_Launcher (ComputeSortProj3bodyGrad) -- STAF/src/grad_finger/ang/reforce.cc:12-31, reforce.cu.cc:13-133.
+ *   prevgrad [nf,Nl,nsmooth_a] = dL/dAF3 -> next_alpha3b_grad [nt_couple,3*nsmooth_a],
+ *   next_emb3b_grad [nt_couple,nsmooth_a] (identically zero, as in the reference). */
+int staf_op_alphagrad_ang_f32(const float* radial_descriptor, const float* angular_descriptor, int nr, int na,
+                              const float* prevgrad, int dimbat, int N_local, const int* intmap3b,
+                              const int* intmap2b, const float* alpha3b, int nsmooth_a, float* next_alpha3b_grad,
+                              const float* type_emb3b, const int* type_map, float* next_emb3b_grad,
+                              const int* num_triplets, int nt_couple, int nt, int ld_atoms, void* stream);
+int staf_op_alphagrad_ang_f64(const double* radial_descriptor, const double* angular_descriptor, int nr, int na,
+                              const double* prevgrad, int dimbat, int N_local, const int* intmap3b,
+                              const int* intmap2b, const double* alpha3b, int nsmooth_a, double* next_alpha3b_grad,
+                              const double* type_emb3b, const int* type_map, double* next_emb3b_grad,
+                              const int* num_triplets, int nt_couple, int nt, int ld_atoms, void* stream);
+
+/* ---- gradients of the force ops ----------------------------------------- */
+
+/* back_prop_grad_force2b_Launcher (ComputeForceRadialGrad) -- STAF/src/grad_force/rad/reforce.cc:42-63,
+ * reforce.cu.cc:46-147, and back_prop_grad_force2b_virial_Launcher (ComputeForceRadialVirialGrad) --
+ * reforce.cc:149-176, reforce.cu.cc:165-261.
+ *   prevgrad [nf,3N] = dL/dF -> grad_net [nf,Nl,num_finger], grad_alpha2b, grad_emb2b [nt,num_finger].
+ *   prevgrad_virial [nf,9] = dL/dW with pos, box for the virial form; NULL for the plain op. */
+int staf_op_gradforce_2b_f32(const float* prevgrad, const float* radiale, int nr, const float* alpha_radiale,
+                             int num_finger, const float* desder, const int* intmap_r, int dimbat, int N,
+                             int N_local, const float* netderiv, const float* type_emb2b, int nt,
+                             const int* type_map, const int* tipos, const int* actual_type, float* grad_net,
+                             float* grad_alpha2b, float* grad_emb2b, const float* prevgrad_virial, const float* pos,
+                             const float* box, int ld_atoms, void* stream);
+int staf_op_gradforce_2b_f64(const double* prevgrad, const double* radiale, int nr, const double* alpha_radiale,
+                             int num_finger, const double* desder, const int* intmap_r, int dimbat, int N,
+                             int N_local, const double* netderiv, const double* type_emb2b, int nt,
+                             const int* type_map, const int* tipos, const int* actual_type, double* grad_net,
+                             double* grad_alpha2b, double* grad_emb2b, const double* prevgrad_virial,
+                             const double* pos, const double* box, int ld_atoms, void* stream);
+
+/* gradforce_tripl_Launcher (ComputeForceTriplGrad) -- STAF/src/grad_force/ang/reforce.cc:39-66, reforce.cu.cc:47-254,
+ * and gradforce_tripl_virial_Launcher (ComputeForceTriplVirialGrad) -- reforce.cc:172-206, reforce.cu.cc:274-477.
+ *   -> gradnet_3b [nf,Nl,num_finger], grad_alpha3b [ntc,3*num_finger], grad_emb3b [ntc,num_finger] (zero). */
+int staf_op_gradforce_tripl_f32(const float* prevgrad, const float* netderiv, const float* desr, const float* desa,
+                                const float* intderiv_r, const float* intderiv_a, const int* intmap_r,
+                                const int* intmap_a, int nr, int na, int N, int dimbat, int num_finger,
+                                const float* type_emb3b, int nt, const int* tipos, const int* actual_type,
+                                const int* num_triplets, const float* smooth_a, const int* type_map, int N_local,
+                                float* gradnet_3b, float* grad_alpha3b, float* grad_emb3b,
+                                const float* prevgrad_virial, const float* pos, const float* box, int ld_atoms,
+                                void* stream);
+int staf_op_gradforce_tripl_f64(const double* prevgrad, const double* netderiv, const double* desr,
+                                const double* desa, const double* intderiv_r, const double* intderiv_a,
+                                const int* intmap_r, const int* intmap_a, int nr, int na, int N, int dimbat,
+                                int num_finger, const double* type_emb3b, int nt, const int* tipos,
+                                const int* actual_type, const int* num_triplets, const double* smooth_a,
+                                const int* type_map, int N_local, double* gradnet_3b, double* grad_alpha3b,
+                                double* grad_emb3b, const double* prevgrad_virial, const double* pos,
+                                const double* box, int ld_atoms, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* STAF_OPS_H */
