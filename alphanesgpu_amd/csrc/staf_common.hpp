@@ -84,7 +84,8 @@ struct DeviceState {
   int* status_h = nullptr;   // pinned host mirror
   Workspace scratch;         // per-slot partial forces / partial sums
   Workspace buckets;         // transpose buckets (counters + entries), kept zeroed between calls
-  size_t bucket_counters = 0;
+  size_t bucket_counters = 0;    // capacity, in ints, of the counter part
+  size_t bucket_entries = 0;     // capacity, in ints, of the entry part
 };
 
 DeviceState* device_state();                                   // for the current device, created on demand

@@ -48,8 +48,7 @@ void* scratch_reserve(DeviceState* st, size_t bytes) {
 // Scatter buckets: n_counters ints (kept all-zero between calls: the gather
 // kernel clears every counter it consumes) followed by n_entries ints.
 int* bucket_reserve(DeviceState* st, size_t n_counters, size_t n_entries, hipStream_t stream, int** entries) {
-  size_t need = (n_counters + n_entries) * sizeof(int);
-  if (need > st->buckets.bytes || n_counters > st->bucket_counters) {
+  if (n_counters > st->bucket_counters || n_entries > st->bucket_entries) {
     if (st->buckets.buf) {
       if (hipFree(st->buckets.buf) != hipSuccess) return nullptr;
       st->buckets.buf = nullptr;
@@ -62,6 +61,7 @@ int* bucket_reserve(DeviceState* st, size_t n_counters, size_t n_entries, hipStr
     if (hipMemset(st->buckets.buf, 0, cnt * sizeof(int)) != hipSuccess) return nullptr;
     st->buckets.bytes = want;
     st->bucket_counters = cnt;
+    st->bucket_entries = ent;
   }
   (void)stream;
   *entries = (int*)st->buckets.buf + st->bucket_counters;

@@ -28,14 +28,12 @@ struct ChanTable {
   int* ch;    // [nsig*Aa] channel id of the compacted entry
   int* nact;  // [nsig]
   int Aa, nsig;
-  __device__ static size_t bytes(int nsig, int Aa) {
-    return (size_t)nsig * Aa * (4 * sizeof(real) + sizeof(int)) + (size_t)nsig * sizeof(int);
-  }
   __device__ unsigned char* carve(unsigned char* p, int nsig_, int Aa_) {
     Aa = Aa_; nsig = nsig_;
     a1 = (real*)p; a2 = a1 + nsig * Aa; be = a2 + nsig * Aa; c3 = be + nsig * Aa;
     ch = (int*)(c3 + nsig * Aa); nact = ch + nsig * Aa;
-    return (unsigned char*)(nact + nsig);
+    // the next carve-out may hold doubles: keep 16-byte alignment
+    return p + ((((size_t)nsig * Aa * (4 * sizeof(real) + sizeof(int)) + (size_t)nsig * sizeof(int)) + 15) & ~(size_t)15);
   }
   // alpha3b [ntc, 3*Aa] as (alpha1, alpha2, beta) per channel, emb3b [ntc, Aa].
   // Waves of the block split the rows; a __syncthreads() must follow.
@@ -68,7 +66,7 @@ struct ChanTable {
 
 template <typename real>
 __host__ __device__ inline size_t chan_table_bytes(int nsig, int Aa) {
-  return (size_t)nsig * Aa * (4 * sizeof(real) + sizeof(int)) + (size_t)nsig * sizeof(int);
+  return (((size_t)nsig * Aa * (4 * sizeof(real) + sizeof(int)) + (size_t)nsig * sizeof(int)) + 15) & ~(size_t)15;
 }
 
 // Slots of one centre grouped by neighbour species (ascending slot inside a

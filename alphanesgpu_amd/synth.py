@@ -34,8 +34,10 @@ def _rot(q):
                      [2 * (x * z - y * w), 2 * (y * z + x * w), 1 - 2 * (x * x + y * y)]])
 
 
-def water_frame(lattice, L, sigma, seed, jitter=0.3):
-    """One frame: -> pos [3N] (all O then all H, unwrapped, centred on 0), box6."""
+def water_frame(lattice, L, sigma, seed, jitter=0.5):
+    """One frame: -> pos [3N] (all O then all H, unwrapped, centred on 0), box6.
+    Molecule centres are stratified: one per lattice cell, uniform inside `jitter` x the cell edge around
+    the cell centre (0.5 = anywhere in its own cell), which gives the ~38 neighbours within 4.5 A of liquid water."""
     rng = _rng(seed)
     nx, ny, nz = lattice
     nmol = nx * ny * nz
@@ -49,7 +51,7 @@ def water_frame(lattice, L, sigma, seed, jitter=0.3):
     for iz in range(nz):
         for iy in range(ny):
             for ix in range(nx):
-                c = (np.array([ix, iy, iz]) + 0.5) * sp + rng.uniform(-jitter, jitter, 3)
+                c = (np.array([ix, iy, iz]) + 0.5) * sp + rng.uniform(-jitter, jitter, 3) * sp
                 for _ in range(200):
                     q = rng.standard_normal(4)
                     q /= np.linalg.norm(q)
