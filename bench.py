@@ -1,0 +1,254 @@
+#!/usr/bin/env python3
+"""Benchmark of the STAF fingerprint hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload water768_f32] [--mode fwd_force|full_step]
+
+One step = one pass of the op sequence over one synthetic batch that is already resident in HBM:
+descriptor op (neighbour list + radial/angular descriptors), then per centre species the 2-body and
+3-body fingerprint ops and the 2-body and 3-body force ops (mode fwd_force); mode full_step adds the four
+parameter-gradient ops (dL/dalpha from the energy branch and from the force branch).  Upstream gradients
+(dE/dAF, dL/dAF, dL/dF) are fixed synthetic tensors: the per-species MLP is not part of this path.
+
+Prints ONE JSON line (metric, value = frames/s, roofline of the dominant kernel, CPU baseline).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+def algorithmic_bytes(N, tipos, nr, na, Ar, Aa, nt, s):
+    """Bytes each op's signature forces through HBM once per frame (inputs read once, outputs written once),
+    per-species calls summed."""
+    ntc = nt * (nt + 1) // 2
+    desc = (N * (8 * nr + 7 * na)) * s + N * (nr + 1 + 2 * na + 1) * 4 + (3 * N + 6) * s
+    af = force = galpha = gforce = 0
+    for Nl in tipos:
+        par2 = 2 * nt * Ar * s
+        par3 = (3 * ntc * Aa + ntc * Aa) * s
+        tm = N * 4
+        af += Nl * nr * s + Nl * (nr + 1) * 4 + par2 + tm + Nl * Ar * s                       # ComputeSortProj
+        af += Nl * (na + nr) * s + Nl * (2 * na + nr + 1 + 1) * 4 + par3 + tm + Nl * Aa * s     # ComputeSortProj3body
+        force += Nl * (Ar + nr + 3 * nr) * s + Nl * (nr + 1) * 4 + par2 + tm + 3 * N * s        # ComputeForceRadial
+        force += (Nl * (Aa + nr + na + 3 * nr + 6 * na) * s + Nl * (nr + 1 + 2 * na + 1) * 4 + par3 + tm
+                  + 3 * N * s)                                                                  # ComputeForceTripl
+        galpha += Nl * (Ar + nr) * s + Nl * (nr + 1) * 4 + par2 + tm + 2 * nt * Ar * s          # ComputeTwoBodyParGrad
+        galpha += (Nl * (Aa + na + nr) * s + Nl * (2 * na + nr + 1 + 1) * 4 + par3 + tm
+                   + (3 * ntc * Aa + ntc * Aa) * s)                                             # ...3bodyGrad
+        gforce += (3 * N * s + Nl * (Ar + nr + 3 * nr) * s + Nl * (nr + 1) * 4 + par2 + tm
+                   + Nl * Ar * s + 2 * nt * Ar * s)                                             # ComputeForceRadialGrad
+        gforce += (3 * N * s + Nl * (Aa + nr + na + 3 * nr + 6 * na) * s + Nl * (nr + 1 + 2 * na + 1) * 4 + par3
+                   + tm + Nl * Aa * s + (3 * ntc * Aa + ntc * Aa) * s)                          # ComputeForceTriplGrad
+    return dict(descriptor=desc, af_fwd=af, force=force, grad_alpha=galpha, grad_force=gforce)
+
+
+def cpu_baseline(batch, params, up, mode, nr, na, max_frames=2):
+    """Times the CPU oracle (single thread) on the first frames of the same batch."""
+    from oracle import staf_oracle as O
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    nfs = min(max_frames, batch["nf"])
+    dt = batch["dtype"]
+    pos, box = batch["pos"][:nfs], batch["box"][:nfs]
+    tipos, type_map = batch["tipos"], batch["type_map"]
+    t0 = time.perf_counter()
+    d = O.compute_descriptors_light(pos, box, 4.5, 4.5, 2.25, nr, na, dtype=dt)
+    o = 0
+    for k, n in enumerate(tipos):
+        s = slice(o, o + int(n))
+        o += int(n)
+        m = params[k]
+        c = lambda a: np.ascontiguousarray(a[:, s])
+        O.radial_afs(c(d["raddescr"]), c(d["intmap2b"]), m["alpha2b"], m["emb2b"], type_map)
+        O.angular_afs(c(d["angdescr"]), c(d["des3bsupp"]), c(d["intmap3b"]), m["alpha3b"], m["emb3b"], type_map,
+                      c(d["numtriplet"]))
+        O.force_radial(up["G2"][k][:nfs], c(d["der2b"]), c(d["intmap2b"]), c(d["raddescr"]), m["alpha2b"], m["emb2b"],
+                       type_map, tipos, k)
+        O.force_tripl(up["G3"][k][:nfs], c(d["des3bsupp"]), c(d["angdescr"]), c(d["der3bsupp"]), c(d["der3b"]),
+                      c(d["intmap2b"]), c(d["intmap3b"]), m["alpha3b"], m["emb3b"], type_map, tipos, k,
+                      c(d["numtriplet"]))
+        if mode == "full_step":
+            O.two_body_par_grad(up["P2"][k][:nfs], c(d["raddescr"]), c(d["intmap2b"]), m["alpha2b"], m["emb2b"],
+                                type_map)
+            O.sort_proj3body_grad(up["P3"][k][:nfs], c(d["angdescr"]), c(d["des3bsupp"]), c(d["intmap3b"]),
+                                  c(d["intmap2b"]), m["alpha3b"], m["emb3b"], type_map, c(d["numtriplet"]))
+            O.force_radial_grad(up["Q"][:nfs], up["G2"][k][:nfs], c(d["der2b"]), c(d["intmap2b"]), c(d["raddescr"]),
+                                m["alpha2b"], m["emb2b"], type_map, tipos, k)
+            O.force_tripl_grad(up["Q"][:nfs], up["G3"][k][:nfs], c(d["des3bsupp"]), c(d["angdescr"]),
+                               c(d["der3bsupp"]), c(d["der3b"]), c(d["intmap2b"]), c(d["intmap3b"]), m["alpha3b"],
+                               m["emb3b"], type_map, tipos, k, c(d["numtriplet"]))
+    el = time.perf_counter() - t0
+    return dict(value=nfs / el, unit="frames/s", cores=1, kind="port",
+                sample=f"{nfs} frame(s) of the same batch, same ops, scalar C++ oracle (-O2 -ffp-contract=off), 1 thread")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="water768_f32")
+    ap.add_argument("--mode", default=None, choices=[None, "fwd_force", "full_step"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--contiguous-splits", action="store_true",
+                    help="copy per-species tensors like tf.split instead of passing views")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (frames are independent; see DESIGN.md for sharding); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from alphanesgpu_amd import ops, synth
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import pipeline
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    batch = synth.water_batch(args.workload)
+    mode = args.mode or ("fwd_force" if args.workload in ("water768_f32", "water6144") else "full_step")
+    dtype = batch["dtype"]
+    tdt = torch.float32 if dtype == np.float32 else torch.float64
+    nr, na = synth.NR, synth.NA
+    nf, N = batch["nf"], batch["N"]
+    tipos = [int(x) for x in batch["tipos"]]
+    nt = len(tipos)
+    params = synth.fingerprint_params(dtype=dtype)
+    Ar, Aa = params[0]["alpha2b"].shape[1], params[0]["alpha3b"].shape[1] // 3
+    up = pipeline.synthetic_upstream(nf, batch["tipos"], params, 11, dtype)
+
+    T = lambda a: torch.as_tensor(np.ascontiguousarray(a)).to(dev)
+    pos, box = T(batch["pos"]), T(batch["box"])
+    tm, tp = T(batch["type_map"]), T(batch["tipos"])
+    P = [{k: T(v) for k, v in m.items()} for m in params]
+    G2, G3 = [T(x) for x in up["G2"]], [T(x) for x in up["G3"]]
+    P2, P3 = [T(x) for x in up["P2"]], [T(x) for x in up["P3"]]
+    Q = T(up["Q"])
+    at = [torch.tensor([k], dtype=torch.int32, device=dev) for k in range(nt)]
+    ops.construct_descriptors_light(synth.RC, nr, na, N, box, synth.RS, synth.RA, nf, dtype=tdt)
+    ops.descriptor_options(dist2_fma=False, zero_padding=False)
+    for f, b in ((ops.init_force_radial, nr), (ops.init_force_tripl, na), (ops.init_grad_force_radial, nr),
+                 (ops.init_grad_force_tripl, na)):
+        f(b)
+    ops.set_sync_errors(False)
+    e = lambda *sh: torch.empty(sh, dtype=tdt, device=dev)
+    ei = lambda *sh: torch.empty(sh, dtype=torch.int32, device=dev)
+    dbuf = (e(nf, N, nr), e(nf, N, na), e(nf, N, nr), ei(nf, N, nr + 1), ei(nf, N, 2 * na), e(nf, N, 3, nr),
+            e(nf, N, 3, 2 * na), e(nf, N, 3, nr), ei(nf, N))
+    slices = []
+    o = 0
+    for n in tipos:
+        slices.append(slice(o, o + n))
+        o += n
+    if args.contiguous_splits:
+        sl = lambda a, s: a[:, s].contiguous()
+    else:
+        sl = lambda a, s: a[:, s]
+
+    timers = {}
+
+    def timed(name, fn, record):
+        if not record:
+            return fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        r = fn()
+        b.record()
+        timers.setdefault(name, []).append((a, b))
+        return r
+
+    def step(record=False):
+        rad, ang, sup, im2, im3, d2, d3, d3s, ntr = timed(
+            "descriptor", lambda: ops.compute_descriptors_light(pos, box, out=dbuf), record)
+        Ftot = None
+        for k, s in enumerate(slices):
+            p = P[k]
+            v = [sl(x, s) for x in (rad, ang, sup, im2, im3, d2, d3, d3s, ntr)]
+            radk, angk, supk, im2k, im3k, d2k, d3k, d3sk, ntrk = v
+            timed("af2", lambda: ops.compute_sort_proj(radk, im2k, p["alpha2b"], p["emb2b"], tm), record)
+            timed("af3", lambda: ops.compute_sort_proj3body(angk, supk, im3k, im2k, p["alpha3b"], p["emb3b"], tm, ntrk,
+                                                            nt=nt), record)
+            f2 = timed("force2", lambda: ops.compute_force_radial(G2[k], d2k, im2k, radk, p["alpha2b"], p["emb2b"], tm,
+                                                                  tp, at[k]), record)
+            f3 = timed("force3", lambda: ops.compute_force_tripl(G3[k], supk, angk, d3sk, d3k, im2k, im3k, p["alpha3b"],
+                                                                 p["emb3b"], tm, tp, at[k], ntrk), record)
+            if mode == "full_step":
+                timed("grad2", lambda: ops.compute_two_body_par_grad(P2[k], radk, im2k, p["alpha2b"], p["emb2b"], tm),
+                      record)
+                timed("grad3", lambda: ops.compute_sort_proj3body_grad(P3[k], angk, supk, im3k, im2k, p["alpha3b"],
+                                                                       p["emb3b"], tm, ntrk, nt=nt), record)
+                timed("gradforce2", lambda: ops.compute_force_radial_grad(Q, G2[k], d2k, im2k, radk, p["alpha2b"],
+                                                                          p["emb2b"], tm, tp, at[k]), record)
+                timed("gradforce3", lambda: ops.compute_force_tripl_grad(Q, G3[k], supk, angk, d3sk, d3k, im2k, im3k,
+                                                                         p["alpha3b"], p["emb3b"], tm, tp, at[k],
+                                                                         ntrk), record)
+            Ftot = f2 + f3 if Ftot is None else Ftot + f2 + f3
+        return Ftot
+
+    for _ in range(args.warmup):
+        step()
+    ops.poll_status()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    el = time.perf_counter() - t0
+    ops.poll_status()
+
+    # per-op GPU time with events on the launch stream (separate pass: events perturb the pipeline slightly)
+    nprof = max(3, min(args.steps, 20))
+    for _ in range(nprof):
+        step(record=True)
+    torch.cuda.synchronize()
+    op_ms = {k: float(np.mean([a.elapsed_time(b) for a, b in v])) for k, v in timers.items()}
+    calls = {k: len(v) // nprof for k, v in timers.items()}
+
+    s = np.dtype(dtype).itemsize
+    ab = algorithmic_bytes(N, tipos, nr, na, Ar, Aa, nt, s)
+    # dominant kernel: the descriptor kernel (the op is a single launch, so the op's event time is the kernel's)
+    desc_ms = op_ms["descriptor"]
+    achieved = ab["descriptor"] * nf / (desc_ms * 1e-3) / 1e9
+    per_step = {k: op_ms[k] * calls[k] for k in op_ms}
+    step_bytes = ab["descriptor"] + ab["af_fwd"] + ab["force"]
+    if mode == "full_step":
+        step_bytes += ab["grad_alpha"] + ab["grad_force"]
+    out = {
+        "metric": "frames/s descriptor fwd+force/alpha bwd, 768-atom water fp32/fp64; % HBM roofline",
+        "value": nf * args.steps / el,
+        "unit": "frames/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": el / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32" if dtype == np.float32 else "f64",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "mode": mode, "atoms": N, "frames_per_step": nf, "Rc": synth.RC,
+                   "radial_buffer": nr, "angular_buffer": na, "Ar": Ar, "Aa": Aa,
+                   "species_tensors": "contiguous copies" if args.contiguous_splits else "views"},
+        "roofline": {"bound": "hbm", "kernel": "desc_kernel", "achieved": achieved, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes_per_launch": ab["descriptor"] * nf, "avg_launch_ms": desc_ms},
+        "whole_step_hbm_frac": step_bytes * nf / (el / args.steps) / 1e9 / HBM_PEAK_GBS,
+        "op_ms_per_step": per_step,
+        "ms_per_frame": el / args.steps * 1e3 / nf,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(batch, params, up, mode, nr, na)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
