@@ -9,6 +9,7 @@
 // fixed-order pass.  There are no floating-point atomics, so results are
 // bit-reproducible from run to run.
 #include "staf_tile.hpp"
+#include "staf_reduce.hpp"
 
 namespace staf {
 
@@ -125,26 +126,6 @@ __global__ __launch_bounds__(AF_BLOCK) void grad2_kernel(const real* __restrict_
     for (int w = 0; w < AF_WAVES; w++) s += w_acc[w * nout + q];
     partial[(size_t)blockIdx.x * nout + q] = s;
   }
-}
-
-// Second pass of every parameter-gradient op: out[e] = sum over the blocks'
-// partials in ascending block order.  out0 takes the first n0 elements, out1
-// (may be null) the next n1.
-template <typename real>
-__global__ void reduce_partials_kernel(const real* __restrict__ partial, int nblocks, int nout, real* out0, int n0,
-                                       real* out1, int n1) {
-  const int e = blockIdx.x * blockDim.x + threadIdx.x;
-  if (e >= nout) return;
-  real s = 0;
-  for (int g = 0; g < nblocks; g++) s += partial[(size_t)g * nout + e];
-  if (e < n0) out0[e] = s;
-  else if (out1 && e - n0 < n1) out1[e - n0] = s;
-}
-
-template <typename real>
-__global__ void fill_zero_kernel(real* p, int n) {
-  const int e = blockIdx.x * blockDim.x + threadIdx.x;
-  if (e < n) p[e] = 0;
 }
 
 // ---------------------------------------------------------------------------
@@ -333,8 +314,7 @@ static int alpha_dist_grad(const real* D, int nr, const real* alpha2b, int Ar, r
   if (lds > 64 * 1024) return STAF_E_LIMIT;
   hipLaunchKernelGGL(grad2_kernel<real>, dim3(nb), dim3(AF_BLOCK), lds, stream, D, im2, alpha2b, emb2b, type_map, P,
                      partial, nf, Nl, ld, nr, Ar, nt);
-  hipLaunchKernelGGL(reduce_partials_kernel<real>, dim3((nout + 127) / 128), dim3(128), 0, stream, partial, nb, nout,
-                     g_alpha, nt * Ar, g_emb, nt * Ar);
+  launch_reduce_partials<real>(partial, nb, nout, g_alpha, nt * Ar, g_emb, nt * Ar, stream);
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }
 
@@ -380,14 +360,11 @@ static int alphagrad_ang(const real* Dsup, const real* Tang, int nr, int na, con
   if (lds > 64 * 1024) return STAF_E_LIMIT;
   // rows sigma >= nsig of the outputs receive no contribution
   const int nall = ntc * Aa * 3;
-  if (nall > nout)
-    hipLaunchKernelGGL(fill_zero_kernel<real>, dim3((nall - nout + 127) / 128), dim3(128), 0, stream, g_alpha + nout,
-                       nall - nout);
-  hipLaunchKernelGGL(fill_zero_kernel<real>, dim3((ntc * Aa + 127) / 128), dim3(128), 0, stream, g_emb, ntc * Aa);
+  launch_fill_zero<real>(g_alpha + nout, nall - nout, stream);
+  launch_fill_zero<real>(g_emb, ntc * Aa, stream);
   hipLaunchKernelGGL((af3_kernel<real, 1>), dim3(nb), dim3(AF_BLOCK), lds, stream, Dsup, Tang, im2, alpha3b, emb3b,
                      type_map, numtriplet, P, partial, nf, Nl, ld, nr, na, Aa, nt);
-  hipLaunchKernelGGL(reduce_partials_kernel<real>, dim3((nout + 127) / 128), dim3(128), 0, stream, partial, nb, nout,
-                     g_alpha, nout, (real*)nullptr, 0);
+  launch_reduce_partials<real>(partial, nb, nout, g_alpha, nout, (real*)nullptr, 0, stream);
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }
 

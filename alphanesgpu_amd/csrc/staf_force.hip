@@ -14,6 +14,7 @@
 // channel and species pair) is gone: der3b is contracted once per triplet with
 // dL/dF into three scalars, and all channels are evaluated from those.
 #include "staf_tile.hpp"
+#include "staf_reduce.hpp"
 
 namespace staf {
 
@@ -543,23 +544,6 @@ __global__ __launch_bounds__(F_BLOCK) void gradforce3_kernel(
   }
 }
 
-template <typename real>
-__global__ void reduce_partials_f_kernel(const real* __restrict__ partial, int nblocks, int nout, real* out0, int n0,
-                                         real* out1, int n1) {
-  const int e = blockIdx.x * blockDim.x + threadIdx.x;
-  if (e >= nout) return;
-  real s = 0;
-  for (int g = 0; g < nblocks; g++) s += partial[(size_t)g * nout + e];
-  if (e < n0) out0[e] = s;
-  else if (out1 && e - n0 < n1) out1[e - n0] = s;
-}
-
-template <typename real>
-__global__ void fill_zero_f_kernel(real* p, int n) {
-  const int e = blockIdx.x * blockDim.x + threadIdx.x;
-  if (e < n) p[e] = 0;
-}
-
 // ---- host launchers --------------------------------------------------------
 
 static inline int grad_blocks_f(int atoms) {
@@ -688,8 +672,7 @@ static int gradforce_2b(const real* Q, const real* D, int nr, const real* alpha2
   if (lds > 64 * 1024) return STAF_E_LIMIT;
   hipLaunchKernelGGL(gradforce2_kernel<real>, dim3(nb), dim3(F_BLOCK), lds, stream, Q, G, D, dD, im2, alpha2b, emb2b,
                      type_map, tipos, actual_type, gnet, partial, nf, N, Nl, ld, nr, Ar, nt);
-  hipLaunchKernelGGL(reduce_partials_f_kernel<real>, dim3((nout + 127) / 128), dim3(128), 0, stream, partial, nb, nout,
-                     g_alpha, nt * Ar, g_emb, nt * Ar);
+  launch_reduce_partials<real>(partial, nb, nout, g_alpha, nt * Ar, g_emb, nt * Ar, stream);
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }
 
@@ -727,15 +710,12 @@ static int gradforce_tripl(const real* Q, const real* G, const real* Dsup, const
   size_t lds = gradforce3_lds<real>(nr, Aa, nt);
   if (lds > 64 * 1024) return STAF_E_LIMIT;
   const int nall = ntc * Aa * 3;
-  if (nall > nout)
-    hipLaunchKernelGGL(fill_zero_f_kernel<real>, dim3((nall - nout + 127) / 128), dim3(128), 0, stream,
-                       g_alpha + nout, nall - nout);
-  hipLaunchKernelGGL(fill_zero_f_kernel<real>, dim3((ntc * Aa + 127) / 128), dim3(128), 0, stream, g_emb, ntc * Aa);
+  launch_fill_zero<real>(g_alpha + nout, nall - nout, stream);
+  launch_fill_zero<real>(g_emb, ntc * Aa, stream);
   hipLaunchKernelGGL(gradforce3_kernel<real>, dim3(nb), dim3(F_BLOCK), lds, stream, Q, G, Dsup, Tang, dDsup, d3b, im2,
                      alpha3b, emb3b, type_map, tipos, actual_type, numtriplet, gnet, partial, nf, N, Nl, ld, nr, na,
                      Aa, nt);
-  hipLaunchKernelGGL(reduce_partials_f_kernel<real>, dim3((nout + 127) / 128), dim3(128), 0, stream, partial, nb, nout,
-                     g_alpha, nout, (real*)nullptr, 0);
+  launch_reduce_partials<real>(partial, nb, nout, g_alpha, nout, (real*)nullptr, 0, stream);
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }
 
