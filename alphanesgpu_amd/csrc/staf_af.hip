@@ -10,6 +10,7 @@
 // bit-reproducible from run to run.
 #include "staf_tile.hpp"
 #include "staf_reduce.hpp"
+#include "staf_tri.hpp"
 
 namespace staf {
 
@@ -128,150 +129,6 @@ __global__ __launch_bounds__(AF_BLOCK) void grad2_kernel(const real* __restrict_
   }
 }
 
-// ---------------------------------------------------------------------------
-// 3-body fingerprints and their parameter gradient.
-//   AF3[b,p,a] = sum_{j<k} T/2 (e^{a1 Dj + a2 Dk} + e^{a2 Dj + a1 Dk}) e^{be T} c3[sigma,a]
-// MODE 0: forward.  MODE 1: gradient wrt (a1,a2,be) given P = dL/dAF3.
-// ---------------------------------------------------------------------------
-template <typename real, int MODE>
-__global__ __launch_bounds__(AF_BLOCK) void af3_kernel(const real* __restrict__ Dsup, const real* __restrict__ Tang,
-                                                       const int* __restrict__ im2, const real* __restrict__ alpha3b,
-                                                       const real* __restrict__ emb3b,
-                                                       const int* __restrict__ type_map,
-                                                       const int* __restrict__ numtriplet,
-                                                       const real* __restrict__ P, real* __restrict__ out, int nf,
-                                                       int Nl, int ld, int nr, int na, int Aa, int nt) {
-  constexpr int CH = (MODE == 0) ? 8 : 4;
-  constexpr int NV = (MODE == 0) ? 1 : 3;
-  extern __shared__ __align__(16) unsigned char smem[];
-  const int nsig = 2 * nt - 1;
-  ChanTable<real> tab;
-  unsigned char* sp = tab.carve(smem, nsig, Aa);
-  const int nacc = (MODE == 0) ? Aa : nsig * Aa * 3;
-  real* w_acc = (real*)sp;                    // [AF_WAVES][nacc]
-  real* w_D = w_acc + AF_WAVES * nacc;        // [AF_WAVES][nr]
-  real* w_P = w_D + AF_WAVES * nr;            // [AF_WAVES][Aa] (MODE 1)
-  int* w_lst = (int*)(w_P + AF_WAVES * Aa);   // [AF_WAVES][nr]
-  int* w_off = w_lst + AF_WAVES * nr;         // [AF_WAVES][NT_MAX+1]
-  tab.build(alpha3b, emb3b);
-  const int wave = threadIdx.x / WAVE, lane = lane_id();
-  real* acc_l = w_acc + wave * nacc;
-  real* myD = w_D + wave * nr;
-  real* myP = w_P + wave * Aa;
-  int* lst = w_lst + wave * nr;
-  int* off = w_off + wave * (NT_MAX + 1);
-  if (MODE == 1)
-    for (int q = lane; q < nacc; q += WAVE) acc_l[q] = 0;
-  __syncthreads();
-
-  const int total = nf * Nl;
-  const int stride = gridDim.x * AF_WAVES;
-  for (int atom = blockIdx.x * AF_WAVES + wave; atom < total; atom += stride) {
-    const int b = atom / Nl, p = atom - b * Nl;
-    const size_t rowAtom = (size_t)b * ld + p;
-    const int* im = im2 + rowAtom * (nr + 1);
-    int m = numtriplet[rowAtom];
-    if (m > nr) m = nr;
-    m = __builtin_amdgcn_readfirstlane(m);
-    const real* Trow = Tang + rowAtom * na;
-    for (int s = lane; s < m; s += WAVE) myD[s] = Dsup[rowAtom * nr + s];
-    if (MODE == 0)
-      for (int q = lane; q < Aa; q += WAVE) acc_l[q] = 0;
-    else
-      for (int q = lane; q < Aa; q += WAVE) myP[q] = P[(size_t)atom * Aa + q];
-    group_slots_by_type(m, nt, im, type_map, lst, off);
-    __builtin_amdgcn_wave_barrier();
-    __threadfence_block();
-
-    for (int ta = 0; ta < nt; ta++) {
-      const int oa = __builtin_amdgcn_readfirstlane(off[ta]);
-      const int na_ = __builtin_amdgcn_readfirstlane(off[ta + 1]) - oa;
-      if (na_ == 0) continue;
-      for (int tb = ta; tb < nt; tb++) {
-        const int ob = __builtin_amdgcn_readfirstlane(off[tb]);
-        const int nb_ = __builtin_amdgcn_readfirstlane(off[tb + 1]) - ob;
-        const bool same = (ta == tb);
-        const int size = same ? (na_ * (na_ - 1)) / 2 : na_ * nb_;
-        if (size == 0) continue;
-        const int sg = ta + tb;
-        const int nch = __builtin_amdgcn_readfirstlane(tab.nact[sg]);
-        const int pb = sg * Aa;
-        for (int c0 = 0; c0 < nch; c0 += CH) {
-          real acc[CH][NV];
-#pragma unroll
-          for (int u = 0; u < CH; u++)
-#pragma unroll
-            for (int v = 0; v < NV; v++) acc[u][v] = 0;
-          for (int q = lane; q < size; q += WAVE) {
-            int j, k, nn;
-            class_pair(q, same, nb_, lst + oa, lst + ob, m, j, k, nn);
-            if (nn >= na) continue;
-            const real T = Trow[nn];
-            const real Dj = myD[j], Dk = myD[k];
-#pragma unroll
-            for (int u = 0; u < CH; u++) {
-              if (c0 + u < nch) {
-                const real a1 = tab.a1[pb + c0 + u], a2 = tab.a2[pb + c0 + u], be = tab.be[pb + c0 + u];
-                const real e1 = r_exp(a1 * Dj + a2 * Dk);
-                const real e2 = r_exp(a2 * Dj + a1 * Dk);
-                const real eb = r_exp(be * T);
-                if (MODE == 0) {
-                  acc[u][0] += T * (e1 + e2) * eb;
-                } else {
-                  const real w = eb * T;
-                  acc[u][0] += (e1 * Dj + e2 * Dk) * w;
-                  acc[u][1] += (e1 * Dk + e2 * Dj) * w;
-                  acc[u][NV - 1] += (e1 + e2) * w * T;
-                }
-              }
-            }
-          }
-#pragma unroll
-          for (int u = 0; u < CH; u++) {
-            if (c0 + u < nch) {
-              const int a = tab.ch[pb + c0 + u];
-              const real c3h = tab.c3[pb + c0 + u] * real(0.5);
-              if (MODE == 0) {
-                const real tot = wave_sum(acc[u][0]);
-                if (lane == 0) acc_l[a] += tot * c3h;
-              } else {
-                const real f = c3h * myP[a];
-#pragma unroll
-                for (int v = 0; v < NV; v++) {
-                  const real tot = wave_sum(acc[u][v]);
-                  if (lane == 0) acc_l[(sg * Aa + a) * 3 + v] += tot * f;
-                }
-              }
-            }
-          }
-        }
-      }
-    }
-    __builtin_amdgcn_wave_barrier();
-    __threadfence_block();
-    if (MODE == 0)
-      for (int q = lane; q < Aa; q += WAVE) out[(size_t)atom * Aa + q] = acc_l[q];
-    __builtin_amdgcn_wave_barrier();
-  }
-  if (MODE == 1) {
-    __syncthreads();
-    for (int q = threadIdx.x; q < nacc; q += blockDim.x) {
-      real s = 0;
-#pragma unroll
-      for (int w = 0; w < AF_WAVES; w++) s += w_acc[w * nacc + q];
-      out[(size_t)blockIdx.x * nacc + q] = s;
-    }
-  }
-}
-
-template <typename real, int MODE>
-static size_t af3_lds(int nr, int Aa, int nt) {
-  const int nsig = 2 * nt - 1;
-  const int nacc = (MODE == 0) ? Aa : nsig * Aa * 3;
-  return chan_table_bytes<real>(nsig, Aa) + (size_t)AF_WAVES * (nacc + nr + Aa) * sizeof(real) +
-         (size_t)AF_WAVES * (nr + NT_MAX + 1) * sizeof(int);
-}
-
 // ---- host launchers --------------------------------------------------------
 
 static inline int grad_blocks(int atoms) {
@@ -328,12 +185,13 @@ static int angular_afs(const real* Dsup, const real* Tang, int nr, int na, real*
     return STAF_E_BAD_ARG;
   if (nt > NT_MAX) return STAF_E_LIMIT;
   if (ld <= 0) ld = Nl;
-  size_t lds = af3_lds<real, 0>(nr, Aa, nt);
+  size_t lds = TriLds<real, 0>::bytes(nr, Aa, nt);
   if (lds > 64 * 1024) return STAF_E_LIMIT;
-  const int atoms = nf * Nl;
-  hipLaunchKernelGGL((af3_kernel<real, 0>), dim3((atoms + AF_WAVES - 1) / AF_WAVES), dim3(AF_BLOCK), lds,
-                     (hipStream_t)stream_, Dsup, Tang, im2, alpha3b, emb3b, type_map, numtriplet, (const real*)nullptr,
-                     out, nf, Nl, ld, nr, na, Aa, nt);
+  TriArgs<real> A = {};
+  A.Dsup = Dsup; A.Tang = Tang; A.im2 = im2; A.alpha3b = alpha3b; A.emb3b = emb3b; A.type_map = type_map;
+  A.numtriplet = numtriplet; A.out = out;
+  A.nf = nf; A.Nl = Nl; A.ld = ld; A.nr = nr; A.na = na; A.Aa = Aa; A.nt = nt;
+  hipLaunchKernelGGL((tri_reduce_kernel<real, 0>), dim3(nf * Nl), dim3(TRI_BLOCK), lds, (hipStream_t)stream_, A);
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }
 
@@ -353,17 +211,20 @@ static int alphagrad_ang(const real* Dsup, const real* Tang, int nr, int na, con
   hipStream_t stream = (hipStream_t)stream_;
   const int nsig = 2 * nt - 1;
   const int nout = nsig * Aa * 3;
-  const int nb = grad_blocks(nf * Nl);
+  const int nb = nf * Nl < TRI_GRID_MAX ? nf * Nl : TRI_GRID_MAX;
   real* partial = (real*)scratch_reserve(st, (size_t)nb * nout * sizeof(real));
   if (!partial) return STAF_E_HIP;
-  size_t lds = af3_lds<real, 1>(nr, Aa, nt);
+  size_t lds = TriLds<real, 1>::bytes(nr, Aa, nt);
   if (lds > 64 * 1024) return STAF_E_LIMIT;
   // rows sigma >= nsig of the outputs receive no contribution
   const int nall = ntc * Aa * 3;
   launch_fill_zero<real>(g_alpha + nout, nall - nout, stream);
   launch_fill_zero<real>(g_emb, ntc * Aa, stream);
-  hipLaunchKernelGGL((af3_kernel<real, 1>), dim3(nb), dim3(AF_BLOCK), lds, stream, Dsup, Tang, im2, alpha3b, emb3b,
-                     type_map, numtriplet, P, partial, nf, Nl, ld, nr, na, Aa, nt);
+  TriArgs<real> A = {};
+  A.Dsup = Dsup; A.Tang = Tang; A.im2 = im2; A.alpha3b = alpha3b; A.emb3b = emb3b; A.type_map = type_map;
+  A.numtriplet = numtriplet; A.P = P; A.partial = partial;
+  A.nf = nf; A.Nl = Nl; A.ld = ld; A.nr = nr; A.na = na; A.Aa = Aa; A.nt = nt;
+  hipLaunchKernelGGL((tri_reduce_kernel<real, 1>), dim3(nb), dim3(TRI_BLOCK), lds, stream, A);
   launch_reduce_partials<real>(partial, nb, nout, g_alpha, nout, (real*)nullptr, 0, stream);
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }

@@ -15,6 +15,7 @@
 // dL/dF into three scalars, and all channels are evaluated from those.
 #include "staf_tile.hpp"
 #include "staf_reduce.hpp"
+#include "staf_tri.hpp"
 
 namespace staf {
 
@@ -98,6 +99,21 @@ __global__ __launch_bounds__(F_BLOCK) void force2_kernel(const real* __restrict_
   }
 }
 
+template <typename real>
+struct Force3Lds {
+  static constexpr int CAPF = sizeof(real) == 8 ? 8 : 16;   // channels tabulated per pass
+  static constexpr int THREADS = sizeof(real) == 8 ? 512 : 256;
+  __host__ __device__ static size_t shared_bytes(int nr) {
+    size_t t = (size_t)2 * CAPF * nr * 2 * sizeof(real);
+    size_t p = (size_t)(F_PARTS * 3 * nr + 3 * nr) * sizeof(real);
+    return ((t > p ? t : p) + 15) & ~(size_t)15;
+  }
+  __host__ __device__ static size_t bytes(int nr, int na, int Aa, int nt) {
+    return chan_table_bytes<real>(2 * nt - 1, Aa) + shared_bytes(nr) +
+           (size_t)(3 * na + nr + 3 * nr + Aa + CAPF) * sizeof(real) + (size_t)(nr + NT_MAX + 1) * sizeof(int);
+  }
+};
+
 // ---------------------------------------------------------------------------
 // 3-body force, pass A.  One 256-thread workgroup per centre.
 // Phase 1 (thread <-> triplet, class-enumerated): channel sums
@@ -108,7 +124,7 @@ __global__ __launch_bounds__(F_BLOCK) void force2_kernel(const real* __restrict_
 //   summed in a fixed order; der3b is read here, once per element.
 // ---------------------------------------------------------------------------
 template <typename real>
-__global__ __launch_bounds__(F_BLOCK) void force3_kernel(const real* __restrict__ G, const real* __restrict__ Dsup,
+__global__ __launch_bounds__(Force3Lds<real>::THREADS) void force3_kernel(const real* __restrict__ G, const real* __restrict__ Dsup,
                                                          const real* __restrict__ Tang,
                                                          const real* __restrict__ dDsup,
                                                          const real* __restrict__ d3b, const int* __restrict__ im2,
@@ -123,14 +139,19 @@ __global__ __launch_bounds__(F_BLOCK) void force3_kernel(const real* __restrict_
   extern __shared__ __align__(16) unsigned char smem[];
   const int nsig = 2 * nt - 1;
   ChanTable<real> tab;
+  constexpr int CAPF = Force3Lds<real>::CAPF;
   unsigned char* sp = tab.carve(smem, nsig, Aa);
-  real* scal = (real*)sp;               // [3*na]
+  // phase-1 pair tables and the phase-2 partial sums never live at the same time: they share one region
+  real2* tabA = (real2*)sp;             // [CAPF*nr]
+  real2* tabB = tabA + CAPF * nr;       // [CAPF*nr]
+  real* part = (real*)sp;               // [F_PARTS*3*nr]   (phase 2)
+  real* fs = part + F_PARTS * 3 * nr;   // [3*nr]           (phase 2)
+  real* scal = (real*)(sp + Force3Lds<real>::shared_bytes(nr));  // [3*na]
   real* bl_D = scal + 3 * na;           // [nr]
   real* bl_g = bl_D + nr;               // [3*nr] grad fc rows (der3bsupp)
   real* bl_G = bl_g + 3 * nr;           // [Aa]
-  real* part = bl_G + Aa;               // [F_PARTS*3*nr]
-  real* fs = part + F_PARTS * 3 * nr;   // [3*nr]
-  int* lst = (int*)(fs + 3 * nr);       // [nr]
+  real* netc = bl_G + Aa;               // [CAPF]
+  int* lst = (int*)(netc + CAPF);       // [nr]
   int* off = lst + nr;                  // [NT_MAX+1]
   tab.build(alpha3b, emb3b);
 
@@ -163,29 +184,78 @@ __global__ __launch_bounds__(F_BLOCK) void force3_kernel(const real* __restrict_
       const int size = same ? (na_ * (na_ - 1)) / 2 : na_ * nb_;
       if (size == 0) continue;
       const int sg = ta + tb;
-      const int nch = tab.nact[sg];
+      const int nact = tab.nact[sg];
       const int pb = sg * Aa;
-      for (int q = tid; q < size; q += blockDim.x) {
-        int j, k, nn;
-        class_pair(q, same, nb_, lst + oa, lst + ob, m, j, k, nn);
-        if (nn >= na) continue;
-        const real T = Trow[nn];
-        const real Dj = bl_D[j], Dk = bl_D[k];
-        real Sd = 0, SBj = 0, SBk = 0;
-        for (int ia = 0; ia < nch; ia++) {
-          const real a1 = tab.a1[pb + ia], a2 = tab.a2[pb + ia], be = tab.be[pb + ia];
-          const real net = real(0.5) * bl_G[tab.ch[pb + ia]] * tab.c3[pb + ia];
-          const real eb = r_exp(be * T);
-          const real sim1 = r_exp(a2 * Dj + a1 * Dk);
-          const real sim2 = r_exp(a1 * Dj + a2 * Dk);
-          const real h = real(0.5) * eb * net;
-          Sd += h * (real(1) + be * T) * (sim1 + sim2);
-          SBj += h * T * (a1 * sim2 + a2 * sim1);
-          SBk += h * T * (a1 * sim1 + a2 * sim2);
+      const int* la = lst + oa;
+      const int* lb = lst + ob;
+      for (int c0 = 0; c0 < nact; c0 += CAPF) {
+        const int nch = (nact - c0) < CAPF ? (nact - c0) : CAPF;
+        __syncthreads();   // readers of the previous tables are done
+        // E[ia][x] = (exp(a1 D), exp(a2 D)) for the slots of both species of the class
+        {
+          const int ea = na_ * nch, eb_ = same ? 0 : nb_ * nch;
+          for (int e = tid; e < ea + eb_; e += blockDim.x) {
+            const bool second = e >= ea;
+            const int ee = second ? e - ea : e;
+            const int n_ = second ? nb_ : na_;
+            const int ia = ee / n_, x = ee - ia * n_;
+            const real d = bl_D[second ? lb[x] : la[x]];
+            real2 v;
+            v.x = r_exp(tab.a1[pb + c0 + ia] * d);
+            v.y = r_exp(tab.a2[pb + c0 + ia] * d);
+            (second ? tabB : tabA)[ia * nr + x] = v;
+          }
+          for (int ia = tid; ia < nch; ia += blockDim.x)
+            netc[ia] = real(0.25) * bl_G[tab.ch[pb + c0 + ia]] * tab.c3[pb + c0 + ia];   // 1/2 of E, 1/2 of T
         }
-        scal[3 * nn] = Sd;
-        scal[3 * nn + 1] = SBj;
-        scal[3 * nn + 2] = SBk;
+        __syncthreads();
+        const real2* tB = same ? tabA : tabB;
+        for (int q = tid; q < size; q += blockDim.x) {
+          int x, y;
+          if (same) tri_decode_xy(q, nb_, x, y);
+          else { x = q / nb_; y = q - x * nb_; }
+          const int s1 = la[x], s2 = lb[y];
+          const bool lo = s1 < s2;
+          const int j = lo ? s1 : s2, k = lo ? s2 : s1;
+          const int nn = tri_rowstart(j, m) + k - j - 1;
+          if (nn >= na) continue;
+          const real T = Trow[nn];
+          real Sd = 0, SB1 = 0, SB2 = 0;
+          for (int ia = 0; ia < nch; ia++) {
+            const real a1 = tab.a1[pb + c0 + ia], a2 = tab.a2[pb + c0 + ia], be = tab.be[pb + c0 + ia];
+            const real2 e1 = tabA[ia * nr + x];
+            const real2 e2 = tB[ia * nr + y];
+            const real sim2 = e1.x * e2.y;   // exp(a1 D1 + a2 D2)
+            const real sim1 = e1.y * e2.x;   // exp(a2 D1 + a1 D2)
+            const real h = r_exp(be * T) * netc[ia];
+            Sd += h * (real(1) + be * T) * (sim1 + sim2);
+            SB1 += h * (a1 * sim2 + a2 * sim1);
+            SB2 += h * (a1 * sim1 + a2 * sim2);
+          }
+          SB1 *= T;
+          SB2 *= T;
+          const real SBj = lo ? SB1 : SB2, SBk = lo ? SB2 : SB1;
+          if (c0 == 0) {
+            scal[3 * nn] = Sd;
+            scal[3 * nn + 1] = SBj;
+            scal[3 * nn + 2] = SBk;
+          } else {
+            scal[3 * nn] += Sd;
+            scal[3 * nn + 1] += SBj;
+            scal[3 * nn + 2] += SBk;
+          }
+        }
+      }
+      if (nact == 0) {
+        // no active channel for this class: its triplets contribute nothing
+        for (int q = tid; q < size; q += blockDim.x) {
+          int j, k, nn;
+          class_pair(q, same, nb_, la, lb, m, j, k, nn);
+          if (nn >= na) continue;
+          scal[3 * nn] = 0;
+          scal[3 * nn + 1] = 0;
+          scal[3 * nn + 2] = 0;
+        }
       }
     }
   }
@@ -377,173 +447,6 @@ __global__ __launch_bounds__(F_BLOCK) void gradforce2_kernel(
   }
 }
 
-// ---------------------------------------------------------------------------
-// gradient of the 3-body force op.  One wave per centre, class-enumerated.
-// Per triplet (j<k), with q_s = Q[atom of slot s] - Q[centre]:
-//   U  = sum_c q_j,c dT/dd_j,c + q_k,c dT/dd_k,c      (der3b contracted once)
-//   V_s = sum_c q_s,c grad fc_s,c                      (per slot)
-// and per channel
-//   dG[a]      += c3/2 (delta U + Bp_j V_j + Bp_k V_k)
-//   dpar[sg,a] += G[a] c3/2 (d delta/dpar U + d Bp_j/dpar V_j + d Bp_k/dpar V_k)
-// ---------------------------------------------------------------------------
-template <typename real>
-__global__ __launch_bounds__(F_BLOCK) void gradforce3_kernel(
-    const real* __restrict__ Q, const real* __restrict__ G, const real* __restrict__ Dsup,
-    const real* __restrict__ Tang, const real* __restrict__ dDsup, const real* __restrict__ d3b,
-    const int* __restrict__ im2, const real* __restrict__ alpha3b, const real* __restrict__ emb3b,
-    const int* __restrict__ type_map, const int* __restrict__ tipos, const int* __restrict__ actual_type,
-    const int* __restrict__ numtriplet, real* __restrict__ gnet, real* __restrict__ partial, int nf, int N, int Nl,
-    int ld, int nr, int na, int Aa, int nt) {
-  using real2 = typename Vec2<real>::type;
-  constexpr int CH = 4;
-  extern __shared__ __align__(16) unsigned char smem[];
-  const int nsig = 2 * nt - 1;
-  ChanTable<real> tab;
-  unsigned char* sp = tab.carve(smem, nsig, Aa);
-  const int nacc = nsig * Aa * 3;
-  real* w_acc = (real*)sp;                     // [F_WAVES][nacc]
-  real* w_D = w_acc + F_WAVES * nacc;          // [F_WAVES][nr]
-  real* w_V = w_D + F_WAVES * nr;              // [F_WAVES][nr]
-  real* w_q = w_V + F_WAVES * nr;              // [F_WAVES][3*nr]
-  real* w_G = w_q + F_WAVES * 3 * nr;          // [F_WAVES][Aa]
-  real* w_o = w_G + F_WAVES * Aa;              // [F_WAVES][Aa]
-  int* w_lst = (int*)(w_o + F_WAVES * Aa);     // [F_WAVES][nr]
-  int* w_off = w_lst + F_WAVES * nr;           // [F_WAVES][NT_MAX+1]
-  tab.build(alpha3b, emb3b);
-  const int wave = threadIdx.x / WAVE, lane = lane_id();
-  real* acc_l = w_acc + wave * nacc;
-  real* myD = w_D + wave * nr;
-  real* myV = w_V + wave * nr;
-  real* myQ = w_q + wave * 3 * nr;
-  real* myG = w_G + wave * Aa;
-  real* myO = w_o + wave * Aa;
-  int* lst = w_lst + wave * nr;
-  int* off = w_off + wave * (NT_MAX + 1);
-  for (int q = lane; q < nacc; q += WAVE) acc_l[q] = 0;
-  const int shift = species_shift(tipos, actual_type);
-  __syncthreads();
-
-  const int total = nf * Nl;
-  const int stride = gridDim.x * F_WAVES;
-  for (int atom = blockIdx.x * F_WAVES + wave; atom < total; atom += stride) {
-    const int b = atom / Nl, p = atom - b * Nl;
-    const size_t rowAtom = (size_t)b * ld + p;
-    const int* im = im2 + rowAtom * (nr + 1);
-    int m = numtriplet[rowAtom];
-    if (m > nr) m = nr;
-    m = __builtin_amdgcn_readfirstlane(m);
-    const real* Trow = Tang + rowAtom * na;
-    const real2* d3 = (const real2*)d3b + rowAtom * 3 * na;
-    const real* Qi = Q + ((size_t)b * N + p + shift) * 3;
-    const real qi0 = Qi[0], qi1 = Qi[1], qi2 = Qi[2];
-    for (int s = lane; s < m; s += WAVE) {
-      const int nj = im[1 + s];
-      const real* Qj = Q + ((size_t)b * N + nj) * 3;
-      const real q0 = Qj[0] - qi0, q1 = Qj[1] - qi1, q2 = Qj[2] - qi2;
-      const real* gr = dDsup + rowAtom * 3 * nr + s;
-      myQ[3 * s] = q0; myQ[3 * s + 1] = q1; myQ[3 * s + 2] = q2;
-      myV[s] = q0 * gr[0] + q1 * gr[nr] + q2 * gr[2 * nr];
-      myD[s] = Dsup[rowAtom * nr + s];
-    }
-    for (int a = lane; a < Aa; a += WAVE) { myG[a] = G[(size_t)atom * Aa + a]; myO[a] = 0; }
-    group_slots_by_type(m, nt, im, type_map, lst, off);
-    __builtin_amdgcn_wave_barrier();
-    __threadfence_block();
-
-    for (int ta = 0; ta < nt; ta++) {
-      const int oa = __builtin_amdgcn_readfirstlane(off[ta]);
-      const int na_ = __builtin_amdgcn_readfirstlane(off[ta + 1]) - oa;
-      if (na_ == 0) continue;
-      for (int tb = ta; tb < nt; tb++) {
-        const int ob = __builtin_amdgcn_readfirstlane(off[tb]);
-        const int nb_ = __builtin_amdgcn_readfirstlane(off[tb + 1]) - ob;
-        const bool same = (ta == tb);
-        const int size = same ? (na_ * (na_ - 1)) / 2 : na_ * nb_;
-        if (size == 0) continue;
-        const int sg = ta + tb;
-        const int nch = __builtin_amdgcn_readfirstlane(tab.nact[sg]);
-        const int pb = sg * Aa;
-        for (int c0 = 0; c0 < nch; c0 += CH) {
-          real acc[CH][4];
-#pragma unroll
-          for (int u = 0; u < CH; u++)
-#pragma unroll
-            for (int v = 0; v < 4; v++) acc[u][v] = 0;
-          for (int q = lane; q < size; q += WAVE) {
-            int j, k, nn;
-            class_pair(q, same, nb_, lst + oa, lst + ob, m, j, k, nn);
-            if (nn >= na) continue;
-            const real T = Trow[nn];
-            const real Dj = myD[j], Dk = myD[k];
-            const real Vj = myV[j], Vk = myV[k];
-            real U = 0;
-#pragma unroll
-            for (int c = 0; c < 3; c++) {
-              const real2 dv = d3[c * na + nn];
-              U += myQ[3 * j + c] * dv.x + myQ[3 * k + c] * dv.y;
-            }
-#pragma unroll
-            for (int u = 0; u < CH; u++) {
-              if (c0 + u < nch) {
-                const real a1 = tab.a1[pb + c0 + u], a2 = tab.a2[pb + c0 + u], be = tab.be[pb + c0 + u];
-                const real eb = r_exp(be * T);
-                const real sim1 = r_exp(a2 * Dj + a1 * Dk);
-                const real sim2 = r_exp(a1 * Dj + a2 * Dk);
-                const real ss = sim1 + sim2;
-                const real opb = real(1) + be * T;
-                const real hT = real(0.5) * eb * T;
-                const real suppj = a1 * sim2 + a2 * sim1;
-                const real suppk = a1 * sim1 + a2 * sim2;
-                // value
-                acc[u][0] += real(0.5) * eb * opb * ss * U + hT * (suppj * Vj + suppk * Vk);
-                // d/d alpha1
-                acc[u][1] += real(0.5) * eb * opb * (sim1 * Dk + sim2 * Dj) * U +
-                             hT * ((sim2 + a1 * sim2 * Dj + a2 * sim1 * Dk) * Vj +
-                                   (sim1 + a1 * sim1 * Dk + a2 * sim2 * Dj) * Vk);
-                // d/d alpha2
-                acc[u][2] += real(0.5) * eb * opb * (sim1 * Dj + sim2 * Dk) * U +
-                             hT * ((sim1 + a2 * sim1 * Dj + a1 * sim2 * Dk) * Vj +
-                                   (sim2 + a2 * sim2 * Dk + a1 * sim1 * Dj) * Vk);
-                // d/d beta
-                acc[u][3] += hT * (real(2) + be * T) * ss * U + hT * T * (suppj * Vj + suppk * Vk);
-              }
-            }
-          }
-#pragma unroll
-          for (int u = 0; u < CH; u++) {
-            if (c0 + u < nch) {
-              const int a = tab.ch[pb + c0 + u];
-              const real c3h = tab.c3[pb + c0 + u] * real(0.5);
-              const real t0 = wave_sum(acc[u][0]);
-              const real t1 = wave_sum(acc[u][1]);
-              const real t2 = wave_sum(acc[u][2]);
-              const real t3 = wave_sum(acc[u][3]);
-              if (lane == 0) {
-                myO[a] += t0 * c3h;
-                const real f = c3h * myG[a];
-                acc_l[(sg * Aa + a) * 3] += t1 * f;
-                acc_l[(sg * Aa + a) * 3 + 1] += t2 * f;
-                acc_l[(sg * Aa + a) * 3 + 2] += t3 * f;
-              }
-            }
-          }
-        }
-      }
-    }
-    __builtin_amdgcn_wave_barrier();
-    __threadfence_block();
-    for (int a = lane; a < Aa; a += WAVE) gnet[(size_t)atom * Aa + a] = myO[a];
-    __builtin_amdgcn_wave_barrier();
-  }
-  __syncthreads();
-  for (int q = threadIdx.x; q < nacc; q += blockDim.x) {
-    real s = 0;
-#pragma unroll
-    for (int w = 0; w < F_WAVES; w++) s += w_acc[w * nacc + q];
-    partial[(size_t)blockIdx.x * nacc + q] = s;
-  }
-}
-
 // ---- host launchers --------------------------------------------------------
 
 static inline int grad_blocks_f(int atoms) {
@@ -611,13 +514,6 @@ static int force_doublets(const real* G, const real* D, const real* dD, const in
 }
 
 template <typename real>
-static size_t force3_lds(int nr, int na, int Aa, int nt) {
-  return chan_table_bytes<real>(2 * nt - 1, Aa) +
-         (size_t)(3 * na + nr + 3 * nr + Aa + F_PARTS * 3 * nr + 3 * nr) * sizeof(real) +
-         (size_t)(nr + NT_MAX + 1) * sizeof(int);
-}
-
-template <typename real>
 static int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* dDsup, const real* d3b,
                        const int* im2, const int* im3, int nr, int na, int N, int nf, int Aa, const real* emb3b,
                        int nt, const int* tipos, const int* actual_type, real* force, const int* numtriplet,
@@ -636,14 +532,14 @@ static int force_tripl(const real* G, const real* Dsup, const real* Tang, const 
   ForceScratch fs;
   int rc = force_scratch<real>(st, nf, N, Nl, nr, stream, &fs);
   if (rc) return rc;
-  size_t lds = force3_lds<real>(nr, na, Aa, nt);
+  size_t lds = Force3Lds<real>::bytes(nr, na, Aa, nt);
   if (lds > 64 * 1024) {
     if (lds > 160 * 1024) return STAF_E_LIMIT;
     if (hipFuncSetAttribute((const void*)force3_kernel<real>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
         hipSuccess)
       return STAF_E_LIMIT;
   }
-  hipLaunchKernelGGL(force3_kernel<real>, dim3(nf * Nl), dim3(F_BLOCK), lds, stream, G, Dsup, Tang, dDsup, d3b, im2,
+  hipLaunchKernelGGL(force3_kernel<real>, dim3(nf * Nl), dim3(Force3Lds<real>::THREADS), lds, stream, G, Dsup, Tang, dDsup, d3b, im2,
                      alpha3b, emb3b, type_map, numtriplet, (real*)fs.gslot, (real*)fs.self, fs.bcnt, fs.bent, fs.cap,
                      st->status_d, nf, N, Nl, ld, nr, na, Aa, nt);
   return launch_gather<real>(st, fs, tipos, actual_type, force, nf, N, Nl, nr, stream);
@@ -677,14 +573,6 @@ static int gradforce_2b(const real* Q, const real* D, int nr, const real* alpha2
 }
 
 template <typename real>
-static size_t gradforce3_lds(int nr, int Aa, int nt) {
-  const int nsig = 2 * nt - 1;
-  return chan_table_bytes<real>(nsig, Aa) +
-         (size_t)F_WAVES * (nsig * Aa * 3 + nr + nr + 3 * nr + Aa + Aa) * sizeof(real) +
-         (size_t)F_WAVES * (nr + NT_MAX + 1) * sizeof(int);
-}
-
-template <typename real>
 static int gradforce_tripl(const real* Q, const real* G, const real* Dsup, const real* Tang, const real* dDsup,
                            const real* d3b, const int* im2, const int* im3, int nr, int na, int N, int nf, int Aa,
                            const real* emb3b, int nt, const int* tipos, const int* actual_type, const int* numtriplet,
@@ -704,17 +592,20 @@ static int gradforce_tripl(const real* Q, const real* G, const real* Dsup, const
   const int ntc = nt * (nt + 1) / 2;
   const int nsig = 2 * nt - 1;
   const int nout = nsig * Aa * 3;
-  const int nb = grad_blocks_f(nf * Nl);
+  const int nb = nf * Nl < TRI_GRID_MAX ? nf * Nl : TRI_GRID_MAX;
   real* partial = (real*)scratch_reserve(st, (size_t)nb * nout * sizeof(real));
   if (!partial) return STAF_E_HIP;
-  size_t lds = gradforce3_lds<real>(nr, Aa, nt);
+  size_t lds = TriLds<real, 2>::bytes(nr, Aa, nt);
   if (lds > 64 * 1024) return STAF_E_LIMIT;
   const int nall = ntc * Aa * 3;
   launch_fill_zero<real>(g_alpha + nout, nall - nout, stream);
   launch_fill_zero<real>(g_emb, ntc * Aa, stream);
-  hipLaunchKernelGGL(gradforce3_kernel<real>, dim3(nb), dim3(F_BLOCK), lds, stream, Q, G, Dsup, Tang, dDsup, d3b, im2,
-                     alpha3b, emb3b, type_map, tipos, actual_type, numtriplet, gnet, partial, nf, N, Nl, ld, nr, na,
-                     Aa, nt);
+  TriArgs<real> A = {};
+  A.Dsup = Dsup; A.Tang = Tang; A.im2 = im2; A.alpha3b = alpha3b; A.emb3b = emb3b; A.type_map = type_map;
+  A.numtriplet = numtriplet; A.P = G; A.Q = Q; A.dDsup = dDsup; A.d3b = d3b; A.tipos = tipos;
+  A.actual_type = actual_type; A.out = gnet; A.partial = partial;
+  A.nf = nf; A.N = N; A.Nl = Nl; A.ld = ld; A.nr = nr; A.na = na; A.Aa = Aa; A.nt = nt;
+  hipLaunchKernelGGL((tri_reduce_kernel<real, 2>), dim3(nb), dim3(TRI_BLOCK), lds, stream, A);
   launch_reduce_partials<real>(partial, nb, nout, g_alpha, nout, (real*)nullptr, 0, stream);
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }
