@@ -7,7 +7,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libstaf_hip.so")
+# STAF_HIP_LIB selects another build of the same library (e.g. an experimental variant)
+LIB_PATH = os.environ.get("STAF_HIP_LIB") or os.path.join(_HERE, "lib", "libstaf_hip.so")
 
 STAF_OK = 0
 ERRORS = {

@@ -52,16 +52,16 @@ struct TriArgs {
 template <typename real, int MODE>
 struct TriLds {
   static constexpr int NV = (MODE == 0) ? 1 : (MODE == 1 ? 3 : 4);
-  // bytes of the staging region: packed pairs + T (+ U), or the per-thread partials of the class reduction
+  // bytes of the staging region (packed pairs + T (+ U)) followed by the per-thread partials of the class reduction
   __host__ __device__ static size_t stage_bytes() {
     size_t st = (size_t)TRI_QB * (sizeof(int) + sizeof(real) * (MODE == 2 ? 2 : 1));
     size_t rd = (size_t)TRI_BLOCK * NV * sizeof(real);
-    return ((st > rd ? st : rd) + 15) & ~(size_t)15;
+    return ((st + 15) & ~(size_t)15) + ((rd + 15) & ~(size_t)15);
   }
   __host__ __device__ static size_t bytes(int nr, int Aa, int nt) {
     const int nsig = 2 * nt - 1;
     size_t b = chan_table_bytes<real>(nsig, Aa);
-    size_t reals = (size_t)Aa /*out_ch*/ + nr /*sD*/ + Aa /*sP*/ + (size_t)2 * nr * TRI_CAP * 2 /*tabA,tabB*/;
+    size_t reals = (size_t)Aa /*out_ch*/ + nr /*sD*/ + Aa /*sP*/ + (size_t)nr * TRI_CAP * 2 /*pair tables*/;
     if (MODE != 0) reals += (size_t)nsig * Aa * 3;
     if (MODE == 2) reals += (size_t)4 * nr;  // sV, sQ
     b += reals * sizeof(real);
@@ -82,8 +82,7 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
   ChanTable<real> tab;
   unsigned char* sp = tab.carve(smem, nsig, Aa);
   real* rp = (real*)sp;   // 16-byte aligned: the pair tables come first
-  real2* tabA = (real2*)rp; rp += (size_t)nr * TRI_CAP * 2;
-  real2* tabB = (real2*)rp; rp += (size_t)nr * TRI_CAP * 2;
+  real2* tabA = (real2*)rp; rp += (size_t)nr * TRI_CAP * 2;   // both species of a class: at most m <= nr rows
   real* out_ch = rp; rp += Aa;
   real* sD = rp; rp += nr;
   real* sP = rp; rp += Aa;
@@ -96,7 +95,7 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
   real* sT = (real*)stg;                       // [TRI_QB]
   real* sU = sT + TRI_QB;                      // [TRI_QB] (MODE 2)
   int* pk = (int*)(sT + TRI_QB * (MODE == 2 ? 2 : 1));   // [TRI_QB]
-  real* red = (real*)stg;                      // aliases the staging arrays
+  real* red = (real*)(stg + (((size_t)TRI_QB * (sizeof(int) + sizeof(real) * (MODE == 2 ? 2 : 1)) + 15) & ~(size_t)15));
   int* lst = (int*)(stg + TriLds<real, MODE>::stage_bytes());
   int* off = lst + nr;
 
@@ -155,6 +154,7 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
         const int pb = sg * Aa;
         const int* la = lst + oa;
         const int* lb = lst + ob;
+        real2* tabB = tabA + (size_t)na_ * TRI_CAP;   // rows of the second species follow the first
         for (int c0 = 0; c0 < nact; c0 += TRI_CAP) {
           const int nch = (nact - c0) < TRI_CAP ? (nact - c0) : TRI_CAP;
           // ---- tables of the class: E[x][ia] = (exp(a1 D), exp(a2 D))
@@ -182,7 +182,7 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
           for (int v = 0; v < NV; v++) acc[v] = 0;
           for (int q0 = 0; q0 < size; q0 += TRI_QB) {
             const int nq = (size - q0) < TRI_QB ? (size - q0) : TRI_QB;
-            __syncthreads();   // tables written / previous block consumed
+            if (q0 > 0) __syncthreads();   // previous block consumed
             // ---- stage a block of triplets
             for (int qq = tid; qq < nq; qq += TRI_BLOCK) {
               const int q = q0 + qq;
@@ -253,8 +253,8 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
               }
             }
           }
-          // ---- combine the subsets of each channel in a fixed order
-          __syncthreads();
+          // ---- combine the subsets of each channel in a fixed order.  `red` is its own region: the
+          // previous pass's combine finished before the barrier that followed this pass's staging.
 #pragma unroll
           for (int v = 0; v < NV; v++) red[tid * NV + v] = acc[v];
           __syncthreads();
