@@ -110,7 +110,7 @@ struct Force3Lds {
   }
   __host__ __device__ static size_t bytes(int nr, int na, int Aa, int nt) {
     return chan_table_bytes<real>(2 * nt - 1, Aa) + shared_bytes(nr) +
-           (size_t)(3 * na + nr + 3 * nr + Aa + CAPF) * sizeof(real) + (size_t)(nr + NT_MAX + 1) * sizeof(int);
+           (size_t)(3 * na + nr + 3 * nr + Aa + CAPF) * sizeof(real) + (size_t)(2 * nr + NT_MAX + 1) * sizeof(int);
   }
 };
 
@@ -152,7 +152,8 @@ __global__ __launch_bounds__(Force3Lds<real>::THREADS) void force3_kernel(const 
   real* bl_G = bl_g + 3 * nr;           // [Aa]
   real* netc = bl_G + Aa;               // [CAPF]
   int* lst = (int*)(netc + CAPF);       // [nr]
-  int* off = lst + nr;                  // [NT_MAX+1]
+  int* stp = lst + nr;                  // [nr] species of every slot
+  int* off = stp + nr;                  // [NT_MAX+1]
   tab.build(alpha3b, emb3b);
 
   const int tid = threadIdx.x;
@@ -164,11 +165,13 @@ __global__ __launch_bounds__(Force3Lds<real>::THREADS) void force3_kernel(const 
   if (m > nr) m = nr;
   for (int s = tid; s < m; s += blockDim.x) {
     bl_D[s] = Dsup[rowAtom * nr + s];
+    stp[s] = type_map[im[1 + s]];
 #pragma unroll
     for (int c = 0; c < 3; c++) bl_g[c * nr + s] = dDsup[rowAtom * 3 * nr + c * nr + s];
   }
   for (int a = tid; a < Aa; a += blockDim.x) bl_G[a] = G[(size_t)atom * Aa + a];
-  if (tid < WAVE) group_slots_by_type(m, nt, im, type_map, lst, off);
+  __syncthreads();
+  if (tid < WAVE) group_slots_by_type(m, nt, stp, lst, off);
   __syncthreads();
 
   const real* Trow = Tang + rowAtom * na;

@@ -71,9 +71,8 @@ __host__ __device__ inline size_t chan_table_bytes(int nsig, int Aa) {
 
 // Slots of one centre grouped by neighbour species (ascending slot inside a
 // species).  lst [m] and off [nt+1] live in LDS (per wave or per block).
-// Called by one full wavefront; types are read through intmap2b + type_map.
-__device__ inline void group_slots_by_type(int m, int nt, const int* im_row /* intmap2b row, slot s at [1+s] */,
-                                           const int* type_map, int* lst, int* off) {
+// Called by one full wavefront; stp [m] holds the species of every slot (LDS).
+__device__ inline void group_slots_by_type(int m, int nt, const int* stp, int* lst, int* off) {
   const int lane = lane_id();
   int base = 0;
   for (int t = 0; t < nt; t++) {
@@ -81,7 +80,7 @@ __device__ inline void group_slots_by_type(int m, int nt, const int* im_row /* i
     for (int s0 = 0; s0 < m; s0 += WAVE) {
       const int s = s0 + lane;
       bool on = false;
-      if (s < m) on = (type_map[im_row[1 + s]] == t);
+      if (s < m) on = (stp[s] == t);
       const unsigned long long mask = __ballot(on);
       if (on) lst[base + __popcll(mask & ((1ull << lane) - 1ull))] = s;
       base += __popcll(mask);

@@ -67,7 +67,7 @@ struct TriLds {
     b += reals * sizeof(real);
     b = (b + 15) & ~(size_t)15;
     b += stage_bytes();
-    b += (size_t)(nr + NT_MAX + 1) * sizeof(int);
+    b += (size_t)(2 * nr + NT_MAX + 1) * sizeof(int);
     return b;
   }
 };
@@ -97,7 +97,8 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
   int* pk = (int*)(sT + TRI_QB * (MODE == 2 ? 2 : 1));   // [TRI_QB]
   real* red = (real*)(stg + (((size_t)TRI_QB * (sizeof(int) + sizeof(real) * (MODE == 2 ? 2 : 1)) + 15) & ~(size_t)15));
   int* lst = (int*)(stg + TriLds<real, MODE>::stage_bytes());
-  int* off = lst + nr;
+  int* stp = lst + nr;
+  int* off = stp + nr;
 
   const int tid = threadIdx.x;
   tab.build(A.alpha3b, A.emb3b);
@@ -122,8 +123,9 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
     // ---- per-atom slot data
     for (int s = tid; s < m; s += TRI_BLOCK) {
       sD[s] = A.Dsup[rowAtom * nr + s];
+      const int nj = im[1 + s];
+      stp[s] = A.type_map[nj];
       if (MODE == 2) {
-        const int nj = im[1 + s];
         const real* Qj = A.Q + ((size_t)b * A.N + nj) * 3;
         const real* Qi = A.Q + ((size_t)b * A.N + p + shift) * 3;
         const real q0 = Qj[0] - Qi[0], q1 = Qj[1] - Qi[1], q2 = Qj[2] - Qi[2];
@@ -136,7 +138,8 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
       out_ch[a] = 0;
       if (MODE != 0) sP[a] = A.P[(size_t)atom * Aa + a];
     }
-    if (tid < WAVE) group_slots_by_type(m, nt, im, A.type_map, lst, off);
+    __syncthreads();
+    if (tid < WAVE) group_slots_by_type(m, nt, stp, lst, off);
     __syncthreads();
 
     for (int ta = 0; ta < nt; ta++) {
