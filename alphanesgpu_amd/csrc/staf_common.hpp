@@ -69,6 +69,28 @@ __device__ inline void tri_decode(int nn, int m, int& j, int& k) {
   k = nn - tri_rowstart(jj, m) + jj + 1;
 }
 
+// Minimum-image Cartesian separation r_i - r_j from Cartesian positions and
+// box6 = [Lx, xy, xz, Ly, yz, Lz]: cart -> frac, rint, back to cart
+// (STAF/include/staf_force_pbc.cuh:16-49; used by the virial forms only).
+template <typename real>
+__device__ inline void mic_cart_from_cart(const real* pi, const real* pj, const real* bx, real* d) {
+  const real i0 = real(1) / bx[0];
+  const real i1 = -bx[1] / (bx[0] * bx[3]);
+  const real i2 = (bx[1] * bx[4]) / (bx[0] * bx[3] * bx[5]) - bx[2] / (bx[0] * bx[5]);
+  const real i3 = real(1) / bx[3];
+  const real i4 = -bx[4] / (bx[3] * bx[5]);
+  const real i5 = real(1) / bx[5];
+  real rx = (i0 * pi[0] + i1 * pi[1] + i2 * pi[2]) - (i0 * pj[0] + i1 * pj[1] + i2 * pj[2]);
+  real ry = (i3 * pi[1] + i4 * pi[2]) - (i3 * pj[1] + i4 * pj[2]);
+  real rz = i5 * pi[2] - i5 * pj[2];
+  rx -= r_rint(rx);
+  ry -= r_rint(ry);
+  rz -= r_rint(rz);
+  d[0] = bx[0] * rx + bx[1] * ry + bx[2] * rz;
+  d[1] = bx[3] * ry + bx[4] * rz;
+  d[2] = bx[5] * rz;
+}
+
 // Pair index q inside an n-item triangle (x<y) -> (x,y); same numbering.
 __device__ inline void tri_decode_xy(int q, int n, int& x, int& y) { tri_decode(q, n, x, y); }
 

@@ -309,6 +309,75 @@ __global__ __launch_bounds__(Force3Lds<real>::THREADS) void force3_kernel(const 
 }
 
 // ---------------------------------------------------------------------------
+// Virial forms (ComputeForceRadialVirial / ComputeForceTriplVirial).  The reference adds W_ab -= g_a r_b for
+// every pair force g it scatters, r = minimum-image r_centre - r_neighbour.  Summed over the triplets of a
+// centre, the pair forces on one slot add up to that slot's entry of gslot, so W = - sum_(centre,slot)
+// gslot (x) r: one wave per centre builds its 3x3 contribution, a second kernel adds the centres of a frame
+// in ascending order.
+// ---------------------------------------------------------------------------
+template <typename real>
+__global__ __launch_bounds__(F_BLOCK) void virial_centre_kernel(const real* __restrict__ gslot,
+                                                                const int* __restrict__ im2,
+                                                                const int* __restrict__ counts,
+                                                                const real* __restrict__ pos,
+                                                                const real* __restrict__ box,
+                                                                const int* __restrict__ tipos,
+                                                                const int* __restrict__ actual_type,
+                                                                real* __restrict__ vpart, int nf, int N, int Nl,
+                                                                int ld, int nr) {
+  const int wave = threadIdx.x / WAVE, lane = lane_id();
+  const int atom = blockIdx.x * F_WAVES + wave;
+  if (atom >= nf * Nl) return;
+  const int b = atom / Nl, p = atom - b * Nl;
+  const size_t rowAtom = (size_t)b * ld + p;
+  const int* im = im2 + rowAtom * (nr + 1);
+  int cnt = counts ? counts[rowAtom] : im[0];
+  if (cnt > nr) cnt = nr;
+  const int shift = species_shift(tipos, actual_type);
+  const real* pi = pos + ((size_t)b * N + p + shift) * 3;
+  const real* bx = box + (size_t)b * 6;
+  real v[9];
+#pragma unroll
+  for (int c = 0; c < 9; c++) v[c] = 0;
+  for (int s = lane; s < cnt; s += WAVE) {
+    const int nj = im[1 + s];
+    real r[3];
+    mic_cart_from_cart(pi, pos + ((size_t)b * N + nj) * 3, bx, r);
+    const real* g = gslot + ((size_t)atom * nr + s) * 3;
+#pragma unroll
+    for (int a = 0; a < 3; a++)
+#pragma unroll
+      for (int e = 0; e < 3; e++) v[a * 3 + e] -= g[a] * r[e];
+  }
+#pragma unroll
+  for (int c = 0; c < 9; c++) {
+    const real t = wave_sum(v[c]);
+    if (lane == 0) vpart[(size_t)atom * 9 + c] = t;
+  }
+}
+
+template <typename real>
+__global__ __launch_bounds__(F_BLOCK) void virial_frame_kernel(const real* __restrict__ vpart,
+                                                               real* __restrict__ virial, int Nl) {
+  __shared__ real sh[F_BLOCK * 9];
+  const int b = blockIdx.x, tid = threadIdx.x;
+  real v[9];
+#pragma unroll
+  for (int c = 0; c < 9; c++) v[c] = 0;
+  for (int p = tid; p < Nl; p += F_BLOCK)
+#pragma unroll
+    for (int c = 0; c < 9; c++) v[c] += vpart[((size_t)b * Nl + p) * 9 + c];
+#pragma unroll
+  for (int c = 0; c < 9; c++) sh[tid * 9 + c] = v[c];
+  __syncthreads();
+  if (tid < 9) {
+    real t = 0;
+    for (int u = 0; u < F_BLOCK; u++) t += sh[u * 9 + tid];
+    virial[b * 9 + tid] = t;
+  }
+}
+
+// ---------------------------------------------------------------------------
 // pass B: one wave per receiving atom.  Bucket entries (keys p*nr+s of the
 // centre slots that point at this atom) are ranked, the slot forces are placed
 // in rank order and summed with a fixed tree; the centre's own force is added
@@ -376,7 +445,9 @@ __global__ __launch_bounds__(F_BLOCK) void gradforce2_kernel(
     const real* __restrict__ Q, const real* __restrict__ G, const real* __restrict__ D, const real* __restrict__ dD,
     const int* __restrict__ im2, const real* __restrict__ alpha2b, const real* __restrict__ emb2b,
     const int* __restrict__ type_map, const int* __restrict__ tipos, const int* __restrict__ actual_type,
-    real* __restrict__ gnet, real* __restrict__ partial, int nf, int N, int Nl, int ld, int nr, int Ar, int nt) {
+    real* __restrict__ gnet, real* __restrict__ partial, const real* __restrict__ Qvir,
+    const real* __restrict__ pos, const real* __restrict__ box, int nf, int N, int Nl, int ld, int nr, int Ar,
+    int nt) {
   extern __shared__ __align__(16) unsigned char smem[];
   real* p_al = (real*)smem;                     // [nt*Ar]
   real* p_c2 = p_al + nt * Ar;                  // [nt*Ar]
@@ -408,7 +479,17 @@ __global__ __launch_bounds__(F_BLOCK) void gradforce2_kernel(
       const int nj = im[1 + s];
       const real* Qj = Q + ((size_t)b * N + nj) * 3;
       const real* dr = dD + rowAtom * 3 * nr + s;
-      myW[s] = real(0.5) * ((Qj[0] - qi0) * dr[0] + (Qj[1] - qi1) * dr[nr] + (Qj[2] - qi2) * dr[2 * nr]);
+      real q0 = Qj[0] - qi0, q1 = Qj[1] - qi1, q2 = Qj[2] - qi2;
+      if (Qvir) {
+        // virial form: dL/dg_a = (dL/dF_j - dL/dF_i)_a - sum_e (dL/dW)_ae r_e  (grad_force/rad/reforce.cu.cc:213-216)
+        real r[3];
+        mic_cart_from_cart(pos + ((size_t)b * N + p + shift) * 3, pos + ((size_t)b * N + nj) * 3, box + (size_t)b * 6, r);
+        const real* Wg = Qvir + (size_t)b * 9;
+        q0 -= Wg[0] * r[0] + Wg[1] * r[1] + Wg[2] * r[2];
+        q1 -= Wg[3] * r[0] + Wg[4] * r[1] + Wg[5] * r[2];
+        q2 -= Wg[6] * r[0] + Wg[7] * r[1] + Wg[8] * r[2];
+      }
+      myW[s] = real(0.5) * (q0 * dr[0] + q1 * dr[nr] + q2 * dr[2 * nr]);
       myD[s] = D[rowAtom * nr + s];
       myT[s] = type_map[nj];
     }
@@ -460,6 +541,7 @@ static inline int grad_blocks_f(int atoms) {
 struct ForceScratch {
   void* gslot;
   void* self;
+  void* vpart;
   int* bcnt;
   int* bent;
   int cap;
@@ -467,15 +549,28 @@ struct ForceScratch {
 
 template <typename real>
 static int force_scratch(DeviceState* st, int nf, int N, int Nl, int nr, hipStream_t stream, ForceScratch* fs) {
-  const size_t ng = (size_t)nf * Nl * nr * 3, ns = (size_t)nf * Nl * 3;
-  real* base = (real*)scratch_reserve(st, (ng + ns) * sizeof(real));
+  const size_t ng = (size_t)nf * Nl * nr * 3, ns = (size_t)nf * Nl * 3, nv = (size_t)nf * Nl * 9;
+  real* base = (real*)scratch_reserve(st, (ng + ns + nv) * sizeof(real));
   if (!base) return STAF_E_HIP;
   fs->gslot = base;
   fs->self = base + ng;
+  fs->vpart = base + ng + ns;
   fs->cap = 4 * nr;
   fs->bcnt = bucket_reserve(st, (size_t)nf * N, (size_t)nf * N * fs->cap, stream, &fs->bent);
   if (!fs->bcnt) return STAF_E_HIP;
   return STAF_OK;
+}
+
+template <typename real>
+static void launch_virial(const ForceScratch& fs, const int* im2, const int* counts, const real* pos, const real* box,
+                          const int* tipos, const int* actual_type, real* virial, int nf, int N, int Nl, int ld,
+                          int nr, hipStream_t stream) {
+  const int atoms = nf * Nl;
+  hipLaunchKernelGGL(virial_centre_kernel<real>, dim3((atoms + F_WAVES - 1) / F_WAVES), dim3(F_BLOCK), 0, stream,
+                     (const real*)fs.gslot, im2, counts, pos, box, tipos, actual_type, (real*)fs.vpart, nf, N, Nl,
+                     ld, nr);
+  hipLaunchKernelGGL(virial_frame_kernel<real>, dim3(nf), dim3(F_BLOCK), 0, stream, (const real*)fs.vpart, virial,
+                     Nl);
 }
 
 template <typename real>
@@ -498,7 +593,7 @@ static int force_doublets(const real* G, const real* D, const real* dD, const in
   if (!G || !D || !dD || !im2 || !alpha2b || !emb2b || !tipos || !actual_type || !force || !type_map || nr <= 0 ||
       N <= 0 || nf <= 0 || Ar <= 0 || nt <= 0 || Nl <= 0 || Nl > N)
     return STAF_E_BAD_ARG;
-  if (virial || pos || box) return STAF_E_LIMIT;  // virial form: not built yet
+  if ((virial || pos || box) && !(virial && pos && box)) return STAF_E_BAD_ARG;
   if (nt > NT_MAX) return STAF_E_LIMIT;
   if (ld <= 0) ld = Nl;
   DeviceState* st = device_state();
@@ -513,6 +608,8 @@ static int force_doublets(const real* G, const real* D, const real* dD, const in
   hipLaunchKernelGGL(force2_kernel<real>, dim3((atoms + F_WAVES - 1) / F_WAVES), dim3(F_BLOCK), lds, stream, G, D, dD,
                      im2, alpha2b, emb2b, type_map, (real*)fs.gslot, (real*)fs.self, fs.bcnt, fs.bent, fs.cap,
                      st->status_d, nf, N, Nl, ld, nr, Ar, nt);
+  if (virial)
+    launch_virial<real>(fs, im2, (const int*)nullptr, pos, box, tipos, actual_type, virial, nf, N, Nl, ld, nr, stream);
   return launch_gather<real>(st, fs, tipos, actual_type, force, nf, N, Nl, nr, stream);
 }
 
@@ -526,7 +623,7 @@ static int force_tripl(const real* G, const real* Dsup, const real* Tang, const 
   if (!G || !Dsup || !Tang || !dDsup || !d3b || !im2 || !emb3b || !tipos || !actual_type || !force || !numtriplet ||
       !alpha3b || !type_map || nr <= 0 || na <= 0 || N <= 0 || nf <= 0 || Aa <= 0 || nt <= 0 || Nl <= 0 || Nl > N)
     return STAF_E_BAD_ARG;
-  if (virial || pos || box) return STAF_E_LIMIT;  // virial form: not built yet
+  if ((virial || pos || box) && !(virial && pos && box)) return STAF_E_BAD_ARG;
   if (nt > NT_MAX) return STAF_E_LIMIT;
   if (ld <= 0) ld = Nl;
   DeviceState* st = device_state();
@@ -545,6 +642,8 @@ static int force_tripl(const real* G, const real* Dsup, const real* Tang, const 
   hipLaunchKernelGGL(force3_kernel<real>, dim3(nf * Nl), dim3(Force3Lds<real>::THREADS), lds, stream, G, Dsup, Tang, dDsup, d3b, im2,
                      alpha3b, emb3b, type_map, numtriplet, (real*)fs.gslot, (real*)fs.self, fs.bcnt, fs.bent, fs.cap,
                      st->status_d, nf, N, Nl, ld, nr, na, Aa, nt);
+  if (virial)
+    launch_virial<real>(fs, im2, numtriplet, pos, box, tipos, actual_type, virial, nf, N, Nl, ld, nr, stream);
   return launch_gather<real>(st, fs, tipos, actual_type, force, nf, N, Nl, nr, stream);
 }
 
@@ -556,7 +655,7 @@ static int gradforce_2b(const real* Q, const real* D, int nr, const real* alpha2
   if (!Q || !D || !alpha2b || !dD || !im2 || !G || !emb2b || !type_map || !tipos || !actual_type || !gnet ||
       !g_alpha || !g_emb || nr <= 0 || Ar <= 0 || nf <= 0 || N <= 0 || Nl <= 0 || Nl > N || nt <= 0)
     return STAF_E_BAD_ARG;
-  if (Qvir || pos || box) return STAF_E_LIMIT;  // virial form: not built yet
+  if ((Qvir || pos || box) && !(Qvir && pos && box)) return STAF_E_BAD_ARG;
   if (nt > NT_MAX) return STAF_E_LIMIT;
   if (ld <= 0) ld = Nl;
   DeviceState* st = device_state();
@@ -570,7 +669,7 @@ static int gradforce_2b(const real* Q, const real* D, int nr, const real* alpha2
                (size_t)F_WAVES * nr * sizeof(int);
   if (lds > 64 * 1024) return STAF_E_LIMIT;
   hipLaunchKernelGGL(gradforce2_kernel<real>, dim3(nb), dim3(F_BLOCK), lds, stream, Q, G, D, dD, im2, alpha2b, emb2b,
-                     type_map, tipos, actual_type, gnet, partial, nf, N, Nl, ld, nr, Ar, nt);
+                     type_map, tipos, actual_type, gnet, partial, Qvir, pos, box, nf, N, Nl, ld, nr, Ar, nt);
   launch_reduce_partials<real>(partial, nb, nout, g_alpha, nt * Ar, g_emb, nt * Ar, stream);
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }
@@ -586,7 +685,7 @@ static int gradforce_tripl(const real* Q, const real* G, const real* Dsup, const
       !alpha3b || !type_map || !gnet || !g_alpha || !g_emb || nr <= 0 || na <= 0 || N <= 0 || nf <= 0 || Aa <= 0 ||
       nt <= 0 || Nl <= 0 || Nl > N)
     return STAF_E_BAD_ARG;
-  if (Qvir || pos || box) return STAF_E_LIMIT;  // virial form: not built yet
+  if ((Qvir || pos || box) && !(Qvir && pos && box)) return STAF_E_BAD_ARG;
   if (nt > NT_MAX) return STAF_E_LIMIT;
   if (ld <= 0) ld = Nl;
   DeviceState* st = device_state();
@@ -606,7 +705,7 @@ static int gradforce_tripl(const real* Q, const real* G, const real* Dsup, const
   TriArgs<real> A = {};
   A.Dsup = Dsup; A.Tang = Tang; A.im2 = im2; A.alpha3b = alpha3b; A.emb3b = emb3b; A.type_map = type_map;
   A.numtriplet = numtriplet; A.P = G; A.Q = Q; A.dDsup = dDsup; A.d3b = d3b; A.tipos = tipos;
-  A.actual_type = actual_type; A.out = gnet; A.partial = partial;
+  A.actual_type = actual_type; A.out = gnet; A.partial = partial; A.Qvir = Qvir; A.pos = pos; A.box = box;
   A.nf = nf; A.N = N; A.Nl = Nl; A.ld = ld; A.nr = nr; A.na = na; A.Aa = Aa; A.nt = nt;
   hipLaunchKernelGGL((tri_reduce_kernel<real, 2>), dim3(nb), dim3(TRI_BLOCK), lds, stream, A);
   launch_reduce_partials<real>(partial, nb, nout, g_alpha, nout, (real*)nullptr, 0, stream);

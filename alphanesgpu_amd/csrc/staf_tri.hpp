@@ -44,6 +44,9 @@ struct TriArgs {
   const real* d3b;        // MODE 2: der3b [nf, ld, 3, na, 2]
   const int* tipos;       // MODE 2
   const int* actual_type; // MODE 2
+  const real* Qvir;       // MODE 2, virial form: dL/dW [nf, 9] (else null)
+  const real* pos;        // MODE 2, virial form: positions [nf, 3N]
+  const real* box;        // MODE 2, virial form: [nf, 6]
   real* out;              // MODE 0: AF3, MODE 2: gradnet  [nf, Nl, Aa] contiguous
   real* partial;          // MODE 1/2: [gridDim.x, nsig*Aa*3]
   int nf, N, Nl, ld, nr, na, Aa, nt;
@@ -128,7 +131,17 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
       if (MODE == 2) {
         const real* Qj = A.Q + ((size_t)b * A.N + nj) * 3;
         const real* Qi = A.Q + ((size_t)b * A.N + p + shift) * 3;
-        const real q0 = Qj[0] - Qi[0], q1 = Qj[1] - Qi[1], q2 = Qj[2] - Qi[2];
+        real q0 = Qj[0] - Qi[0], q1 = Qj[1] - Qi[1], q2 = Qj[2] - Qi[2];
+        if (A.Qvir) {
+          // virial form: dL/dg_a = (dL/dF_j - dL/dF_i)_a - sum_e (dL/dW)_ae r_e (grad_force/ang/reforce.cu.cc:391-394)
+          real r[3];
+          mic_cart_from_cart(A.pos + ((size_t)b * A.N + p + shift) * 3, A.pos + ((size_t)b * A.N + nj) * 3,
+                             A.box + (size_t)b * 6, r);
+          const real* Wg = A.Qvir + (size_t)b * 9;
+          q0 -= Wg[0] * r[0] + Wg[1] * r[1] + Wg[2] * r[2];
+          q1 -= Wg[3] * r[0] + Wg[4] * r[1] + Wg[5] * r[2];
+          q2 -= Wg[6] * r[0] + Wg[7] * r[1] + Wg[8] * r[2];
+        }
         const real* gr = A.dDsup + rowAtom * 3 * nr + s;
         sQ[3 * s] = q0; sQ[3 * s + 1] = q1; sQ[3 * s + 2] = q2;
         sV[s] = q0 * gr[0] + q1 * gr[nr] + q2 * gr[2 * nr];

@@ -408,3 +408,23 @@ def compute_force_tripl_grad(prevgrad, netderiv, radial_descriptor, angular_desc
          ptr(None if prevgrad_virial is None else _dense(prevgrad_virial)),
          ptr(None if pos is None else _dense(pos)), ptr(None if box is None else _dense(box)), _I(v.ld), _stream())
     return gn, ga, ge
+
+
+def compute_force_radial_virial_grad(prevgrad, prevgrad_virial, netderiv, descriptor_derivative_rad,
+                                     interaction_map_rad, radial_descriptor, alpha2b_parameters,
+                                     type_emb2b_parameters, type_map, tipos, actual_type, pos, box):
+    """ComputeForceRadialVirialGrad (STAF/src/grad_force/rad/reforce.cc:160-176)."""
+    return compute_force_radial_grad(prevgrad, netderiv, descriptor_derivative_rad, interaction_map_rad,
+                                     radial_descriptor, alpha2b_parameters, type_emb2b_parameters, type_map, tipos,
+                                     actual_type, prevgrad_virial, pos, box)
+
+
+def compute_force_tripl_virial_grad(prevgrad, prevgrad_virial, netderiv, radial_descriptor, angular_descriptor,
+                                    descriptor_derivative_rad, descriptor_derivative_ang, interaction_map_rad,
+                                    interaction_map_ang, alpha3b_parameters, type_emb3b_parameters, type_map, tipos,
+                                    actual_type, num_triplets, pos, box):
+    """ComputeForceTriplVirialGrad (STAF/src/grad_force/ang/reforce.cc:186-206)."""
+    return compute_force_tripl_grad(prevgrad, netderiv, radial_descriptor, angular_descriptor,
+                                    descriptor_derivative_rad, descriptor_derivative_ang, interaction_map_rad,
+                                    interaction_map_ang, alpha3b_parameters, type_emb3b_parameters, type_map, tipos,
+                                    actual_type, num_triplets, prevgrad_virial, pos, box)

@@ -210,3 +210,63 @@ def test_full_size_properties(oracle):
             assert abs(lhs - rhs) <= 1e-10 * max(abs(lhs), 1.0), (key, k, lhs, rhs)
     ntr = got["desc"]["numtriplet"]
     assert got["desc"]["intmap2b"][..., 0].max() <= NR and (ntr * (ntr - 1) // 2).max() <= NA
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_virial_forms(oracle, dtype):
+    """ComputeForce{Radial,Tripl}Virial and their *VirialGrad ops against the oracle: forces unchanged, W [nf,9],
+    and gradients with a non-zero dL/dW.  Two frames of the 768-atom generator (periodic images matter)."""
+    import torch
+    from alphanesgpu_amd import ops
+    from util import species_slices
+    dtype = np.dtype(dtype)
+    tol = TOL[dtype]
+    b = _synth("water768_f64", nf=2)
+    params = _params(dtype, dense=True)
+    pos, box = b["pos"].astype(dtype), b["box"].astype(dtype)
+    nf = 2
+    up = pipeline.synthetic_upstream(nf, b["tipos"], params, 21, dtype)
+    rng = np.random.Generator(np.random.Philox(5))
+    Wg = rng.standard_normal((nf, 9)).astype(dtype)
+    d = oracle.compute_descriptors_light(pos, box, 4.5, 4.5, 2.25, NR, NA, dtype=dtype)
+    dev = torch.device("cuda:0")
+    T = lambda a: torch.as_tensor(np.ascontiguousarray(a)).to(dev)
+    tdt = torch.float32 if dtype == np.float32 else torch.float64
+    ops.construct_descriptors_light(4.5, NR, NA, b["N"], None, 2.25, 4.5, nf, dtype=tdt)
+    ops.descriptor_options(False, True)
+    names = ["raddescr", "angdescr", "des3bsupp", "intmap2b", "intmap3b", "der2b", "der3b", "der3bsupp", "numtriplet"]
+    g = dict(zip(names, ops.compute_descriptors_light(T(pos), T(box))))
+    tm, tp = T(b["type_map"]), T(b["tipos"])
+    Q, tWg, tpos, tbox = T(up["Q"]), T(Wg), T(pos), T(box)
+    P64 = lambda x: x.astype(np.float64)
+    for k, s in enumerate(species_slices(b["tipos"])):
+        m = params[k]
+        c = lambda a: np.ascontiguousarray(a[:, s])
+        v = lambda key: g[key][:, s]
+        tk = {kk: T(vv) for kk, vv in m.items()}
+        at = torch.tensor([k], dtype=torch.int32, device=dev)
+        a2 = (c(d["der2b"]), c(d["intmap2b"]), c(d["raddescr"]), m["alpha2b"], m["emb2b"], b["type_map"], b["tipos"], k)
+        a3 = (c(d["des3bsupp"]), c(d["angdescr"]), c(d["der3bsupp"]), c(d["der3b"]), c(d["intmap2b"]),
+              c(d["intmap3b"]), m["alpha3b"], m["emb3b"], b["type_map"], b["tipos"], k, c(d["numtriplet"]))
+        f2r, w2r = oracle.force_radial(up["G2"][k], *a2, pos=pos, box=box)
+        f3r, w3r = oracle.force_tripl(up["G3"][k], *a3, pos=pos, box=box)
+        g2r = oracle.force_radial_grad(up["Q"], up["G2"][k], *a2, prevgrad_virial=Wg, pos=pos, box=box)
+        g3r = oracle.force_tripl_grad(up["Q"], up["G3"][k], *a3, prevgrad_virial=Wg, pos=pos, box=box)
+        f2, w2 = ops.compute_force_radial_virial(T(up["G2"][k]), v("der2b"), v("intmap2b"), v("raddescr"),
+                                                 tk["alpha2b"], tk["emb2b"], tm, tp, at, tpos, tbox)
+        f3, w3 = ops.compute_force_tripl_virial(T(up["G3"][k]), v("des3bsupp"), v("angdescr"), v("der3bsupp"),
+                                                v("der3b"), v("intmap2b"), v("intmap3b"), tk["alpha3b"], tk["emb3b"],
+                                                tm, tp, at, v("numtriplet"), tpos, tbox)
+        g2 = ops.compute_force_radial_virial_grad(Q, tWg, T(up["G2"][k]), v("der2b"), v("intmap2b"), v("raddescr"),
+                                                  tk["alpha2b"], tk["emb2b"], tm, tp, at, tpos, tbox)
+        g3 = ops.compute_force_tripl_virial_grad(Q, tWg, T(up["G3"][k]), v("des3bsupp"), v("angdescr"),
+                                                 v("der3bsupp"), v("der3b"), v("intmap2b"), v("intmap3b"),
+                                                 tk["alpha3b"], tk["emb3b"], tm, tp, at, v("numtriplet"), tpos, tbox)
+        # fp32 long sums: allow the fp32 oracle's own summation error on top of the tolerance (see compare())
+        slack = 0.0 if dtype == np.float64 else 2e-5
+        for name, x, y in (("f2", f2, f2r), ("w2", w2, w2r), ("f3", f3, f3r), ("w3", w3, w3r),
+                           ("g2.net", g2[0], g2r[0]), ("g2.alpha", g2[1], g2r[1]), ("g2.emb", g2[2], g2r[2]),
+                           ("g3.net", g3[0], g3r[0]), ("g3.alpha", g3[1], g3r[1])):
+            e = nerr(x.cpu().numpy(), y)
+            assert e <= tol + slack, (name, k, e)
+        assert torch.all(g3[2] == 0)
