@@ -14,8 +14,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libstaf_hip.so")
-SOURCES = ["staf_runtime.hip", "staf_desc.hip", "staf_af.hip", "staf_force.hip"]
-HEADERS = ["staf_common.hpp", "staf_tile.hpp", "staf_reduce.hpp", "staf_tri.hpp", os.path.join("..", "..", "include", "staf_ops.h")]
+SOURCES = ["staf_runtime.hip", "staf_desc.hip", "staf_af.hip", "staf_force.hip", "staf_api.hip", "staf_mlp.cpp"]
+HEADERS = ["staf_common.hpp", "staf_tile.hpp", "staf_reduce.hpp", "staf_tri.hpp", os.path.join("..", "..", "include", "staf_ops.h"),
+           os.path.join("..", "..", "include", "staf.h"), os.path.join("..", "..", "include", "staf_mlp.h")]
 ARCH = "gfx950"
 # packed-fp32 instructions are switched off for all device code
 HIPCC_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",
@@ -45,7 +46,7 @@ def build(force=False, verbose=True):
     objs = []
     for s in SOURCES:
         src = os.path.join(CSRC, s)
-        obj = os.path.join(objdir, s.replace(".hip", ".o"))
+        obj = os.path.join(objdir, os.path.splitext(s)[0] + ".o")
         objs.append(obj)
         if force or _stale(obj, [src] + hdrs):
             jobs.append([_hipcc()] + HIPCC_FLAGS + ["-c", src, "-o", obj])

@@ -1,0 +1,465 @@
+// MD-facing entry (LAMMPS `pair_style staf`): staf_load / staf_compute / staf_free of include/staf.h.
+//
+// Host logic follows libstaf/src/staf_api.cpp:192-412 (validation and return codes, species-sorted packing of
+// the owned atoms, ghosts appended, neighbour-index remapping, un-packing of forces) and the step order of
+// calculateforces (libstaf/vendor/jmd/nn_nn_mlp.cu:838-889): neighbour list (own, or the caller's with no
+// periodic wrap) -> descriptors -> fingerprints of every species -> MLP -> 2-body + 3-body forces with virial.
+// Everything on the GPU runs in float64 through the same kernels as the training ops; the MLP is the per-species
+// Dense stack of staf_mlp.cpp evaluated on the host between the fingerprint and the force kernels.
+#include "staf_common.hpp"
+#include "staf_reduce.hpp"
+#include "../../include/staf.h"
+#include "../../include/staf_mlp.h"
+
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <string>
+#include <vector>
+
+extern "C" void staf_op_force_set_skip_pbc(int skip);
+
+namespace {
+
+template <typename T>
+struct DevBuf {
+  T* p = nullptr;
+  size_t n = 0;
+  bool reserve(size_t want) {
+    if (want <= n) return true;
+    if (p) (void)hipFree(p);
+    p = nullptr;
+    n = 0;
+    if (hipMalloc((void**)&p, want * sizeof(T)) != hipSuccess) return false;
+    n = want;
+    return true;
+  }
+  void release() {
+    if (p) (void)hipFree(p);
+    p = nullptr;
+    n = 0;
+  }
+};
+
+__global__ void add_into_kernel(double* dst, const double* src, int n) {
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e < n) dst[e] += src[e];
+}
+
+bool read_numbers(const std::string& path, std::vector<double>& out, int* rows) {
+  FILE* f = fopen(path.c_str(), "r");
+  if (!f) return false;
+  out.clear();
+  int nrows = 0;
+  char line[1 << 16];
+  while (fgets(line, sizeof(line), f)) {
+    char* s = line;
+    int got = 0;
+    for (;;) {
+      char* e;
+      double v = strtod(s, &e);
+      if (e == s) break;
+      out.push_back(v);
+      s = e;
+      got++;
+    }
+    if (got) nrows++;
+  }
+  fclose(f);
+  if (rows) *rows = nrows;
+  return !out.empty();
+}
+
+}  // namespace
+
+struct StafModel {
+  StafOptions opt;
+  std::string dir;
+  StafMlp* mlp = nullptr;
+  int nt = 0, ntc = 0, nr = 60, na = 1770;
+  double Rc = 4.5, Ra = 4.5, Rs = 2.25;
+  std::vector<int> Ar, Aa;
+  std::vector<DevBuf<double>> alpha2b, alpha3b, emb2b, emb3b;
+  staf::DescConfig<double> cfg;
+  hipStream_t stream = nullptr;
+  // device buffers
+  DevBuf<double> pos, box, force, force_op, virial_op, af2, af3, g2, g3;
+  DevBuf<double> raddescr, angdescr, des3bsupp, der2b, der3b, der3bsupp;
+  DevBuf<int> intmap2b, intmap3b, numtriplet, type_map, tipos, actual_type, how, with;
+  // host staging
+  std::vector<double> pos_h, force_h, af_h, gr_h, tmp2, tmp3;
+  std::vector<float> af_f, gr_f;
+  std::vector<int> order_to_slot, slot_to_order, type_map_h, how_h, with_h;
+};
+
+static bool load_species_params(StafModel* m) {
+  const int nt = m->nt, ntc = m->ntc;
+  m->Ar.assign(nt, 0);
+  m->Aa.assign(nt, 0);
+  m->alpha2b.resize(nt);
+  m->alpha3b.resize(nt);
+  m->emb2b.resize(nt);
+  m->emb3b.resize(nt);
+  for (int k = 0; k < nt; k++) {
+    const std::string pre = m->dir + "/type" + std::to_string(k) + "_";
+    std::vector<double> a2, a3, e2, e3;
+    int rows = 0;
+    if (!read_numbers(pre + "alpha_2body.dat", a2, &rows) || rows != nt || a2.size() % nt) return false;
+    if (!read_numbers(pre + "alpha_3body.dat", a3, &rows) || rows != ntc || a3.size() % (3 * ntc)) return false;
+    m->Ar[k] = (int)(a2.size() / nt);
+    m->Aa[k] = (int)(a3.size() / (3 * ntc));
+    // the kernels take the squared embeddings (what the reference's Python layers feed its ops)
+    if (!read_numbers(pre + "type_emb_2b_sq.dat", e2, nullptr)) {
+      if (!read_numbers(pre + "type_emb_2b.dat", e2, nullptr)) return false;
+      for (double& v : e2) v *= v;
+    }
+    if (!read_numbers(pre + "type_emb_3b_sq.dat", e3, nullptr)) {
+      if (!read_numbers(pre + "type_emb_3b.dat", e3, nullptr)) return false;
+      for (double& v : e3) v *= v;
+    }
+    if ((int)e2.size() != nt * m->Ar[k] || (int)e3.size() != ntc * m->Aa[k]) return false;
+    struct { DevBuf<double>* d; std::vector<double>* h; } up[4] = {
+        {&m->alpha2b[k], &a2}, {&m->alpha3b[k], &a3}, {&m->emb2b[k], &e2}, {&m->emb3b[k], &e3}};
+    for (auto& u : up) {
+      if (!u.d->reserve(u.h->size())) return false;
+      if (hipMemcpy(u.d->p, u.h->data(), u.h->size() * sizeof(double), hipMemcpyHostToDevice) != hipSuccess)
+        return false;
+    }
+  }
+  return true;
+}
+
+// staf_jmd.cfg: "key = value" lines (test/test-lammps-smoke/staf_jmd.cfg); missing file or keys -> the defaults
+// the reference writes into its auto-generated cfg (libstaf/src/staf_api.cpp:139-148).
+static void read_cfg(StafModel* m) {
+  FILE* f = fopen((m->dir + "/staf_jmd.cfg").c_str(), "r");
+  if (!f) return;
+  char line[4096];
+  while (fgets(line, sizeof(line), f)) {
+    char key[256];
+    double v;
+    if (sscanf(line, " %255[A-Za-z_] = %lf", key, &v) != 2) continue;
+    if (!strcmp(key, "Buffer_radial_descriptors")) m->nr = (int)v;
+    else if (!strcmp(key, "Buffer_angular_descriptors")) m->na = (int)v;
+    else if (!strcmp(key, "Cutoff")) m->Rc = v;
+    else if (!strcmp(key, "Cutoff_Angular")) m->Ra = v;
+    else if (!strcmp(key, "Hardcore_Cutoff")) m->Rs = v;
+    else if (!strcmp(key, "number_of_types")) m->nt = (int)v;
+  }
+  fclose(f);
+}
+
+extern "C" {
+
+void staf_options_default(StafOptions* opt) {
+  if (!opt) return;
+  memset(opt, 0, sizeof(*opt));
+  opt->mlp_backend = STAF_MLP_ORT;
+  opt->device_id = 0;
+  opt->precision = 0;
+}
+
+int staf_cuda_set_device(int device_id) {
+  int ndev = 0;
+  if (hipGetDeviceCount(&ndev) != hipSuccess || ndev <= 0) {
+    fprintf(stderr, "staf_cuda_set_device: no GPU\n");
+    return -1;
+  }
+  if (device_id < 0) device_id = 0;
+  device_id %= ndev;
+  if (hipSetDevice(device_id) != hipSuccess) return -1;
+  return device_id;
+}
+
+void staf_free(StafModel* m) {
+  if (!m) return;
+  if (m->mlp) staf_mlp_destroy(m->mlp);
+  for (auto* v : {&m->alpha2b, &m->alpha3b, &m->emb2b, &m->emb3b})
+    for (auto& b : *v) b.release();
+  for (DevBuf<double>* b : {&m->pos, &m->box, &m->force, &m->force_op, &m->virial_op, &m->af2, &m->af3, &m->g2, &m->g3,
+                            &m->raddescr, &m->angdescr, &m->des3bsupp, &m->der2b, &m->der3b, &m->der3bsupp})
+    b->release();
+  for (DevBuf<int>* b : {&m->intmap2b, &m->intmap3b, &m->numtriplet, &m->type_map, &m->tipos, &m->actual_type, &m->how,
+                         &m->with})
+    b->release();
+  delete m;
+}
+
+StafModel* staf_load(const char* model_dir, const StafOptions* opt) {
+  if (!model_dir) return NULL;
+  StafModel* m = new StafModel();
+  staf_options_default(&m->opt);
+  if (opt) m->opt = *opt;
+  const int dev = staf_cuda_set_device(m->opt.device_id);
+  if (dev < 0) { delete m; return NULL; }
+  m->opt.device_id = dev;
+  m->dir = model_dir;
+  m->mlp = staf_mlp_create(m->opt.mlp_backend, model_dir, m->opt.precision, dev);
+  if (!m->mlp) {
+    fprintf(stderr, "staf_load: staf_mlp_create failed for %s\n", model_dir);
+    staf_free(m);
+    return NULL;
+  }
+  m->nt = staf_mlp_ntypes(m->mlp);
+  read_cfg(m);
+  if (m->nt != staf_mlp_ntypes(m->mlp) || m->nt < 1 || m->nt > staf::NT_MAX) {
+    fprintf(stderr, "staf_load: %d species in staf_jmd.cfg, %d MLP files\n", m->nt, staf_mlp_ntypes(m->mlp));
+    staf_free(m);
+    return NULL;
+  }
+  m->ntc = m->nt * (m->nt + 1) / 2;
+  if (!load_species_params(m)) {
+    fprintf(stderr, "staf_load: cannot read the type*_alpha_*.dat / type*_type_emb_*.dat files of %s\n", model_dir);
+    staf_free(m);
+    return NULL;
+  }
+  for (int k = 0; k < m->nt; k++)
+    if (staf_mlp_n_af(m->mlp, k) != m->Ar[k] + m->Aa[k]) {
+      fprintf(stderr, "staf_load: species %d: MLP input width %d != %d + %d fingerprints\n", k,
+              staf_mlp_n_af(m->mlp, k), m->Ar[k], m->Aa[k]);
+      staf_free(m);
+      return NULL;
+    }
+  if (staf::desc_configure<double>(m->cfg, m->Rc, m->nr, m->na, m->Rs, m->Ra) != STAF_OK) {
+    staf_free(m);
+    return NULL;
+  }
+  return m;
+}
+
+#define STAF_HIP_OK(x) do { if ((x) != hipSuccess) return -20; } while (0)
+
+int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const double* box, const int* type,
+                 const int* howmany, const int* with, int maxneigh, double* e_rank, double* f, double* virial) {
+  if (!m || !m->mlp) return -1;
+  const bool ext = (howmany != NULL);
+  const int nall = ext ? (nlocal + nghost) : nlocal;
+  if (nlocal <= 0) return -3;
+  if (!x || !box || (ext && !with)) return -1;
+  if (box[0] == 0.0 || box[3] == 0.0 || box[5] == 0.0) return -7;
+  if (hipSetDevice(m->opt.device_id) != hipSuccess) return -20;
+  const int nt = m->nt, nr = m->nr, na = m->na;
+
+  // ---- owned atoms species-sorted into slots [0, nlocal), ghosts keep their order behind them
+  std::vector<int> tipos(nt, 0), cursor(nt, 0);
+  for (int i = 0; i < nlocal; i++) {
+    const int sp = type ? type[i] : 0;
+    if (sp < 0 || sp >= nt) {
+      fprintf(stderr, "staf_compute: unsupported type %d at atom %d\n", sp, i);
+      return -8;
+    }
+    tipos[sp]++;
+  }
+  for (int t = 1; t < nt; t++) cursor[t] = cursor[t - 1] + tipos[t - 1];
+  m->order_to_slot.resize(nall);
+  m->slot_to_order.resize(nall);
+  m->type_map_h.resize(nall);
+  for (int i = 0; i < nlocal; i++) {
+    const int sp = type ? type[i] : 0;
+    const int slot = cursor[sp]++;
+    m->order_to_slot[i] = slot;
+    m->slot_to_order[slot] = i;
+    m->type_map_h[slot] = sp;
+  }
+  for (int i = nlocal; i < nall; i++) {
+    const int sp = type ? type[i] : 0;
+    if (sp < 0 || sp >= nt) return -8;
+    m->order_to_slot[i] = i;
+    m->slot_to_order[i] = i;
+    m->type_map_h[i] = sp;
+  }
+  if (ext) {
+    m->how_h.assign(nlocal, 0);
+    m->with_h.assign((size_t)nlocal * nr, 0);
+    for (int i = 0; i < nlocal; i++) {
+      const int slot = m->order_to_slot[i];
+      int nn = howmany[i];
+      if (nn < 0) nn = 0;
+      if (nn > nr) nn = nr;   // truncated like the reference (staf_api.cpp:321-323)
+      if (nn > maxneigh) nn = maxneigh;
+      m->how_h[slot] = nn;
+      for (int k = 0; k < nn; k++) {
+        const int j = with[(size_t)i * maxneigh + k];
+        if (j < 0 || j >= nall) {
+          fprintf(stderr, "staf_compute: neighbor index %d out of range [0,%d)\n", j, nall);
+          return -9;
+        }
+        m->with_h[(size_t)slot * nr + k] = m->order_to_slot[j];
+      }
+    }
+  }
+  m->pos_h.resize((size_t)nall * 3);
+  for (int i = 0; i < nall; i++) {
+    const int s = m->order_to_slot[i];
+    m->pos_h[3 * s] = x[3 * i];
+    m->pos_h[3 * s + 1] = x[3 * i + 1];
+    m->pos_h[3 * s + 2] = x[3 * i + 2];
+  }
+
+  // ---- device buffers
+  const size_t L = (size_t)nlocal;
+  int amax2 = 0, amax3 = 0;
+  for (int k = 0; k < nt; k++) { amax2 = m->Ar[k] > amax2 ? m->Ar[k] : amax2; amax3 = m->Aa[k] > amax3 ? m->Aa[k] : amax3; }
+  bool ok = m->pos.reserve((size_t)nall * 3) && m->box.reserve(6) && m->force.reserve((size_t)nall * 3) &&
+            m->force_op.reserve((size_t)nall * 3) && m->virial_op.reserve(9) && m->af2.reserve(L * amax2) &&
+            m->af3.reserve(L * amax3) && m->g2.reserve(L * amax2) && m->g3.reserve(L * amax3) &&
+            m->raddescr.reserve(L * nr) && m->angdescr.reserve(L * na) && m->des3bsupp.reserve(L * nr) &&
+            m->der2b.reserve(L * 3 * nr) && m->der3b.reserve(L * 6 * na) && m->der3bsupp.reserve(L * 3 * nr) &&
+            m->intmap2b.reserve(L * (nr + 1)) && m->intmap3b.reserve(L * 2 * na) && m->numtriplet.reserve(L) &&
+            m->type_map.reserve(nall) && m->tipos.reserve(nt) && m->actual_type.reserve(nt) &&
+            (!ext || (m->how.reserve(L) && m->with.reserve(L * nr)));
+  if (!ok) return -1;
+  hipStream_t st = m->stream;
+  STAF_HIP_OK(hipMemcpyAsync(m->pos.p, m->pos_h.data(), (size_t)nall * 3 * sizeof(double), hipMemcpyHostToDevice, st));
+  STAF_HIP_OK(hipMemcpyAsync(m->box.p, box, 6 * sizeof(double), hipMemcpyHostToDevice, st));
+  STAF_HIP_OK(hipMemcpyAsync(m->type_map.p, m->type_map_h.data(), (size_t)nall * sizeof(int), hipMemcpyHostToDevice, st));
+  STAF_HIP_OK(hipMemcpyAsync(m->tipos.p, tipos.data(), nt * sizeof(int), hipMemcpyHostToDevice, st));
+  std::vector<int> ats(nt);
+  for (int k = 0; k < nt; k++) ats[k] = k;
+  STAF_HIP_OK(hipMemcpyAsync(m->actual_type.p, ats.data(), nt * sizeof(int), hipMemcpyHostToDevice, st));
+  if (ext) {
+    STAF_HIP_OK(hipMemcpyAsync(m->how.p, m->how_h.data(), L * sizeof(int), hipMemcpyHostToDevice, st));
+    STAF_HIP_OK(hipMemcpyAsync(m->with.p, m->with_h.data(), L * nr * sizeof(int), hipMemcpyHostToDevice, st));
+  }
+  STAF_HIP_OK(hipStreamSynchronize(st));   // the host vectors above may be reused by the next call
+
+  // ---- descriptors (own minimum-image list, or the caller's list with explicit images)
+  int rc = staf::desc_launch<double>(m->cfg, m->pos.p, m->box.p, 1, nlocal, nall, ext ? m->how.p : nullptr,
+                                     ext ? m->with.p : nullptr, ext ? 1 : 0, m->raddescr.p, m->angdescr.p,
+                                     m->des3bsupp.p, m->intmap2b.p, m->intmap3b.p, m->der2b.p, m->der3b.p,
+                                     m->der3bsupp.p, m->numtriplet.p, st);
+  if (rc == STAF_OK && !staf::sync_errors_enabled()) rc = staf_ops_poll_status(st);
+  if (rc == STAF_E_RADIAL_OVERFLOW) return -10;
+  if (rc != STAF_OK) return -20;
+
+  // ---- fingerprints of every species, packed rows [Ar+Aa] for the MLP
+  size_t total = 0;
+  for (int k = 0; k < nt; k++) total += (size_t)tipos[k] * (m->Ar[k] + m->Aa[k]);
+  m->af_h.resize(total);
+  m->gr_h.assign(total, 0.0);
+  size_t off = 0;
+  int shift = 0;
+  for (int k = 0; k < nt; shift += tipos[k], k++) {
+    const int Nl = tipos[k], Ar = m->Ar[k], Aa = m->Aa[k];
+    if (Nl == 0) continue;
+    const size_t o = (size_t)shift;
+    rc = staf_op_radial_afs_f64(m->raddescr.p + o * nr, nr, m->alpha2b[k].p, Ar, m->af2.p, 1, Nl,
+                                m->intmap2b.p + o * (nr + 1), m->emb2b[k].p, m->type_map.p, nt, nlocal, st);
+    if (rc == STAF_OK)
+      rc = staf_op_angular_afs_f64(m->des3bsupp.p + o * nr, m->angdescr.p + o * na, nr, na, m->af3.p, 1, Nl,
+                                   m->intmap3b.p + o * 2 * na, m->intmap2b.p + o * (nr + 1), m->alpha3b[k].p, Aa,
+                                   m->emb3b[k].p, m->type_map.p, m->numtriplet.p + o, nt, nlocal, st);
+    if (rc != STAF_OK) return -20;
+    m->tmp2.resize((size_t)Nl * Ar);
+    m->tmp3.resize((size_t)Nl * Aa);
+    STAF_HIP_OK(hipMemcpyAsync(m->tmp2.data(), m->af2.p, m->tmp2.size() * sizeof(double), hipMemcpyDeviceToHost, st));
+    STAF_HIP_OK(hipMemcpyAsync(m->tmp3.data(), m->af3.p, m->tmp3.size() * sizeof(double), hipMemcpyDeviceToHost, st));
+    STAF_HIP_OK(hipStreamSynchronize(st));
+    for (int a = 0; a < Nl; a++) {
+      double* row = &m->af_h[off + (size_t)a * (Ar + Aa)];
+      memcpy(row, &m->tmp2[(size_t)a * Ar], Ar * sizeof(double));
+      memcpy(row + Ar, &m->tmp3[(size_t)a * Aa], Aa * sizeof(double));
+    }
+    off += (size_t)Nl * (Ar + Aa);
+  }
+
+  // ---- MLP on the host (libstaf/vendor/jmd/nn_nn_mlp.cu:657-768): float32 nets see float32 fingerprints
+  std::vector<int> n_af(nt);
+  for (int k = 0; k < nt; k++) n_af[k] = m->Ar[k] + m->Aa[k];
+  StafMlpEval ev;
+  memset(&ev, 0, sizeof(ev));
+  ev.n_type = nt;
+  ev.n_atoms = tipos.data();
+  ev.n_af = n_af.data();
+  double energy = 0.0;
+  if (staf_mlp_precision(m->mlp) == 0) {
+    m->af_f.resize(total);
+    m->gr_f.assign(total, 0.f);
+    for (size_t i = 0; i < total; i++) m->af_f[i] = (float)m->af_h[i];
+    float e_f = 0.f;
+    ev.af_f32 = m->af_f.data();
+    ev.energy_f32 = &e_f;
+    ev.dE_daf_f32 = m->gr_f.data();
+    if (staf_mlp_eval(m->mlp, &ev) != 0) return -20;
+    energy = (double)e_f;
+    for (size_t i = 0; i < total; i++) m->gr_h[i] = (double)m->gr_f[i];
+  } else {
+    ev.af_f64 = m->af_h.data();
+    ev.energy_f64 = &energy;
+    ev.dE_daf_f64 = m->gr_h.data();
+    if (staf_mlp_eval(m->mlp, &ev) != 0) return -20;
+  }
+  if (!isfinite(energy))
+    fprintf(stderr, "staf_compute: non-finite energy=%g nlocal=%d nghost=%d\n", energy, nlocal, nghost);
+
+  // ---- forces: 2-body + 3-body of every centre species, with the virial
+  staf_op_force_set_skip_pbc(ext ? 1 : 0);
+  staf::launch_fill_zero<double>(m->force.p, nall * 3, st);
+  double W[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0}, Wk[9];
+  off = 0;
+  shift = 0;
+  const int n3 = nall * 3;
+  for (int k = 0; k < nt; shift += tipos[k], k++) {
+    const int Nl = tipos[k], Ar = m->Ar[k], Aa = m->Aa[k];
+    if (Nl == 0) continue;
+    const size_t o = (size_t)shift;
+    m->tmp2.resize((size_t)Nl * Ar);
+    m->tmp3.resize((size_t)Nl * Aa);
+    for (int a = 0; a < Nl; a++) {
+      const double* row = &m->gr_h[off + (size_t)a * (Ar + Aa)];
+      memcpy(&m->tmp2[(size_t)a * Ar], row, Ar * sizeof(double));
+      memcpy(&m->tmp3[(size_t)a * Aa], row + Ar, Aa * sizeof(double));
+    }
+    off += (size_t)Nl * (Ar + Aa);
+    STAF_HIP_OK(hipMemcpyAsync(m->g2.p, m->tmp2.data(), m->tmp2.size() * sizeof(double), hipMemcpyHostToDevice, st));
+    STAF_HIP_OK(hipMemcpyAsync(m->g3.p, m->tmp3.data(), m->tmp3.size() * sizeof(double), hipMemcpyHostToDevice, st));
+    STAF_HIP_OK(hipStreamSynchronize(st));
+    for (int body = 2; body <= 3; body++) {
+      if (body == 2)
+        rc = staf_op_force_doublets_f64(m->g2.p, m->raddescr.p + o * nr, m->der2b.p + o * 3 * nr,
+                                        m->intmap2b.p + o * (nr + 1), nr, nall, 1, Ar, m->alpha2b[k].p, m->emb2b[k].p,
+                                        nt, m->tipos.p, m->actual_type.p + k, m->force_op.p, m->type_map.p, Nl,
+                                        m->virial_op.p, m->pos.p, m->box.p, nlocal, st);
+      else
+        rc = staf_op_force_tripl_f64(m->g3.p, m->des3bsupp.p + o * nr, m->angdescr.p + o * na,
+                                     m->der3bsupp.p + o * 3 * nr, m->der3b.p + o * 6 * na,
+                                     m->intmap2b.p + o * (nr + 1), m->intmap3b.p + o * 2 * na, nr, na, nall, 1, Aa,
+                                     m->emb3b[k].p, nt, m->tipos.p, m->actual_type.p + k, m->force_op.p,
+                                     m->numtriplet.p + o, m->alpha3b[k].p, m->type_map.p, Nl, m->virial_op.p,
+                                     m->pos.p, m->box.p, nlocal, st);
+      if (rc != STAF_OK) return -20;
+      hipLaunchKernelGGL(add_into_kernel, dim3((n3 + 255) / 256), dim3(256), 0, st, m->force.p, m->force_op.p, n3);
+      STAF_HIP_OK(hipMemcpyAsync(Wk, m->virial_op.p, 9 * sizeof(double), hipMemcpyDeviceToHost, st));
+      STAF_HIP_OK(hipStreamSynchronize(st));
+      for (int c = 0; c < 9; c++) W[c] += Wk[c];
+    }
+  }
+  m->force_h.resize((size_t)n3);
+  STAF_HIP_OK(hipMemcpyAsync(m->force_h.data(), m->force.p, (size_t)n3 * sizeof(double), hipMemcpyDeviceToHost, st));
+  STAF_HIP_OK(hipStreamSynchronize(st));
+
+  if (e_rank) *e_rank = energy;
+  if (f)
+    for (int s = 0; s < nall; s++) {
+      const int i = m->slot_to_order[s];
+      f[3 * i] = m->force_h[3 * s];
+      f[3 * i + 1] = m->force_h[3 * s + 1];
+      f[3 * i + 2] = m->force_h[3 * s + 2];
+    }
+  if (virial) {
+    virial[0] = W[0];
+    virial[1] = W[4];
+    virial[2] = W[8];
+    virial[3] = virial[4] = virial[5] = 0.0;   // the reference fills the diagonal only (staf_api.cpp:398-403)
+    if (m->opt.reserved & 1) {
+      virial[3] = 0.5 * (W[1] + W[3]);
+      virial[4] = 0.5 * (W[2] + W[6]);
+      virial[5] = 0.5 * (W[5] + W[7]);
+    }
+  }
+  return 0;
+}
+
+}  // extern "C"

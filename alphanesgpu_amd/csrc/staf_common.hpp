@@ -71,9 +71,10 @@ __device__ inline void tri_decode(int nn, int m, int& j, int& k) {
 
 // Minimum-image Cartesian separation r_i - r_j from Cartesian positions and
 // box6 = [Lx, xy, xz, Ly, yz, Lz]: cart -> frac, rint, back to cart
-// (STAF/include/staf_force_pbc.cuh:16-49; used by the virial forms only).
+// (STAF/include/staf_force_pbc.cuh:16-49; used by the virial forms only).  skip_pbc: no wrap, the neighbour
+// already carries its periodic image (staf_force_skip_pbc there).
 template <typename real>
-__device__ inline void mic_cart_from_cart(const real* pi, const real* pj, const real* bx, real* d) {
+__device__ inline void mic_cart_from_cart(const real* pi, const real* pj, const real* bx, int skip_pbc, real* d) {
   const real i0 = real(1) / bx[0];
   const real i1 = -bx[1] / (bx[0] * bx[3]);
   const real i2 = (bx[1] * bx[4]) / (bx[0] * bx[3] * bx[5]) - bx[2] / (bx[0] * bx[5]);
@@ -83,9 +84,11 @@ __device__ inline void mic_cart_from_cart(const real* pi, const real* pj, const 
   real rx = (i0 * pi[0] + i1 * pi[1] + i2 * pi[2]) - (i0 * pj[0] + i1 * pj[1] + i2 * pj[2]);
   real ry = (i3 * pi[1] + i4 * pi[2]) - (i3 * pj[1] + i4 * pj[2]);
   real rz = i5 * pi[2] - i5 * pj[2];
-  rx -= r_rint(rx);
-  ry -= r_rint(ry);
-  rz -= r_rint(rz);
+  if (!skip_pbc) {
+    rx -= r_rint(rx);
+    ry -= r_rint(ry);
+    rz -= r_rint(rz);
+  }
   d[0] = bx[0] * rx + bx[1] * ry + bx[2] * rz;
   d[1] = bx[3] * ry + bx[4] * rz;
   d[2] = bx[5] * rz;
@@ -126,5 +129,15 @@ struct DescConfig {
   int dist2_fma = 0;
   int zero_padding = 0;
 };
+
+// Internal launchers shared with the MD entry (staf_api): descriptor op with an explicit configuration, an
+// optional caller-supplied neighbour list (owned centres only, Npos >= N positions) and optional no-wrap mode.
+template <typename real>
+int desc_configure(DescConfig<real>& c, real Rc, int nr, int na, real Rs, real Ra);
+template <typename real>
+int desc_launch(const DescConfig<real>& c, const real* pos, const real* box, int nf, int N, int Npos,
+                const int* inj_howmany, const int* inj_with, int skip_pbc, real* raddescr, real* angdescr,
+                real* des3bsupp, int* intmap2b, int* intmap3b, real* der2b, real* der3b, real* der3bsupp,
+                int* numtriplet, hipStream_t stream);
 
 }  // namespace staf

@@ -27,9 +27,12 @@ namespace staf {
 
 template <typename real>
 struct DescArgs {
-  const real* pos;
+  const real* pos;         // [nf, 3*Npos] Cartesian
   const real* box;
-  int nf, N, nr, na;
+  const int* inj_howmany;  // injected neighbour list (else null): [nf, N]
+  const int* inj_with;     // [nf, N, nr], sorted by distance, indices into the Npos atoms
+  int nf, N, Npos, nr, na;
+  int skip_pbc;            // no minimum-image wrap (neighbours carry their periodic image)
   real Rc, Ra, Rs, cA, cB, cC, pa, pb;
   int dist2_fma, zero_padding;
   real* raddescr;
@@ -69,12 +72,14 @@ __device__ inline void to_frac(const real* inv, real px, real py, real pz, real*
 
 // d = H * ((sa - sb) - rint(sa - sb)), returns |d|^2 as the neighbour test sees it.
 template <typename real>
-__device__ inline real mic_delta(const real* box, const real* sa, const real* sb, int fma_mode, real* d) {
+__device__ inline real mic_delta(const real* box, const real* sa, const real* sb, int fma_mode, int skip_pbc, real* d) {
 #pragma clang fp contract(off)
   real ox = sa[0] - sb[0], oy = sa[1] - sb[1], oz = sa[2] - sb[2];
-  ox -= r_rint(ox);
-  oy -= r_rint(oy);
-  oz -= r_rint(oz);
+  if (!skip_pbc) {
+    ox -= r_rint(ox);
+    oy -= r_rint(oy);
+    oz -= r_rint(oz);
+  }
   d[0] = box[0] * ox + box[1] * oy + box[2] * oz;
   d[1] = box[3] * oy + box[4] * oz;
   d[2] = box[5] * oz;
@@ -116,25 +121,42 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
 #pragma unroll
   for (int c = 0; c < 6; c++) box[c] = sbox[c];
   inverse_box(box, inv);
-  const real* pf = A.pos + (size_t)b * N * 3;
+  const real* pf = A.pos + (size_t)b * A.Npos * 3;
   real si[3];
   to_frac(inv, pf[3 * i], pf[3 * i + 1], pf[3 * i + 2], si);
   const real rc2 = A.Rc * A.Rc;
 
-  // 1. candidate scan
-  for (int j = tid; j < N; j += blockDim.x) {
-    real sj[3], d[3];
-    to_frac(inv, pf[3 * j], pf[3 * j + 1], pf[3 * j + 2], sj);
-    real d2 = mic_delta(box, sj, si, A.dist2_fma, d);
-    if (d2 < rc2 && j != i) {
-      int slot = atomicAdd(&cnt_all, 1);
-      if (slot < nr) {
-        c_j[slot] = j;
-        c_d2[slot] = d2;
-        c_d[3 * slot] = d[0];
-        c_d[3 * slot + 1] = d[1];
-        c_d[3 * slot + 2] = d[2];
+  // 1. candidate scan -- or the caller's list (already cut off and sorted by distance)
+  const bool injected = A.inj_howmany != nullptr;
+  if (!injected) {
+    for (int j = tid; j < A.Npos; j += blockDim.x) {
+      real sj[3], d[3];
+      to_frac(inv, pf[3 * j], pf[3 * j + 1], pf[3 * j + 2], sj);
+      real d2 = mic_delta(box, sj, si, A.dist2_fma, A.skip_pbc, d);
+      if (d2 < rc2 && j != i) {
+        int slot = atomicAdd(&cnt_all, 1);
+        if (slot < nr) {
+          c_j[slot] = j;
+          c_d2[slot] = d2;
+          c_d[3 * slot] = d[0];
+          c_d[3 * slot + 1] = d[1];
+          c_d[3 * slot + 2] = d[2];
+        }
       }
+    }
+  } else {
+    const int cnt = A.inj_howmany[(size_t)b * N + i];
+    if (tid == 0) cnt_all = cnt;
+    const int* wl = A.inj_with + ((size_t)b * N + i) * nr;
+    for (int e = tid; e < cnt && e < nr; e += blockDim.x) {
+      const int j = wl[e];
+      real sj[3], d[3];
+      to_frac(inv, pf[3 * j], pf[3 * j + 1], pf[3 * j + 2], sj);
+      c_d2[e] = mic_delta(box, sj, si, A.dist2_fma, A.skip_pbc, d);
+      c_j[e] = j;
+      c_d[3 * e] = d[0];
+      c_d[3 * e + 1] = d[1];
+      c_d[3 * e + 2] = d[2];
     }
   }
   __syncthreads();
@@ -154,10 +176,14 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
       const real d2 = c_d2[e];
       const int j = c_j[e];
       int rank = 0;
-      for (int o = 0; o < n; o++) {
-        const real od2 = c_d2[o];
-        const int oj = c_j[o];
-        rank += (od2 < d2 || (od2 == d2 && oj < j)) ? 1 : 0;
+      if (injected) {
+        rank = e;   // the caller's order is kept
+      } else {
+        for (int o = 0; o < n; o++) {
+          const real od2 = c_d2[o];
+          const int oj = c_j[o];
+          rank += (od2 < d2 || (od2 == d2 && oj < j)) ? 1 : 0;
+        }
       }
       // centre - neighbour: exact negation of the scan's neighbour - centre
       real d[3] = {-c_d[3 * e], -c_d[3 * e + 1], -c_d[3 * e + 2]};
@@ -332,23 +358,19 @@ static int construct(real Rc, int nr, int na, int numpar, real Rs, real Ra, int 
 }
 
 template <typename real>
-static int compute(const real* pos, const real* box, int nf, int N, real* raddescr, real* angdescr, real* des3bsupp,
-                   int* intmap2b, int* intmap3b, real* der2b, real* der3b, real* der3bsupp, int* numtriplet,
-                   void* stream_) {
-  DescConfig<real> c;
-  {
-    std::lock_guard<std::mutex> lock(g_cfg_mu);
-    c = cfg<real>();
-  }
+int desc_launch(const DescConfig<real>& c, const real* pos, const real* box, int nf, int N, int Npos,
+                const int* inj_howmany, const int* inj_with, int skip_pbc, real* raddescr, real* angdescr,
+                real* des3bsupp, int* intmap2b, int* intmap3b, real* der2b, real* der3b, real* der3bsupp,
+                int* numtriplet, hipStream_t stream) {
   if (!c.ready) return STAF_E_NOT_CONSTRUCTED;
   if (!pos || !box || !raddescr || !angdescr || !des3bsupp || !intmap2b || !intmap3b || !der2b || !der3b ||
-      !der3bsupp || !numtriplet || nf <= 0 || N <= 0)
+      !der3bsupp || !numtriplet || nf <= 0 || N <= 0 || Npos < N || (inj_howmany && !inj_with))
     return STAF_E_BAD_ARG;
   DeviceState* st = device_state();
   if (!st) return STAF_E_HIP;
-  hipStream_t stream = (hipStream_t)stream_;
   DescArgs<real> A;
-  A.pos = pos; A.box = box; A.nf = nf; A.N = N; A.nr = c.nr; A.na = c.na;
+  A.pos = pos; A.box = box; A.nf = nf; A.N = N; A.Npos = Npos; A.nr = c.nr; A.na = c.na;
+  A.inj_howmany = inj_howmany; A.inj_with = inj_with; A.skip_pbc = skip_pbc;
   A.Rc = c.Rc; A.Ra = c.Ra; A.Rs = c.Rs; A.cA = c.cA; A.cB = c.cB; A.cC = c.cC; A.pa = c.pa; A.pb = c.pb;
   A.dist2_fma = c.dist2_fma; A.zero_padding = c.zero_padding;
   A.raddescr = raddescr; A.angdescr = angdescr; A.des3bsupp = des3bsupp; A.intmap2b = intmap2b;
@@ -358,6 +380,37 @@ static int compute(const real* pos, const real* box, int nf, int N, real* raddes
   if (lds > 60 * 1024) return STAF_E_LIMIT;
   hipLaunchKernelGGL(desc_kernel<real>, dim3((unsigned)(nf * N)), dim3(256), lds, stream, A);
   return finish_op(st, stream);
+}
+template int desc_launch<float>(const DescConfig<float>&, const float*, const float*, int, int, int, const int*,
+                                const int*, int, float*, float*, float*, int*, int*, float*, float*, float*, int*,
+                                hipStream_t);
+template int desc_launch<double>(const DescConfig<double>&, const double*, const double*, int, int, int, const int*,
+                                 const int*, int, double*, double*, double*, int*, int*, double*, double*, double*,
+                                 int*, hipStream_t);
+
+template <typename real>
+int desc_configure(DescConfig<real>& c, real Rc, int nr, int na, real Rs, real Ra) {
+  if (nr <= 0 || na <= 0 || !(Rc > 0) || !(Ra > 0)) return STAF_E_BAD_ARG;
+  if (nr > 1024) return STAF_E_LIMIT;
+  c = DescConfig<real>();
+  c.nr = nr; c.na = na; c.Rc = Rc; c.Rs = Rs; c.Ra = Ra;
+  repulsion_coefficients(c);
+  c.ready = true;
+  return STAF_OK;
+}
+template int desc_configure<double>(DescConfig<double>&, double, int, int, double, double);
+
+template <typename real>
+static int compute(const real* pos, const real* box, int nf, int N, real* raddescr, real* angdescr, real* des3bsupp,
+                   int* intmap2b, int* intmap3b, real* der2b, real* der3b, real* der3bsupp, int* numtriplet,
+                   void* stream_) {
+  DescConfig<real> c;
+  {
+    std::lock_guard<std::mutex> lock(g_cfg_mu);
+    c = cfg<real>();
+  }
+  return desc_launch<real>(c, pos, box, nf, N, N, nullptr, nullptr, 0, raddescr, angdescr, des3bsupp, intmap2b,
+                           intmap3b, der2b, der3b, der3bsupp, numtriplet, (hipStream_t)stream_);
 }
 
 }  // namespace staf

@@ -24,6 +24,11 @@ constexpr int F_WAVES = F_BLOCK / WAVE;
 constexpr int F_PARTS = 4;  // partner split of the per-slot sums in the 3-body force
 constexpr int GRAD_MAX_BLOCKS_F = 1024;
 
+// Process-wide switch of the virial forms: 0 = minimum-image wrap of r_i - r_j (periodic box, default),
+// 1 = no wrap (neighbours are explicit periodic images).  Same role as staf_force_skip_pbc of the reference
+// (STAF/include/staf_force_pbc.cuh:5-10, libstaf/vendor/jmd/src_nn/staf_force_pbc.cu).
+static int g_force_skip_pbc = 0;
+
 __device__ inline int species_shift(const int* tipos, const int* actual_type) {
   const int at = actual_type[0];
   int s = 0;
@@ -324,7 +329,7 @@ __global__ __launch_bounds__(F_BLOCK) void virial_centre_kernel(const real* __re
                                                                 const int* __restrict__ tipos,
                                                                 const int* __restrict__ actual_type,
                                                                 real* __restrict__ vpart, int nf, int N, int Nl,
-                                                                int ld, int nr) {
+                                                                int ld, int nr, int skip_pbc) {
   const int wave = threadIdx.x / WAVE, lane = lane_id();
   const int atom = blockIdx.x * F_WAVES + wave;
   if (atom >= nf * Nl) return;
@@ -342,7 +347,7 @@ __global__ __launch_bounds__(F_BLOCK) void virial_centre_kernel(const real* __re
   for (int s = lane; s < cnt; s += WAVE) {
     const int nj = im[1 + s];
     real r[3];
-    mic_cart_from_cart(pi, pos + ((size_t)b * N + nj) * 3, bx, r);
+    mic_cart_from_cart(pi, pos + ((size_t)b * N + nj) * 3, bx, skip_pbc, r);
     const real* g = gslot + ((size_t)atom * nr + s) * 3;
 #pragma unroll
     for (int a = 0; a < 3; a++)
@@ -446,8 +451,8 @@ __global__ __launch_bounds__(F_BLOCK) void gradforce2_kernel(
     const int* __restrict__ im2, const real* __restrict__ alpha2b, const real* __restrict__ emb2b,
     const int* __restrict__ type_map, const int* __restrict__ tipos, const int* __restrict__ actual_type,
     real* __restrict__ gnet, real* __restrict__ partial, const real* __restrict__ Qvir,
-    const real* __restrict__ pos, const real* __restrict__ box, int nf, int N, int Nl, int ld, int nr, int Ar,
-    int nt) {
+    const real* __restrict__ pos, const real* __restrict__ box, int skip_pbc, int nf, int N, int Nl, int ld, int nr,
+    int Ar, int nt) {
   extern __shared__ __align__(16) unsigned char smem[];
   real* p_al = (real*)smem;                     // [nt*Ar]
   real* p_c2 = p_al + nt * Ar;                  // [nt*Ar]
@@ -483,7 +488,8 @@ __global__ __launch_bounds__(F_BLOCK) void gradforce2_kernel(
       if (Qvir) {
         // virial form: dL/dg_a = (dL/dF_j - dL/dF_i)_a - sum_e (dL/dW)_ae r_e  (grad_force/rad/reforce.cu.cc:213-216)
         real r[3];
-        mic_cart_from_cart(pos + ((size_t)b * N + p + shift) * 3, pos + ((size_t)b * N + nj) * 3, box + (size_t)b * 6, r);
+        mic_cart_from_cart(pos + ((size_t)b * N + p + shift) * 3, pos + ((size_t)b * N + nj) * 3, box + (size_t)b * 6,
+                           skip_pbc, r);
         const real* Wg = Qvir + (size_t)b * 9;
         q0 -= Wg[0] * r[0] + Wg[1] * r[1] + Wg[2] * r[2];
         q1 -= Wg[3] * r[0] + Wg[4] * r[1] + Wg[5] * r[2];
@@ -568,7 +574,7 @@ static void launch_virial(const ForceScratch& fs, const int* im2, const int* cou
   const int atoms = nf * Nl;
   hipLaunchKernelGGL(virial_centre_kernel<real>, dim3((atoms + F_WAVES - 1) / F_WAVES), dim3(F_BLOCK), 0, stream,
                      (const real*)fs.gslot, im2, counts, pos, box, tipos, actual_type, (real*)fs.vpart, nf, N, Nl,
-                     ld, nr);
+                     ld, nr, g_force_skip_pbc);
   hipLaunchKernelGGL(virial_frame_kernel<real>, dim3(nf), dim3(F_BLOCK), 0, stream, (const real*)fs.vpart, virial,
                      Nl);
 }
@@ -669,7 +675,8 @@ static int gradforce_2b(const real* Q, const real* D, int nr, const real* alpha2
                (size_t)F_WAVES * nr * sizeof(int);
   if (lds > 64 * 1024) return STAF_E_LIMIT;
   hipLaunchKernelGGL(gradforce2_kernel<real>, dim3(nb), dim3(F_BLOCK), lds, stream, Q, G, D, dD, im2, alpha2b, emb2b,
-                     type_map, tipos, actual_type, gnet, partial, Qvir, pos, box, nf, N, Nl, ld, nr, Ar, nt);
+                     type_map, tipos, actual_type, gnet, partial, Qvir, pos, box, g_force_skip_pbc, nf, N, Nl, ld, nr,
+                     Ar, nt);
   launch_reduce_partials<real>(partial, nb, nout, g_alpha, nt * Ar, g_emb, nt * Ar, stream);
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }
@@ -706,6 +713,7 @@ static int gradforce_tripl(const real* Q, const real* G, const real* Dsup, const
   A.Dsup = Dsup; A.Tang = Tang; A.im2 = im2; A.alpha3b = alpha3b; A.emb3b = emb3b; A.type_map = type_map;
   A.numtriplet = numtriplet; A.P = G; A.Q = Q; A.dDsup = dDsup; A.d3b = d3b; A.tipos = tipos;
   A.actual_type = actual_type; A.out = gnet; A.partial = partial; A.Qvir = Qvir; A.pos = pos; A.box = box;
+  A.skip_pbc = g_force_skip_pbc;
   A.nf = nf; A.N = N; A.Nl = Nl; A.ld = ld; A.nr = nr; A.na = na; A.Aa = Aa; A.nt = nt;
   hipLaunchKernelGGL((tri_reduce_kernel<real, 2>), dim3(nb), dim3(TRI_BLOCK), lds, stream, A);
   launch_reduce_partials<real>(partial, nb, nout, g_alpha, nout, (real*)nullptr, 0, stream);
@@ -715,6 +723,8 @@ static int gradforce_tripl(const real* Q, const real* G, const real* Dsup, const
 }  // namespace staf
 
 extern "C" {
+
+void staf_op_force_set_skip_pbc(int skip) { staf::g_force_skip_pbc = skip ? 1 : 0; }
 
 #define STAF_FORCE_ENTRY(real, SFX)                                                                                    \
   int staf_op_force_doublets_##SFX(const real* netderiv, const real* des_r, const real* intderiv_r,                    \

@@ -47,6 +47,7 @@ struct TriArgs {
   const real* Qvir;       // MODE 2, virial form: dL/dW [nf, 9] (else null)
   const real* pos;        // MODE 2, virial form: positions [nf, 3N]
   const real* box;        // MODE 2, virial form: [nf, 6]
+  int skip_pbc;           // MODE 2, virial form: no minimum-image wrap
   real* out;              // MODE 0: AF3, MODE 2: gradnet  [nf, Nl, Aa] contiguous
   real* partial;          // MODE 1/2: [gridDim.x, nsig*Aa*3]
   int nf, N, Nl, ld, nr, na, Aa, nt;
@@ -136,7 +137,7 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
           // virial form: dL/dg_a = (dL/dF_j - dL/dF_i)_a - sum_e (dL/dW)_ae r_e (grad_force/ang/reforce.cu.cc:391-394)
           real r[3];
           mic_cart_from_cart(A.pos + ((size_t)b * A.N + p + shift) * 3, A.pos + ((size_t)b * A.N + nj) * 3,
-                             A.box + (size_t)b * 6, r);
+                             A.box + (size_t)b * 6, A.skip_pbc, r);
           const real* Wg = A.Qvir + (size_t)b * 9;
           q0 -= Wg[0] * r[0] + Wg[1] * r[1] + Wg[2] * r[2];
           q1 -= Wg[3] * r[0] + Wg[4] * r[1] + Wg[5] * r[2];

@@ -137,6 +137,11 @@ int staf_op_init_force_tripl(int buffdim);
 int staf_op_init_grad_force_radial(int buffdim);
 int staf_op_init_grad_force_tripl(int buffdim);
 
+/* Virial forms only: 0 (default) = r_i - r_j is wrapped to the minimum image of the periodic box; 1 = no wrap, the
+ * neighbour positions already are the periodic images (domain-decomposed MD with ghost atoms).  Process-wide, like
+ * staf_force_skip_pbc of the reference (STAF/include/staf_force_pbc.cuh:5-10). */
+void staf_op_force_set_skip_pbc(int skip);
+
 /* computeforce_doublets_Launcher (ComputeForceRadial) -- STAF/src/force/rad/reforce.cc:39-57, reforce.cu.cc:45-172
  * and computeforce_doublets_virial_Launcher (ComputeForceRadialVirial) -- reforce.cc:124-146, reforce.cu.cc:174-314.
  *   forces2b [nf,3N] (all atoms; fully written).  virial [nf,9] row-major W_ab -= g_a r_b, pos [nf,3N]
