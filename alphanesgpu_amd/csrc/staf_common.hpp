@@ -46,6 +46,36 @@ __device__ inline T wave_sum(T v) {
   for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
   return v;
 }
+// Data-parallel-primitive lane moves: lane l receives the value of another lane of its row of 16 (or of the
+// previous rows for the broadcasts); lanes without a source receive 0.
+template <int CTRL, int ROW_MASK>
+__device__ inline float dpp_get(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
+}
+template <int CTRL, int ROW_MASK>
+__device__ inline double dpp_get(double v) {
+  const long long b = __double_as_longlong(v);
+  const int lo = __builtin_amdgcn_update_dpp(0, (int)(b & 0xffffffffll), CTRL, ROW_MASK, 0xf, false);
+  const int hi = __builtin_amdgcn_update_dpp(0, (int)(b >> 32), CTRL, ROW_MASK, 0xf, false);
+  return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+}
+// Sum over the 64 lanes with register-to-register lane moves only; the total is valid in lane 63 alone.
+// Fixed tree: prefix steps 1,2,3,4,8 inside each row of 16, then row 0->1, 2->3, and rows 0-1 -> 2-3.
+template <typename T>
+__device__ inline T wave_sum_to_last(T v) {
+  T s = v + dpp_get<0x111, 0xf>(v);
+  s += dpp_get<0x112, 0xf>(v);
+  s += dpp_get<0x113, 0xf>(v);
+  s += dpp_get<0x114, 0xf>(s);
+  s += dpp_get<0x118, 0xf>(s);
+  s += dpp_get<0x142, 0xa>(s);   // lane 15 of a row -> every lane of the next row (rows 1 and 3 take it)
+  s += dpp_get<0x143, 0xc>(s);   // lane 31 -> rows 2 and 3
+  return s;
+}
+// Wave-uniform value loaded through a vector path (e.g. from LDS) moved to a scalar register, so that loop
+// bounds and addresses derived from it stay scalar.
+__device__ inline int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
 __device__ inline int wave_max(int v) {
 #pragma unroll
   for (int o = WAVE / 2; o > 0; o >>= 1) v = max(v, __shfl_xor(v, o, WAVE));
@@ -96,6 +126,44 @@ __device__ inline void mic_cart_from_cart(const real* pi, const real* pj, const 
 
 // Pair index q inside an n-item triangle (x<y) -> (x,y); same numbering.
 __device__ inline void tri_decode_xy(int q, int n, int& x, int& y) { tri_decode(q, n, x, y); }
+
+// Phase clock (profiling builds only, -DSTAF_PHASE_CLOCK): thread 0 of every workgroup adds the shader-clock
+// cycles between consecutive marks to a per-phase total when it ends.  Every translation unit has its own totals, read back
+// and cleared with the staf_debug_phase_clock_<unit>() it defines through PHASE_CLOCK_READER.
+#ifdef STAF_PHASE_CLOCK
+static __device__ unsigned long long g_phase_clock[32];
+#define PHASE_CLOCK_READER(name)                                                                            \
+  extern "C" int name(unsigned long long* out) {                                                            \
+    if (hipDeviceSynchronize() != hipSuccess) return STAF_E_HIP;                                            \
+    if (hipMemcpyFromSymbol(out, HIP_SYMBOL(staf::g_phase_clock), 32 * sizeof(unsigned long long)) !=       \
+        hipSuccess)                                                                                         \
+      return STAF_E_HIP;                                                                                    \
+    unsigned long long zero[32] = {0};                                                                      \
+    if (hipMemcpyToSymbol(HIP_SYMBOL(staf::g_phase_clock), zero, sizeof(zero)) != hipSuccess)               \
+      return STAF_E_HIP;                                                                                    \
+    return STAF_OK;                                                                                         \
+  }
+#define PHASE_CLOCK_BEGIN()                     \
+  unsigned long long phase_acc_[16] = {0};      \
+  unsigned long long phase_t_ = clock64()
+#define PHASE_MARK(i)                                   \
+  do {                                                  \
+    const unsigned long long now_ = clock64();          \
+    phase_acc_[i] += now_ - phase_t_;                   \
+    phase_t_ = now_;                                    \
+  } while (0)
+#define PHASE_CLOCK_END()                                                   \
+  do {                                                                      \
+    if (threadIdx.x == 0)                                                   \
+      for (int i_ = 0; i_ < 16; i_++)                                       \
+        if (phase_acc_[i_]) atomicAdd(&g_phase_clock[i_], phase_acc_[i_]);  \
+  } while (0)
+#else
+#define PHASE_CLOCK_READER(name)
+#define PHASE_CLOCK_BEGIN() do {} while (0)
+#define PHASE_MARK(i) do {} while (0)
+#define PHASE_CLOCK_END() do {} while (0)
+#endif
 
 // ---- library-owned device state (per device) -------------------------------
 struct Workspace {

@@ -1,7 +1,9 @@
 // Triplet kernels that reduce over an atom's triplets: 3-body fingerprints
 // (MODE 0), their parameter gradient (MODE 1) and the gradient of the 3-body
 // force op (MODE 2).  One 256-thread workgroup per centre atom (persistent
-// over atoms for the gradient modes).
+// over atoms for the gradient modes).  These kernels are bound by vector-ALU
+// issue, so the layout below is chosen to keep the instruction count per
+// (triplet, channel) item low.
 //
 // Work decomposition inside a species class (ta,tb) of the centre's triplets
 // (see staf_tile.hpp for the class enumeration):
@@ -10,13 +12,15 @@
 //     multiplies instead of an exp: O(m * channels) transcendental calls for
 //     the pair factors instead of O(m^2 * channels).  Only exp(beta*T) stays
 //     per (triplet, channel).
-//   * thread <-> (channel, triplet subset): the threads of a wave that share a
-//     subset walk the same triplets and differ in the channel, so every thread
-//     accumulates its own channel privately -- no cross-lane reduction per
-//     channel, parameters live in registers, table reads are contiguous in the
-//     channel.  Subsets are combined once per class through LDS in a fixed
-//     order (bit-reproducible).
-//   * triplets are staged in LDS in blocks (packed pair index, T, and for
+//   * thread <-> (channel ia = tid & 15, triplet subset sub = tid >> 4): the
+//     16 lanes of a subset walk the same triplets and differ in the channel,
+//     so every thread accumulates its own channel privately with its
+//     parameters in registers, and table reads are contiguous in the channel.
+//     The four subsets of a wave are combined with two cross-lane adds and
+//     added into per-wave accumulators in LDS; the waves are summed once per
+//     atom in a fixed order (bit-reproducible).  No barrier per class for the
+//     reduction.
+//   * triplets are staged in LDS in blocks (table row offsets, T, and for
 //     MODE 2 the contraction U of der3b with dL/dF), so tensors laid out by
 //     the storage index nn are read exactly once.
 #pragma once
@@ -25,9 +29,32 @@
 namespace staf {
 
 constexpr int TRI_BLOCK = 256;
-constexpr int TRI_CAP = 16;    // channels tabulated per pass
+constexpr int TRI_WAVES = TRI_BLOCK / WAVE;
+constexpr int TRI_CAP = 16;    // channels tabulated per pass = lanes of a subset
+constexpr int TRI_SUBS = TRI_BLOCK / TRI_CAP;
 constexpr int TRI_QB = 512;    // triplets staged per block
 constexpr int TRI_GRID_MAX = 2048;  // workgroups of the persistent gradient modes (one partial row each)
+
+// Exponential of the hot loops.  float: the argument is pre-scaled by log2(e) and fed to the hardware exp2
+// (two instructions; the rounding of the scaled product is of the same size as the rounding of the unscaled
+// product inside expf).  double: the library routine.
+template <typename real> struct HotExp;
+template <> struct HotExp<float> {
+  __device__ static float scale(float a) { return a * 1.44269504088896341f; }
+  __device__ static float eval(float t) { return __builtin_amdgcn_exp2f(t); }
+};
+template <> struct HotExp<double> {
+  __device__ static double scale(double a) { return a; }
+  __device__ static double eval(double t) { return exp(t); }
+};
+
+// q / n for 0 <= q < 2^22, 1 <= n <= 2^11 without the integer-division sequence
+__device__ inline int small_div(int q, int n, float inv_n) {
+  int x = (int)(((float)q + 0.5f) * inv_n);
+  if (x * n > q) --x;
+  else if ((x + 1) * n <= q) ++x;
+  return x;
+}
 
 template <typename real>
 struct TriArgs {
@@ -56,63 +83,68 @@ struct TriArgs {
 template <typename real, int MODE>
 struct TriLds {
   static constexpr int NV = (MODE == 0) ? 1 : (MODE == 1 ? 3 : 4);
-  // bytes of the staging region (packed pairs + T (+ U)) followed by the per-thread partials of the class reduction
-  __host__ __device__ static size_t stage_bytes() {
-    size_t st = (size_t)TRI_QB * (sizeof(int) + sizeof(real) * (MODE == 2 ? 2 : 1));
-    size_t rd = (size_t)TRI_BLOCK * NV * sizeof(real);
-    return ((st + 15) & ~(size_t)15) + ((rd + 15) & ~(size_t)15);
+  __host__ __device__ static size_t n_reals(int nr, int Aa, int nt) {
+    const int nsig = 2 * nt - 1;
+    size_t r = (size_t)nr * TRI_CAP * 2;                    // pair tables (real2 per (row, channel))
+    r += (size_t)nr * (MODE == 2 ? 2 : 1);                  // D (and V) by table row
+    r += nr;                                                // sD
+    r += Aa;                                                // sP
+    r += (size_t)TRI_WAVES * Aa;                            // per-wave channel sums
+    if (MODE != 0) r += (size_t)TRI_WAVES * nsig * Aa * 3;  // per-wave parameter-gradient sums
+    if (MODE == 2) r += (size_t)4 * nr;                     // sV, sQ
+    r += (size_t)TRI_QB * (MODE == 2 ? 2 : 1);              // staged T (and U)
+    return r;
   }
   __host__ __device__ static size_t bytes(int nr, int Aa, int nt) {
-    const int nsig = 2 * nt - 1;
-    size_t b = chan_table_bytes<real>(nsig, Aa);
-    size_t reals = (size_t)Aa /*out_ch*/ + nr /*sD*/ + Aa /*sP*/ + (size_t)nr * TRI_CAP * 2 /*pair tables*/;
-    if (MODE != 0) reals += (size_t)nsig * Aa * 3;
-    if (MODE == 2) reals += (size_t)4 * nr;  // sV, sQ
-    b += reals * sizeof(real);
-    b = (b + 15) & ~(size_t)15;
-    b += stage_bytes();
-    b += (size_t)(2 * nr + NT_MAX + 1) * sizeof(int);
-    return b;
+    size_t b = chan_table_bytes<real>(2 * nt - 1, Aa) + n_reals(nr, Aa, nt) * sizeof(real);
+    b += (size_t)(2 * TRI_QB + 2 * nr + NT_MAX + 1) * sizeof(int);
+    return (b + 15) & ~(size_t)15;
   }
 };
 
 template <typename real, int MODE>
 __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) {
   using real2 = typename Vec2<real>::type;
+  using HE = HotExp<real>;
   constexpr int NV = TriLds<real, MODE>::NV;
   extern __shared__ __align__(16) unsigned char smem[];
   const int nr = A.nr, na = A.na, Aa = A.Aa, nt = A.nt;
   const int nsig = 2 * nt - 1;
+  const int nacc = nsig * Aa * 3;
   ChanTable<real> tab;
   unsigned char* sp = tab.carve(smem, nsig, Aa);
   real* rp = (real*)sp;   // 16-byte aligned: the pair tables come first
-  real2* tabA = (real2*)rp; rp += (size_t)nr * TRI_CAP * 2;   // both species of a class: at most m <= nr rows
-  real* out_ch = rp; rp += Aa;
+  real2* tabE = (real2*)rp; rp += (size_t)nr * TRI_CAP * 2;   // rows of both species of a class: at most m <= nr
+  real* Drow = rp; rp += nr;
+  real* Vrow = rp; if (MODE == 2) rp += nr;
   real* sD = rp; rp += nr;
   real* sP = rp; rp += Aa;
-  real* acc_par = rp;
-  if (MODE != 0) rp += (size_t)nsig * Aa * 3;
+  real* outw = rp; rp += (size_t)TRI_WAVES * Aa;
+  real* accw = rp; if (MODE != 0) rp += (size_t)TRI_WAVES * nacc;
   real* sV = rp;
   real* sQ = rp + nr;
   if (MODE == 2) rp += (size_t)4 * nr;
-  unsigned char* stg = (unsigned char*)((((size_t)rp) + 15) & ~(size_t)15);
-  real* sT = (real*)stg;                       // [TRI_QB]
-  real* sU = sT + TRI_QB;                      // [TRI_QB] (MODE 2)
-  int* pk = (int*)(sT + TRI_QB * (MODE == 2 ? 2 : 1));   // [TRI_QB]
-  real* red = (real*)(stg + (((size_t)TRI_QB * (sizeof(int) + sizeof(real) * (MODE == 2 ? 2 : 1)) + 15) & ~(size_t)15));
-  int* lst = (int*)(stg + TriLds<real, MODE>::stage_bytes());
+  real* sT = rp; rp += TRI_QB;
+  real* sU = rp; if (MODE == 2) rp += TRI_QB;
+  int* offA = (int*)rp;          // [TRI_QB] first table row of the staged triplet, times TRI_CAP
+  int* offB = offA + TRI_QB;     // [TRI_QB] second
+  int* lst = offB + TRI_QB;
   int* stp = lst + nr;
   int* off = stp + nr;
 
   const int tid = threadIdx.x;
+  const int lane = tid & (WAVE - 1), wave = tid / WAVE;
+  const int ia = tid & (TRI_CAP - 1), sub = tid / TRI_CAP;
   tab.build(A.alpha3b, A.emb3b);
   if (MODE != 0)
-    for (int q = tid; q < nsig * Aa * 3; q += TRI_BLOCK) acc_par[q] = 0;
+    for (int q = tid; q < TRI_WAVES * nacc; q += TRI_BLOCK) accw[q] = 0;
   int shift = 0;
   if (MODE == 2) {
     const int at = A.actual_type[0];
     for (int y = 0; y < at; y++) shift += A.tipos[y];
   }
+  real* my_out = outw + wave * Aa;
+  real* my_acc = accw + (size_t)wave * nacc;
   __syncthreads();
 
   const int total = A.nf * A.Nl;
@@ -148,14 +180,14 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
         sV[s] = q0 * gr[0] + q1 * gr[nr] + q2 * gr[2 * nr];
       }
     }
-    for (int a = tid; a < Aa; a += TRI_BLOCK) {
-      out_ch[a] = 0;
+    for (int a = tid; a < Aa; a += TRI_BLOCK)
       if (MODE != 0) sP[a] = A.P[(size_t)atom * Aa + a];
-    }
+    for (int q = tid; q < TRI_WAVES * Aa; q += TRI_BLOCK) outw[q] = 0;
     __syncthreads();
     if (tid < WAVE) group_slots_by_type(m, nt, stp, lst, off);
     __syncthreads();
 
+    bool first = true;
     for (int ta = 0; ta < nt; ta++) {
       const int oa = off[ta];
       const int na_ = off[ta + 1] - oa;
@@ -171,29 +203,32 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
         const int pb = sg * Aa;
         const int* la = lst + oa;
         const int* lb = lst + ob;
-        real2* tabB = tabA + (size_t)na_ * TRI_CAP;   // rows of the second species follow the first
+        const int nrows = same ? na_ : na_ + nb_;   // rows of the second species follow the first
+        const int rowB0 = same ? 0 : na_;
+        const float inv_nb = 1.0f / (float)nb_;
         for (int c0 = 0; c0 < nact; c0 += TRI_CAP) {
           const int nch = (nact - c0) < TRI_CAP ? (nact - c0) : TRI_CAP;
-          // ---- tables of the class: E[x][ia] = (exp(a1 D), exp(a2 D))
-          {
-            const int ea = na_ * nch, eb_ = same ? 0 : nb_ * nch;
-            for (int e = tid; e < ea + eb_; e += TRI_BLOCK) {
-              const bool second = e >= ea;
-              const int ee = second ? e - ea : e;
-              const int x = ee / nch, ia = ee - x * nch;
-              const real d = sD[second ? lb[x] : la[x]];
+          const bool chan = ia < nch;
+          real a1 = 0, a2 = 0, be = 0;
+          if (chan) { a1 = tab.a1[pb + c0 + ia]; a2 = tab.a2[pb + c0 + ia]; be = tab.be[pb + c0 + ia]; }
+          const real a1s = HE::scale(a1), a2s = HE::scale(a2), bes = HE::scale(be);
+          if (!first) __syncthreads();   // tables and staged block of the previous pass fully consumed
+          first = false;
+          // ---- tables of the class: E[row][ia] = (exp(a1 D), exp(a2 D)), D (and V) by row
+          for (int row = sub; row < nrows; row += TRI_SUBS) {
+            const int s = row < na_ ? la[row] : lb[row - na_];
+            const real d = sD[s];
+            if (chan) {
               real2 v;
-              v.x = r_exp(tab.a1[pb + c0 + ia] * d);
-              v.y = r_exp(tab.a2[pb + c0 + ia] * d);
-              (second ? tabB : tabA)[x * TRI_CAP + ia] = v;
+              v.x = HE::eval(a1s * d);
+              v.y = HE::eval(a2s * d);
+              tabE[row * TRI_CAP + ia] = v;
+            }
+            if (ia == 0) {
+              Drow[row] = d;
+              if (MODE == 2) Vrow[row] = sV[s];
             }
           }
-          const real2* tB = same ? tabA : tabB;
-          const int S = TRI_BLOCK / nch;
-          const int sub = tid / nch, ia = tid - sub * nch;
-          const bool worker = sub < S;
-          real be = 0;
-          if (worker) be = tab.be[pb + c0 + ia];
           real acc[NV];
 #pragma unroll
           for (int v = 0; v < NV; v++) acc[v] = 0;
@@ -205,12 +240,13 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
               const int q = q0 + qq;
               int x, y;
               if (same) tri_decode_xy(q, nb_, x, y);
-              else { x = q / nb_; y = q - x * nb_; }
+              else { x = small_div(q, nb_, inv_nb); y = q - x * nb_; }
               const int s1 = la[x], s2 = lb[y];
               const int j = s1 < s2 ? s1 : s2, k = s1 < s2 ? s2 : s1;
               const int nn = tri_rowstart(j, m) + k - j - 1;
               const bool ok = nn < na;
-              pk[qq] = x | (y << 16);
+              offA[qq] = x * TRI_CAP;
+              offB[qq] = (rowB0 + y) * TRI_CAP;
               real T = 0;
               if (ok) T = Trow[nn];
               sT[qq] = T;
@@ -228,30 +264,27 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
             }
             __syncthreads();
             // ---- thread <-> (channel ia, subset sub)
-            if (worker) {
-              for (int qq = sub; qq < nq; qq += S) {
-                const int xy = pk[qq];
-                const int x = xy & 0xffff, y = xy >> 16;
+            if (chan) {
+              for (int qq = sub; qq < nq; qq += TRI_SUBS) {
+                const int ra = offA[qq], rb = offB[qq];
                 const real T = sT[qq];
-                const real2 e1 = tabA[x * TRI_CAP + ia];
-                const real2 e2 = tB[y * TRI_CAP + ia];
-                const real ebt = r_exp(be * T);
+                const real2 e1 = tabE[ra + ia];
+                const real2 e2 = tabE[rb + ia];
+                const real ebt = HE::eval(bes * T);
                 const real sim2 = e1.x * e2.y;   // exp(a1 D1 + a2 D2)
                 const real sim1 = e1.y * e2.x;   // exp(a2 D1 + a1 D2)
                 if (MODE == 0) {
                   acc[0] += T * (sim1 + sim2) * ebt;
                 } else if (MODE == 1) {
-                  const real D1 = sD[la[x]], D2 = sD[lb[y]];
+                  const real D1 = Drow[ra / TRI_CAP], D2 = Drow[rb / TRI_CAP];
                   const real w = ebt * T;
                   acc[0] += (sim2 * D1 + sim1 * D2) * w;
                   acc[1] += (sim2 * D2 + sim1 * D1) * w;
                   acc[NV - 1] += (sim1 + sim2) * w * T;
                 } else {
-                  const int s1 = la[x], s2 = lb[y];
-                  const real D1 = sD[s1], D2 = sD[s2];
-                  const real V1 = sV[s1], V2 = sV[s2];
+                  const real D1 = Drow[ra / TRI_CAP], D2 = Drow[rb / TRI_CAP];
+                  const real V1 = Vrow[ra / TRI_CAP], V2 = Vrow[rb / TRI_CAP];
                   const real U = sU[qq];
-                  const real a1 = tab.a1[pb + c0 + ia], a2 = tab.a2[pb + c0 + ia];
                   const real ss = sim1 + sim2;
                   const real opb = real(1) + be * T;
                   const real hT = real(0.5) * ebt * T;
@@ -270,38 +303,50 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
               }
             }
           }
-          // ---- combine the subsets of each channel in a fixed order.  `red` is its own region: the
-          // previous pass's combine finished before the barrier that followed this pass's staging.
+          // ---- the wave's four subsets of every channel, then the wave's own accumulators (fixed order)
 #pragma unroll
-          for (int v = 0; v < NV; v++) red[tid * NV + v] = acc[v];
-          __syncthreads();
-          if (tid < nch * NV) {
-            const int ia2 = tid / NV, v = tid - ia2 * NV;
-            real s = 0;
-            for (int u = 0; u < S; u++) s += red[(u * nch + ia2) * NV + v];
-            const int a = tab.ch[pb + c0 + ia2];
-            const real c3h = tab.c3[pb + c0 + ia2] * real(0.5);
+          for (int v = 0; v < NV; v++) {
+            real s = acc[v];
+            s += __shfl_xor(s, 16, WAVE);
+            s += __shfl_xor(s, 32, WAVE);
+            acc[v] = s;
+          }
+          if (lane < TRI_CAP && chan) {
+            const int a = tab.ch[pb + c0 + ia];
+            const real c3h = tab.c3[pb + c0 + ia] * real(0.5);
             if (MODE == 0) {
-              out_ch[a] += s * c3h;
+              my_out[a] += acc[0] * c3h;
             } else if (MODE == 1) {
-              acc_par[(sg * Aa + a) * 3 + v] += s * c3h * sP[a];
+              const real f = c3h * sP[a];
+#pragma unroll
+              for (int v = 0; v < 3; v++) my_acc[(sg * Aa + a) * 3 + v] += acc[v] * f;
             } else {
-              if (v == 0) out_ch[a] += s * c3h;
-              else acc_par[(sg * Aa + a) * 3 + (v - 1)] += s * c3h * sP[a];
+              my_out[a] += acc[0] * c3h;
+              const real f = c3h * sP[a];
+#pragma unroll
+              for (int v = 0; v < 3; v++) my_acc[(sg * Aa + a) * 3 + v] += acc[v + 1] * f;
             }
           }
-          // the next pass starts with a __syncthreads() before red/staging/tables are rewritten
         }
       }
     }
     __syncthreads();
     if (MODE != 1)
-      for (int a = tid; a < Aa; a += TRI_BLOCK) A.out[(size_t)atom * Aa + a] = out_ch[a];
+      for (int a = tid; a < Aa; a += TRI_BLOCK) {
+        real s = 0;
+#pragma unroll
+        for (int w = 0; w < TRI_WAVES; w++) s += outw[w * Aa + a];
+        A.out[(size_t)atom * Aa + a] = s;
+      }
     __syncthreads();
   }
   if (MODE != 0) {
-    const int nacc = nsig * Aa * 3;
-    for (int q = tid; q < nacc; q += TRI_BLOCK) A.partial[(size_t)blockIdx.x * nacc + q] = acc_par[q];
+    for (int q = tid; q < nacc; q += TRI_BLOCK) {
+      real s = 0;
+#pragma unroll
+      for (int w = 0; w < TRI_WAVES; w++) s += accw[(size_t)w * nacc + q];
+      A.partial[(size_t)blockIdx.x * nacc + q] = s;
+    }
   }
 }
 
