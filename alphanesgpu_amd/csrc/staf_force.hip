@@ -42,6 +42,10 @@ __device__ inline void bucket_push(int* bcnt, int* bent, int cap, size_t recv, i
   else atomicOr(status, 2);
 }
 
+}  // namespace staf
+#include "staf_force3.hpp"
+namespace staf {
+
 // ---------------------------------------------------------------------------
 // 2-body force, pass A.  One wave per centre, lane <-> slot.
 //   g_s = 1/2 sum_a G[a] c2[t_s,a] e^{alpha D}(1 + alpha D) * grad D_s
@@ -101,313 +105,6 @@ __global__ __launch_bounds__(F_BLOCK) void force2_kernel(const real* __restrict_
     const real tot = wave_sum(sf[c]);
     if (lane == 0) self[rowScr * 3 + c] = tot;
   }
-}
-
-template <typename real>
-struct Force3Lds {
-  static constexpr int CAPF = sizeof(real) == 8 ? 8 : 16;   // channels tabulated per pass
-  static constexpr int THREADS = 256;
-  static constexpr int NW = THREADS / WAVE;
-  static constexpr int MIN_WAVES = sizeof(real) == 8 ? 3 : 5;   // waves per SIMD the register budget must allow
-  static constexpr int WIN = 1024;   // triplets whose three scalars are held in LDS at a time
-  __host__ __device__ static int window(int na) { return na < WIN ? na : WIN; }
-  // The phase-1 pair tables and the phase-2 per-wave column sums share one region when every slot has a lane
-  // (nr <= 64: the column sums are written once, after the last window).
-  __host__ __device__ static size_t table_reals(int nr) { return (size_t)CAPF * nr * 2; }
-  __host__ __device__ static size_t wf_reals(int nr) { return (size_t)NW * 4 * nr; }
-  __host__ __device__ static size_t shared_reals(int nr) {
-    const size_t t = table_reals(nr), p = wf_reals(nr);
-    return nr > WAVE ? t + p : (t > p ? t : p);
-  }
-  __host__ __device__ static size_t bytes(int nr, int na, int Aa, int nt) {
-    size_t reals = shared_reals(nr) + (size_t)3 * window(na) + 4 * nr /*rowsum*/ + nr + 3 * nr + Aa + 4 * CAPF + 3 * nr;
-    return chan_table_bytes<real>(2 * nt - 1, Aa) + reals * sizeof(real) + (size_t)(2 * nr + NT_MAX + 1) * sizeof(int);
-  }
-};
-
-// ---------------------------------------------------------------------------
-// 3-body force, pass A.  One workgroup per centre.
-// Phase 1 (thread <-> triplet, class-enumerated): channel sums
-//     Sd  = sum_a net_a delta_a,  SBj = sum_a net_a Bp_j,a,  SBk = sum_a net_a Bp_k,a
-//   kept in LDS by storage index nn.
-// Phase 2 (wave <-> row j of the triplet triangle, lane <-> k): der3b is read here, once, in storage order
-//   (a row is contiguous).  The force on slot k from the rows a wave owns accumulates in lane k's registers;
-//   the force on slot j is the row sum, taken with register lane moves.  Per-wave results meet in LDS and are
-//   added in a fixed order:
-//     F_s = sum_p Sd(s,p) dT/dd_s(s,p) + (sum_p SB_s(s,p)) grad fc_s
-// The kernel is bound by latency and by how many workgroups fit a compute unit, so LDS is kept small: the
-// scalars of at most WIN triplets are resident; a centre with more triplets runs both phases once per window
-// of storage indices.  All global reads of a phase are issued together.
-// ---------------------------------------------------------------------------
-template <typename real>
-__global__ __launch_bounds__(Force3Lds<real>::THREADS, Force3Lds<real>::MIN_WAVES) void force3_kernel(const real* __restrict__ G, const real* __restrict__ Dsup,
-                                                         const real* __restrict__ Tang,
-                                                         const real* __restrict__ dDsup,
-                                                         const real* __restrict__ d3b, const int* __restrict__ im2,
-                                                         const real* __restrict__ alpha3b,
-                                                         const real* __restrict__ emb3b,
-                                                         const int* __restrict__ type_map,
-                                                         const int* __restrict__ numtriplet,
-                                                         real* __restrict__ gslot, real* __restrict__ self, int* bcnt,
-                                                         int* bent, int cap, int* status, int nf, int N, int Nl,
-                                                         int ld, int nr, int na, int Aa, int nt) {
-  using real2 = typename Vec2<real>::type;
-  using HE = HotExp<real>;
-  using L = Force3Lds<real>;
-  extern __shared__ __align__(16) unsigned char smem[];
-  const int nsig = 2 * nt - 1;
-  ChanTable<real> tab;
-  constexpr int CAPF = L::CAPF;
-  constexpr int NW = L::NW;
-  constexpr int THREADS = L::THREADS;
-  const int win = L::window(na);
-  unsigned char* sp = tab.carve(smem, nsig, Aa);
-  real2* tabE = (real2*)sp;             // [CAPF][nr]: rows of the class's second species follow the first
-  real* wf = (real*)sp + (nr > WAVE ? L::table_reals(nr) : 0);   // [NW][4][nr] per-wave column sums: 3 components + SBk
-  real* scal = (real*)sp + L::shared_reals(nr);                  // [3*win]
-  real* rowsum = scal + 3 * win;        // [4][nr] row sums: 3 components + SBj
-  real* bl_D = rowsum + 4 * nr;         // [nr]
-  real* bl_g = bl_D + nr;               // [3*nr] grad fc rows (der3bsupp)
-  real* bl_G = bl_g + 3 * nr;           // [Aa]
-  real* prm = bl_G + Aa;                // [CAPF][4] = a1, a2, beta, 1/4 G c3 of the tabulated channels
-  real* fs = prm + 4 * CAPF;            // [3*nr]
-  int* lst = (int*)(fs + 3 * nr);       // [nr]
-  int* stp = lst + nr;                  // [nr] species of every slot
-  int* off = stp + nr;                  // [NT_MAX+1]
-  PHASE_CLOCK_BEGIN();
-
-  const int tid = threadIdx.x;
-  const int lane = tid & (WAVE - 1), wave = tid / WAVE;
-  const int atom = blockIdx.x;
-  const int b = atom / Nl, p = atom - b * Nl;
-  const size_t rowAtom = (size_t)b * ld + p;
-  const int* im = im2 + rowAtom * (nr + 1);
-  int m = numtriplet[rowAtom];
-  if (m > nr) m = nr;
-  int ntri = (m * (m - 1)) / 2;
-  if (ntri > na) ntri = na;
-  const real* Trow = Tang + rowAtom * na;
-  const real2* d3 = (const real2*)d3b + rowAtom * 3 * na;
-  // Every global read of the set-up is issued here, back to back: the centre's T row (parked in the first of
-  // the three scalars of each triplet until phase 1 replaces it), slot data, and the registration of the slots
-  // with their receiving atoms (integer atomics whose return is only needed for a store).  One read per 128
-  // bytes of the centre's der3b rows starts their way from HBM long before phase 2 needs them.
-  for (int q = tid; q < ntri && q < win; q += THREADS) scal[3 * q] = Trow[q];
-  real warm = 0;
-  {
-    constexpr int STEP = 128 / sizeof(real2);
-    for (int q = tid * STEP; q < ntri; q += THREADS * STEP)
-      warm += d3[q].x + d3[na + q].x + d3[2 * na + q].x;
-  }
-  for (int s = tid; s < m; s += THREADS) {
-    const int nj = im[1 + s];
-    bl_D[s] = Dsup[rowAtom * nr + s];
-#pragma unroll
-    for (int c = 0; c < 3; c++) bl_g[c * nr + s] = dDsup[rowAtom * 3 * nr + c * nr + s];
-    stp[s] = type_map[nj];
-    bucket_push(bcnt, bent, cap, (size_t)b * N + nj, p * nr + s, status);
-  }
-  for (int a = tid; a < Aa; a += THREADS) bl_G[a] = G[(size_t)atom * Aa + a];
-  for (int q = tid; q < 4 * nr; q += THREADS) rowsum[q] = 0;
-  tab.build(alpha3b, emb3b);
-  __syncthreads();
-  PHASE_MARK(0);
-  if (tid < WAVE) group_slots_by_type(m, nt, stp, lst, off);
-  __syncthreads();
-  PHASE_MARK(1);
-
-  real* my_wf = wf + wave * 4 * nr;
-  if (m > WAVE)
-    for (int q = WAVE + lane; q < m; q += WAVE) {
-#pragma unroll
-      for (int c = 0; c < 4; c++) my_wf[c * nr + q] = 0;
-    }
-  real colk[4] = {0, 0, 0, 0};   // column sums of slot k = lane
-
-  for (int w0 = 0; w0 < ntri; w0 += win) {
-    const int w1 = (w0 + win) < ntri ? (w0 + win) : ntri;
-    if (w0 > 0) {
-      __syncthreads();   // phase 2 of the previous window is done with scal
-      for (int q = w0 + tid; q < w1; q += THREADS) scal[3 * (q - w0)] = Trow[q];
-    }
-    // ---- phase 1
-    for (int ta = 0; ta < nt; ta++) {
-      const int oa = uniform(off[ta]);
-      const int na_ = uniform(off[ta + 1]) - oa;
-      if (na_ == 0) continue;
-      for (int tb = ta; tb < nt; tb++) {
-        const int ob = uniform(off[tb]);
-        const int nb_ = uniform(off[tb + 1]) - ob;
-        const bool same = (ta == tb);
-        const int size = same ? (na_ * (na_ - 1)) / 2 : na_ * nb_;
-        if (size == 0) continue;
-        const int sg = ta + tb;
-        const int nact = uniform(tab.nact[sg]);
-        const int pb = sg * Aa;
-        const int* la = lst + oa;
-        const int* lb = lst + ob;
-        const int rowB0 = same ? 0 : na_;
-        const int nrows = same ? na_ : na_ + nb_;
-        const float inv_rows = 1.0f / (float)nrows, inv_nb = 1.0f / (float)nb_;
-        for (int c0 = 0; c0 < nact; c0 += CAPF) {
-          const int nch = (nact - c0) < CAPF ? (nact - c0) : CAPF;
-          __syncthreads();   // readers of the previous tables are done (and, for the first class, T is parked)
-          // E[ia][row] = (exp(a1 D), exp(a2 D)) for the slots of both species of the class
-          for (int e = tid; e < nrows * nch; e += THREADS) {
-            const int ia = small_div(e, nrows, inv_rows), row = e - ia * nrows;
-            const real d = bl_D[row < na_ ? la[row] : lb[row - na_]];
-            real2 v;
-            v.x = HE::eval(HE::scale(tab.a1[pb + c0 + ia]) * d);
-            v.y = HE::eval(HE::scale(tab.a2[pb + c0 + ia]) * d);
-            tabE[ia * nr + row] = v;
-          }
-          if (tid < nch) {
-            prm[4 * tid] = tab.a1[pb + c0 + tid];
-            prm[4 * tid + 1] = tab.a2[pb + c0 + tid];
-            prm[4 * tid + 2] = tab.be[pb + c0 + tid];
-            prm[4 * tid + 3] = real(0.25) * bl_G[tab.ch[pb + c0 + tid]] * tab.c3[pb + c0 + tid];   // 1/2 of E, 1/2 of T
-          }
-          __syncthreads();
-          PHASE_MARK(2);
-          for (int q = tid; q < size; q += THREADS) {
-            int x, y;
-            if (same) tri_decode_xy(q, nb_, x, y);
-            else { x = small_div(q, nb_, inv_nb); y = q - x * nb_; }
-            const int s1 = la[x], s2 = lb[y];
-            const bool lo = s1 < s2;
-            const int j = lo ? s1 : s2, k = lo ? s2 : s1;
-            const int nn = tri_rowstart(j, m) + k - j - 1;
-            if (nn < w0 || nn >= w1) continue;
-            real* sc = scal + 3 * (nn - w0);
-            const real T = c0 == 0 ? sc[0] : Trow[nn];
-            real Sd = 0, SB1 = 0, SB2 = 0;
-            const real2* pa = tabE + x;
-            const real2* pb2 = tabE + rowB0 + y;
-            for (int ia = 0; ia < nch; ia++) {
-              const real a1 = prm[4 * ia], a2 = prm[4 * ia + 1], be = prm[4 * ia + 2], nc = prm[4 * ia + 3];
-              const real2 e1 = pa[ia * nr];
-              const real2 e2 = pb2[ia * nr];
-              const real sim2 = e1.x * e2.y;   // exp(a1 D1 + a2 D2)
-              const real sim1 = e1.y * e2.x;   // exp(a2 D1 + a1 D2)
-              const real bt = be * T;
-              const real h = HE::eval(HE::scale(bt)) * nc;
-              Sd += h * (real(1) + bt) * (sim1 + sim2);
-              SB1 += h * (a1 * sim2 + a2 * sim1);
-              SB2 += h * (a1 * sim1 + a2 * sim2);
-            }
-            SB1 *= T;
-            SB2 *= T;
-            const real SBj = lo ? SB1 : SB2, SBk = lo ? SB2 : SB1;
-            if (c0 == 0) {
-              sc[0] = Sd; sc[1] = SBj; sc[2] = SBk;
-            } else {
-              sc[0] += Sd; sc[1] += SBj; sc[2] += SBk;
-            }
-          }
-          PHASE_MARK(3);
-        }
-        if (nact == 0) {
-          // no active channel for this class: its triplets contribute nothing
-          __syncthreads();   // T of the window is parked
-          for (int q = tid; q < size; q += THREADS) {
-            int j, k, nn;
-            class_pair(q, same, nb_, la, lb, m, j, k, nn);
-            if (nn < w0 || nn >= w1) continue;
-            scal[3 * (nn - w0)] = 0;
-            scal[3 * (nn - w0) + 1] = 0;
-            scal[3 * (nn - w0) + 2] = 0;
-          }
-        }
-      }
-    }
-    __syncthreads();
-    PHASE_MARK(4);
-
-    // ---- phase 2
-    constexpr int RB = 2;   // rows in flight per wave: their der3b loads are issued together
-    for (int j0 = wave * RB; j0 < m - 1; j0 += NW * RB) {
-      real2 dv[RB][3];
-      real Sd[RB], Bj[RB], Bk[RB];
-#pragma unroll
-      for (int r = 0; r < RB; r++) {
-        const int j = j0 + r;
-        const int nn = tri_rowstart(j, m) - j - 1 + lane;   // k = lane
-        const bool on = j < m - 1 && lane > j && lane < m && nn >= w0 && nn < w1;
-#pragma unroll
-        for (int c = 0; c < 3; c++) { dv[r][c].x = 0; dv[r][c].y = 0; }
-        Sd[r] = 0; Bj[r] = 0; Bk[r] = 0;
-        if (on) {
-#pragma unroll
-          for (int c = 0; c < 3; c++) dv[r][c] = d3[c * na + nn];
-          const real* sc = scal + 3 * (nn - w0);
-          Sd[r] = sc[0]; Bj[r] = sc[1]; Bk[r] = sc[2];
-        }
-      }
-#pragma unroll
-      for (int r = 0; r < RB; r++) {
-        const int j = j0 + r;
-        if (j >= m - 1) break;
-        real rj[4];
-#pragma unroll
-        for (int c = 0; c < 3; c++) { rj[c] = Sd[r] * dv[r][c].x; colk[c] += Sd[r] * dv[r][c].y; }
-        rj[3] = Bj[r];
-        colk[3] += Bk[r];
-        if (m > WAVE) {   // more than 64 slots: the rest of the row accumulates in LDS
-          const int rs = tri_rowstart(j, m) - j - 1;
-          for (int k = WAVE + lane; k < m; k += WAVE) {
-            const int nn = rs + k;
-            if (nn >= w0 && nn < w1) {
-              const real2 d0 = d3[nn], d1 = d3[na + nn], d2 = d3[2 * na + nn];
-              const real* sc = scal + 3 * (nn - w0);
-              rj[0] += sc[0] * d0.x; rj[1] += sc[0] * d1.x; rj[2] += sc[0] * d2.x; rj[3] += sc[1];
-              my_wf[k] += sc[0] * d0.y; my_wf[nr + k] += sc[0] * d1.y; my_wf[2 * nr + k] += sc[0] * d2.y;
-              my_wf[3 * nr + k] += sc[2];
-            }
-          }
-        }
-#pragma unroll
-        for (int c = 0; c < 4; c++) {
-          const real t = wave_sum_to_last(rj[c]);
-          if (lane == WAVE - 1) rowsum[c * nr + j] += t;   // row j belongs to this wave alone
-        }
-      }
-    }
-    PHASE_MARK(5);
-  }
-  // the tables are dead: when the column sums share their region it is free now
-  __syncthreads();
-  if (lane < m) {
-#pragma unroll
-    for (int c = 0; c < 4; c++) my_wf[c * nr + lane] = colk[c];
-  }
-  __syncthreads();
-  PHASE_MARK(6);
-  const size_t rowScr = (size_t)atom;
-  for (int s = tid; s < m; s += THREADS) {
-    real B = rowsum[3 * nr + s];
-    for (int w = 0; w < NW; w++) B += wf[(w * 4 + 3) * nr + s];
-#pragma unroll
-    for (int c = 0; c < 3; c++) {
-      real f = rowsum[c * nr + s];
-      for (int w = 0; w < NW; w++) f += wf[(w * 4 + c) * nr + s];
-      f += B * bl_g[c * nr + s];
-      fs[c * nr + s] = f;
-      gslot[(rowScr * nr + s) * 3 + c] = f;
-    }
-  }
-  __syncthreads();
-  if (tid < WAVE) {
-#pragma unroll
-    for (int c = 0; c < 3; c++) {
-      real a = 0;
-      for (int s = tid; s < m; s += WAVE) a -= fs[c * nr + s];
-      a = wave_sum(a);
-      if (tid == 0) self[rowScr * 3 + c] = a;
-    }
-  }
-  if (warm == real(12345.678)) status[0] |= 0;   // keeps the warm-up reads alive; never true for finite data
-  PHASE_MARK(7);
-  PHASE_CLOCK_END();
 }
 
 // ---------------------------------------------------------------------------
@@ -735,16 +432,17 @@ static int force_tripl(const real* G, const real* Dsup, const real* Tang, const 
   ForceScratch fs;
   int rc = force_scratch<real>(st, nf, N, Nl, nr, stream, &fs);
   if (rc) return rc;
-  size_t lds = Force3Lds<real>::bytes(nr, na, Aa, nt);
+  if (!Force3Cfg<real>::fits(nr, nt)) return STAF_E_LIMIT;
+  const size_t lds = Force3Cfg<real>::bytes(nr, Aa, nt);
   if (lds > 64 * 1024) {
-    if (lds > 160 * 1024) return STAF_E_LIMIT;
-    if (hipFuncSetAttribute((const void*)force3_kernel<real>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
-        hipSuccess)
+    if (lds > 160 * 1024 ||
+        hipFuncSetAttribute((const void*)force3_kernel<real>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
+            hipSuccess)
       return STAF_E_LIMIT;
   }
-  hipLaunchKernelGGL(force3_kernel<real>, dim3(nf * Nl), dim3(Force3Lds<real>::THREADS), lds, stream, G, Dsup, Tang, dDsup, d3b, im2,
-                     alpha3b, emb3b, type_map, numtriplet, (real*)fs.gslot, (real*)fs.self, fs.bcnt, fs.bent, fs.cap,
-                     st->status_d, nf, N, Nl, ld, nr, na, Aa, nt);
+  hipLaunchKernelGGL(force3_kernel<real>, dim3(nf * Nl), dim3(Force3Cfg<real>::THREADS), lds, stream, G, Dsup, Tang,
+                     dDsup, d3b, im2, alpha3b, emb3b, type_map, numtriplet, (real*)fs.gslot, (real*)fs.self, fs.bcnt,
+                     fs.bent, fs.cap, st->status_d, nf, N, Nl, ld, nr, na, Aa, nt);
   if (virial)
     launch_virial<real>(fs, im2, numtriplet, pos, box, tipos, actual_type, virial, nf, N, Nl, ld, nr, stream);
   return launch_gather<real>(st, fs, tipos, actual_type, force, nf, N, Nl, nr, stream);

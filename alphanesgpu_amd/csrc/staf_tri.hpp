@@ -42,10 +42,12 @@ template <typename real> struct HotExp;
 template <> struct HotExp<float> {
   __device__ static float scale(float a) { return a * 1.44269504088896341f; }
   __device__ static float eval(float t) { return __builtin_amdgcn_exp2f(t); }
+  __device__ static float unscale() { return 0.693147180559945309f; }   // scaled argument -> natural argument
 };
 template <> struct HotExp<double> {
   __device__ static double scale(double a) { return a; }
   __device__ static double eval(double t) { return exp(t); }
+  __device__ static double unscale() { return 1.0; }
 };
 
 // q / n for 0 <= q < 2^22, 1 <= n <= 2^11 without the integer-division sequence
