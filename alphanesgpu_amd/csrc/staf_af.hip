@@ -146,8 +146,11 @@ static int radial_afs(const real* D, int nr, const real* alpha2b, int Ar, real* 
   size_t lds = (size_t)2 * nt * Ar * sizeof(real) + (size_t)AF_WAVES * nr * (sizeof(real) + sizeof(int));
   if (lds > 64 * 1024) return STAF_E_LIMIT;
   const int atoms = nf * Nl;
-  hipLaunchKernelGGL(af2_kernel<real>, dim3((atoms + AF_WAVES - 1) / AF_WAVES), dim3(AF_BLOCK), lds,
-                     (hipStream_t)stream_, D, im2, alpha2b, emb2b, type_map, out, nf, Nl, ld, nr, Ar, nt);
+  {
+    KernelTimer kt_("af2_kernel", (hipStream_t)stream_);
+    hipLaunchKernelGGL(af2_kernel<real>, dim3((atoms + AF_WAVES - 1) / AF_WAVES), dim3(AF_BLOCK), lds,
+                       (hipStream_t)stream_, D, im2, alpha2b, emb2b, type_map, out, nf, Nl, ld, nr, Ar, nt);
+  }
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }
 
@@ -165,13 +168,17 @@ static int alpha_dist_grad(const real* D, int nr, const real* alpha2b, int Ar, r
   hipStream_t stream = (hipStream_t)stream_;
   const int nout = 2 * nt * Ar;
   const int nb = grad_blocks(nf * Nl);
-  real* partial = (real*)scratch_reserve(st, (size_t)nb * nout * sizeof(real));
+  real* partial = (real*)scratch_reserve(st, ((size_t)nb + RED_SLICES) * nout * sizeof(real));
+  real* red_tmp = partial ? partial + (size_t)nb * nout : nullptr;
   if (!partial) return STAF_E_HIP;
   size_t lds = (size_t)(2 * nt * Ar + AF_WAVES * nout + AF_WAVES * nr) * sizeof(real) + (size_t)AF_WAVES * nr * sizeof(int);
   if (lds > 64 * 1024) return STAF_E_LIMIT;
-  hipLaunchKernelGGL(grad2_kernel<real>, dim3(nb), dim3(AF_BLOCK), lds, stream, D, im2, alpha2b, emb2b, type_map, P,
-                     partial, nf, Nl, ld, nr, Ar, nt);
-  launch_reduce_partials<real>(partial, nb, nout, g_alpha, nt * Ar, g_emb, nt * Ar, stream);
+  {
+    KernelTimer kt_("grad2_kernel", stream);
+    hipLaunchKernelGGL(grad2_kernel<real>, dim3(nb), dim3(AF_BLOCK), lds, stream, D, im2, alpha2b, emb2b, type_map, P,
+                       partial, nf, Nl, ld, nr, Ar, nt);
+  }
+  launch_reduce_partials<real>(partial, nb, nout, g_alpha, nt * Ar, nt * Ar, g_emb, nt * Ar, nt * Ar, red_tmp, stream);
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }
 
@@ -191,7 +198,10 @@ static int angular_afs(const real* Dsup, const real* Tang, int nr, int na, real*
   A.Dsup = Dsup; A.Tang = Tang; A.im2 = im2; A.alpha3b = alpha3b; A.emb3b = emb3b; A.type_map = type_map;
   A.numtriplet = numtriplet; A.out = out;
   A.nf = nf; A.Nl = Nl; A.ld = ld; A.nr = nr; A.na = na; A.Aa = Aa; A.nt = nt;
-  hipLaunchKernelGGL((tri_reduce_kernel<real, 0>), dim3(nf * Nl), dim3(TRI_BLOCK), lds, (hipStream_t)stream_, A);
+  {
+    KernelTimer kt_("af3_kernel", (hipStream_t)stream_);
+    hipLaunchKernelGGL((tri_reduce_kernel<real, 0>), dim3(nf * Nl), dim3(TRI_BLOCK), lds, (hipStream_t)stream_, A);
+  }
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }
 
@@ -212,20 +222,23 @@ static int alphagrad_ang(const real* Dsup, const real* Tang, int nr, int na, con
   const int nsig = 2 * nt - 1;
   const int nout = nsig * Aa * 3;
   const int nb = nf * Nl < TRI_GRID_MAX ? nf * Nl : TRI_GRID_MAX;
-  real* partial = (real*)scratch_reserve(st, (size_t)nb * nout * sizeof(real));
+  real* partial = (real*)scratch_reserve(st, ((size_t)nb + RED_SLICES) * nout * sizeof(real));
+  real* red_tmp = partial ? partial + (size_t)nb * nout : nullptr;
   if (!partial) return STAF_E_HIP;
   size_t lds = TriLds<real, 1>::bytes(nr, Aa, nt);
   if (lds > 64 * 1024) return STAF_E_LIMIT;
   // rows sigma >= nsig of the outputs receive no contribution
   const int nall = ntc * Aa * 3;
-  launch_fill_zero<real>(g_alpha + nout, nall - nout, stream);
-  launch_fill_zero<real>(g_emb, ntc * Aa, stream);
   TriArgs<real> A = {};
   A.Dsup = Dsup; A.Tang = Tang; A.im2 = im2; A.alpha3b = alpha3b; A.emb3b = emb3b; A.type_map = type_map;
   A.numtriplet = numtriplet; A.P = P; A.partial = partial;
   A.nf = nf; A.Nl = Nl; A.ld = ld; A.nr = nr; A.na = na; A.Aa = Aa; A.nt = nt;
-  hipLaunchKernelGGL((tri_reduce_kernel<real, 1>), dim3(nb), dim3(TRI_BLOCK), lds, stream, A);
-  launch_reduce_partials<real>(partial, nb, nout, g_alpha, nout, (real*)nullptr, 0, stream);
+  {
+    KernelTimer kt_("grad3_kernel", stream);
+    hipLaunchKernelGGL((tri_reduce_kernel<real, 1>), dim3(nb), dim3(TRI_BLOCK), lds, stream, A);
+  }
+  // parameter rows sigma >= nsig and the embedding gradient (identically zero in the reference) are zero-filled here
+  launch_reduce_partials<real>(partial, nb, nout, g_alpha, nout, nall, g_emb, 0, ntc * Aa, red_tmp, stream);
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }
 

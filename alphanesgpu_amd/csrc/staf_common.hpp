@@ -187,6 +187,26 @@ int* bucket_reserve(DeviceState* st, size_t n_counters, size_t n_entries, hipStr
 int finish_op(DeviceState* st, hipStream_t stream);            // launch check (+ optional sync & status fetch)
 bool sync_errors_enabled();
 
+// Optional timing of single kernels with HIP events on the stream they are launched on (off by default; switched on
+// with staf_ops_kernel_timing).  A KernelTimer brackets one launch; the pairs are summed by staf_ops_kernel_time.
+bool kernel_timing_enabled();
+void kernel_timing_record(const char* kernel, hipEvent_t a, hipEvent_t b);
+struct KernelTimer {
+  hipEvent_t a = nullptr, b = nullptr;
+  hipStream_t stream;
+  const char* name;
+  KernelTimer(const char* kernel, hipStream_t s) : stream(s), name(kernel) {
+    if (!kernel_timing_enabled()) return;
+    if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) { a = b = nullptr; return; }
+    (void)hipEventRecord(a, stream);
+  }
+  ~KernelTimer() {
+    if (!a) return;
+    (void)hipEventRecord(b, stream);
+    kernel_timing_record(name, a, b);
+  }
+};
+
 // Descriptor geometry shared by all devices (set by construct_descriptors_light).
 template <typename real>
 struct DescConfig {

@@ -378,7 +378,10 @@ int desc_launch(const DescConfig<real>& c, const real* pos, const real* box, int
   A.status = st->status_d;
   size_t lds = desc_lds_bytes<real>(c.nr);
   if (lds > 60 * 1024) return STAF_E_LIMIT;
-  hipLaunchKernelGGL(desc_kernel<real>, dim3((unsigned)(nf * N)), dim3(256), lds, stream, A);
+  {
+    KernelTimer kt_("desc_kernel", stream);
+    hipLaunchKernelGGL(desc_kernel<real>, dim3((unsigned)(nf * N)), dim3(256), lds, stream, A);
+  }
   return finish_op(st, stream);
 }
 template int desc_launch<float>(const DescConfig<float>&, const float*, const float*, int, int, int, const int*,

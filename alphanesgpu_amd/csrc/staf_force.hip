@@ -379,9 +379,12 @@ static int launch_gather(DeviceState* st, const ForceScratch& fs, const int* tip
   size_t lds = (size_t)F_WAVES * fs.cap * (3 * sizeof(real) + sizeof(int));
   if (lds > 64 * 1024) return STAF_E_LIMIT;
   const int recv = nf * N;
-  hipLaunchKernelGGL(gather_kernel<real>, dim3((recv + F_WAVES - 1) / F_WAVES), dim3(F_BLOCK), lds, stream,
-                     (const real*)fs.gslot, (const real*)fs.self, fs.bcnt, (const int*)fs.bent, fs.cap, tipos,
-                     actual_type, force, nf, N, Nl, nr);
+  {
+    KernelTimer kt_("gather_kernel", stream);
+    hipLaunchKernelGGL(gather_kernel<real>, dim3((recv + F_WAVES - 1) / F_WAVES), dim3(F_BLOCK), lds, stream,
+                       (const real*)fs.gslot, (const real*)fs.self, fs.bcnt, (const int*)fs.bent, fs.cap, tipos,
+                       actual_type, force, nf, N, Nl, nr);
+  }
   return finish_op(st, stream);
 }
 
@@ -405,9 +408,12 @@ static int force_doublets(const real* G, const real* D, const real* dD, const in
   size_t lds = (size_t)(2 * nt * Ar + F_WAVES * Ar) * sizeof(real);
   if (lds > 64 * 1024) return STAF_E_LIMIT;
   const int atoms = nf * Nl;
-  hipLaunchKernelGGL(force2_kernel<real>, dim3((atoms + F_WAVES - 1) / F_WAVES), dim3(F_BLOCK), lds, stream, G, D, dD,
-                     im2, alpha2b, emb2b, type_map, (real*)fs.gslot, (real*)fs.self, fs.bcnt, fs.bent, fs.cap,
-                     st->status_d, nf, N, Nl, ld, nr, Ar, nt);
+  {
+    KernelTimer kt_("force2_kernel", stream);
+    hipLaunchKernelGGL(force2_kernel<real>, dim3((atoms + F_WAVES - 1) / F_WAVES), dim3(F_BLOCK), lds, stream, G, D, dD,
+                       im2, alpha2b, emb2b, type_map, (real*)fs.gslot, (real*)fs.self, fs.bcnt, fs.bent, fs.cap,
+                       st->status_d, nf, N, Nl, ld, nr, Ar, nt);
+  }
   if (virial)
     launch_virial<real>(fs, im2, (const int*)nullptr, pos, box, tipos, actual_type, virial, nf, N, Nl, ld, nr, stream);
   return launch_gather<real>(st, fs, tipos, actual_type, force, nf, N, Nl, nr, stream);
@@ -440,9 +446,12 @@ static int force_tripl(const real* G, const real* Dsup, const real* Tang, const 
             hipSuccess)
       return STAF_E_LIMIT;
   }
-  hipLaunchKernelGGL(force3_kernel<real>, dim3(nf * Nl), dim3(Force3Cfg<real>::THREADS), lds, stream, G, Dsup, Tang,
-                     dDsup, d3b, im2, alpha3b, emb3b, type_map, numtriplet, (real*)fs.gslot, (real*)fs.self, fs.bcnt,
-                     fs.bent, fs.cap, st->status_d, nf, N, Nl, ld, nr, na, Aa, nt);
+  {
+    KernelTimer kt_("force3_kernel", stream);
+    hipLaunchKernelGGL(force3_kernel<real>, dim3(nf * Nl), dim3(Force3Cfg<real>::THREADS), lds, stream, G, Dsup, Tang,
+                       dDsup, d3b, im2, alpha3b, emb3b, type_map, numtriplet, (real*)fs.gslot, (real*)fs.self, fs.bcnt,
+                       fs.bent, fs.cap, st->status_d, nf, N, Nl, ld, nr, na, Aa, nt);
+  }
   if (virial)
     launch_virial<real>(fs, im2, numtriplet, pos, box, tipos, actual_type, virial, nf, N, Nl, ld, nr, stream);
   return launch_gather<real>(st, fs, tipos, actual_type, force, nf, N, Nl, nr, stream);
@@ -464,15 +473,19 @@ static int gradforce_2b(const real* Q, const real* D, int nr, const real* alpha2
   hipStream_t stream = (hipStream_t)stream_;
   const int nout = 2 * nt * Ar;
   const int nb = grad_blocks_f(nf * Nl);
-  real* partial = (real*)scratch_reserve(st, (size_t)nb * nout * sizeof(real));
+  real* partial = (real*)scratch_reserve(st, ((size_t)nb + RED_SLICES) * nout * sizeof(real));
+  real* red_tmp = partial ? partial + (size_t)nb * nout : nullptr;
   if (!partial) return STAF_E_HIP;
   size_t lds = (size_t)(2 * nt * Ar + F_WAVES * nout + 2 * F_WAVES * nr) * sizeof(real) +
                (size_t)F_WAVES * nr * sizeof(int);
   if (lds > 64 * 1024) return STAF_E_LIMIT;
-  hipLaunchKernelGGL(gradforce2_kernel<real>, dim3(nb), dim3(F_BLOCK), lds, stream, Q, G, D, dD, im2, alpha2b, emb2b,
-                     type_map, tipos, actual_type, gnet, partial, Qvir, pos, box, g_force_skip_pbc, nf, N, Nl, ld, nr,
-                     Ar, nt);
-  launch_reduce_partials<real>(partial, nb, nout, g_alpha, nt * Ar, g_emb, nt * Ar, stream);
+  {
+    KernelTimer kt_("gradforce2_kernel", stream);
+    hipLaunchKernelGGL(gradforce2_kernel<real>, dim3(nb), dim3(F_BLOCK), lds, stream, Q, G, D, dD, im2, alpha2b, emb2b,
+                       type_map, tipos, actual_type, gnet, partial, Qvir, pos, box, g_force_skip_pbc, nf, N, Nl, ld, nr,
+                       Ar, nt);
+  }
+  launch_reduce_partials<real>(partial, nb, nout, g_alpha, nt * Ar, nt * Ar, g_emb, nt * Ar, nt * Ar, red_tmp, stream);
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }
 
@@ -497,21 +510,24 @@ static int gradforce_tripl(const real* Q, const real* G, const real* Dsup, const
   const int nsig = 2 * nt - 1;
   const int nout = nsig * Aa * 3;
   const int nb = nf * Nl < TRI_GRID_MAX ? nf * Nl : TRI_GRID_MAX;
-  real* partial = (real*)scratch_reserve(st, (size_t)nb * nout * sizeof(real));
+  real* partial = (real*)scratch_reserve(st, ((size_t)nb + RED_SLICES) * nout * sizeof(real));
+  real* red_tmp = partial ? partial + (size_t)nb * nout : nullptr;
   if (!partial) return STAF_E_HIP;
   size_t lds = TriLds<real, 2>::bytes(nr, Aa, nt);
   if (lds > 64 * 1024) return STAF_E_LIMIT;
   const int nall = ntc * Aa * 3;
-  launch_fill_zero<real>(g_alpha + nout, nall - nout, stream);
-  launch_fill_zero<real>(g_emb, ntc * Aa, stream);
   TriArgs<real> A = {};
   A.Dsup = Dsup; A.Tang = Tang; A.im2 = im2; A.alpha3b = alpha3b; A.emb3b = emb3b; A.type_map = type_map;
   A.numtriplet = numtriplet; A.P = G; A.Q = Q; A.dDsup = dDsup; A.d3b = d3b; A.tipos = tipos;
   A.actual_type = actual_type; A.out = gnet; A.partial = partial; A.Qvir = Qvir; A.pos = pos; A.box = box;
   A.skip_pbc = g_force_skip_pbc;
   A.nf = nf; A.N = N; A.Nl = Nl; A.ld = ld; A.nr = nr; A.na = na; A.Aa = Aa; A.nt = nt;
-  hipLaunchKernelGGL((tri_reduce_kernel<real, 2>), dim3(nb), dim3(TRI_BLOCK), lds, stream, A);
-  launch_reduce_partials<real>(partial, nb, nout, g_alpha, nout, (real*)nullptr, 0, stream);
+  {
+    KernelTimer kt_("gradforce3_kernel", stream);
+    hipLaunchKernelGGL((tri_reduce_kernel<real, 2>), dim3(nb), dim3(TRI_BLOCK), lds, stream, A);
+  }
+  // parameter rows sigma >= nsig and the embedding gradient (identically zero in the reference) are zero-filled here
+  launch_reduce_partials<real>(partial, nb, nout, g_alpha, nout, nall, g_emb, 0, ntc * Aa, red_tmp, stream);
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }
 

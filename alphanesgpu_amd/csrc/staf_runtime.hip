@@ -5,6 +5,9 @@
 #include <unordered_map>
 #include <memory>
 #include <stdio.h>
+#include <string>
+#include <utility>
+#include <vector>
 
 namespace staf {
 
@@ -13,6 +16,14 @@ static std::unordered_map<int, std::unique_ptr<DeviceState>> g_state;
 static int g_sync_errors = 1;
 
 bool sync_errors_enabled() { return g_sync_errors != 0; }
+
+static int g_kernel_timing = 0;
+static std::unordered_map<std::string, std::vector<std::pair<hipEvent_t, hipEvent_t>>> g_kernel_events;
+bool kernel_timing_enabled() { return g_kernel_timing != 0; }
+void kernel_timing_record(const char* kernel, hipEvent_t a, hipEvent_t b) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  g_kernel_events[kernel].emplace_back(a, b);
+}
 
 DeviceState* device_state() {
   int dev = 0;
@@ -104,6 +115,26 @@ int staf_ops_poll_status(void* stream) {
   staf::DeviceState* st = staf::device_state();
   if (!st) return STAF_E_HIP;
   return staf::fetch_status(st, (hipStream_t)stream);
+}
+
+void staf_ops_kernel_timing(int enable) { staf::g_kernel_timing = enable ? 1 : 0; }
+
+int staf_ops_kernel_time(const char* kernel, double* total_ms, int* launches) {
+  if (!kernel || !total_ms || !launches) return STAF_E_BAD_ARG;
+  if (hipDeviceSynchronize() != hipSuccess) return STAF_E_HIP;
+  std::lock_guard<std::mutex> lock(staf::g_mu);
+  *total_ms = 0.0;
+  *launches = 0;
+  auto it = staf::g_kernel_events.find(kernel);
+  if (it == staf::g_kernel_events.end()) return STAF_OK;
+  for (auto& ev : it->second) {
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, ev.first, ev.second) == hipSuccess) { *total_ms += ms; ++*launches; }
+    (void)hipEventDestroy(ev.first);
+    (void)hipEventDestroy(ev.second);
+  }
+  it->second.clear();
+  return STAF_OK;
 }
 
 void staf_ops_release(void) {

@@ -275,9 +275,9 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
                 const real ebt = HE::eval(bes * T);
                 const real sim2 = e1.x * e2.y;   // exp(a1 D1 + a2 D2)
                 const real sim1 = e1.y * e2.x;   // exp(a2 D1 + a1 D2)
-                if (MODE == 0) {
+                if constexpr (MODE == 0) {
                   acc[0] += T * (sim1 + sim2) * ebt;
-                } else if (MODE == 1) {
+                } else if constexpr (MODE == 1) {
                   const real D1 = Drow[ra / TRI_CAP], D2 = Drow[rb / TRI_CAP];
                   const real w = ebt * T;
                   acc[0] += (sim2 * D1 + sim1 * D2) * w;
@@ -316,9 +316,9 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
           if (lane < TRI_CAP && chan) {
             const int a = tab.ch[pb + c0 + ia];
             const real c3h = tab.c3[pb + c0 + ia] * real(0.5);
-            if (MODE == 0) {
+            if constexpr (MODE == 0) {
               my_out[a] += acc[0] * c3h;
-            } else if (MODE == 1) {
+            } else if constexpr (MODE == 1) {
               const real f = c3h * sP[a];
 #pragma unroll
               for (int v = 0; v < 3; v++) my_acc[(sg * Aa + a) * 3 + v] += acc[v] * f;

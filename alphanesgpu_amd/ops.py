@@ -88,6 +88,18 @@ def poll_status():
     call("staf_ops_poll_status", _stream())
 
 
+def kernel_timing(on=True):
+    """Brackets every kernel the library launches with HIP events on its launch stream (measurement aid)."""
+    _lib.lib().staf_ops_kernel_timing(_I(1 if on else 0))
+
+
+def kernel_time(kernel):
+    """(summed milliseconds, launches) of the named kernel since the last call for that name; waits for the device."""
+    ms, n = C.c_double(0.0), C.c_int(0)
+    call("staf_ops_kernel_time", C.c_char_p(kernel.encode()), C.byref(ms), C.byref(n))
+    return ms.value, n.value
+
+
 def version():
     return _lib.lib().staf_ops_version().decode()
 

@@ -24,30 +24,39 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (see profiles/),
+# scaled by what the same counters read for a copy kernel of known size; None where no such run was made.
+TRAFFIC = {}
+
 
 def algorithmic_bytes(N, tipos, nr, na, Ar, Aa, nt, s):
     """Bytes each op's signature forces through HBM once per frame (inputs read once, outputs written once),
-    per-species calls summed."""
+    per-species calls summed.  Keys are the kernels that do the op's work."""
     ntc = nt * (nt + 1) // 2
-    desc = (N * (8 * nr + 7 * na)) * s + N * (nr + 1 + 2 * na + 1) * 4 + (3 * N + 6) * s
-    af = force = galpha = gforce = 0
+    out = dict(desc_kernel=(N * (8 * nr + 7 * na)) * s + N * (nr + 1 + 2 * na + 1) * 4 + (3 * N + 6) * s)
+    for k in ("af2", "af3", "force2", "force3", "grad2", "grad3", "gradforce2", "gradforce3"):
+        out[k + "_kernel"] = 0
     for Nl in tipos:
         par2 = 2 * nt * Ar * s
         par3 = (3 * ntc * Aa + ntc * Aa) * s
         tm = N * 4
-        af += Nl * nr * s + Nl * (nr + 1) * 4 + par2 + tm + Nl * Ar * s                       # ComputeSortProj
-        af += Nl * (na + nr) * s + Nl * (2 * na + nr + 1 + 1) * 4 + par3 + tm + Nl * Aa * s     # ComputeSortProj3body
-        force += Nl * (Ar + nr + 3 * nr) * s + Nl * (nr + 1) * 4 + par2 + tm + 3 * N * s        # ComputeForceRadial
-        force += (Nl * (Aa + nr + na + 3 * nr + 6 * na) * s + Nl * (nr + 1 + 2 * na + 1) * 4 + par3 + tm
-                  + 3 * N * s)                                                                  # ComputeForceTripl
-        galpha += Nl * (Ar + nr) * s + Nl * (nr + 1) * 4 + par2 + tm + 2 * nt * Ar * s          # ComputeTwoBodyParGrad
-        galpha += (Nl * (Aa + na + nr) * s + Nl * (2 * na + nr + 1 + 1) * 4 + par3 + tm
-                   + (3 * ntc * Aa + ntc * Aa) * s)                                             # ...3bodyGrad
-        gforce += (3 * N * s + Nl * (Ar + nr + 3 * nr) * s + Nl * (nr + 1) * 4 + par2 + tm
-                   + Nl * Ar * s + 2 * nt * Ar * s)                                             # ComputeForceRadialGrad
-        gforce += (3 * N * s + Nl * (Aa + nr + na + 3 * nr + 6 * na) * s + Nl * (nr + 1 + 2 * na + 1) * 4 + par3
-                   + tm + Nl * Aa * s + (3 * ntc * Aa + ntc * Aa) * s)                          # ComputeForceTriplGrad
-    return dict(descriptor=desc, af_fwd=af, force=force, grad_alpha=galpha, grad_force=gforce)
+        out["af2_kernel"] += Nl * nr * s + Nl * (nr + 1) * 4 + par2 + tm + Nl * Ar * s            # ComputeSortProj
+        out["af3_kernel"] += (Nl * (na + nr) * s + Nl * (2 * na + nr + 1 + 1) * 4 + par3 + tm
+                              + Nl * Aa * s)                                                      # ComputeSortProj3body
+        out["force2_kernel"] += (Nl * (Ar + nr + 3 * nr) * s + Nl * (nr + 1) * 4 + par2 + tm
+                                 + 3 * N * s)                                                     # ComputeForceRadial
+        out["force3_kernel"] += (Nl * (Aa + nr + na + 3 * nr + 6 * na) * s + Nl * (nr + 1 + 2 * na + 1) * 4 + par3
+                                 + tm + 3 * N * s)                                                # ComputeForceTripl
+        out["grad2_kernel"] += (Nl * (Ar + nr) * s + Nl * (nr + 1) * 4 + par2 + tm
+                                + 2 * nt * Ar * s)                                                # ComputeTwoBodyParGrad
+        out["grad3_kernel"] += (Nl * (Aa + na + nr) * s + Nl * (2 * na + nr + 1 + 1) * 4 + par3 + tm
+                                + (3 * ntc * Aa + ntc * Aa) * s)                                  # ...3bodyGrad
+        out["gradforce2_kernel"] += (3 * N * s + Nl * (Ar + nr + 3 * nr) * s + Nl * (nr + 1) * 4 + par2 + tm
+                                     + Nl * Ar * s + 2 * nt * Ar * s)                             # ComputeForceRadialGrad
+        out["gradforce3_kernel"] += (3 * N * s + Nl * (Aa + nr + na + 3 * nr + 6 * na) * s
+                                     + Nl * (nr + 1 + 2 * na + 1) * 4 + par3 + tm + Nl * Aa * s
+                                     + (3 * ntc * Aa + ntc * Aa) * s)                             # ComputeForceTriplGrad
+    return out
 
 
 def cpu_baseline(batch, params, up, mode, nr, na, max_frames=2):
@@ -213,15 +222,24 @@ def main():
     op_ms = {k: float(np.mean([a.elapsed_time(b) for a, b in v])) for k, v in timers.items()}
     calls = {k: len(v) // nprof for k, v in timers.items()}
 
+    # per-kernel GPU time from the library's own HIP events, recorded on the stream each kernel is launched on
+    ops.kernel_timing(True)
+    for _ in range(nprof):
+        step()
+    ops.kernel_timing(False)
     s = np.dtype(dtype).itemsize
     ab = algorithmic_bytes(N, tipos, nr, na, Ar, Aa, nt, s)
-    # dominant kernel: the descriptor kernel (the op is a single launch, so the op's event time is the kernel's)
-    desc_ms = op_ms["descriptor"]
-    achieved = ab["descriptor"] * nf / (desc_ms * 1e-3) / 1e9
+    kern = {}
+    for name in list(ab) + ["gather_kernel"]:
+        ms, n = ops.kernel_time(name)
+        if n:
+            kern[name] = dict(ms_per_step=ms / nprof, launches_per_step=n // nprof, avg_launch_ms=ms / n)
     per_step = {k: op_ms[k] * calls[k] for k in op_ms}
-    step_bytes = ab["descriptor"] + ab["af_fwd"] + ab["force"]
-    if mode == "full_step":
-        step_bytes += ab["grad_alpha"] + ab["grad_force"]
+    step_bytes = sum(ab[k] for k in kern if k in ab)
+    # the kernel the step spends most of its time in, priced against HBM with the bytes its op signature moves
+    dom = max((k for k in kern if k in ab), key=lambda k: kern[k]["ms_per_step"])
+    dom_bytes_per_launch = ab[dom] * nf / kern[dom]["launches_per_step"]
+    achieved = dom_bytes_per_launch / (kern[dom]["avg_launch_ms"] * 1e-3) / 1e9
     out = {
         "metric": "frames/s descriptor fwd+force/alpha bwd, 768-atom water fp32/fp64; % HBM roofline",
         "value": nf * args.steps / el,
@@ -238,9 +256,14 @@ def main():
         "config": {"workload": args.workload, "mode": mode, "atoms": N, "frames_per_step": nf, "Rc": synth.RC,
                    "radial_buffer": nr, "angular_buffer": na, "Ar": Ar, "Aa": Aa,
                    "species_tensors": "contiguous copies" if args.contiguous_splits else "views"},
-        "roofline": {"bound": "hbm", "kernel": "desc_kernel", "achieved": achieved, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "algorithmic_bytes_per_launch": ab["descriptor"] * nf, "avg_launch_ms": desc_ms},
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": TRAFFIC.get((dom, args.workload)),
+                     "algorithmic_bytes_per_launch": dom_bytes_per_launch,
+                     "avg_launch_ms": kern[dom]["avg_launch_ms"],
+                     "launches_per_step": kern[dom]["launches_per_step"]},
+        "kernel_hbm_frac": {k: ab[k] * nf / (kern[k]["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS
+                            for k in kern if k in ab},
+        "kernel_ms_per_step": {k: v["ms_per_step"] for k, v in kern.items()},
         "whole_step_hbm_frac": step_bytes * nf / (el / args.steps) / 1e9 / HBM_PEAK_GBS,
         "op_ms_per_step": per_step,
         "ms_per_frame": el / args.steps * 1e3 / nf,
