@@ -87,14 +87,16 @@ __device__ inline int wave_max(int v) {
 // STAF/src/descriptor_builder/reforce.cu.cc:137-146.
 __device__ inline int tri_rowstart(int j, int m) { return j * m - (j * (j + 1)) / 2; }
 
-// Inverse of the numbering: nn -> (j,k), 0 <= nn < m(m-1)/2.
+// Inverse of the numbering: nn -> (j,k), 0 <= nn < m(m-1)/2, m <= 2048.  The hardware square root (1 ulp) puts
+// the row estimate within one of the exact row; the comparisons with the exact integer row starts settle it.
 __device__ inline void tri_decode(int nn, int m, int& j, int& k) {
   const int t = 2 * m - 1;
-  int jj = (int)(((float)t - sqrtf((float)(t * t - 8 * nn))) * 0.5f);
-  if (jj < 0) jj = 0;
-  if (jj > m - 2) jj = m - 2;
-  while (jj < m - 2 && tri_rowstart(jj + 1, m) <= nn) ++jj;
-  while (jj > 0 && tri_rowstart(jj, m) > nn) --jj;
+  int jj = (int)(((float)t - __builtin_amdgcn_sqrtf((float)(t * t - 8 * nn))) * 0.5f);
+  jj = jj < 0 ? 0 : (jj > m - 2 ? m - 2 : jj);
+  if (jj > 0 && tri_rowstart(jj, m) > nn) --jj;
+  if (jj > 0 && tri_rowstart(jj, m) > nn) --jj;
+  if (jj < m - 2 && tri_rowstart(jj + 1, m) <= nn) ++jj;
+  if (jj < m - 2 && tri_rowstart(jj + 1, m) <= nn) ++jj;
   j = jj;
   k = nn - tri_rowstart(jj, m) + jj + 1;
 }

@@ -221,7 +221,17 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
       PHASE_MARK(3);
     }
 
-    // ---- contraction with der3b, slot sums of this wave
+    // ---- contraction with der3b, slot sums of this wave.  The reads of all passes are issued together.
+    real2 dv[NP][3];
+#pragma unroll
+    for (int p = 0; p < NP; p++) {
+      const int nn = w0 + (p * NW + wave) * WAVE + lane;
+#pragma unroll
+      for (int c = 0; c < 3; c++) {
+        dv[p][c].x = 0; dv[p][c].y = 0;
+        if (nn < ntri) dv[p][c] = d3[c * na + nn];
+      }
+    }
 #pragma unroll
     for (int p = 0; p < NP; p++) {
       const int nn0 = w0 + (p * NW + wave) * WAVE;   // first storage index of the pass
@@ -231,7 +241,7 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
       const int j = jk[p] & 0xff, k = (jk[p] >> 8) & 0xff;
       real vj[4] = {0, 0, 0, 0}, vk[4] = {0, 0, 0, 0};
       if (valid) {
-        const real2 d0 = d3[nn], d1 = d3[na + nn], d2 = d3[2 * na + nn];
+        const real2 d0 = dv[p][0], d1 = dv[p][1], d2 = dv[p][2];
         vj[0] = Sd[p] * d0.x; vj[1] = Sd[p] * d1.x; vj[2] = Sd[p] * d2.x; vj[3] = S1[p] * T[p];
         vk[0] = Sd[p] * d0.y; vk[1] = Sd[p] * d1.y; vk[2] = Sd[p] * d2.y; vk[3] = S2[p] * T[p];
       }
@@ -283,13 +293,14 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
       t4[c] = t;
     }
 #pragma unroll
-    for (int c = 0; c < 3; c++) {
-      const real f = t4[c] + t4[3] * sg[c * nr + s];
-      gslot[((size_t)atom * nr + s) * 3 + c] = f;
-      fs[c * nr + s] = f;
-    }
+    for (int c = 0; c < 3; c++) fs[c * nr + s] = t4[c] + t4[3] * sg[c * nr + s];
   }
   __syncthreads();
+  // global stores after the last barrier: nothing waits for them
+  for (int s = tid; s < m; s += THREADS) {
+#pragma unroll
+    for (int c = 0; c < 3; c++) gslot[((size_t)atom * nr + s) * 3 + c] = fs[c * nr + s];
+  }
   if (tid < WAVE) {
 #pragma unroll
     for (int c = 0; c < 3; c++) {
