@@ -26,7 +26,13 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (see profiles/),
 # scaled by what the same counters read for a copy kernel of known size; None where no such run was made.
-TRAFFIC = {}
+TRAFFIC = {
+    # (FETCH_SIZE KiB x 2.0 + WRITE_SIZE KiB x 1.0) x 1024, averaged over the two per-species launches of a step;
+    # factors from a 256 MiB device copy in the same runs (profiles/force3_kernel_water768_f32_hbm_counters.txt,
+    # profiles/gradforce3_kernel_water768_f64_hbm_counters.txt)
+    ("force3_kernel", "water768_f32"): 39.9e6,
+    ("gradforce3_kernel", "water768_f64"): 77.8e6,
+}
 
 
 def algorithmic_bytes(N, tipos, nr, na, Ar, Aa, nt, s):
@@ -106,6 +112,8 @@ def main():
     ap.add_argument("--workload", default="water768_f32")
     ap.add_argument("--mode", default=None, choices=[None, "fwd_force", "full_step"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
+                    help="also run a plain device copy of this size three times (reference point for HBM counters)")
     ap.add_argument("--contiguous-splits", action="store_true",
                     help="copy per-species tensors like tf.split instead of passing views")
     args = ap.parse_args()
@@ -202,6 +210,14 @@ def main():
                                                                          ntrk), record)
             Ftot = f2 + f3 if Ftot is None else Ftot + f2 + f3
         return Ftot
+
+    if args.calibrate_copy:
+        src = torch.ones(args.calibrate_copy * (1 << 20) // 4, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step()
