@@ -8,6 +8,7 @@
 // Dense stack of staf_mlp.cpp evaluated on the host between the fingerprint and the force kernels.
 #include "staf_common.hpp"
 #include "staf_reduce.hpp"
+#include "staf_mlp_dev.hpp"
 #include "../../include/staf.h"
 #include "../../include/staf_mlp.h"
 
@@ -85,7 +86,11 @@ struct StafModel {
   staf::DescConfig<double> cfg;
   hipStream_t stream = nullptr;
   // device buffers
-  DevBuf<double> pos, box, force, force_op, virial_op, af2, af3, g2, g3;
+  DevBuf<double> pos, box, force, force_op, virial_op, af2, af3, g2, g3, e_atom, virial_acc;
+  // device-resident MLP (default); false: the host evaluation of staf_mlp.cpp between the kernels
+  bool dev_mlp = false;
+  std::vector<staf::DevMlpNet> dnets;
+  std::vector<double> e_atom_h;
   DevBuf<double> raddescr, angdescr, des3bsupp, der2b, der3b, der3bsupp;
   DevBuf<int> intmap2b, intmap3b, numtriplet, type_map, tipos, actual_type, how, with;
   // host staging
@@ -176,9 +181,11 @@ int staf_cuda_set_device(int device_id) {
 void staf_free(StafModel* m) {
   if (!m) return;
   if (m->mlp) staf_mlp_destroy(m->mlp);
+  for (auto& n : m->dnets) staf::dev_mlp_free(&n);
   for (auto* v : {&m->alpha2b, &m->alpha3b, &m->emb2b, &m->emb3b})
     for (auto& b : *v) b.release();
-  for (DevBuf<double>* b : {&m->pos, &m->box, &m->force, &m->force_op, &m->virial_op, &m->af2, &m->af3, &m->g2, &m->g3,
+  for (DevBuf<double>* b : {&m->pos, &m->box, &m->force, &m->force_op, &m->virial_op, &m->af2, &m->af3, &m->g2, &m->g3, &m->e_atom,
+                            &m->virial_acc,
                             &m->raddescr, &m->angdescr, &m->des3bsupp, &m->der2b, &m->der3b, &m->der3bsupp})
     b->release();
   for (DevBuf<int>* b : {&m->intmap2b, &m->intmap3b, &m->numtriplet, &m->type_map, &m->tipos, &m->actual_type, &m->how,
@@ -222,6 +229,18 @@ StafModel* staf_load(const char* model_dir, const StafOptions* opt) {
       staf_free(m);
       return NULL;
     }
+  // The MLP runs on the GPU between the fingerprint and the force kernels unless the caller asks for the host
+  // evaluation (StafOptions.reserved bit 1, or STAF_MLP_HOST=1 in the environment).
+  if (!(m->opt.reserved & 2) && !getenv("STAF_MLP_HOST")) {
+    m->dnets.resize(m->nt);
+    m->dev_mlp = true;
+    for (int k = 0; k < m->nt && m->dev_mlp; k++) m->dev_mlp = staf::dev_mlp_upload(m->mlp, k, &m->dnets[k]);
+    if (!m->dev_mlp) {
+      for (auto& n : m->dnets) staf::dev_mlp_free(&n);
+      m->dnets.clear();
+      fprintf(stderr, "staf_load: MLP not representable on the device path, evaluating it on the host\n");
+    }
+  }
   if (staf::desc_configure<double>(m->cfg, m->Rc, m->nr, m->na, m->Rs, m->Ra) != STAF_OK) {
     staf_free(m);
     return NULL;
@@ -305,6 +324,7 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
   bool ok = m->pos.reserve((size_t)nall * 3) && m->box.reserve(6) && m->force.reserve((size_t)nall * 3) &&
             m->force_op.reserve((size_t)nall * 3) && m->virial_op.reserve(9) && m->af2.reserve(L * amax2) &&
             m->af3.reserve(L * amax3) && m->g2.reserve(L * amax2) && m->g3.reserve(L * amax3) &&
+            m->e_atom.reserve(L) && m->virial_acc.reserve(9) &&
             m->raddescr.reserve(L * nr) && m->angdescr.reserve(L * na) && m->des3bsupp.reserve(L * nr) &&
             m->der2b.reserve(L * 3 * nr) && m->der3b.reserve(L * 6 * na) && m->der3bsupp.reserve(L * 3 * nr) &&
             m->intmap2b.reserve(L * (nr + 1)) && m->intmap3b.reserve(L * 2 * na) && m->numtriplet.reserve(L) &&
@@ -334,106 +354,154 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
   if (rc == STAF_E_RADIAL_OVERFLOW) return -10;
   if (rc != STAF_OK) return -20;
 
-  // ---- fingerprints of every species, packed rows [Ar+Aa] for the MLP
-  size_t total = 0;
-  for (int k = 0; k < nt; k++) total += (size_t)tipos[k] * (m->Ar[k] + m->Aa[k]);
-  m->af_h.resize(total);
-  m->gr_h.assign(total, 0.0);
-  size_t off = 0;
-  int shift = 0;
-  for (int k = 0; k < nt; shift += tipos[k], k++) {
-    const int Nl = tipos[k], Ar = m->Ar[k], Aa = m->Aa[k];
-    if (Nl == 0) continue;
-    const size_t o = (size_t)shift;
-    rc = staf_op_radial_afs_f64(m->raddescr.p + o * nr, nr, m->alpha2b[k].p, Ar, m->af2.p, 1, Nl,
-                                m->intmap2b.p + o * (nr + 1), m->emb2b[k].p, m->type_map.p, nt, nlocal, st);
-    if (rc == STAF_OK)
-      rc = staf_op_angular_afs_f64(m->des3bsupp.p + o * nr, m->angdescr.p + o * na, nr, na, m->af3.p, 1, Nl,
-                                   m->intmap3b.p + o * 2 * na, m->intmap2b.p + o * (nr + 1), m->alpha3b[k].p, Aa,
-                                   m->emb3b[k].p, m->type_map.p, m->numtriplet.p + o, nt, nlocal, st);
-    if (rc != STAF_OK) return -20;
-    m->tmp2.resize((size_t)Nl * Ar);
-    m->tmp3.resize((size_t)Nl * Aa);
-    STAF_HIP_OK(hipMemcpyAsync(m->tmp2.data(), m->af2.p, m->tmp2.size() * sizeof(double), hipMemcpyDeviceToHost, st));
-    STAF_HIP_OK(hipMemcpyAsync(m->tmp3.data(), m->af3.p, m->tmp3.size() * sizeof(double), hipMemcpyDeviceToHost, st));
-    STAF_HIP_OK(hipStreamSynchronize(st));
-    for (int a = 0; a < Nl; a++) {
-      double* row = &m->af_h[off + (size_t)a * (Ar + Aa)];
-      memcpy(row, &m->tmp2[(size_t)a * Ar], Ar * sizeof(double));
-      memcpy(row + Ar, &m->tmp3[(size_t)a * Aa], Aa * sizeof(double));
-    }
-    off += (size_t)Nl * (Ar + Aa);
-  }
-
-  // ---- MLP on the host (libstaf/vendor/jmd/nn_nn_mlp.cu:657-768): float32 nets see float32 fingerprints
-  std::vector<int> n_af(nt);
-  for (int k = 0; k < nt; k++) n_af[k] = m->Ar[k] + m->Aa[k];
-  StafMlpEval ev;
-  memset(&ev, 0, sizeof(ev));
-  ev.n_type = nt;
-  ev.n_atoms = tipos.data();
-  ev.n_af = n_af.data();
   double energy = 0.0;
-  if (staf_mlp_precision(m->mlp) == 0) {
-    m->af_f.resize(total);
-    m->gr_f.assign(total, 0.f);
-    for (size_t i = 0; i < total; i++) m->af_f[i] = (float)m->af_h[i];
-    float e_f = 0.f;
-    ev.af_f32 = m->af_f.data();
-    ev.energy_f32 = &e_f;
-    ev.dE_daf_f32 = m->gr_f.data();
-    if (staf_mlp_eval(m->mlp, &ev) != 0) return -20;
-    energy = (double)e_f;
-    for (size_t i = 0; i < total; i++) m->gr_h[i] = (double)m->gr_f[i];
-  } else {
-    ev.af_f64 = m->af_h.data();
-    ev.energy_f64 = &energy;
-    ev.dE_daf_f64 = m->gr_h.data();
-    if (staf_mlp_eval(m->mlp, &ev) != 0) return -20;
-  }
-  if (!isfinite(energy))
-    fprintf(stderr, "staf_compute: non-finite energy=%g nlocal=%d nghost=%d\n", energy, nlocal, nghost);
-
-  // ---- forces: 2-body + 3-body of every centre species, with the virial
-  staf_op_force_set_skip_pbc(ext ? 1 : 0);
-  staf::launch_fill_zero<double>(m->force.p, nall * 3, st);
-  double W[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0}, Wk[9];
-  off = 0;
-  shift = 0;
+  double W[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
   const int n3 = nall * 3;
-  for (int k = 0; k < nt; shift += tipos[k], k++) {
-    const int Nl = tipos[k], Ar = m->Ar[k], Aa = m->Aa[k];
-    if (Nl == 0) continue;
-    const size_t o = (size_t)shift;
-    m->tmp2.resize((size_t)Nl * Ar);
-    m->tmp3.resize((size_t)Nl * Aa);
-    for (int a = 0; a < Nl; a++) {
-      const double* row = &m->gr_h[off + (size_t)a * (Ar + Aa)];
-      memcpy(&m->tmp2[(size_t)a * Ar], row, Ar * sizeof(double));
-      memcpy(&m->tmp3[(size_t)a * Aa], row + Ar, Aa * sizeof(double));
-    }
-    off += (size_t)Nl * (Ar + Aa);
-    STAF_HIP_OK(hipMemcpyAsync(m->g2.p, m->tmp2.data(), m->tmp2.size() * sizeof(double), hipMemcpyHostToDevice, st));
-    STAF_HIP_OK(hipMemcpyAsync(m->g3.p, m->tmp3.data(), m->tmp3.size() * sizeof(double), hipMemcpyHostToDevice, st));
-    STAF_HIP_OK(hipStreamSynchronize(st));
-    for (int body = 2; body <= 3; body++) {
-      if (body == 2)
-        rc = staf_op_force_doublets_f64(m->g2.p, m->raddescr.p + o * nr, m->der2b.p + o * 3 * nr,
-                                        m->intmap2b.p + o * (nr + 1), nr, nall, 1, Ar, m->alpha2b[k].p, m->emb2b[k].p,
-                                        nt, m->tipos.p, m->actual_type.p + k, m->force_op.p, m->type_map.p, Nl,
-                                        m->virial_op.p, m->pos.p, m->box.p, nlocal, st);
-      else
-        rc = staf_op_force_tripl_f64(m->g3.p, m->des3bsupp.p + o * nr, m->angdescr.p + o * na,
-                                     m->der3bsupp.p + o * 3 * nr, m->der3b.p + o * 6 * na,
-                                     m->intmap2b.p + o * (nr + 1), m->intmap3b.p + o * 2 * na, nr, na, nall, 1, Aa,
-                                     m->emb3b[k].p, nt, m->tipos.p, m->actual_type.p + k, m->force_op.p,
-                                     m->numtriplet.p + o, m->alpha3b[k].p, m->type_map.p, Nl, m->virial_op.p,
-                                     m->pos.p, m->box.p, nlocal, st);
+  staf_op_force_set_skip_pbc(ext ? 1 : 0);
+  if (m->dev_mlp) {
+    // ---- everything stays on the device: per species fingerprints -> MLP -> forces; one synchronisation at the end
+    staf::launch_fill_zero<double>(m->force.p, n3, st);
+    staf::launch_fill_zero<double>(m->virial_acc.p, 9, st);
+    int shift = 0;
+    for (int k = 0; k < nt; shift += tipos[k], k++) {
+      const int Nl = tipos[k], Ar = m->Ar[k], Aa = m->Aa[k];
+      if (Nl == 0) continue;
+      const size_t o = (size_t)shift;
+      rc = staf_op_radial_afs_f64(m->raddescr.p + o * nr, nr, m->alpha2b[k].p, Ar, m->af2.p, 1, Nl,
+                                  m->intmap2b.p + o * (nr + 1), m->emb2b[k].p, m->type_map.p, nt, nlocal, st);
+      if (rc == STAF_OK)
+        rc = staf_op_angular_afs_f64(m->des3bsupp.p + o * nr, m->angdescr.p + o * na, nr, na, m->af3.p, 1, Nl,
+                                     m->intmap3b.p + o * 2 * na, m->intmap2b.p + o * (nr + 1), m->alpha3b[k].p, Aa,
+                                     m->emb3b[k].p, m->type_map.p, m->numtriplet.p + o, nt, nlocal, st);
+      if (rc == STAF_OK)
+        rc = staf::dev_mlp_eval(m->dnets[k], m->af2.p, Ar, m->af3.p, Aa, Nl, m->e_atom.p + o, m->g2.p, m->g3.p, st);
       if (rc != STAF_OK) return -20;
-      hipLaunchKernelGGL(add_into_kernel, dim3((n3 + 255) / 256), dim3(256), 0, st, m->force.p, m->force_op.p, n3);
-      STAF_HIP_OK(hipMemcpyAsync(Wk, m->virial_op.p, 9 * sizeof(double), hipMemcpyDeviceToHost, st));
+      for (int body = 2; body <= 3; body++) {
+        if (body == 2)
+          rc = staf_op_force_doublets_f64(m->g2.p, m->raddescr.p + o * nr, m->der2b.p + o * 3 * nr,
+                                          m->intmap2b.p + o * (nr + 1), nr, nall, 1, Ar, m->alpha2b[k].p,
+                                          m->emb2b[k].p, nt, m->tipos.p, m->actual_type.p + k, m->force_op.p,
+                                          m->type_map.p, Nl, m->virial_op.p, m->pos.p, m->box.p, nlocal, st);
+        else
+          rc = staf_op_force_tripl_f64(m->g3.p, m->des3bsupp.p + o * nr, m->angdescr.p + o * na,
+                                       m->der3bsupp.p + o * 3 * nr, m->der3b.p + o * 6 * na,
+                                       m->intmap2b.p + o * (nr + 1), m->intmap3b.p + o * 2 * na, nr, na, nall, 1, Aa,
+                                       m->emb3b[k].p, nt, m->tipos.p, m->actual_type.p + k, m->force_op.p,
+                                       m->numtriplet.p + o, m->alpha3b[k].p, m->type_map.p, Nl, m->virial_op.p,
+                                       m->pos.p, m->box.p, nlocal, st);
+        if (rc != STAF_OK) return -20;
+        hipLaunchKernelGGL(add_into_kernel, dim3((n3 + 255) / 256), dim3(256), 0, st, m->force.p, m->force_op.p, n3);
+        hipLaunchKernelGGL(add_into_kernel, dim3(1), dim3(64), 0, st, m->virial_acc.p, m->virial_op.p, 9);
+      }
+    }
+    m->e_atom_h.resize(nlocal);
+    STAF_HIP_OK(hipMemcpyAsync(m->e_atom_h.data(), m->e_atom.p, L * sizeof(double), hipMemcpyDeviceToHost, st));
+    STAF_HIP_OK(hipMemcpyAsync(W, m->virial_acc.p, 9 * sizeof(double), hipMemcpyDeviceToHost, st));
+    STAF_HIP_OK(hipStreamSynchronize(st));
+    for (int a = 0; a < nlocal; a++) energy += m->e_atom_h[a];   // slot order: fixed
+    energy *= 0.5;
+    if (!isfinite(energy))
+      fprintf(stderr, "staf_compute: non-finite energy=%g nlocal=%d nghost=%d\n", energy, nlocal, nghost);
+  } else {
+    // ---- fingerprints of every species, packed rows [Ar+Aa] for the MLP
+    size_t total = 0;
+    for (int k = 0; k < nt; k++) total += (size_t)tipos[k] * (m->Ar[k] + m->Aa[k]);
+    m->af_h.resize(total);
+    m->gr_h.assign(total, 0.0);
+    size_t off = 0;
+    int shift = 0;
+    for (int k = 0; k < nt; shift += tipos[k], k++) {
+      const int Nl = tipos[k], Ar = m->Ar[k], Aa = m->Aa[k];
+      if (Nl == 0) continue;
+      const size_t o = (size_t)shift;
+      rc = staf_op_radial_afs_f64(m->raddescr.p + o * nr, nr, m->alpha2b[k].p, Ar, m->af2.p, 1, Nl,
+                                  m->intmap2b.p + o * (nr + 1), m->emb2b[k].p, m->type_map.p, nt, nlocal, st);
+      if (rc == STAF_OK)
+        rc = staf_op_angular_afs_f64(m->des3bsupp.p + o * nr, m->angdescr.p + o * na, nr, na, m->af3.p, 1, Nl,
+                                     m->intmap3b.p + o * 2 * na, m->intmap2b.p + o * (nr + 1), m->alpha3b[k].p, Aa,
+                                     m->emb3b[k].p, m->type_map.p, m->numtriplet.p + o, nt, nlocal, st);
+      if (rc != STAF_OK) return -20;
+      m->tmp2.resize((size_t)Nl * Ar);
+      m->tmp3.resize((size_t)Nl * Aa);
+      STAF_HIP_OK(hipMemcpyAsync(m->tmp2.data(), m->af2.p, m->tmp2.size() * sizeof(double), hipMemcpyDeviceToHost, st));
+      STAF_HIP_OK(hipMemcpyAsync(m->tmp3.data(), m->af3.p, m->tmp3.size() * sizeof(double), hipMemcpyDeviceToHost, st));
       STAF_HIP_OK(hipStreamSynchronize(st));
-      for (int c = 0; c < 9; c++) W[c] += Wk[c];
+      for (int a = 0; a < Nl; a++) {
+        double* row = &m->af_h[off + (size_t)a * (Ar + Aa)];
+        memcpy(row, &m->tmp2[(size_t)a * Ar], Ar * sizeof(double));
+        memcpy(row + Ar, &m->tmp3[(size_t)a * Aa], Aa * sizeof(double));
+      }
+      off += (size_t)Nl * (Ar + Aa);
+    }
+
+    // ---- MLP on the host (libstaf/vendor/jmd/nn_nn_mlp.cu:657-768): float32 nets see float32 fingerprints
+    std::vector<int> n_af(nt);
+    for (int k = 0; k < nt; k++) n_af[k] = m->Ar[k] + m->Aa[k];
+    StafMlpEval ev;
+    memset(&ev, 0, sizeof(ev));
+    ev.n_type = nt;
+    ev.n_atoms = tipos.data();
+    ev.n_af = n_af.data();
+    energy = 0.0;
+    if (staf_mlp_precision(m->mlp) == 0) {
+      m->af_f.resize(total);
+      m->gr_f.assign(total, 0.f);
+      for (size_t i = 0; i < total; i++) m->af_f[i] = (float)m->af_h[i];
+      float e_f = 0.f;
+      ev.af_f32 = m->af_f.data();
+      ev.energy_f32 = &e_f;
+      ev.dE_daf_f32 = m->gr_f.data();
+      if (staf_mlp_eval(m->mlp, &ev) != 0) return -20;
+      energy = (double)e_f;
+      for (size_t i = 0; i < total; i++) m->gr_h[i] = (double)m->gr_f[i];
+    } else {
+      ev.af_f64 = m->af_h.data();
+      ev.energy_f64 = &energy;
+      ev.dE_daf_f64 = m->gr_h.data();
+      if (staf_mlp_eval(m->mlp, &ev) != 0) return -20;
+    }
+    if (!isfinite(energy))
+      fprintf(stderr, "staf_compute: non-finite energy=%g nlocal=%d nghost=%d\n", energy, nlocal, nghost);
+
+    // ---- forces: 2-body + 3-body of every centre species, with the virial
+    staf::launch_fill_zero<double>(m->force.p, nall * 3, st);
+    double Wk[9];
+    off = 0;
+    shift = 0;
+    for (int k = 0; k < nt; shift += tipos[k], k++) {
+      const int Nl = tipos[k], Ar = m->Ar[k], Aa = m->Aa[k];
+      if (Nl == 0) continue;
+      const size_t o = (size_t)shift;
+      m->tmp2.resize((size_t)Nl * Ar);
+      m->tmp3.resize((size_t)Nl * Aa);
+      for (int a = 0; a < Nl; a++) {
+        const double* row = &m->gr_h[off + (size_t)a * (Ar + Aa)];
+        memcpy(&m->tmp2[(size_t)a * Ar], row, Ar * sizeof(double));
+        memcpy(&m->tmp3[(size_t)a * Aa], row + Ar, Aa * sizeof(double));
+      }
+      off += (size_t)Nl * (Ar + Aa);
+      STAF_HIP_OK(hipMemcpyAsync(m->g2.p, m->tmp2.data(), m->tmp2.size() * sizeof(double), hipMemcpyHostToDevice, st));
+      STAF_HIP_OK(hipMemcpyAsync(m->g3.p, m->tmp3.data(), m->tmp3.size() * sizeof(double), hipMemcpyHostToDevice, st));
+      STAF_HIP_OK(hipStreamSynchronize(st));
+      for (int body = 2; body <= 3; body++) {
+        if (body == 2)
+          rc = staf_op_force_doublets_f64(m->g2.p, m->raddescr.p + o * nr, m->der2b.p + o * 3 * nr,
+                                          m->intmap2b.p + o * (nr + 1), nr, nall, 1, Ar, m->alpha2b[k].p, m->emb2b[k].p,
+                                          nt, m->tipos.p, m->actual_type.p + k, m->force_op.p, m->type_map.p, Nl,
+                                          m->virial_op.p, m->pos.p, m->box.p, nlocal, st);
+        else
+          rc = staf_op_force_tripl_f64(m->g3.p, m->des3bsupp.p + o * nr, m->angdescr.p + o * na,
+                                       m->der3bsupp.p + o * 3 * nr, m->der3b.p + o * 6 * na,
+                                       m->intmap2b.p + o * (nr + 1), m->intmap3b.p + o * 2 * na, nr, na, nall, 1, Aa,
+                                       m->emb3b[k].p, nt, m->tipos.p, m->actual_type.p + k, m->force_op.p,
+                                       m->numtriplet.p + o, m->alpha3b[k].p, m->type_map.p, Nl, m->virial_op.p,
+                                       m->pos.p, m->box.p, nlocal, st);
+        if (rc != STAF_OK) return -20;
+        hipLaunchKernelGGL(add_into_kernel, dim3((n3 + 255) / 256), dim3(256), 0, st, m->force.p, m->force_op.p, n3);
+        STAF_HIP_OK(hipMemcpyAsync(Wk, m->virial_op.p, 9 * sizeof(double), hipMemcpyDeviceToHost, st));
+        STAF_HIP_OK(hipStreamSynchronize(st));
+        for (int c = 0; c < 9; c++) W[c] += Wk[c];
+      }
     }
   }
   m->force_h.resize((size_t)n3);

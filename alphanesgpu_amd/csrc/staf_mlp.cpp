@@ -198,4 +198,30 @@ int staf_mlp_n_af(const StafMlp* mlp, int type) {
 
 int staf_mlp_precision(const StafMlp* mlp) { return mlp ? mlp->precision : -1; }
 
+// ---- library-internal access to the loaded weights (staf_mlp_internal.h): the device-resident evaluation of the
+// MD entry uploads them once at load time.
+int staf_mlp_internal_nlayers(const StafMlp* mlp, int type) {
+  if (!mlp || type < 0 || type >= staf_mlp_ntypes(mlp)) return -1;
+  return (int)(mlp->precision ? mlp->nets_d[type].layers.size() : mlp->nets_f[type].layers.size());
+}
+
+const void* staf_mlp_internal_mu(const StafMlp* mlp, int type) {
+  if (staf_mlp_internal_nlayers(mlp, type) < 0) return NULL;
+  return mlp->precision ? (const void*)mlp->nets_d[type].mu.data() : (const void*)mlp->nets_f[type].mu.data();
+}
+
+int staf_mlp_internal_layer(const StafMlp* mlp, int type, int layer, int* act, int* in_f, int* out_f, const void** W,
+                            const void** b) {
+  const int nl = staf_mlp_internal_nlayers(mlp, type);
+  if (nl < 0 || layer < 0 || layer >= nl) return -1;
+  if (mlp->precision) {
+    const auto& L = mlp->nets_d[type].layers[layer];
+    *act = L.act; *in_f = L.in_f; *out_f = L.out_f; *W = L.W.data(); *b = L.b.data();
+  } else {
+    const auto& L = mlp->nets_f[type].layers[layer];
+    *act = L.act; *in_f = L.in_f; *out_f = L.out_f; *W = L.W.data(); *b = L.b.data();
+  }
+  return 0;
+}
+
 }  // extern "C"

@@ -224,6 +224,27 @@ def test_compute_with_injected_list_and_ghosts_matches_own_list():
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("prec,tol", [("double", 1e-11), ("float", 2e-5)])
+def test_device_mlp_matches_host_mlp(prec, tol):
+    """The MLP evaluated on the GPU between the kernels (default) against the host evaluation of the same weights
+    (reserved bit 1): energy, forces, virial.  float64 nets: 1e-11; float32 nets: the two evaluations sum in
+    different orders, 2e-5 of the largest force."""
+    from alphanesgpu_amd import libstaf
+    pos, box, types = load_water_smoke(np.float64)
+    pos = pos.reshape(-1, 3)
+    p = 1 if prec == "double" else 0
+    dev = libstaf.StafModel(os.path.join(GOLDEN, f"model_{prec}"), precision=p, full_virial=True)
+    host = libstaf.StafModel(os.path.join(GOLDEN, f"model_{prec}"), precision=p, full_virial=True, host_mlp=True)
+    e0, f0, v0 = host.compute(pos, box[0], types)
+    e1, f1, v1 = dev.compute(pos, box[0], types)
+    assert abs(e1 - e0) <= max(tol, 1e-6 if p == 0 else 0) * abs(e0)
+    assert nerr(f1, f0) <= tol
+    assert nerr(v1, v0) <= tol
+    dev.close()
+    host.close()
+
+
+@pytest.mark.gpu
 def test_compute_return_codes():
     """Validation order and codes of libstaf/src/staf_api.cpp:196-337."""
     from alphanesgpu_amd import libstaf
