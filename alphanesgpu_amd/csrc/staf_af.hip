@@ -168,7 +168,7 @@ static int alpha_dist_grad(const real* D, int nr, const real* alpha2b, int Ar, r
   hipStream_t stream = (hipStream_t)stream_;
   const int nout = 2 * nt * Ar;
   const int nb = grad_blocks(nf * Nl);
-  real* partial = (real*)scratch_reserve(st, ((size_t)nb + RED_SLICES) * nout * sizeof(real));
+  real* partial = (real*)scratch_reserve(st, stream, ((size_t)nb + RED_SLICES) * nout * sizeof(real));
   real* red_tmp = partial ? partial + (size_t)nb * nout : nullptr;
   if (!partial) return STAF_E_HIP;
   size_t lds = (size_t)(2 * nt * Ar + AF_WAVES * nout + AF_WAVES * nr) * sizeof(real) + (size_t)AF_WAVES * nr * sizeof(int);
@@ -222,7 +222,7 @@ static int alphagrad_ang(const real* Dsup, const real* Tang, int nr, int na, con
   const int nsig = 2 * nt - 1;
   const int nout = nsig * Aa * 3;
   const int nb = nf * Nl < TRI_GRID_MAX ? nf * Nl : TRI_GRID_MAX;
-  real* partial = (real*)scratch_reserve(st, ((size_t)nb + RED_SLICES) * nout * sizeof(real));
+  real* partial = (real*)scratch_reserve(st, stream, ((size_t)nb + RED_SLICES) * nout * sizeof(real));
   real* red_tmp = partial ? partial + (size_t)nb * nout : nullptr;
   if (!partial) return STAF_E_HIP;
   size_t lds = TriLds<real, 1>::bytes(nr, Aa, nt);

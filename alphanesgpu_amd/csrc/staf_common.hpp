@@ -8,6 +8,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <unordered_map>
+
 #include "../../include/staf_ops.h"
 
 namespace staf {
@@ -173,18 +175,24 @@ struct Workspace {
   size_t bytes = 0;
 };
 
-struct DeviceState {
-  int device = -1;
-  int* status_d = nullptr;   // device word, error bits OR-ed in by kernels
-  int* status_h = nullptr;   // pinned host mirror
+// Work areas are kept per stream: ops issued on different streams of one device (e.g. the per-species op chains,
+// which do not depend on each other) never share scratch, so they may run concurrently.
+struct StreamWork {
   Workspace scratch;         // per-slot partial forces / partial sums
   Workspace buckets;         // transpose buckets (counters + entries), kept zeroed between calls
   size_t bucket_counters = 0;    // capacity, in ints, of the counter part
   size_t bucket_entries = 0;     // capacity, in ints, of the entry part
 };
 
+struct DeviceState {
+  int device = -1;
+  int* status_d = nullptr;   // device word, error bits OR-ed in by kernels
+  int* status_h = nullptr;   // pinned host mirror
+  std::unordered_map<hipStream_t, StreamWork> work;
+};
+
 DeviceState* device_state();                                   // for the current device, created on demand
-void* scratch_reserve(DeviceState* st, size_t bytes);          // grows, never shrinks
+void* scratch_reserve(DeviceState* st, hipStream_t stream, size_t bytes);   // grows, never shrinks
 int* bucket_reserve(DeviceState* st, size_t n_counters, size_t n_entries, hipStream_t stream, int** entries);
 int finish_op(DeviceState* st, hipStream_t stream);            // launch check (+ optional sync & status fetch)
 bool sync_errors_enabled();

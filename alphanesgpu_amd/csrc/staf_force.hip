@@ -350,7 +350,7 @@ struct ForceScratch {
 template <typename real>
 static int force_scratch(DeviceState* st, int nf, int N, int Nl, int nr, hipStream_t stream, ForceScratch* fs) {
   const size_t ng = (size_t)nf * Nl * nr * 3, ns = (size_t)nf * Nl * 3, nv = (size_t)nf * Nl * 9;
-  real* base = (real*)scratch_reserve(st, (ng + ns + nv) * sizeof(real));
+  real* base = (real*)scratch_reserve(st, stream, (ng + ns + nv) * sizeof(real));
   if (!base) return STAF_E_HIP;
   fs->gslot = base;
   fs->self = base + ng;
@@ -473,7 +473,7 @@ static int gradforce_2b(const real* Q, const real* D, int nr, const real* alpha2
   hipStream_t stream = (hipStream_t)stream_;
   const int nout = 2 * nt * Ar;
   const int nb = grad_blocks_f(nf * Nl);
-  real* partial = (real*)scratch_reserve(st, ((size_t)nb + RED_SLICES) * nout * sizeof(real));
+  real* partial = (real*)scratch_reserve(st, stream, ((size_t)nb + RED_SLICES) * nout * sizeof(real));
   real* red_tmp = partial ? partial + (size_t)nb * nout : nullptr;
   if (!partial) return STAF_E_HIP;
   size_t lds = (size_t)(2 * nt * Ar + F_WAVES * nout + 2 * F_WAVES * nr) * sizeof(real) +
@@ -510,7 +510,7 @@ static int gradforce_tripl(const real* Q, const real* G, const real* Dsup, const
   const int nsig = 2 * nt - 1;
   const int nout = nsig * Aa * 3;
   const int nb = nf * Nl < TRI_GRID_MAX ? nf * Nl : TRI_GRID_MAX;
-  real* partial = (real*)scratch_reserve(st, ((size_t)nb + RED_SLICES) * nout * sizeof(real));
+  real* partial = (real*)scratch_reserve(st, stream, ((size_t)nb + RED_SLICES) * nout * sizeof(real));
   real* red_tmp = partial ? partial + (size_t)nb * nout : nullptr;
   if (!partial) return STAF_E_HIP;
   size_t lds = TriLds<real, 2>::bytes(nr, Aa, nt);

@@ -42,41 +42,47 @@ DeviceState* device_state() {
   return raw;
 }
 
-void* scratch_reserve(DeviceState* st, size_t bytes) {
-  if (bytes <= st->scratch.bytes) return st->scratch.buf;
-  if (st->scratch.buf) {
+static StreamWork* stream_work(DeviceState* st, hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  return &st->work[stream];   // references into an unordered_map stay valid when it grows
+}
+
+void* scratch_reserve(DeviceState* st, hipStream_t stream, size_t bytes) {
+  StreamWork* w = stream_work(st, stream);
+  if (bytes <= w->scratch.bytes) return w->scratch.buf;
+  if (w->scratch.buf) {
     // hipFree waits for in-flight work that may still read the old block
-    if (hipFree(st->scratch.buf) != hipSuccess) return nullptr;
-    st->scratch.buf = nullptr;
-    st->scratch.bytes = 0;
+    if (hipFree(w->scratch.buf) != hipSuccess) return nullptr;
+    w->scratch.buf = nullptr;
+    w->scratch.bytes = 0;
   }
   size_t want = bytes + bytes / 4;
-  if (hipMalloc(&st->scratch.buf, want) != hipSuccess) return nullptr;
-  st->scratch.bytes = want;
-  return st->scratch.buf;
+  if (hipMalloc(&w->scratch.buf, want) != hipSuccess) return nullptr;
+  w->scratch.bytes = want;
+  return w->scratch.buf;
 }
 
 // Scatter buckets: n_counters ints (kept all-zero between calls: the gather
 // kernel clears every counter it consumes) followed by n_entries ints.
 int* bucket_reserve(DeviceState* st, size_t n_counters, size_t n_entries, hipStream_t stream, int** entries) {
-  if (n_counters > st->bucket_counters || n_entries > st->bucket_entries) {
-    if (st->buckets.buf) {
-      if (hipFree(st->buckets.buf) != hipSuccess) return nullptr;
-      st->buckets.buf = nullptr;
-      st->buckets.bytes = 0;
+  StreamWork* w = stream_work(st, stream);
+  if (n_counters > w->bucket_counters || n_entries > w->bucket_entries) {
+    if (w->buckets.buf) {
+      if (hipFree(w->buckets.buf) != hipSuccess) return nullptr;
+      w->buckets.buf = nullptr;
+      w->buckets.bytes = 0;
     }
     size_t cnt = n_counters + n_counters / 4;
     size_t ent = n_entries + n_entries / 4;
     size_t want = (cnt + ent) * sizeof(int);
-    if (hipMalloc(&st->buckets.buf, want) != hipSuccess) return nullptr;
-    if (hipMemset(st->buckets.buf, 0, cnt * sizeof(int)) != hipSuccess) return nullptr;
-    st->buckets.bytes = want;
-    st->bucket_counters = cnt;
-    st->bucket_entries = ent;
+    if (hipMalloc(&w->buckets.buf, want) != hipSuccess) return nullptr;
+    if (hipMemset(w->buckets.buf, 0, cnt * sizeof(int)) != hipSuccess) return nullptr;
+    w->buckets.bytes = want;
+    w->bucket_counters = cnt;
+    w->bucket_entries = ent;
   }
-  (void)stream;
-  *entries = (int*)st->buckets.buf + st->bucket_counters;
-  return (int*)st->buckets.buf;
+  *entries = (int*)w->buckets.buf + w->bucket_counters;
+  return (int*)w->buckets.buf;
 }
 
 static int decode_status(int bits) {
@@ -145,8 +151,10 @@ void staf_ops_release(void) {
   if (it == staf::g_state.end()) return;
   staf::DeviceState* st = it->second.get();
   (void)hipDeviceSynchronize();
-  if (st->scratch.buf) (void)hipFree(st->scratch.buf);
-  if (st->buckets.buf) (void)hipFree(st->buckets.buf);
+  for (auto& kv : st->work) {
+    if (kv.second.scratch.buf) (void)hipFree(kv.second.scratch.buf);
+    if (kv.second.buckets.buf) (void)hipFree(kv.second.buckets.buf);
+  }
   if (st->status_d) (void)hipFree(st->status_d);
   if (st->status_h) (void)hipHostFree(st->status_h);
   staf::g_state.erase(it);

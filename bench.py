@@ -114,6 +114,11 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
                     help="also run a plain device copy of this size three times (reference point for HBM counters)")
+    ap.add_argument("--streams", type=int, default=2, choices=[1, 2],
+                    help="2: the per-species op chains (independent until the forces are summed) are issued on one "
+                         "HIP stream per species; 1: everything on one stream")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="launch every op of every step from Python instead of replaying one captured HIP graph")
     ap.add_argument("--contiguous-splits", action="store_true",
                     help="copy per-species tensors like tf.split instead of passing views")
     args = ap.parse_args()
@@ -183,32 +188,52 @@ def main():
         timers.setdefault(name, []).append((a, b))
         return r
 
-    def step(record=False):
-        rad, ang, sup, im2, im3, d2, d3, d3s, ntr = timed(
-            "descriptor", lambda: ops.compute_descriptors_light(pos, box, out=dbuf), record)
-        Ftot = None
-        for k, s in enumerate(slices):
-            p = P[k]
-            v = [sl(x, s) for x in (rad, ang, sup, im2, im3, d2, d3, d3s, ntr)]
-            radk, angk, supk, im2k, im3k, d2k, d3k, d3sk, ntrk = v
-            timed("af2", lambda: ops.compute_sort_proj(radk, im2k, p["alpha2b"], p["emb2b"], tm), record)
-            timed("af3", lambda: ops.compute_sort_proj3body(angk, supk, im3k, im2k, p["alpha3b"], p["emb3b"], tm, ntrk,
-                                                            nt=nt), record)
-            f2 = timed("force2", lambda: ops.compute_force_radial(G2[k], d2k, im2k, radk, p["alpha2b"], p["emb2b"], tm,
-                                                                  tp, at[k]), record)
-            f3 = timed("force3", lambda: ops.compute_force_tripl(G3[k], supk, angk, d3sk, d3k, im2k, im3k, p["alpha3b"],
-                                                                 p["emb3b"], tm, tp, at[k], ntrk), record)
-            if mode == "full_step":
-                timed("grad2", lambda: ops.compute_two_body_par_grad(P2[k], radk, im2k, p["alpha2b"], p["emb2b"], tm),
-                      record)
-                timed("grad3", lambda: ops.compute_sort_proj3body_grad(P3[k], angk, supk, im3k, im2k, p["alpha3b"],
-                                                                       p["emb3b"], tm, ntrk, nt=nt), record)
-                timed("gradforce2", lambda: ops.compute_force_radial_grad(Q, G2[k], d2k, im2k, radk, p["alpha2b"],
-                                                                          p["emb2b"], tm, tp, at[k]), record)
-                timed("gradforce3", lambda: ops.compute_force_tripl_grad(Q, G3[k], supk, angk, d3sk, d3k, im2k, im3k,
-                                                                         p["alpha3b"], p["emb3b"], tm, tp, at[k],
-                                                                         ntrk), record)
-            Ftot = f2 + f3 if Ftot is None else Ftot + f2 + f3
+    side = [torch.cuda.Stream() for _ in range(nt)] if args.streams > 1 else None
+
+    def species_chain(k, s, d, record):
+        rad, ang, sup, im2, im3, d2, d3, d3s, ntr = d
+        p = P[k]
+        v = [sl(x, s) for x in (rad, ang, sup, im2, im3, d2, d3, d3s, ntr)]
+        radk, angk, supk, im2k, im3k, d2k, d3k, d3sk, ntrk = v
+        timed("af2", lambda: ops.compute_sort_proj(radk, im2k, p["alpha2b"], p["emb2b"], tm), record)
+        timed("af3", lambda: ops.compute_sort_proj3body(angk, supk, im3k, im2k, p["alpha3b"], p["emb3b"], tm, ntrk,
+                                                        nt=nt), record)
+        f2 = timed("force2", lambda: ops.compute_force_radial(G2[k], d2k, im2k, radk, p["alpha2b"], p["emb2b"], tm,
+                                                              tp, at[k]), record)
+        f3 = timed("force3", lambda: ops.compute_force_tripl(G3[k], supk, angk, d3sk, d3k, im2k, im3k, p["alpha3b"],
+                                                             p["emb3b"], tm, tp, at[k], ntrk), record)
+        if mode == "full_step":
+            timed("grad2", lambda: ops.compute_two_body_par_grad(P2[k], radk, im2k, p["alpha2b"], p["emb2b"], tm),
+                  record)
+            timed("grad3", lambda: ops.compute_sort_proj3body_grad(P3[k], angk, supk, im3k, im2k, p["alpha3b"],
+                                                                   p["emb3b"], tm, ntrk, nt=nt), record)
+            timed("gradforce2", lambda: ops.compute_force_radial_grad(Q, G2[k], d2k, im2k, radk, p["alpha2b"],
+                                                                      p["emb2b"], tm, tp, at[k]), record)
+            timed("gradforce3", lambda: ops.compute_force_tripl_grad(Q, G3[k], supk, angk, d3sk, d3k, im2k, im3k,
+                                                                     p["alpha3b"], p["emb3b"], tm, tp, at[k],
+                                                                     ntrk), record)
+        return f2 + f3
+
+    def step(record=False, streams=side):
+        d = timed("descriptor", lambda: ops.compute_descriptors_light(pos, box, out=dbuf), record)
+        if streams is None:
+            parts = [species_chain(k, s, d, record) for k, s in enumerate(slices)]
+        else:
+            main_stream = torch.cuda.current_stream()   # the capture stream while a graph is recorded
+            ready = main_stream.record_event()
+            parts, done = [], []
+            for k, s in enumerate(slices):
+                with torch.cuda.stream(streams[k]):
+                    streams[k].wait_event(ready)
+                    f = species_chain(k, s, d, record)
+                    f.record_stream(main_stream)
+                    parts.append(f)
+                    done.append(streams[k].record_event())
+            for ev in done:
+                main_stream.wait_event(ev)
+        Ftot = parts[0]
+        for f in parts[1:]:
+            Ftot = Ftot + f
         return Ftot
 
     if args.calibrate_copy:
@@ -219,21 +244,54 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    for _ in range(args.warmup):
+    # One step = one replay of a HIP graph that holds the whole op sequence (the ops run on the stream they are
+    # called on, so stream capture records their kernels; scratch is grown by the eager warm-up steps first).
+    graph = None
+    run = step
+    for _ in range(2):
         step()
+    ops.poll_status()
+    if not args.no_graph:
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            graph_out = step()
+        run = graph.replay
+    for _ in range(args.warmup):
+        run()
     ops.poll_status()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        step()
+        run()
     torch.cuda.synchronize()
     el = time.perf_counter() - t0
     ops.poll_status()
+    if graph is not None:
+        # the replayed graph must reproduce the eager step bit for bit (all reductions have a fixed order)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = graph_out.clone()
+        want = step(streams=None)
+        torch.cuda.synchronize()
+        if not torch.equal(got, want):
+            print("bench.py: HIP graph replay differs from the eager step", file=sys.stderr)
+            sys.exit(1)
 
-    # per-op GPU time with events on the launch stream (separate pass: events perturb the pipeline slightly)
+    # the same step with everything on one stream (reported beside the main figure)
     nprof = max(3, min(args.steps, 20))
+    el1 = el
+    if side is not None:
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(nprof):
+            step(streams=None)
+        torch.cuda.synchronize()
+        el1 = (time.perf_counter() - t1) * args.steps / nprof
+
+    # per-op GPU time with events on the launch stream, one stream (separate pass: events perturb the pipeline)
     for _ in range(nprof):
-        step(record=True)
+        step(record=True, streams=None)
     torch.cuda.synchronize()
     op_ms = {k: float(np.mean([a.elapsed_time(b) for a, b in v])) for k, v in timers.items()}
     calls = {k: len(v) // nprof for k, v in timers.items()}
@@ -241,7 +299,7 @@ def main():
     # per-kernel GPU time from the library's own HIP events, recorded on the stream each kernel is launched on
     ops.kernel_timing(True)
     for _ in range(nprof):
-        step()
+        step(streams=None)
     ops.kernel_timing(False)
     s = np.dtype(dtype).itemsize
     ab = algorithmic_bytes(N, tipos, nr, na, Ar, Aa, nt, s)
@@ -271,7 +329,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": args.workload, "mode": mode, "atoms": N, "frames_per_step": nf, "Rc": synth.RC,
                    "radial_buffer": nr, "angular_buffer": na, "Ar": Ar, "Aa": Aa,
-                   "species_tensors": "contiguous copies" if args.contiguous_splits else "views"},
+                   "species_tensors": "contiguous copies" if args.contiguous_splits else "views",
+                   "species_streams": args.streams, "launch": "python per op" if graph is None else "hip graph replay"},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": TRAFFIC.get((dom, args.workload)),
                      "algorithmic_bytes_per_launch": dom_bytes_per_launch,
@@ -283,6 +342,7 @@ def main():
         "whole_step_hbm_frac": step_bytes * nf / (el / args.steps) / 1e9 / HBM_PEAK_GBS,
         "op_ms_per_step": per_step,
         "ms_per_frame": el / args.steps * 1e3 / nf,
+        "single_stream": {"value": nf * args.steps / el1, "ms_per_step": el1 / args.steps * 1e3},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(batch, params, up, mode, nr, na)

@@ -270,3 +270,89 @@ def test_virial_forms(oracle, dtype):
             e = nerr(x.cpu().numpy(), y)
             assert e <= tol + slack, (name, k, e)
         assert torch.all(g3[2] == 0)
+
+
+@pytest.mark.gpu
+def test_hip_graph_replay_with_two_streams_matches_eager():
+    """The whole op sequence captured once in a HIP graph, the two per-species chains forked onto their own streams
+    (per-stream scratch inside the library): every replay, with eager calls and synchronisations in between, gives
+    the eager result bit for bit."""
+    import torch
+    from alphanesgpu_amd import ops, synth
+    import pipeline
+    dev = torch.device("cuda:0")
+    batch = synth.water_batch("water96")
+    dt = batch["dtype"]
+    tdt = torch.float64
+    nr, na = synth.NR, synth.NA
+    nf, N = batch["nf"], batch["N"]
+    tipos = [int(x) for x in batch["tipos"]]
+    nt = len(tipos)
+    params = synth.fingerprint_params(dtype=dt)
+    up = pipeline.synthetic_upstream(nf, batch["tipos"], params, 3, dt)
+    T = lambda a: torch.as_tensor(np.ascontiguousarray(a)).to(dev)
+    pos, box, tm, tp = T(batch["pos"]), T(batch["box"]), T(batch["type_map"]), T(batch["tipos"])
+    P = [{k: T(v) for k, v in m.items()} for m in params]
+    G2, G3 = [T(x) for x in up["G2"]], [T(x) for x in up["G3"]]
+    Q = T(up["Q"])
+    at = [torch.tensor([k], dtype=torch.int32, device=dev) for k in range(nt)]
+    ops.construct_descriptors_light(synth.RC, nr, na, N, box, synth.RS, synth.RA, nf, dtype=tdt)
+    ops.set_sync_errors(False)
+    side = [torch.cuda.Stream() for _ in range(nt)]
+    sl, o = [], 0
+    for n in tipos:
+        sl.append(slice(o, o + n))
+        o += n
+
+    def chain(k, d):
+        rad, ang, sup, im2, im3, d2, d3, d3s, ntr = [x[:, sl[k]] for x in d]
+        p = P[k]
+        a3 = ops.compute_sort_proj3body(ang, sup, im3, im2, p["alpha3b"], p["emb3b"], tm, ntr, nt=nt)
+        f2 = ops.compute_force_radial(G2[k], d2, im2, rad, p["alpha2b"], p["emb2b"], tm, tp, at[k])
+        f3 = ops.compute_force_tripl(G3[k], sup, ang, d3s, d3, im2, im3, p["alpha3b"], p["emb3b"], tm, tp, at[k], ntr)
+        ga = ops.compute_force_tripl_grad(Q, G3[k], sup, ang, d3s, d3, im2, im3, p["alpha3b"], p["emb3b"], tm, tp,
+                                          at[k], ntr)
+        return [a3, f2 + f3, ga[0], ga[1]]
+
+    def step(streams):
+        d = ops.compute_descriptors_light(pos, box)
+        if streams is None:
+            return [chain(k, d) for k in range(nt)]
+        main = torch.cuda.current_stream()
+        ready = main.record_event()
+        outs, done = [], []
+        for k in range(nt):
+            with torch.cuda.stream(streams[k]):
+                streams[k].wait_event(ready)
+                r = chain(k, d)
+                for t in r:
+                    t.record_stream(main)
+                outs.append(r)
+                done.append(streams[k].record_event())
+        for ev in done:
+            main.wait_event(ev)
+        return outs
+
+    try:
+        want = step(None)
+        step(side)                      # grows the per-stream scratch before the capture
+        ops.poll_status()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            held = step(side)
+        for rep in range(3):
+            g.replay()
+            torch.cuda.synchronize()
+            for a, b in zip(held, want):
+                for x, y in zip(a, b):
+                    assert torch.equal(x, y), f"replay {rep}"
+            again = step(None)          # eager work between the replays, on the default stream
+            ops.poll_status()
+            torch.cuda.synchronize()
+            for a, b in zip(again, want):
+                for x, y in zip(a, b):
+                    assert torch.equal(x, y)
+    finally:
+        ops.set_sync_errors(True)
+
