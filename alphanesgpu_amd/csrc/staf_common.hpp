@@ -30,6 +30,8 @@ __device__ inline float r_cos(float x) { return cosf(x); }
 __device__ inline double r_cos(double x) { return cos(x); }
 __device__ inline float r_sin(float x) { return sinf(x); }
 __device__ inline double r_sin(double x) { return sin(x); }
+__device__ inline void r_sincos(float x, float* s, float* c) { sincosf(x, s, c); }
+__device__ inline void r_sincos(double x, double* s, double* c) { sincos(x, s, c); }
 __device__ inline float r_sqrt(float x) { return sqrtf(x); }
 __device__ inline double r_sqrt(double x) { return sqrt(x); }
 __device__ inline float r_pow(float x, float n) { return powf(x, n); }

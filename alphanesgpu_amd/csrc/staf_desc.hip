@@ -101,12 +101,12 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
   // LDS carve-up
   real* c_d2 = (real*)smem;            // [nr] candidate dist2
   real* c_d = c_d2 + nr;               // [3*nr] candidate delta (neighbour - centre)
-  real* s_u = c_d + 3 * nr;            // [3*nr] unit vector centre - neighbour, sorted
-  real* s_g = s_u + 3 * nr;            // [3*nr] grad of fc wrt d, sorted
-  real* s_invr = s_g + 3 * nr;         // [nr]
-  real* s_fc = s_invr + nr;            // [nr]
-  int* c_j = (int*)(s_fc + nr);        // [nr] candidate index
+  // [nr][8] per sorted neighbour: unit vector centre - neighbour (3), 1/r, grad of fc wrt d (3), fc -- one record,
+  // so the angular fill reads a neighbour with two (fp32) or four (fp64) 16-byte LDS reads
+  real* s_rec = c_d + 3 * nr;
+  int* c_j = (int*)(s_rec + 8 * nr);   // [nr] candidate index
   int* s_j = c_j + nr;                 // [nr] sorted neighbour index
+  int* s_rank = s_j + nr;              // [nr] rank of every candidate
   __shared__ int cnt_all, cnt_ang;
   __shared__ real sbox[6];
 
@@ -114,6 +114,7 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
   const int b = blockIdx.x / N;
   const int i = blockIdx.x - b * N;
   if (tid == 0) { cnt_all = 0; cnt_ang = 0; }
+  for (int e = tid; e < nr; e += blockDim.x) s_rank[e] = 0;
   if (tid < 6) sbox[tid] = A.box[b * 6 + tid];
   __syncthreads();
 
@@ -129,18 +130,31 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
   // 1. candidate scan -- or the caller's list (already cut off and sorted by distance)
   const bool injected = A.inj_howmany != nullptr;
   if (!injected) {
-    for (int j = tid; j < A.Npos; j += blockDim.x) {
-      real sj[3], d[3];
-      to_frac(inv, pf[3 * j], pf[3 * j + 1], pf[3 * j + 2], sj);
-      real d2 = mic_delta(box, sj, si, A.dist2_fma, A.skip_pbc, d);
-      if (d2 < rc2 && j != i) {
-        int slot = atomicAdd(&cnt_all, 1);
-        if (slot < nr) {
-          c_j[slot] = j;
-          c_d2[slot] = d2;
-          c_d[3 * slot] = d[0];
-          c_d[3 * slot + 1] = d[1];
-          c_d[3 * slot + 2] = d[2];
+    // the position reads of four candidates per thread are issued together
+    for (int j0 = tid; j0 < A.Npos; j0 += 4 * 256) {
+      real px[4], py[4], pz[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int j = j0 + u * 256;
+        px[u] = py[u] = pz[u] = 0;
+        if (j < A.Npos) { px[u] = pf[3 * j]; py[u] = pf[3 * j + 1]; pz[u] = pf[3 * j + 2]; }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int j = j0 + u * 256;
+        if (j >= A.Npos) break;
+        real sj[3], d[3];
+        to_frac(inv, px[u], py[u], pz[u], sj);
+        real d2 = mic_delta(box, sj, si, A.dist2_fma, A.skip_pbc, d);
+        if (d2 < rc2 && j != i) {
+          int slot = atomicAdd(&cnt_all, 1);
+          if (slot < nr) {
+            c_j[slot] = j;
+            c_d2[slot] = d2;
+            c_d[3 * slot] = d[0];
+            c_d[3 * slot + 1] = d[1];
+            c_d[3 * slot + 2] = d[2];
+          }
         }
       }
     }
@@ -170,54 +184,75 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
   int* im = A.intmap2b + atom * (nr + 1);
   const real PI = pi_ref<real>();
 
-  // 2+3. rank sort and radial fill
-  for (int e = tid; e < nr; e += blockDim.x) {
-    if (e < n) {
-      const real d2 = c_d2[e];
-      const int j = c_j[e];
-      int rank = 0;
-      if (injected) {
-        rank = e;   // the caller's order is kept
-      } else {
-        for (int o = 0; o < n; o++) {
+  // 2. rank of every candidate in (dist2, index) order: the four waves each count a quarter of the others
+  if (!injected) {
+    const int e = tid & (WAVE - 1), part = tid / WAVE;
+    for (int e0 = 0; e0 < n; e0 += WAVE) {
+      const int ee = e0 + e;
+      if (ee < n) {
+        const real d2 = c_d2[ee];
+        const int j = c_j[ee];
+        int rank = 0;
+        for (int o = part; o < n; o += 4) {
           const real od2 = c_d2[o];
           const int oj = c_j[o];
           rank += (od2 < d2 || (od2 == d2 && oj < j)) ? 1 : 0;
         }
+        if (rank) atomicAdd(&s_rank[ee], rank);
       }
+    }
+    __syncthreads();
+  }
+  // 3. radial fill
+  const bool same_cut = A.Ra == A.Rc;
+  const bool std_pow = A.pa == real(1) && A.pb == real(-30);   // the exponents fill_repulsion uses
+  for (int e = tid; e < nr; e += blockDim.x) {
+    if (e < n) {
+      const int j = c_j[e];
+      const int rank = injected ? e : s_rank[e];   // the caller's order is kept
       // centre - neighbour: exact negation of the scan's neighbour - centre
       real d[3] = {-c_d[3 * e], -c_d[3 * e + 1], -c_d[3 * e + 2]};
       const real r = norm_plain(d);
       const real invr = real(1) / r;
+      real sc, cc;
+      r_sincos(PI * r / A.Rc, &sc, &cc);
       real fc = 0, dfc = 0;
       if (r < A.Ra) {
         atomicAdd(&cnt_ang, 1);
-        const real x = PI * r / A.Ra;
-        fc = real(0.5) * (r_cos(x) + real(1));
-        dfc = -real(0.5) * r_sin(x) * PI / A.Ra;
+        real sa = sc, ca = cc;
+        if (!same_cut) r_sincos(PI * r / A.Ra, &sa, &ca);
+        fc = real(0.5) * (ca + real(1));
+        dfc = -real(0.5) * sa * PI / A.Ra;
       }
       real D, dD;
       if (r < A.Rs) {
-        D = A.cA / r_pow(r, A.pa) + A.cB / r_pow(r, A.pb) + A.cC;
-        dD = -A.pa * A.cA / r_pow(r, A.pa + real(1)) - A.pb * A.cB / r_pow(r, A.pb + real(1));
+        if (std_pow) {
+          // A/r + B r^30 + C and its derivative, r^30 by squarings
+          const real r2 = r * r, r4 = r2 * r2, r8 = r4 * r4, r16 = r8 * r8;
+          const real r28 = r16 * r8 * r4, r29 = r28 * r;
+          D = A.cA * invr + A.cB * (r29 * r) + A.cC;
+          dD = -A.cA * invr * invr + real(30) * A.cB * r29;
+        } else {
+          D = A.cA / r_pow(r, A.pa) + A.cB / r_pow(r, A.pb) + A.cC;
+          dD = -A.pa * A.cA / r_pow(r, A.pa + real(1)) - A.pb * A.cB / r_pow(r, A.pb + real(1));
+        }
       } else {
-        const real x = PI * r / A.Rc;
-        D = real(0.5) * (r_cos(x) + real(1));
-        dD = -real(0.5) * r_sin(x) * PI / A.Rc;
+        D = real(0.5) * (cc + real(1));
+        dD = -real(0.5) * sc * PI / A.Rc;
       }
       A.raddescr[row + rank] = D;
       A.des3bsupp[row + rank] = fc;
       im[1 + rank] = j;
       s_j[rank] = j;
-      s_invr[rank] = invr;
-      s_fc[rank] = fc;
+      s_rec[8 * rank + 3] = invr;
+      s_rec[8 * rank + 7] = fc;
 #pragma unroll
       for (int c = 0; c < 3; c++) {
         const real u = d[c] * invr;
         A.der2b[row3 + c * nr + rank] = dD * u;
         A.der3bsupp[row3 + c * nr + rank] = dfc * u;
-        s_u[3 * rank + c] = u;
-        s_g[3 * rank + c] = dfc * u;
+        s_rec[8 * rank + c] = u;
+        s_rec[8 * rank + 4 + c] = dfc * u;
       }
     } else {
       A.raddescr[row + e] = 0;
@@ -247,25 +282,28 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
     if (nn < ntr) {
       int j, k;
       tri_decode(nn, m, j, k);
-      const real uj0 = s_u[3 * j], uj1 = s_u[3 * j + 1], uj2 = s_u[3 * j + 2];
-      const real uk0 = s_u[3 * k], uk1 = s_u[3 * k + 1], uk2 = s_u[3 * k + 2];
+      real rj[8], rk[8];
+#pragma unroll
+      for (int c = 0; c < 8; c++) { rj[c] = s_rec[8 * j + c]; rk[c] = s_rec[8 * k + c]; }
+      const real uj0 = rj[0], uj1 = rj[1], uj2 = rj[2];
+      const real uk0 = rk[0], uk1 = rk[1], uk2 = rk[2];
       const real cs = uj0 * uk0 + uj1 * uk1 + uj2 * uk2;
-      const real fj = s_fc[j], fk = s_fc[k];
+      const real fj = rj[7], fk = rk[7];
       const real half = real(0.5) * (cs + real(1));
       const real ff = fj * fk;
-      const real aj = real(0.5) * s_invr[j] * ff, ak = real(0.5) * s_invr[k] * ff;
+      const real aj = real(0.5) * rj[3] * ff, ak = real(0.5) * rk[3] * ff;
       const real hk = half * fk, hj = half * fj;
       ang[nn] = half * ff;
       im3[nn] = make_int2(s_j[j], s_j[k]);
       real2 o;
-      o.x = aj * (uk0 - cs * uj0) + hk * s_g[3 * j];
-      o.y = ak * (uj0 - cs * uk0) + hj * s_g[3 * k];
+      o.x = aj * (uk0 - cs * uj0) + hk * rj[4];
+      o.y = ak * (uj0 - cs * uk0) + hj * rk[4];
       d3[nn] = o;
-      o.x = aj * (uk1 - cs * uj1) + hk * s_g[3 * j + 1];
-      o.y = ak * (uj1 - cs * uk1) + hj * s_g[3 * k + 1];
+      o.x = aj * (uk1 - cs * uj1) + hk * rj[5];
+      o.y = ak * (uj1 - cs * uk1) + hj * rk[5];
       d3[na + nn] = o;
-      o.x = aj * (uk2 - cs * uj2) + hk * s_g[3 * j + 2];
-      o.y = ak * (uj2 - cs * uk2) + hj * s_g[3 * k + 2];
+      o.x = aj * (uk2 - cs * uj2) + hk * rj[6];
+      o.y = ak * (uj2 - cs * uk2) + hj * rk[6];
       d3[2 * na + nn] = o;
     } else {
       ang[nn] = 0;
@@ -284,7 +322,7 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
 
 template <typename real>
 size_t desc_lds_bytes(int nr) {
-  return (size_t)nr * (12 * sizeof(real) + 2 * sizeof(int));
+  return (size_t)nr * (12 * sizeof(real) + 3 * sizeof(int));
 }
 
 // ---- host side -------------------------------------------------------------
