@@ -272,6 +272,78 @@ def test_virial_forms(oracle, dtype):
         assert torch.all(g3[2] == 0)
 
 
+def _generic_case(oracle, pos, box, tipos, dtype, nr, na, rc, ra, rs, nt, seed=5, dense=False, maps=None):
+    """All ops on an arbitrary configuration: oracle and library with the same synthetic parameters."""
+    from alphanesgpu_amd import synth
+    dtype = np.dtype(dtype)
+    tipos = np.asarray(tipos, np.int32)
+    type_map = np.concatenate([np.full(n, k, np.int32) for k, n in enumerate(tipos)])
+    kw = {} if maps is None else dict(ar_map=maps[0], aa_map=maps[1])   # one block per species / species pair
+    params = synth.fingerprint_params(nt=nt, dtype=dtype, dense_embedding=dense, seed=seed, **kw)
+    pos, box = pos.astype(dtype), box.astype(dtype)
+    up = pipeline.synthetic_upstream(box.shape[0], tipos, params, seed, dtype)
+    ref = pipeline.run_oracle(oracle, pos, box, tipos, type_map, params, up, nr, na, dtype, rc=rc, ra=ra, rs=rs)
+    got = pipeline.run_hip(pos, box, tipos, type_map, params, up, nr, na, dtype, rc=rc, ra=ra, rs=rs)
+    truth = None
+    if dtype == np.float32:
+        d, p, u = pipeline.promote(ref, params, up)
+        truth = pipeline.run_oracle(oracle, None, None, tipos, type_map, p, u, nr, na, np.float64, desc=d)
+    return compare(ref, got, dtype, nr=nr, na=na, truth=truth), ref
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_single_species_example(oracle, dtype):
+    """The reference's single-species example (STAF/example_inference: 50 atoms, Rc = Ra = 22, Rs = 11, nr = 50,
+    na = 1225): nt = 1, one parameter row, Ra = Rc so every neighbour is an angular one."""
+    import os
+    from util import GOLDEN
+    d = os.path.join(GOLDEN, "frame_single_species")
+    pos = np.loadtxt(os.path.join(d, "pos_0")).reshape(1, -1)
+    box = np.loadtxt(os.path.join(d, "box_0")).reshape(1, 6)
+    _generic_case(oracle, pos, box, [pos.shape[1] // 3], dtype, nr=50, na=1225, rc=22.0, ra=22.0, rs=11.0, nt=1,
+                  maps=((20,), (40,)))
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_three_species_with_isolated_atoms(oracle, dtype):
+    """nt = 3 (five parameter rows sigma, six species classes), dense embeddings, Ra < Rc, a triclinic box, and the
+    ragged cases: an atom with no neighbour at all, a pair that only sees each other (no triplet), an atom with
+    neighbours but fewer than two inside Ra."""
+    rng = np.random.default_rng(2)
+    tip = [7, 9, 8]
+    n = sum(tip)
+    L = 14.0
+    pts = []
+    while len(pts) < n - 4:                      # a loose cluster around the origin
+        c = rng.uniform(-3.2, 3.2, 3)
+        if all(np.linalg.norm(c - q) > 1.0 for q in pts):
+            pts.append(c)
+    pts += [np.array([6.5, 6.5, 6.5]),            # isolated
+            np.array([-6.0, 6.0, 0.0]), np.array([-6.0, 6.0, 1.1]),   # a dimer far from everything
+            np.array([0.0, -6.2, -6.2])]          # sees the cluster only beyond Ra, if at all
+    pos = np.array(pts)
+    order = rng.permutation(n)                    # species assigned at random, then stored species-sorted
+    pos = pos[order].reshape(1, -1)
+    box = np.array([[L, 0.7, -0.4, L + 1.0, 0.5, L + 2.0]])
+    errs, ref = _generic_case(oracle, pos, box, tip, dtype, nr=24, na=276, rc=4.5, ra=3.2, rs=1.6, nt=3, dense=True,
+                              maps=((5, 4, 6), (4, 3, 5, 3, 4, 3)))
+    hm = ref["desc"]["intmap2b"][0, :, 0]
+    ntr = ref["desc"]["numtriplet"][0]
+    assert hm.min() == 0 and (hm == 1).sum() >= 2 and (ntr < hm).any()
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_angular_buffer_smaller_than_triplet_count(oracle, dtype):
+    """angular_buffer below m(m-1)/2: the reference silently drops the triplets beyond it (its kernels span only na
+    storage indices); the library must drop exactly the same ones in every op."""
+    b = _synth("water96")
+    ntr = None
+    errs, ref = _generic_case(oracle, b["pos"], b["box"], b["tipos"], dtype, nr=60, na=400, rc=4.5, ra=4.5, rs=2.25,
+                              nt=2)
+    m = ref["desc"]["numtriplet"].astype(np.int64)
+    assert ((m * (m - 1)) // 2 > 400).any()
+
+
 @pytest.mark.gpu
 def test_hip_graph_replay_with_two_streams_matches_eager():
     """The whole op sequence captured once in a HIP graph, the two per-species chains forked onto their own streams
