@@ -106,7 +106,6 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
   }
   if (tid >= nsig && tid < 16) nact[tid] = 0;
   for (int q = tid; q < NW * 8 * nr; q += THREADS) acc[q] = 0;
-  for (int q = tid; q < CAP * RT * 2; q += THREADS) ((real*)E)[q] = 0;   // entries no channel writes stay finite
   for (int sgm = wave; sgm < nsig; sgm += NW) {
     int base = 0;
     for (int a0 = 0; a0 < Aa; a0 += WAVE) {
@@ -185,14 +184,16 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
         const int ia = small_div(e, mrows, inv_mrows), r = e - ia * mrows;
         const int tb = small_div(r, m, inv_m), s = r - tb * m;
         const int sgm = stp[s] + tb;
+        // an entry without a channel is read by lanes of another sigma (and weighted with 0): it must be finite
+        real2 v;
+        v.x = 0; v.y = 0;
         if (c0 + ia < nact[sgm]) {
           const real* o = prm + ((size_t)sgm * Aa + c0 + ia) * 4;
           const real d = sD[s];
-          real2 v;
           v.x = HE::eval(HE::scale(o[0]) * d);
           v.y = HE::eval(HE::scale(o[1]) * d);
-          E[ia * RT + tb * nr + s] = v;
         }
+        E[ia * RT + tb * nr + s] = v;
       }
       __syncthreads();
       PHASE_MARK(2);

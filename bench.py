@@ -65,43 +65,57 @@ def algorithmic_bytes(N, tipos, nr, na, Ar, Aa, nt, s):
     return out
 
 
-def cpu_baseline(batch, params, up, mode, nr, na, max_frames=2):
-    """Times the CPU oracle (single thread) on the first frames of the same batch."""
+def cpu_baseline(batch, params, up, mode, nr, na, max_frames=2, threads=16):
+    """Times the CPU oracle on the first frames of the same batch: one thread (the reported value), and one frame per
+    thread on `threads` threads (frames are independent; ctypes releases the GIL inside the oracle's C++ calls)."""
+    from concurrent.futures import ThreadPoolExecutor
+
     from oracle import staf_oracle as O
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
-    nfs = min(max_frames, batch["nf"])
     dt = batch["dtype"]
-    pos, box = batch["pos"][:nfs], batch["box"][:nfs]
     tipos, type_map = batch["tipos"], batch["type_map"]
+
+    def frames(lo, hi):
+        pos, box = batch["pos"][lo:hi], batch["box"][lo:hi]
+        d = O.compute_descriptors_light(pos, box, 4.5, 4.5, 2.25, nr, na, dtype=dt)
+        o = 0
+        for k, n in enumerate(tipos):
+            s = slice(o, o + int(n))
+            o += int(n)
+            m = params[k]
+            c = lambda a: np.ascontiguousarray(a[:, s])
+            u = lambda name: up[name][k][lo:hi]
+            O.radial_afs(c(d["raddescr"]), c(d["intmap2b"]), m["alpha2b"], m["emb2b"], type_map)
+            O.angular_afs(c(d["angdescr"]), c(d["des3bsupp"]), c(d["intmap3b"]), m["alpha3b"], m["emb3b"], type_map,
+                          c(d["numtriplet"]))
+            O.force_radial(u("G2"), c(d["der2b"]), c(d["intmap2b"]), c(d["raddescr"]), m["alpha2b"], m["emb2b"],
+                           type_map, tipos, k)
+            O.force_tripl(u("G3"), c(d["des3bsupp"]), c(d["angdescr"]), c(d["der3bsupp"]), c(d["der3b"]),
+                          c(d["intmap2b"]), c(d["intmap3b"]), m["alpha3b"], m["emb3b"], type_map, tipos, k,
+                          c(d["numtriplet"]))
+            if mode == "full_step":
+                O.two_body_par_grad(u("P2"), c(d["raddescr"]), c(d["intmap2b"]), m["alpha2b"], m["emb2b"], type_map)
+                O.sort_proj3body_grad(u("P3"), c(d["angdescr"]), c(d["des3bsupp"]), c(d["intmap3b"]),
+                                      c(d["intmap2b"]), m["alpha3b"], m["emb3b"], type_map, c(d["numtriplet"]))
+                O.force_radial_grad(up["Q"][lo:hi], u("G2"), c(d["der2b"]), c(d["intmap2b"]), c(d["raddescr"]),
+                                    m["alpha2b"], m["emb2b"], type_map, tipos, k)
+                O.force_tripl_grad(up["Q"][lo:hi], u("G3"), c(d["des3bsupp"]), c(d["angdescr"]), c(d["der3bsupp"]),
+                                   c(d["der3b"]), c(d["intmap2b"]), c(d["intmap3b"]), m["alpha3b"], m["emb3b"],
+                                   type_map, tipos, k, c(d["numtriplet"]))
+
+    nfs = min(max_frames, batch["nf"])
     t0 = time.perf_counter()
-    d = O.compute_descriptors_light(pos, box, 4.5, 4.5, 2.25, nr, na, dtype=dt)
-    o = 0
-    for k, n in enumerate(tipos):
-        s = slice(o, o + int(n))
-        o += int(n)
-        m = params[k]
-        c = lambda a: np.ascontiguousarray(a[:, s])
-        O.radial_afs(c(d["raddescr"]), c(d["intmap2b"]), m["alpha2b"], m["emb2b"], type_map)
-        O.angular_afs(c(d["angdescr"]), c(d["des3bsupp"]), c(d["intmap3b"]), m["alpha3b"], m["emb3b"], type_map,
-                      c(d["numtriplet"]))
-        O.force_radial(up["G2"][k][:nfs], c(d["der2b"]), c(d["intmap2b"]), c(d["raddescr"]), m["alpha2b"], m["emb2b"],
-                       type_map, tipos, k)
-        O.force_tripl(up["G3"][k][:nfs], c(d["des3bsupp"]), c(d["angdescr"]), c(d["der3bsupp"]), c(d["der3b"]),
-                      c(d["intmap2b"]), c(d["intmap3b"]), m["alpha3b"], m["emb3b"], type_map, tipos, k,
-                      c(d["numtriplet"]))
-        if mode == "full_step":
-            O.two_body_par_grad(up["P2"][k][:nfs], c(d["raddescr"]), c(d["intmap2b"]), m["alpha2b"], m["emb2b"],
-                                type_map)
-            O.sort_proj3body_grad(up["P3"][k][:nfs], c(d["angdescr"]), c(d["des3bsupp"]), c(d["intmap3b"]),
-                                  c(d["intmap2b"]), m["alpha3b"], m["emb3b"], type_map, c(d["numtriplet"]))
-            O.force_radial_grad(up["Q"][:nfs], up["G2"][k][:nfs], c(d["der2b"]), c(d["intmap2b"]), c(d["raddescr"]),
-                                m["alpha2b"], m["emb2b"], type_map, tipos, k)
-            O.force_tripl_grad(up["Q"][:nfs], up["G3"][k][:nfs], c(d["des3bsupp"]), c(d["angdescr"]),
-                               c(d["der3bsupp"]), c(d["der3b"]), c(d["intmap2b"]), c(d["intmap3b"]), m["alpha3b"],
-                               m["emb3b"], type_map, tipos, k, c(d["numtriplet"]))
+    frames(0, nfs)
     el = time.perf_counter() - t0
+    threads = max(1, min(threads, os.cpu_count() or 1))
+    nfr = batch["nf"]
+    t0 = time.perf_counter()
+    with ThreadPoolExecutor(threads) as ex:
+        list(ex.map(lambda i: frames(i % nfr, i % nfr + 1), range(threads)))
+    elm = time.perf_counter() - t0
     return dict(value=nfs / el, unit="frames/s", cores=1, kind="port",
-                sample=f"{nfs} frame(s) of the same batch, same ops, scalar C++ oracle (-O2 -ffp-contract=off), 1 thread")
+                sample=f"{nfs} frame(s) of the same batch, same ops, scalar C++ oracle (-O2 -ffp-contract=off), 1 thread",
+                multicore=dict(value=threads / elm, unit="frames/s", cores=threads,
+                               sample=f"{threads} frames, one per thread, same oracle"))
 
 
 def main():
@@ -236,6 +250,19 @@ def main():
             Ftot = Ftot + f
         return Ftot
 
+    # what a plain device copy reaches on this GPU (bytes read + bytes written per second): second roofline denominator
+    src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    ev[0].record()
+    for _ in range(5):
+        dst.copy_(src)
+    ev[1].record()
+    torch.cuda.synchronize()
+    copy_gbs = 5 * 2 * src.numel() * 4 / (ev[0].elapsed_time(ev[1]) * 1e-3) / 1e9
+    del src, dst
+
     if args.calibrate_copy:
         src = torch.ones(args.calibrate_copy * (1 << 20) // 4, dtype=torch.float32, device=dev)
         dst = torch.empty_like(src)
@@ -333,6 +360,7 @@ def main():
                    "species_streams": args.streams, "launch": "python per op" if graph is None else "hip graph replay"},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": TRAFFIC.get((dom, args.workload)),
+                     "measured_copy_GBs": copy_gbs, "frac_of_measured_copy": achieved / copy_gbs,
                      "algorithmic_bytes_per_launch": dom_bytes_per_launch,
                      "avg_launch_ms": kern[dom]["avg_launch_ms"],
                      "launches_per_step": kern[dom]["launches_per_step"]},
@@ -340,6 +368,7 @@ def main():
                             for k in kern if k in ab},
         "kernel_ms_per_step": {k: v["ms_per_step"] for k, v in kern.items()},
         "whole_step_hbm_frac": step_bytes * nf / (el / args.steps) / 1e9 / HBM_PEAK_GBS,
+        "whole_step_frac_of_measured_copy": step_bytes * nf / (el / args.steps) / 1e9 / copy_gbs,
         "op_ms_per_step": per_step,
         "ms_per_frame": el / args.steps * 1e3 / nf,
         "single_stream": {"value": nf * args.steps / el1, "ms_per_step": el1 / args.steps * 1e3},
