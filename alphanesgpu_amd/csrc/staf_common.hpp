@@ -20,6 +20,9 @@ constexpr int NT_MAX = 8;  // species supported by the per-type bookkeeping
 template <typename real> struct Vec2;
 template <> struct Vec2<float> { using type = float2; };
 template <> struct Vec2<double> { using type = double2; };
+template <typename real> struct Vec4;
+template <> struct Vec4<float> { using type = float4; };
+template <> struct Vec4<double> { using type = double4; };
 
 // The reference's value of pi (STAF/src/descriptor_builder/reforce.cu.cc:15).
 template <typename real> __host__ __device__ inline real pi_ref() { return real(3.141592654); }

@@ -10,14 +10,21 @@
 //     per centre (a row per (tb, s): the parameter row is sigma = t_s + tb; channels whose squared embedding is
 //     exactly 0 are compacted away), so that exp(a1 Dj + a2 Dk) = E[ia][tk,j].x * E[ia][tj,k].y costs two
 //     multiplies.  Per triplet and channel only exp(beta T) remains: one multiply and the hardware exp2 in fp32.
-//       Sd  += h (1 + beta T)(sim1 + sim2)              h = 1/4 G c3 e^{beta T}   (1/2 of E, 1/2 of T)
-//       SBj += h (a1 sim2 + a2 sim1)  SBk += h (a1 sim1 + a2 sim2)               (times T at the end)
+//     With sim2 = exp(a1 Dj + a2 Dk), sim1 = exp(a2 Dj + a1 Dk), P = sim1 + sim2, M = sim2 - sim1:
+//       Sd += h (1 + beta T) P                          h = 1/4 G c3 e^{beta T}   (1/2 of E, 1/2 of T)
+//       U  += h (a1 + a2) P     V += h (a1 - a2) M
+//       SBj = (U + V)/2 = sum h (a1 sim2 + a2 sim1)     SBk = (U - V)/2          (times T at the end)
+//     The table is stored row-major ([row][channel], rows padded by one entry against bank conflicts) and the
+//     channel loop is unrolled, so that every LDS read of the loop is a per-triplet base address plus an
+//     immediate offset.
 //   * der3b contraction in the same lanes: the contributions to slot j of a pass form contiguous lane groups
 //     (rows of the triplet triangle) and are summed with one inclusive scan per value; the contributions to
 //     slot k are added to the wave's own LDS accumulators row by row (inside a row the k are distinct).  The
 //     four waves' accumulators are added in a fixed order: results are bit-reproducible.
 //     F_s = sum_p Sd(s,p) dT/dd_s(s,p) + (sum_p SB_s(s,p)) grad fc_s
 #pragma once
+#include <type_traits>
+
 #include "staf_tri.hpp"
 
 namespace staf {
@@ -32,11 +39,14 @@ struct Force3Cfg {
   static constexpr int NW = THREADS / WAVE;
   static constexpr int NP = 4;                              // passes of 64 triplets a wave holds in registers
   static constexpr int CAP = sizeof(real) == 8 ? 8 : 16;    // channels tabulated at a time
+  static constexpr int CAPP = CAP + 1;                      // table row pitch in entries
   __host__ __device__ static bool fits(int nr, int nt) { return nr <= 255 && nt <= NT_MAX; }   // slots packed in 8 bits
+  __host__ __device__ static int pitch(int Aa) { return (Aa + 3) & ~3; }   // parameter row pitch (channels)
   __host__ __device__ static size_t n_reals(int nr, int Aa, int nt) {
     const int nsig = 2 * nt - 1;
-    return (size_t)CAP * nt * nr * 2 /*E*/ + (size_t)nsig * Aa * 4 /*prm*/ + (size_t)NW * 8 * nr /*accJ, accK per wave*/ +
-           nr /*D*/ + 3 * nr /*grad fc*/ + (size_t)NW * 4 * WAVE /*scan exchange per wave*/ + 3 * nr /*fs*/;
+    return (size_t)nsig * pitch(Aa) * 6 /*prm, prE*/ + (size_t)CAPP * nt * nr * 2 /*E*/ +
+           (size_t)NW * 8 * nr /*accJ, accK per wave*/ + nr /*D*/ + 3 * nr /*grad fc*/ +
+           (size_t)NW * 4 * WAVE /*scan exchange per wave*/;
   }
   __host__ __device__ static size_t bytes(int nr, int Aa, int nt) {
     return n_reals(nr, Aa, nt) * sizeof(real) + (size_t)(16 + nr) * sizeof(int);
@@ -51,25 +61,27 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
     const int* __restrict__ numtriplet, real* __restrict__ gslot, real* __restrict__ self, int* bcnt, int* bent,
     int cap, int* status, int nf, int N, int Nl, int ld, int nr, int na, int Aa, int nt) {
   using real2 = typename Vec2<real>::type;
+  using real4 = typename Vec4<real>::type;
   using HE = HotExp<real>;
   using L = Force3Cfg<real>;
-  constexpr int NP = L::NP, NW = L::NW, THREADS = L::THREADS, CAP = L::CAP;
+  constexpr int NP = L::NP, NW = L::NW, THREADS = L::THREADS, CAP = L::CAP, CAPP = L::CAPP;
   extern __shared__ __align__(16) unsigned char smem[];
   const int nsig = 2 * nt - 1;
   const int RT = nt * nr;                                  // table rows (tb, s)
-  real2* E = (real2*)smem;                                 // [CAP][RT]
-  real* prm = (real*)(E + (size_t)CAP * RT);               // [nsig*Aa][4] = a1, a2, scaled beta, 1/4 G c3 (active channels)
-  real* acc = prm + (size_t)nsig * Aa * 4;                 // [NW][8][nr]: per wave, slot sums as j (4) and as k (4)
+  const int Ap = L::pitch(Aa);
+  real* prm = (real*)smem;                                 // [nsig*Ap][4] = a1+a2, a1-a2, scaled beta, 1/4 G c3 (active channels)
+  real* prE = prm + (size_t)nsig * Ap * 4;                 // [nsig*Ap][2] = a1, a2 in the units of the hot exponential
+  real2* E = (real2*)(prE + (size_t)nsig * Ap * 2);        // [RT][CAPP]
+  real* acc = (real*)(E + (size_t)RT * CAPP);              // [NW][8][nr]: per wave, slot sums as j (4) and as k (4)
   real* sD = acc + (size_t)NW * 8 * nr;                    // [nr]
   real* sg = sD + nr;                                      // [3*nr] grad fc (der3bsupp)
   real* xch = sg + 3 * nr;                                 // [NW][4][64] prefix sums of a pass
-  real* fs = xch + NW * 4 * WAVE;                          // [3*nr]
-  int* nact = (int*)(fs + 3 * nr);                         // [16] active channels per sigma (0 beyond nsig)
+  int* nact = (int*)(xch + NW * 4 * WAVE);                 // [16] active channels per sigma (0 beyond nsig)
   int* stp = nact + 16;                                    // [nr] species of every slot
   PHASE_CLOCK_BEGIN();
 
   const int tid = threadIdx.x;
-  const int lane = tid & (WAVE - 1), wave = tid / WAVE;
+  const int lane = tid & (WAVE - 1), wave = uniform(tid / WAVE);
   const int atom = blockIdx.x;
   const int b = atom / Nl, p_ = atom - b * Nl;
   const size_t rowAtom = (size_t)b * ld + p_;
@@ -84,16 +96,14 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
   real* accK = accJ + 4 * nr;
   real* myx = xch + wave * 4 * WAVE;
 
-  // ---- set-up.  Global reads are issued level by level, back to back: (1) everything addressed by the centre
-  // alone -- slot rows (read up to nr: padded slots hold index 0), the T of the first sweep, the parameter rows;
-  // (2) what needs a neighbour index -- its species and its registration with the receiving atom (an integer
-  // atomic whose return is only used for a store at the very end).  Holding the der3b rows of the first sweep in
-  // registers from here on was measured and is slower: it only adds to the burst of reads every workgroup of
-  // the launch issues at the same moment.
-  int nj = 0;
+  // ---- set-up.  Global reads are issued back to back in two levels: (1) everything addressed by the centre alone,
+  // the neighbour index first (read up to nr: padded slots are never used); (2) the neighbour's species, which
+  // needs only that index and overlaps the parameter rows.
+  // Holding the der3b rows of the first sweep in registers from here on was measured and is slower.
+  unsigned nj = 0;   // unsigned: no sign extension (and so no wait for the read) ahead of the reads that follow
   real d_s = 0, g_s[3] = {0, 0, 0};
   if (tid < nr) {
-    nj = im[1 + tid];
+    nj = (unsigned)im[1 + tid];
     d_s = Dsup[rowAtom * nr + tid];
 #pragma unroll
     for (int c = 0; c < 3; c++) g_s[c] = dDsup[rowAtom * 3 * nr + c * nr + tid];
@@ -104,6 +114,9 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
     const int nn = (p * NW + wave) * WAVE + lane;
     Tpre[p] = nn < na ? Trow[nn] : real(0);
   }
+  const bool slot = tid < m;
+  int t_s = 0;
+  if (slot) t_s = type_map[nj];
   if (tid >= nsig && tid < 16) nact[tid] = 0;
   for (int q = tid; q < NW * 8 * nr; q += THREADS) acc[q] = 0;
   for (int sgm = wave; sgm < nsig; sgm += NW) {
@@ -120,29 +133,33 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
       const bool on = (a < Aa) && (c != real(0));
       const unsigned long long mask = __ballot(on);
       if (on) {
-        real* o = prm + ((size_t)sgm * Aa + base + __popcll(mask & ((1ull << lane) - 1ull))) * 4;
-        o[0] = al0;
-        o[1] = al1;
-        o[2] = HE::scale(al2);   // beta in the units of the hot exponential
-        o[3] = real(0.25) * gv * c;
+        const int ch = sgm * Ap + base + __popcll(mask & ((1ull << lane) - 1ull));
+        real4 o;
+        o.x = al0 + al1;
+        o.y = al0 - al1;
+        o.z = HE::scale(al2);   // beta in the units of the hot exponential
+        o.w = real(0.25) * gv * c;
+        *(real4*)(prm + (size_t)ch * 4) = o;
+        real2 e;
+        e.x = HE::scale(al0);
+        e.y = HE::scale(al1);
+        *(real2*)(prE + (size_t)ch * 2) = e;
       }
       base += __popcll(mask);
     }
-    // parameter rows beyond the active ones are read (and weighted with 0) by lanes of another sigma
-    for (int q = base * 4 + lane; q < Aa * 4; q += WAVE) prm[(size_t)sgm * Aa * 4 + q] = 0;
+    // Rows are Ap long and zero beyond the active channels: a triplet whose sigma has fewer channels than the
+    // workgroup's maximum reads weight 0 (and exponent 0: table entries 1) there.
+    for (int q = base * 4 + lane; q < Ap * 4; q += WAVE) prm[(size_t)sgm * Ap * 4 + q] = 0;
+    for (int q = base * 2 + lane; q < Ap * 2; q += WAVE) prE[(size_t)sgm * Ap * 2 + q] = 0;
     if (lane == 0) nact[sgm] = base;
-  }
-  int bpos = 0;
-  const bool slot = tid < m;
-  if (slot) {
-    stp[tid] = type_map[nj];
-    bpos = atomicAdd(&bcnt[(size_t)b * N + nj], 1);
   }
   if (tid < nr) {
     sD[tid] = d_s;
 #pragma unroll
     for (int c = 0; c < 3; c++) sg[c * nr + tid] = g_s[c];
   }
+  if (slot) stp[tid] = t_s;
+  int bpos = 0;   // place in the receiving atom's bucket (see below)
   __syncthreads();
   PHASE_MARK(0);
   int maxact = 0;
@@ -154,75 +171,101 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
   const float inv_mrows = mrows > 0 ? 1.0f / (float)mrows : 0.f, inv_m = m > 0 ? 1.0f / (float)m : 0.f;
 
   for (int w0 = 0; w0 < ntri; w0 += NW * NP * WAVE) {
-    // ---- this wave's triplets of the sweep: T, packed table rows / sigma, packed slots / active-channel count
-    real T[NP], Sd[NP], S1[NP], S2[NP];
-    int rj[NP], rk[NP], rp[NP], jk[NP];   // table rows of slot j and slot k, first parameter row of sigma, packed j|k|count
+    // ---- this wave's triplets of the sweep: T, table rows of slot j and slot k, parameter row of sigma, packed j|k
+    real T[NP], Sd[NP], U[NP], V[NP];
+    int rj[NP], rk[NP], rp[NP], jk[NP];
+    int npass = 0;   // passes of the sweep this wave has triplets in (a prefix of the NP)
 #pragma unroll
     for (int p = 0; p < NP; p++) {
-      const int nn = w0 + (p * NW + wave) * WAVE + lane;
-      T[p] = 0; Sd[p] = 0; S1[p] = 0; S2[p] = 0;
-      rj[p] = 0; rk[p] = 0; rp[p] = 0;
-      jk[p] = 0;                // count 0: no active channel
+      const int nn0 = w0 + (p * NW + wave) * WAVE, nn = nn0 + lane;
+      if (nn0 < ntri) npass = p + 1;
+      T[p] = 0; Sd[p] = 0; U[p] = 0; V[p] = 0;
+      rj[p] = 0; rk[p] = 0; rp[p] = 0; jk[p] = 0;   // lanes past the last triplet compute on row 0: finite, never used
       if (nn < ntri) {
         int j, k;
         tri_decode(nn, m, j, k);
         T[p] = w0 == 0 ? Tpre[p] : Trow[nn];
         const int tj = stp[j], tk = stp[k];
-        rj[p] = tk * nr + j;
-        rk[p] = tj * nr + k;
-        rp[p] = (tj + tk) * Aa;
-        jk[p] = j | (k << 8) | (nact[tj + tk] << 16);
+        rj[p] = (tk * nr + j) * CAPP;
+        rk[p] = (tj * nr + k) * CAPP;
+        rp[p] = (tj + tk) * Ap * 4;
+        jk[p] = j | (k << 8);
       }
     }
     PHASE_MARK(1);
 
     for (int c0 = 0; c0 < maxact; c0 += CAP) {
       const int nch = (maxact - c0) < CAP ? (maxact - c0) : CAP;
-      if (c0 > 0 || w0 > 0) __syncthreads();   // readers of the previous tables are done
-      // E[ia][(tb, s)] = (exp(a1 D_s), exp(a2 D_s)) with the parameters of sigma = t_s + tb
-      for (int e = tid; e < nch * mrows; e += THREADS) {
+      const int nch4 = (nch + 3) & ~3;            // the channel loop runs in groups of four (c0 + nch4 <= Ap)
+      if (c0 > 0 || w0 > 0) __syncthreads();      // readers of the previous tables are done
+      // E[(tb, s)][ia] = (exp(a1 D_s), exp(a2 D_s)) with the parameters of sigma = t_s + tb
+      for (int e = tid; e < nch4 * mrows; e += THREADS) {
         const int ia = small_div(e, mrows, inv_mrows), r = e - ia * mrows;
         const int tb = small_div(r, m, inv_m), s = r - tb * m;
-        const int sgm = stp[s] + tb;
-        // an entry without a channel is read by lanes of another sigma (and weighted with 0): it must be finite
+        const real2 o = *(const real2*)(prE + ((size_t)(stp[s] + tb) * Ap + c0 + ia) * 2);
+        const real d = sD[s];
         real2 v;
-        v.x = 0; v.y = 0;
-        if (c0 + ia < nact[sgm]) {
-          const real* o = prm + ((size_t)sgm * Aa + c0 + ia) * 4;
-          const real d = sD[s];
-          v.x = HE::eval(HE::scale(o[0]) * d);
-          v.y = HE::eval(HE::scale(o[1]) * d);
-        }
-        E[ia * RT + tb * nr + s] = v;
+        v.x = HE::eval(o.x * d);
+        v.y = HE::eval(o.y * d);
+        E[(tb * nr + s) * CAPP + ia] = v;
       }
       __syncthreads();
       PHASE_MARK(2);
-      for (int ia = 0; ia < nch; ia++) {
-        const real2* Ei = E + ia * RT;
-        const real* prmi = prm + (size_t)(c0 + ia) * 4;
+      // The slot registers with its receiving atom: an integer atomic whose return is only needed for a store at
+      // the very end.  Issued here, ahead of the longest stretch without global reads, its latency is covered by
+      // the channel loop; the next wait on the (in-order) memory counter is the one for the der3b rows.
+      if (w0 == 0 && c0 == 0 && slot) bpos = atomicAdd(&bcnt[(size_t)b * N + nj], 1);
+      // One copy of the loop per number of passes, so that no branch separates the (triplet, channel) items and
+      // the LDS reads of the next items are in flight while the current ones are computed.
+      auto channels = [&](auto npass_c) {
+        constexpr int NPASS = decltype(npass_c)::value;
+        const real2* pj[NPASS];
+        const real2* pk[NPASS];
+        const real* po[NPASS];
 #pragma unroll
-        for (int p = 0; p < NP; p++) {
-          if (w0 + (p * NW + wave) * WAVE >= ntri) break;   // this wave has no further pass in the sweep
-          // A lane whose sigma has no channel c0+ia reads parameters and table entries that are not its own
-          // (finite values of another channel or the zeros the table starts with) and weights them with 0.
-          const real* o = prmi + rp[p] * 4;
-          const real a1 = o[0], a2 = o[1], bes = o[2];
-          const real nc = (c0 + ia) < (jk[p] >> 16) ? o[3] : real(0);
-          const real2 e1 = Ei[rj[p]];
-          const real2 e2 = Ei[rk[p]];
-          const real sim2 = e1.x * e2.y;   // exp(a1 Dj + a2 Dk)
-          const real sim1 = e1.y * e2.x;   // exp(a2 Dj + a1 Dk)
-          const real bts = bes * T[p];
-          const real h = HE::eval(bts) * nc;
-          Sd[p] += h * r_fma(bts, HE::unscale(), real(1)) * (sim1 + sim2);
-          S1[p] += h * (a1 * sim2 + a2 * sim1);
-          S2[p] += h * (a1 * sim1 + a2 * sim2);
+        for (int p = 0; p < NPASS; p++) {
+          pj[p] = E + rj[p];
+          pk[p] = E + rk[p];
+          po[p] = prm + rp[p] + c0 * 4;
         }
+        for (int ia = 0; ia < nch4; ia += 4) {
+#pragma unroll
+          for (int u = 0; u < 4; u++) {
+            // the reads of one channel's items are in flight together; hoisting those of all four channels
+            // would cost more registers than the occupancy can afford
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int p = 0; p < NPASS; p++) {
+              const real4 o = *(const real4*)(po[p] + (ia + u) * 4);   // a1+a2, a1-a2, scaled beta, weight
+              const real2 e1 = pj[p][ia + u];
+              const real2 e2 = pk[p][ia + u];
+              const real bts = o.z * T[p];
+              const real h = HE::eval(bts) * o.w;
+              const real sim1 = e1.y * e2.x;                      // exp(a2 Dj + a1 Dk)
+              const real P = r_fma(e1.x, e2.y, sim1);             // + exp(a1 Dj + a2 Dk)
+              const real M = r_fma(e1.x, e2.y, -sim1);
+              const real hp = h * P, hm = h * M;
+              Sd[p] = r_fma(hp, r_fma(bts, HE::unscale(), real(1)), Sd[p]);
+              U[p] = r_fma(hp, o.x, U[p]);
+              V[p] = r_fma(hm, o.y, V[p]);
+            }
+          }
+        }
+      };
+      static_assert(NP == 4, "one case per pass count below");
+      switch (npass) {
+        case 1: channels(std::integral_constant<int, 1>{}); break;
+        case 2: channels(std::integral_constant<int, 2>{}); break;
+        case 3: channels(std::integral_constant<int, 3>{}); break;
+        case 4: channels(std::integral_constant<int, 4>{}); break;
+        default: break;
       }
       PHASE_MARK(3);
     }
 
-    // ---- contraction with der3b, slot sums of this wave.  The reads of all passes are issued together.
+    // ---- contraction with der3b, slot sums of this wave.  The reads of all passes are issued together and
+    // multiplied in straight-line code (every path waits for them before the sweep loop closes; lanes past the
+    // last triplet hold T = 0, finite sums and read nothing: all their products are 0).
     real2 dv[NP][3];
 #pragma unroll
     for (int p = 0; p < NP; p++) {
@@ -233,19 +276,28 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
         if (nn < ntri) dv[p][c] = d3[c * na + nn];
       }
     }
+    real vjs[NP][4], vks[NP][4];
 #pragma unroll
     for (int p = 0; p < NP; p++) {
+      const real hT = real(0.5) * T[p];
+#pragma unroll
+      for (int c = 0; c < 3; c++) {
+        vjs[p][c] = Sd[p] * dv[p][c].x;
+        vks[p][c] = Sd[p] * dv[p][c].y;
+      }
+      vjs[p][3] = (U[p] + V[p]) * hT;
+      vks[p][3] = (U[p] - V[p]) * hT;
+    }
+#pragma unroll
+    for (int p = 0; p < NP; p++) {
+      if (p >= npass) break;
       const int nn0 = w0 + (p * NW + wave) * WAVE;   // first storage index of the pass
-      if (nn0 >= ntri) break;
       const int nn = nn0 + lane;
       const bool valid = nn < ntri;
-      const int j = jk[p] & 0xff, k = (jk[p] >> 8) & 0xff;
-      real vj[4] = {0, 0, 0, 0}, vk[4] = {0, 0, 0, 0};
-      if (valid) {
-        const real2 d0 = dv[p][0], d1 = dv[p][1], d2 = dv[p][2];
-        vj[0] = Sd[p] * d0.x; vj[1] = Sd[p] * d1.x; vj[2] = Sd[p] * d2.x; vj[3] = S1[p] * T[p];
-        vk[0] = Sd[p] * d0.y; vk[1] = Sd[p] * d1.y; vk[2] = Sd[p] * d2.y; vk[3] = S2[p] * T[p];
-      }
+      const int j = jk[p] & 0xff, k = jk[p] >> 8;
+      real vj[4], vk[4];
+#pragma unroll
+      for (int c = 0; c < 4; c++) { vj[c] = vjs[p][c]; vk[c] = vks[p][c]; }
       // slot j: the lanes of a row are contiguous.  Row sum = prefix at the row's last lane minus prefix
       // before its first lane of this pass.
       __builtin_amdgcn_wave_barrier();
@@ -280,36 +332,43 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
     }
     PHASE_MARK(4);
   }
+  if (ntri <= 0 && slot) bpos = atomicAdd(&bcnt[(size_t)b * N + nj], 1);   // no triplet: not registered yet
+  // The atomic's return is taken here, while no store is in flight: the memory counter is in order, so waiting for
+  // it after the stores below would wait for them as well.
+  asm volatile("" : "+v"(bpos));
   __syncthreads();
   PHASE_MARK(5);
 
-  // ---- slot forces (waves added in a fixed order), centre's own force
-  for (int s = tid; s < m; s += THREADS) {
+  // ---- slot forces (waves added in a fixed order; one slot per thread: m <= nr < THREADS), centre's own force
+  real f3[3] = {0, 0, 0};
+  if (slot) {
     real t4[4];
 #pragma unroll
     for (int c = 0; c < 4; c++) {
       real t = 0;
 #pragma unroll
-      for (int w = 0; w < NW; w++) t += acc[((size_t)w * 8 + c) * nr + s] + acc[((size_t)w * 8 + 4 + c) * nr + s];
+      for (int w = 0; w < NW; w++) t += acc[((size_t)w * 8 + c) * nr + tid] + acc[((size_t)w * 8 + 4 + c) * nr + tid];
       t4[c] = t;
     }
 #pragma unroll
-    for (int c = 0; c < 3; c++) fs[c * nr + s] = t4[c] + t4[3] * sg[c * nr + s];
+    for (int c = 0; c < 3; c++) f3[c] = t4[c] + t4[3] * sg[c * nr + tid];
+  }
+#pragma unroll
+  for (int c = 0; c < 3; c++) {
+    const real t = wave_sum_to_last(f3[c]);
+    if (lane == WAVE - 1) xch[wave * 4 + c] = t;
   }
   __syncthreads();
   // global stores after the last barrier: nothing waits for them
-  for (int s = tid; s < m; s += THREADS) {
+  if (slot) {
 #pragma unroll
-    for (int c = 0; c < 3; c++) gslot[((size_t)atom * nr + s) * 3 + c] = fs[c * nr + s];
+    for (int c = 0; c < 3; c++) gslot[((size_t)atom * nr + tid) * 3 + c] = f3[c];
   }
-  if (tid < WAVE) {
+  if (tid < 3) {
+    real a = 0;
 #pragma unroll
-    for (int c = 0; c < 3; c++) {
-      real a = 0;
-      for (int s = tid; s < m; s += WAVE) a -= fs[c * nr + s];
-      a = wave_sum(a);
-      if (tid == 0) self[(size_t)atom * 3 + c] = a;
-    }
+    for (int w = 0; w < NW; w++) a += xch[w * 4 + tid];
+    self[(size_t)atom * 3 + tid] = -a;
   }
   if (slot) {   // the slot's place in the bucket of its receiving atom
     if (bpos < cap) bent[((size_t)b * N + nj) * cap + bpos] = p_ * nr + tid;
