@@ -152,8 +152,9 @@ static __device__ unsigned long long g_phase_clock[32];
       return STAF_E_HIP;                                                                                    \
     return STAF_OK;                                                                                         \
   }
-#define PHASE_CLOCK_BEGIN()                     \
-  unsigned long long phase_acc_[16] = {0};      \
+#define PHASE_CLOCK_BEGIN()                           \
+  unsigned long long phase_acc_[16] = {0};            \
+  const unsigned long long phase_w0_ = wall_clock64(); \
   unsigned long long phase_t_ = clock64()
 #define PHASE_MARK(i)                                   \
   do {                                                  \
@@ -163,9 +164,17 @@ static __device__ unsigned long long g_phase_clock[32];
   } while (0)
 #define PHASE_CLOCK_END()                                                   \
   do {                                                                      \
-    if (threadIdx.x == 0)                                                   \
+    if (threadIdx.x == 0) {                                                 \
       for (int i_ = 0; i_ < 16; i_++)                                       \
         if (phase_acc_[i_]) atomicAdd(&g_phase_clock[i_], phase_acc_[i_]);  \
+      /* wall-clock (100 MHz) extremes of workgroup start and end; entry 16 holds ~min start */ \
+      const unsigned long long w1_ = wall_clock64();                        \
+      atomicMax(&g_phase_clock[16], ~phase_w0_);                            \
+      atomicMax(&g_phase_clock[17], phase_w0_);                             \
+      atomicMax(&g_phase_clock[18], ~w1_);                                  \
+      atomicMax(&g_phase_clock[19], w1_);                                   \
+      atomicAdd(&g_phase_clock[20], w1_ - phase_w0_);                       \
+    }                                                                       \
   } while (0)
 #else
 #define PHASE_CLOCK_READER(name)

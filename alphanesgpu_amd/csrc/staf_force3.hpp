@@ -40,11 +40,14 @@ struct Force3Cfg {
   static constexpr int NP = 4;                              // passes of 64 triplets a wave holds in registers
   static constexpr int CAP = sizeof(real) == 8 ? 8 : 16;    // channels tabulated at a time
   static constexpr int CAPP = CAP + 1;                      // table row pitch in entries
+  // der3b rows requested one sweep ahead and held in registers across the channel loop: measured, no gain in
+  // fp32 (the kernel is bound by vector-ALU issue) and slower in fp64 (a third of the resident waves lost)
+  static constexpr bool PREFETCH = false;
   __host__ __device__ static bool fits(int nr, int nt) { return nr <= 255 && nt <= NT_MAX; }   // slots packed in 8 bits
   __host__ __device__ static int pitch(int Aa) { return (Aa + 3) & ~3; }   // parameter row pitch (channels)
   __host__ __device__ static size_t n_reals(int nr, int Aa, int nt) {
     const int nsig = 2 * nt - 1;
-    return (size_t)nsig * pitch(Aa) * 6 /*prm, prE*/ + (size_t)CAPP * nt * nr * 2 /*E*/ +
+    return (size_t)nsig * pitch(Aa) * 6 /*prm, prE*/ + (((size_t)CAPP * nt * nr + 1) & ~(size_t)1) * 2 /*E*/ +
            (size_t)NW * 8 * nr /*accJ, accK per wave*/ + nr /*D*/ + 3 * nr /*grad fc*/ +
            (size_t)NW * 4 * WAVE /*scan exchange per wave*/;
   }
@@ -72,7 +75,7 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
   real* prm = (real*)smem;                                 // [nsig*Ap][4] = a1+a2, a1-a2, scaled beta, 1/4 G c3 (active channels)
   real* prE = prm + (size_t)nsig * Ap * 4;                 // [nsig*Ap][2] = a1, a2 in the units of the hot exponential
   real2* E = (real2*)(prE + (size_t)nsig * Ap * 2);        // [RT][CAPP]
-  real* acc = (real*)(E + (size_t)RT * CAPP);              // [NW][8][nr]: per wave, slot sums as j (4) and as k (4)
+  real* acc = (real*)(E + (((size_t)RT * CAPP + 1) & ~(size_t)1));   // [NW][2][nr][4]: per wave, slot sums as j and as k
   real* sD = acc + (size_t)NW * 8 * nr;                    // [nr]
   real* sg = sD + nr;                                      // [3*nr] grad fc (der3bsupp)
   real* xch = sg + 3 * nr;                                 // [NW][4][64] prefix sums of a pass
@@ -92,8 +95,8 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
   if (ntri > na) ntri = na;
   const real* Trow = Tang + rowAtom * na;
   const real2* d3 = (const real2*)d3b + rowAtom * 3 * na;
-  real* accJ = acc + (size_t)wave * 8 * nr;
-  real* accK = accJ + 4 * nr;
+  real4* accJ = (real4*)(acc + (size_t)wave * 8 * nr);   // [nr] x (force x, y, z, radial factor)
+  real4* accK = accJ + nr;
   real* myx = xch + wave * 4 * WAVE;
 
   // ---- set-up.  Global reads are issued back to back in two levels: (1) everything addressed by the centre alone,
@@ -108,11 +111,15 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
 #pragma unroll
     for (int c = 0; c < 3; c++) g_s[c] = dDsup[rowAtom * 3 * nr + c * nr + tid];
   }
-  real Tpre[NP];
+  // Reads of per-triplet rows are never predicated: a lane past the last triplet re-reads the last one (row element
+  // 0 if there is none) and its value is masked where it is used.  With every read issued on every path the waits
+  // can name how many later reads may stay in flight, which is what lets the prefetches below overlap.
+  const int nlast = ntri > 0 ? ntri - 1 : 0;
+  real Tn[NP];
 #pragma unroll
   for (int p = 0; p < NP; p++) {
     const int nn = (p * NW + wave) * WAVE + lane;
-    Tpre[p] = nn < na ? Trow[nn] : real(0);
+    Tn[p] = Trow[nn < nlast ? nn : nlast];
   }
   const bool slot = tid < m;
   int t_s = 0;
@@ -167,8 +174,18 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
     const int n_ = uniform(nact[sgm]);
     maxact = n_ > maxact ? n_ : maxact;
   }
-  const int mrows = nt * m;
-  const float inv_mrows = mrows > 0 ? 1.0f / (float)mrows : 0.f, inv_m = m > 0 ? 1.0f / (float)m : 0.f;
+  // The der3b rows of a sweep are requested one sweep ahead (those of the first here, after the last wait of the
+  // set-up): all workgroups of a launch run in step, so reads issued only where they are needed arrive as one
+  // burst with the vector units idle.
+  real2 dn[NP][3];
+  if constexpr (L::PREFETCH) {
+#pragma unroll
+    for (int p = 0; p < NP; p++) {
+      const int nn = (p * NW + wave) * WAVE + lane;
+#pragma unroll
+      for (int c = 0; c < 3; c++) dn[p][c] = d3[c * na + (nn < nlast ? nn : nlast)];
+    }
+  }
 
   for (int w0 = 0; w0 < ntri; w0 += NW * NP * WAVE) {
     // ---- this wave's triplets of the sweep: T, table rows of slot j and slot k, parameter row of sigma, packed j|k
@@ -184,7 +201,7 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
       if (nn < ntri) {
         int j, k;
         tri_decode(nn, m, j, k);
-        T[p] = w0 == 0 ? Tpre[p] : Trow[nn];
+        T[p] = Tn[p];
         const int tj = stp[j], tk = stp[k];
         rj[p] = (tk * nr + j) * CAPP;
         rk[p] = (tj * nr + k) * CAPP;
@@ -196,18 +213,25 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
 
     for (int c0 = 0; c0 < maxact; c0 += CAP) {
       const int nch = (maxact - c0) < CAP ? (maxact - c0) : CAP;
-      const int nch4 = (nch + 3) & ~3;            // the channel loop runs in groups of four (c0 + nch4 <= Ap)
+      const int nch2 = (nch + 1) & ~1;            // the channel loop runs in pairs (c0 + nch2 <= Ap)
       if (c0 > 0 || w0 > 0) __syncthreads();      // readers of the previous tables are done
       // E[(tb, s)][ia] = (exp(a1 D_s), exp(a2 D_s)) with the parameters of sigma = t_s + tb
-      for (int e = tid; e < nch4 * mrows; e += THREADS) {
-        const int ia = small_div(e, mrows, inv_mrows), r = e - ia * mrows;
-        const int tb = small_div(r, m, inv_m), s = r - tb * m;
-        const real2 o = *(const real2*)(prE + ((size_t)(stp[s] + tb) * Ap + c0 + ia) * 2);
-        const real d = sD[s];
-        real2 v;
-        v.x = HE::eval(o.x * d);
-        v.y = HE::eval(o.y * d);
-        E[(tb * nr + s) * CAPP + ia] = v;
+      // thread <-> (channel ia, rows r0, r0 + RPI, ...): no index division, a row's channels written contiguously
+      {
+        constexpr int RPI = THREADS / CAP;
+        const int ia = tid & (CAP - 1), r0 = tid / CAP;
+        if (ia < nch2) {
+          for (int tb = 0; tb < nt; tb++) {
+            for (int s_ = r0; s_ < m; s_ += RPI) {
+              const real2 o = *(const real2*)(prE + ((size_t)(stp[s_] + tb) * Ap + c0 + ia) * 2);
+              const real d = sD[s_];
+              real2 v;
+              v.x = HE::eval(o.x * d);
+              v.y = HE::eval(o.y * d);
+              E[(tb * nr + s_) * CAPP + ia] = v;
+            }
+          }
+        }
       }
       __syncthreads();
       PHASE_MARK(2);
@@ -228,11 +252,11 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
           pk[p] = E + rk[p];
           po[p] = prm + rp[p] + c0 * 4;
         }
-        for (int ia = 0; ia < nch4; ia += 4) {
+        for (int ia = 0; ia < nch2; ia += 2) {
 #pragma unroll
-          for (int u = 0; u < 4; u++) {
-            // the reads of one channel's items are in flight together; hoisting those of all four channels
-            // would cost more registers than the occupancy can afford
+          for (int u = 0; u < 2; u++) {
+            // the reads of one channel's items are in flight together; hoisting those of more channels would
+            // cost more registers than the occupancy can afford
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int p = 0; p < NPASS; p++) {
@@ -263,30 +287,44 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
       PHASE_MARK(3);
     }
 
-    // ---- contraction with der3b, slot sums of this wave.  The reads of all passes are issued together and
-    // multiplied in straight-line code (every path waits for them before the sweep loop closes; lanes past the
-    // last triplet hold T = 0, finite sums and read nothing: all their products are 0).
-    real2 dv[NP][3];
+    // ---- contraction with der3b, slot sums of this wave.  Lanes past the last triplet hold T = 0 and finite sums
+    // computed on row 0: their products are forced to 0.
+    if constexpr (!L::PREFETCH) {
 #pragma unroll
-    for (int p = 0; p < NP; p++) {
-      const int nn = w0 + (p * NW + wave) * WAVE + lane;
+      for (int p = 0; p < NP; p++) {
+        const int nn = w0 + (p * NW + wave) * WAVE + lane;
 #pragma unroll
-      for (int c = 0; c < 3; c++) {
-        dv[p][c].x = 0; dv[p][c].y = 0;
-        if (nn < ntri) dv[p][c] = d3[c * na + nn];
+        for (int c = 0; c < 3; c++) dn[p][c] = d3[c * na + (nn < nlast ? nn : nlast)];
       }
     }
     real vjs[NP][4], vks[NP][4];
 #pragma unroll
     for (int p = 0; p < NP; p++) {
+      const bool valid = w0 + (p * NW + wave) * WAVE + lane < ntri;
+      const real sd = valid ? Sd[p] : real(0);
       const real hT = real(0.5) * T[p];
 #pragma unroll
       for (int c = 0; c < 3; c++) {
-        vjs[p][c] = Sd[p] * dv[p][c].x;
-        vks[p][c] = Sd[p] * dv[p][c].y;
+        vjs[p][c] = sd * dn[p][c].x;
+        vks[p][c] = sd * dn[p][c].y;
       }
       vjs[p][3] = (U[p] + V[p]) * hT;
       vks[p][3] = (U[p] - V[p]) * hT;
+    }
+    if (w0 + NW * NP * WAVE < ntri) {   // rows of the next sweep
+#pragma unroll
+      for (int p = 0; p < NP; p++) {
+        const int nn = w0 + NW * NP * WAVE + (p * NW + wave) * WAVE + lane;
+        Tn[p] = Trow[nn < nlast ? nn : nlast];
+      }
+      if constexpr (L::PREFETCH) {
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+          const int nn = w0 + NW * NP * WAVE + (p * NW + wave) * WAVE + lane;
+#pragma unroll
+          for (int c = 0; c < 3; c++) dn[p][c] = d3[c * na + (nn < nlast ? nn : nlast)];
+        }
+      }
     }
 #pragma unroll
     for (int p = 0; p < NP; p++) {
@@ -311,21 +349,25 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
       const bool row_end = valid && (lane == WAVE - 1 || jn != j);
       if (row_end) {
         const int first = lane - (k - j - 1);   // lane of the row's first triplet (not positive: starts earlier)
+        real sj[4];
 #pragma unroll
         for (int c = 0; c < 4; c++) {
-          real s = vj[c];
-          if (first > 0) s -= myx[c * WAVE + first - 1];
-          accJ[c * nr + j] += s;
+          sj[c] = vj[c];
+          if (first > 0) sj[c] -= myx[c * WAVE + first - 1];
         }
+        real4 t = accJ[j];
+        t.x += sj[0]; t.y += sj[1]; t.z += sj[2]; t.w += sj[3];
+        accJ[j] = t;
       }
       // slot k: row by row (the k of one row are distinct)
       const int jlo = __builtin_amdgcn_readfirstlane(j);
-      const int nlast = (ntri - 1 - nn0) < (WAVE - 1) ? (ntri - 1 - nn0) : (WAVE - 1);
-      const int jhi = __builtin_amdgcn_readlane(j, nlast);
+      const int llast = (ntri - 1 - nn0) < (WAVE - 1) ? (ntri - 1 - nn0) : (WAVE - 1);
+      const int jhi = __builtin_amdgcn_readlane(j, llast);
       for (int g = jlo; g <= jhi; g++) {
         if (valid && j == g) {
-#pragma unroll
-          for (int c = 0; c < 4; c++) accK[c * nr + k] += vk[c];
+          real4 t = accK[k];
+          t.x += vk[0]; t.y += vk[1]; t.z += vk[2]; t.w += vk[3];
+          accK[k] = t;
         }
         __builtin_amdgcn_wave_barrier();
       }
@@ -342,13 +384,12 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
   // ---- slot forces (waves added in a fixed order; one slot per thread: m <= nr < THREADS), centre's own force
   real f3[3] = {0, 0, 0};
   if (slot) {
-    real t4[4];
+    real t4[4] = {0, 0, 0, 0};
 #pragma unroll
-    for (int c = 0; c < 4; c++) {
-      real t = 0;
-#pragma unroll
-      for (int w = 0; w < NW; w++) t += acc[((size_t)w * 8 + c) * nr + tid] + acc[((size_t)w * 8 + 4 + c) * nr + tid];
-      t4[c] = t;
+    for (int w = 0; w < NW; w++) {
+      const real4 a = ((const real4*)(acc + (size_t)w * 8 * nr))[tid];
+      const real4 c_ = ((const real4*)(acc + (size_t)w * 8 * nr))[nr + tid];
+      t4[0] += a.x + c_.x; t4[1] += a.y + c_.y; t4[2] += a.z + c_.z; t4[3] += a.w + c_.w;
     }
 #pragma unroll
     for (int c = 0; c < 3; c++) f3[c] = t4[c] + t4[3] * sg[c * nr + tid];
