@@ -257,8 +257,18 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
           for (int v = 0; v < NV; v++) acc[v] = 0;
           for (int q0 = 0; q0 < size; q0 += TRI_QB) {
             const int nq = (size - q0) < TRI_QB ? (size - q0) : TRI_QB;
+            // The block is padded to a whole number of rounds of the TRI_SUBS subsets with triplets of T = U = 0 on
+            // table row 0 (they add exact zeros): every subset then makes the same number of steps, and the loop below
+            // runs on a scalar counter.
+            const int nq_pad = (nq + TRI_SUBS - 1) & ~(TRI_SUBS - 1);
             if (q0 > 0) __syncthreads();   // previous block consumed
             // ---- stage a block of triplets
+            for (int qq = nq + tid; qq < nq_pad; qq += TRI_BLOCK) {
+              offA[qq] = 0;
+              offB[qq] = 0;
+              sT[qq] = 0;
+              if (MODE == 2) sU[qq] = 0;
+            }
             for (int qq = tid; qq < nq; qq += TRI_BLOCK) {
               const int q = q0 + qq;
               int x, y;
@@ -288,7 +298,10 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
             __syncthreads();
             // ---- thread <-> (channel ia, subset sub)
             if (chan) {
-              for (int qq = sub; qq < nq; qq += TRI_SUBS) {
+              const int rounds = nq_pad / TRI_SUBS;
+#pragma unroll 2
+              for (int it = 0; it < rounds; it++) {
+                const int qq = sub + it * TRI_SUBS;
                 const int ra = offA[qq], rb = offB[qq];
                 const real T = sT[qq];
                 const real2 e1 = tabE[ra + ia];
