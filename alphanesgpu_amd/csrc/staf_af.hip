@@ -20,7 +20,6 @@ constexpr int GRAD_MAX_BLOCKS = 1024;
 
 // ---------------------------------------------------------------------------
 // 2-body fingerprints: AF2[b,p,a] = sum_s D_s exp(alpha[t_s,a] D_s) c2[t_s,a]
-// lane <-> channel, sequential over the slots (same order as the slot index).
 // ---------------------------------------------------------------------------
 template <typename real>
 __global__ __launch_bounds__(AF_BLOCK) void af2_kernel(const real* __restrict__ D, const int* __restrict__ im2,
@@ -28,12 +27,13 @@ __global__ __launch_bounds__(AF_BLOCK) void af2_kernel(const real* __restrict__ 
                                                        const real* __restrict__ emb2b,
                                                        const int* __restrict__ type_map, real* __restrict__ out,
                                                        int nf, int Nl, int ld, int nr, int Ar, int nt) {
+  using HE = HotExp<real>;
   extern __shared__ __align__(16) unsigned char smem[];
-  real* p_al = (real*)smem;          // [nt*Ar]
+  real* p_al = (real*)smem;          // [nt*Ar] alpha in the units of the hot exponential
   real* p_c2 = p_al + nt * Ar;       // [nt*Ar]
   real* w_D = p_c2 + nt * Ar;        // [AF_WAVES][nr]
   int* w_t = (int*)(w_D + AF_WAVES * nr);  // [AF_WAVES][nr]
-  for (int q = threadIdx.x; q < nt * Ar; q += blockDim.x) { p_al[q] = alpha2b[q]; p_c2[q] = emb2b[q]; }
+  for (int q = threadIdx.x; q < nt * Ar; q += blockDim.x) { p_al[q] = HE::scale(alpha2b[q]); p_c2[q] = emb2b[q]; }
   const int wave = threadIdx.x / WAVE, lane = lane_id();
   real* myD = w_D + wave * nr;
   int* myT = w_t + wave * nr;
@@ -46,25 +46,32 @@ __global__ __launch_bounds__(AF_BLOCK) void af2_kernel(const real* __restrict__ 
     const int* im = im2 + rowAtom * (nr + 1);
     cnt = im[0];
     if (cnt > nr) cnt = nr;
-    for (int s = lane; s < cnt; s += WAVE) { myD[s] = D[rowAtom * nr + s]; myT[s] = type_map[im[1 + s]]; }
+    for (int s = lane; s < cnt; s += WAVE) { myD[s] = D[rowAtom * nr + s]; myT[s] = type_map[im[1 + s]] * Ar; }
   }
   __syncthreads();
   if (atom >= nf * Nl) return;
-  for (int a = lane; a < Ar; a += WAVE) {
+  const ChanSub cs(lane, Ar);
+  for (int a0 = 0; a0 < Ar; a0 += cs.chunk) {
+    const int a = a0 + cs.a;
+    const bool on = cs.sub < cs.nsub && a < Ar;
     real acc = 0;
-    for (int s = 0; s < cnt; s++) {
-      const real d = myD[s];
-      const int t = myT[s];
-      acc += d * (r_exp(p_al[t * Ar + a] * d) * p_c2[t * Ar + a]);
+    if (on) {
+      for (int s = cs.sub; s < cnt; s += cs.nsub) {
+        const real d = myD[s];
+        const int ta = myT[s] + a;
+        acc += d * (HE::eval(p_al[ta] * d) * p_c2[ta]);
+      }
     }
-    out[(size_t)atom * Ar + a] = acc;
+    acc = cs.combine(acc, lane);
+    if (on && cs.sub == 0) out[(size_t)atom * Ar + a] = acc;
   }
 }
 
 // ---------------------------------------------------------------------------
 // dL/dalpha2b, dL/demb2b from P = dL/dAF2:
 //   dalpha[t,a] += P c2 D^2 e^{alpha D},  demb[t,a] += P D e^{alpha D}
-// lane <-> channel; per-species accumulators in registers; workgroup partials.
+// The slots of a centre are grouped by neighbour species, so that a lane's running sums belong to one species at
+// a time; workgroup partials.
 // ---------------------------------------------------------------------------
 template <typename real>
 __global__ __launch_bounds__(AF_BLOCK) void grad2_kernel(const real* __restrict__ D, const int* __restrict__ im2,
@@ -73,19 +80,25 @@ __global__ __launch_bounds__(AF_BLOCK) void grad2_kernel(const real* __restrict_
                                                          const int* __restrict__ type_map,
                                                          const real* __restrict__ P, real* __restrict__ partial,
                                                          int nf, int Nl, int ld, int nr, int Ar, int nt) {
+  using HE = HotExp<real>;
   extern __shared__ __align__(16) unsigned char smem[];
-  real* p_al = (real*)smem;                 // [nt*Ar]
+  real* p_al = (real*)smem;                 // [nt*Ar] alpha in the units of the hot exponential
   real* p_c2 = p_al + nt * Ar;              // [nt*Ar]
   real* w_acc = p_c2 + nt * Ar;             // [AF_WAVES][2*nt*Ar]
-  real* w_D = w_acc + AF_WAVES * 2 * nt * Ar;  // [AF_WAVES][nr]
-  int* w_t = (int*)(w_D + AF_WAVES * nr);   // [AF_WAVES][nr]
-  for (int q = threadIdx.x; q < nt * Ar; q += blockDim.x) { p_al[q] = alpha2b[q]; p_c2[q] = emb2b[q]; }
+  real* w_D = w_acc + AF_WAVES * 2 * nt * Ar;  // [AF_WAVES][nr] D of the slots in grouped order
+  int* w_t = (int*)(w_D + AF_WAVES * nr);   // [AF_WAVES][nr] species of the slot
+  int* w_l = w_t + AF_WAVES * nr;           // [AF_WAVES][nr] slots grouped by species
+  int* w_o = w_l + AF_WAVES * nr;           // [AF_WAVES][NT_MAX+1] first grouped position of a species
+  for (int q = threadIdx.x; q < nt * Ar; q += blockDim.x) { p_al[q] = HE::scale(alpha2b[q]); p_c2[q] = emb2b[q]; }
   const int wave = threadIdx.x / WAVE, lane = lane_id();
   real* myD = w_D + wave * nr;
   int* myT = w_t + wave * nr;
+  int* myL = w_l + wave * nr;
+  int* myO = w_o + wave * (NT_MAX + 1);
   real* myAcc = w_acc + wave * 2 * nt * Ar;
   for (int q = lane; q < 2 * nt * Ar; q += WAVE) myAcc[q] = 0;
   __syncthreads();
+  const ChanSub cs(lane, Ar);
   const int total = nf * Nl;
   const int stride = gridDim.x * AF_WAVES;
   for (int atom = blockIdx.x * AF_WAVES + wave; atom < total; atom += stride) {
@@ -94,27 +107,38 @@ __global__ __launch_bounds__(AF_BLOCK) void grad2_kernel(const real* __restrict_
     const int* im = im2 + rowAtom * (nr + 1);
     int cnt = im[0];
     if (cnt > nr) cnt = nr;
-    for (int s = lane; s < cnt; s += WAVE) { myD[s] = D[rowAtom * nr + s]; myT[s] = type_map[im[1 + s]]; }
+    for (int s = lane; s < cnt; s += WAVE) myT[s] = type_map[im[1 + s]];
     __builtin_amdgcn_wave_barrier();
     __threadfence_block();
-    for (int a = lane; a < Ar; a += WAVE) {
-      const real pg = P[(size_t)atom * Ar + a];
-      real ga[NT_MAX], ge[NT_MAX];
-#pragma unroll
-      for (int t = 0; t < NT_MAX; t++) { ga[t] = 0; ge[t] = 0; }
-      for (int s = 0; s < cnt; s++) {
-        const real d = myD[s];
-        const int t = __builtin_amdgcn_readfirstlane(myT[s]);
-        const real e = r_exp(p_al[t * Ar + a] * d) * pg;
-        const real va = d * d * e * p_c2[t * Ar + a];
-        const real ve = d * e;
-#pragma unroll
-        for (int u = 0; u < NT_MAX; u++)
-          if (u == t) { ga[u] += va; ge[u] += ve; }
+    group_slots_by_type(cnt, nt, myT, myL, myO);
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
+    for (int q = lane; q < cnt; q += WAVE) myD[q] = D[rowAtom * nr + myL[q]];
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
+    for (int a0 = 0; a0 < Ar; a0 += cs.chunk) {
+      const int a = a0 + cs.a;
+      const bool on = cs.sub < cs.nsub && a < Ar;
+      const real pg = on ? P[(size_t)atom * Ar + a] : real(0);
+      for (int t = 0; t < nt; t++) {
+        const int q0 = uniform(myO[t]), q1 = uniform(myO[t + 1]);
+        if (q0 == q1) continue;
+        real ga = 0, ge = 0;
+        if (on) {
+          const real al = p_al[t * Ar + a];
+          for (int q = q0 + cs.sub; q < q1; q += cs.nsub) {
+            const real d = myD[q];
+            const real de = d * HE::eval(al * d);
+            ge += de;
+            ga += d * de;
+          }
+          ga *= p_c2[t * Ar + a] * pg;
+          ge *= pg;
+        }
+        ga = cs.combine(ga, lane);
+        ge = cs.combine(ge, lane);
+        if (on && cs.sub == 0) { myAcc[t * Ar + a] += ga; myAcc[nt * Ar + t * Ar + a] += ge; }
       }
-#pragma unroll
-      for (int u = 0; u < NT_MAX; u++)
-        if (u < nt) { myAcc[u * Ar + a] += ga[u]; myAcc[nt * Ar + u * Ar + a] += ge[u]; }
     }
     __builtin_amdgcn_wave_barrier();
     __threadfence_block();
@@ -171,7 +195,8 @@ static int alpha_dist_grad(const real* D, int nr, const real* alpha2b, int Ar, r
   real* partial = (real*)scratch_reserve(st, stream, ((size_t)nb + RED_SLICES) * nout * sizeof(real));
   real* red_tmp = partial ? partial + (size_t)nb * nout : nullptr;
   if (!partial) return STAF_E_HIP;
-  size_t lds = (size_t)(2 * nt * Ar + AF_WAVES * nout + AF_WAVES * nr) * sizeof(real) + (size_t)AF_WAVES * nr * sizeof(int);
+  size_t lds = (size_t)(2 * nt * Ar + AF_WAVES * nout + AF_WAVES * nr) * sizeof(real) +
+               (size_t)AF_WAVES * (2 * nr + NT_MAX + 1) * sizeof(int);
   if (lds > 64 * 1024) return STAF_E_LIMIT;
   {
     KernelTimer kt_("grad2_kernel", stream);

@@ -59,6 +59,7 @@ __global__ __launch_bounds__(F_BLOCK) void force2_kernel(const real* __restrict_
                                                          real* __restrict__ self, int* bcnt, int* bent, int cap,
                                                          int* status, int nf, int N, int Nl, int ld, int nr, int Ar,
                                                          int nt) {
+  using HE = HotExp<real>;
   extern __shared__ __align__(16) unsigned char smem[];
   real* p_al = (real*)smem;      // [nt*Ar]
   real* p_c2 = p_al + nt * Ar;   // [nt*Ar]
@@ -88,8 +89,8 @@ __global__ __launch_bounds__(F_BLOCK) void force2_kernel(const real* __restrict_
     const real d = D[rowAtom * nr + s];
     real w = 0;
     for (int a = 0; a < Ar; a++) {
-      const real al = p_al[t * Ar + a];
-      w += myG[a] * (p_c2[t * Ar + a] * r_exp(al * d) * (real(1) + al * d));
+      const real ad = p_al[t * Ar + a] * d;
+      w += myG[a] * (p_c2[t * Ar + a] * HE::eval(HE::scale(ad)) * (real(1) + ad));
     }
     w *= real(0.5);
 #pragma unroll
@@ -247,23 +248,29 @@ __global__ __launch_bounds__(F_BLOCK) void gradforce2_kernel(
     real* __restrict__ gnet, real* __restrict__ partial, const real* __restrict__ Qvir,
     const real* __restrict__ pos, const real* __restrict__ box, int skip_pbc, int nf, int N, int Nl, int ld, int nr,
     int Ar, int nt) {
+  using HE = HotExp<real>;
   extern __shared__ __align__(16) unsigned char smem[];
   real* p_al = (real*)smem;                     // [nt*Ar]
   real* p_c2 = p_al + nt * Ar;                  // [nt*Ar]
   real* w_acc = p_c2 + nt * Ar;                 // [F_WAVES][2*nt*Ar]
-  real* w_D = w_acc + F_WAVES * 2 * nt * Ar;    // [F_WAVES][nr]
+  real* w_D = w_acc + F_WAVES * 2 * nt * Ar;    // [F_WAVES][nr]  D, w of the slots in grouped order
   real* w_w = w_D + F_WAVES * nr;               // [F_WAVES][nr]
-  int* w_t = (int*)(w_w + F_WAVES * nr);        // [F_WAVES][nr]
+  int* w_t = (int*)(w_w + F_WAVES * nr);        // [F_WAVES][nr]  species of the slot
+  int* w_l = w_t + F_WAVES * nr;                // [F_WAVES][nr]  slots grouped by species
+  int* w_o = w_l + F_WAVES * nr;                // [F_WAVES][NT_MAX+1]
   for (int q = threadIdx.x; q < nt * Ar; q += blockDim.x) { p_al[q] = alpha2b[q]; p_c2[q] = emb2b[q]; }
   const int wave = threadIdx.x / WAVE, lane = lane_id();
   real* myD = w_D + wave * nr;
   real* myW = w_w + wave * nr;
   int* myT = w_t + wave * nr;
+  int* myL = w_l + wave * nr;
+  int* myO = w_o + wave * (NT_MAX + 1);
   const int nout = 2 * nt * Ar;
   real* myAcc = w_acc + wave * nout;
   for (int q = lane; q < nout; q += WAVE) myAcc[q] = 0;
   const int shift = species_shift(tipos, actual_type);
   __syncthreads();
+  const ChanSub cs(lane, Ar);
   const int total = nf * Nl;
   const int stride = gridDim.x * F_WAVES;
   for (int atom = blockIdx.x * F_WAVES + wave; atom < total; atom += stride) {
@@ -272,9 +279,16 @@ __global__ __launch_bounds__(F_BLOCK) void gradforce2_kernel(
     const int* im = im2 + rowAtom * (nr + 1);
     int cnt = im[0];
     if (cnt > nr) cnt = nr;
+    for (int s = lane; s < cnt; s += WAVE) myT[s] = type_map[im[1 + s]];
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
+    group_slots_by_type(cnt, nt, myT, myL, myO);
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
     const real* Qi = Q + ((size_t)b * N + p + shift) * 3;
     const real qi0 = Qi[0], qi1 = Qi[1], qi2 = Qi[2];
-    for (int s = lane; s < cnt; s += WAVE) {
+    for (int q = lane; q < cnt; q += WAVE) {
+      const int s = myL[q];
       const int nj = im[1 + s];
       const real* Qj = Q + ((size_t)b * N + nj) * 3;
       const real* dr = dD + rowAtom * 3 * nr + s;
@@ -289,35 +303,40 @@ __global__ __launch_bounds__(F_BLOCK) void gradforce2_kernel(
         q1 -= Wg[3] * r[0] + Wg[4] * r[1] + Wg[5] * r[2];
         q2 -= Wg[6] * r[0] + Wg[7] * r[1] + Wg[8] * r[2];
       }
-      myW[s] = real(0.5) * (q0 * dr[0] + q1 * dr[nr] + q2 * dr[2 * nr]);
-      myD[s] = D[rowAtom * nr + s];
-      myT[s] = type_map[nj];
+      myW[q] = real(0.5) * (q0 * dr[0] + q1 * dr[nr] + q2 * dr[2 * nr]);
+      myD[q] = D[rowAtom * nr + s];
     }
     __builtin_amdgcn_wave_barrier();
     __threadfence_block();
-    for (int a = lane; a < Ar; a += WAVE) {
-      const real g = G[(size_t)atom * Ar + a];
+    for (int a0 = 0; a0 < Ar; a0 += cs.chunk) {
+      const int a = a0 + cs.a;
+      const bool on = cs.sub < cs.nsub && a < Ar;
+      const real g = on ? G[(size_t)atom * Ar + a] : real(0);
       real dg = 0;
-      real ga[NT_MAX], ge[NT_MAX];
-#pragma unroll
-      for (int t = 0; t < NT_MAX; t++) { ga[t] = 0; ge[t] = 0; }
-      for (int s = 0; s < cnt; s++) {
-        const real d = myD[s], w = myW[s];
-        const int t = __builtin_amdgcn_readfirstlane(myT[s]);
-        const real al = p_al[t * Ar + a], c2 = p_c2[t * Ar + a];
-        const real e = r_exp(al * d);
-        const real sds = e * (real(1) + al * d);
-        dg += w * c2 * sds;
-        const real va = w * g * c2 * e * d * (real(2) + al * d);
-        const real ve = w * g * sds;
-#pragma unroll
-        for (int u = 0; u < NT_MAX; u++)
-          if (u == t) { ga[u] += va; ge[u] += ve; }
+      for (int t = 0; t < nt; t++) {
+        const int q0 = uniform(myO[t]), q1 = uniform(myO[t + 1]);
+        if (q0 == q1) continue;
+        real ga = 0, ge = 0;
+        if (on) {
+          const real al = p_al[t * Ar + a], c2 = p_c2[t * Ar + a];
+          const real als = HE::scale(al);
+          for (int q = q0 + cs.sub; q < q1; q += cs.nsub) {
+            const real d = myD[q], w = myW[q];
+            const real ad = al * d;
+            const real we = w * HE::eval(als * d);
+            ge += we * (real(1) + ad);           // sum w e (1 + alpha D)
+            ga += we * d * (real(2) + ad);       // sum w e D (2 + alpha D)
+          }
+          dg += c2 * ge;
+          ga *= g * c2;
+          ge *= g;
+        }
+        ga = cs.combine(ga, lane);
+        ge = cs.combine(ge, lane);
+        if (on && cs.sub == 0) { myAcc[t * Ar + a] += ga; myAcc[nt * Ar + t * Ar + a] += ge; }
       }
-      gnet[(size_t)atom * Ar + a] = dg;
-#pragma unroll
-      for (int u = 0; u < NT_MAX; u++)
-        if (u < nt) { myAcc[u * Ar + a] += ga[u]; myAcc[nt * Ar + u * Ar + a] += ge[u]; }
+      dg = cs.combine(dg, lane);
+      if (on && cs.sub == 0) gnet[(size_t)atom * Ar + a] = dg;
     }
     __builtin_amdgcn_wave_barrier();
     __threadfence_block();
@@ -477,7 +496,7 @@ static int gradforce_2b(const real* Q, const real* D, int nr, const real* alpha2
   real* red_tmp = partial ? partial + (size_t)nb * nout : nullptr;
   if (!partial) return STAF_E_HIP;
   size_t lds = (size_t)(2 * nt * Ar + F_WAVES * nout + 2 * F_WAVES * nr) * sizeof(real) +
-               (size_t)F_WAVES * nr * sizeof(int);
+               (size_t)F_WAVES * (2 * nr + NT_MAX + 1) * sizeof(int);
   if (lds > 64 * 1024) return STAF_E_LIMIT;
   {
     KernelTimer kt_("gradforce2_kernel", stream);

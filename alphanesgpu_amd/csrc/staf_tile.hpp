@@ -107,4 +107,24 @@ __device__ inline void class_pair(int q, bool same, int nb_, const int* la, cons
   nn = tri_rowstart(j, m) + k - j - 1;
 }
 
+// Lane <-> (channel, slot subset) for the 2-body kernels: with Ar channels the 64 lanes hold 64 / Ar subsets that
+// walk the slots with that stride, so most lanes work even for few channels (Ar = 20: 60 lanes).  More than 64
+// channels are taken in chunks of 64 with one subset.
+struct ChanSub {
+  int chunk, nsub, sub, a;
+  __device__ ChanSub(int lane, int Ar) {
+    chunk = Ar < WAVE ? Ar : WAVE;
+    nsub = WAVE / chunk;
+    sub = lane / chunk;
+    a = lane - sub * chunk;
+  }
+  // sum over the subsets of a channel, valid in the lanes of subset 0 (fixed order)
+  template <typename real>
+  __device__ real combine(real v, int lane) const {
+    real tot = v;
+    for (int k = 1; k < nsub; k++) tot += __shfl(v, lane + k * chunk, WAVE);
+    return tot;
+  }
+};
+
 }  // namespace staf
