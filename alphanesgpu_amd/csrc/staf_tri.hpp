@@ -31,6 +31,7 @@ namespace staf {
 constexpr int TRI_BLOCK = 256;
 constexpr int TRI_WAVES = TRI_BLOCK / WAVE;
 constexpr int TRI_CAP = 16;    // channels tabulated per pass = lanes of a subset
+constexpr int TRI_CAPP = TRI_CAP + 1;   // table row pitch: the entry after a row's channels holds (D, V) of its slot
 constexpr int TRI_SUBS = TRI_BLOCK / TRI_CAP;
 constexpr int TRI_QB = 512;    // triplets staged per block
 constexpr int TRI_GRID_MAX = 2048;  // workgroups of the persistent gradient modes (one partial row each)
@@ -108,8 +109,7 @@ struct TriLds {
   static constexpr int NV = (MODE == 0) ? 1 : (MODE == 1 ? 3 : 4);
   __host__ __device__ static size_t n_reals(int nr, int Aa, int nt) {
     const int nsig = 2 * nt - 1;
-    size_t r = (size_t)nr * TRI_CAP * 2;                    // pair tables (real2 per (row, channel))
-    r += (size_t)nr * (MODE == 2 ? 2 : 1);                  // D (and V) by table row
+    size_t r = (size_t)nr * TRI_CAPP * 2;                   // pair tables (real2 per (row, channel)), + (D, V) per row
     r += nr;                                                // sD
     r += Aa;                                                // sP
     r += (size_t)TRI_WAVES * Aa;                            // per-wave channel sums
@@ -137,9 +137,7 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
   ChanTable<real> tab;
   unsigned char* sp = tab.carve(smem, nsig, Aa);
   real* rp = (real*)sp;   // 16-byte aligned: the pair tables come first
-  real2* tabE = (real2*)rp; rp += (size_t)nr * TRI_CAP * 2;   // rows of both species of a class: at most m <= nr
-  real* Drow = rp; rp += nr;
-  real* Vrow = rp; if (MODE == 2) rp += nr;
+  real2* tabE = (real2*)rp; rp += (size_t)nr * TRI_CAPP * 2;   // rows of both species of a class: at most m <= nr
   real* sD = rp; rp += nr;
   real* sP = rp; rp += Aa;
   real* outw = rp; rp += (size_t)TRI_WAVES * Aa;
@@ -149,7 +147,7 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
   if (MODE == 2) rp += (size_t)4 * nr;
   real* sT = rp; rp += TRI_QB;
   real* sU = rp; if (MODE == 2) rp += TRI_QB;
-  int* offA = (int*)rp;          // [TRI_QB] first table row of the staged triplet, times TRI_CAP
+  int* offA = (int*)rp;          // [TRI_QB] first table row of the staged triplet, times TRI_CAPP
   int* offB = offA + TRI_QB;     // [TRI_QB] second
   int* lst = offB + TRI_QB;
   int* stp = lst + nr;
@@ -245,11 +243,13 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
               real2 v;
               v.x = HE::eval(a1s * d);
               v.y = HE::eval(a2s * d);
-              tabE[row * TRI_CAP + ia] = v;
+              tabE[row * TRI_CAPP + ia] = v;
             }
             if (ia == 0) {
-              Drow[row] = d;
-              if (MODE == 2) Vrow[row] = sV[s];
+              real2 v;
+              v.x = d;
+              v.y = MODE == 2 ? sV[s] : real(0);
+              tabE[row * TRI_CAPP + TRI_CAP] = v;
             }
           }
           real acc[NV];
@@ -278,8 +278,8 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
               const int j = s1 < s2 ? s1 : s2, k = s1 < s2 ? s2 : s1;
               const int nn = tri_rowstart(j, m) + k - j - 1;
               const bool ok = nn < na;
-              offA[qq] = x * TRI_CAP;
-              offB[qq] = (rowB0 + y) * TRI_CAP;
+              offA[qq] = x * TRI_CAPP;
+              offB[qq] = (rowB0 + y) * TRI_CAPP;
               real T = 0;
               if (ok) T = Trow[nn];
               sT[qq] = T;
@@ -302,24 +302,25 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
 #pragma unroll 2
               for (int it = 0; it < rounds; it++) {
                 const int qq = sub + it * TRI_SUBS;
-                const int ra = offA[qq], rb = offB[qq];
+                const real2* r1 = tabE + (unsigned)offA[qq];
+                const real2* r2 = tabE + (unsigned)offB[qq];
                 const real T = sT[qq];
-                const real2 e1 = tabE[ra + ia];
-                const real2 e2 = tabE[rb + ia];
+                const real2 e1 = r1[ia];
+                const real2 e2 = r2[ia];
                 const real ebt = HE::eval(bes * T);
                 const real sim2 = e1.x * e2.y;   // exp(a1 D1 + a2 D2)
                 const real sim1 = e1.y * e2.x;   // exp(a2 D1 + a1 D2)
                 if constexpr (MODE == 0) {
                   acc[0] += T * (sim1 + sim2) * ebt;
                 } else if constexpr (MODE == 1) {
-                  const real D1 = Drow[ra / TRI_CAP], D2 = Drow[rb / TRI_CAP];
+                  const real D1 = r1[TRI_CAP].x, D2 = r2[TRI_CAP].x;
                   const real w = ebt * T;
                   acc[0] += (sim2 * D1 + sim1 * D2) * w;
                   acc[1] += (sim2 * D2 + sim1 * D1) * w;
                   acc[NV - 1] += (sim1 + sim2) * w * T;
                 } else {
-                  const real D1 = Drow[ra / TRI_CAP], D2 = Drow[rb / TRI_CAP];
-                  const real V1 = Vrow[ra / TRI_CAP], V2 = Vrow[rb / TRI_CAP];
+                  const real2 g1 = r1[TRI_CAP], g2 = r2[TRI_CAP];
+                  const real D1 = g1.x, D2 = g2.x, V1 = g1.y, V2 = g2.y;
                   const real U = sU[qq];
                   const real ss = sim1 + sim2;
                   const real opb = real(1) + be * T;
