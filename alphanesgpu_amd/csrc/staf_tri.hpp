@@ -322,20 +322,30 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
                   const real2 g1 = r1[TRI_CAP], g2 = r2[TRI_CAP];
                   const real D1 = g1.x, D2 = g2.x, V1 = g1.y, V2 = g2.y;
                   const real U = sU[qq];
+                  // With X1 = sim2 V1 + sim1 V2, X2 = sim1 V1 + sim2 V2, W = a1 X1 + a2 X2 (the factor 1/2 of both
+                  // weights is applied once per channel at the end):
+                  //   d/dG      : hU ss + hT W                         hT = e^{bT} T,  hU = e^{bT} (1 + bT) U
+                  //   d/da1     : hU (p + q) + hT (X1 + a1 (p V1 + q V2) + a2 (q V1 + p V2)),  p = sim2 D1, q = sim1 D2
+                  //   d/da2     : hU (r + t) + hT (X2 + a2 (r V1 + t V2) + a1 (t V1 + r V2)),  r = sim1 D1, t = sim2 D2
+                  //   d/dbeta   : hT ((2 + bT) ss U + T W)
+                  const real bT = be * T;
+                  const real hT = ebt * T;
+                  const real eU = ebt * U;
+                  const real hU = r_fma(eU, bT, eU);
                   const real ss = sim1 + sim2;
-                  const real opb = real(1) + be * T;
-                  const real hT = real(0.5) * ebt * T;
-                  const real hU = real(0.5) * ebt * opb * U;
-                  const real sup1 = a1 * sim2 + a2 * sim1;   // multiplies V1 (slot paired with a1 in sim2)
-                  const real sup2 = a1 * sim1 + a2 * sim2;
-                  acc[0] += hU * ss + hT * (sup1 * V1 + sup2 * V2);
-                  acc[1] += hU * (sim1 * D2 + sim2 * D1) +
-                            hT * ((sim2 + a1 * sim2 * D1 + a2 * sim1 * D2) * V1 +
-                                  (sim1 + a1 * sim1 * D2 + a2 * sim2 * D1) * V2);
-                  acc[2] += hU * (sim1 * D1 + sim2 * D2) +
-                            hT * ((sim1 + a2 * sim1 * D1 + a1 * sim2 * D2) * V1 +
-                                  (sim2 + a2 * sim2 * D2 + a1 * sim1 * D1) * V2);
-                  acc[NV - 1] += hT * (real(2) + be * T) * ss * U + hT * T * (sup1 * V1 + sup2 * V2);
+                  const real X1 = r_fma(sim2, V1, sim1 * V2);
+                  const real X2 = r_fma(sim1, V1, sim2 * V2);
+                  const real W = r_fma(a1, X1, a2 * X2);
+                  acc[0] = r_fma(hU, ss, acc[0]);
+                  acc[0] = r_fma(hT, W, acc[0]);
+                  const real p_ = sim2 * D1, q_ = sim1 * D2, r_ = sim1 * D1, t_ = sim2 * D2;
+                  const real Y1 = r_fma(p_, V1, q_ * V2), Y2 = r_fma(q_, V1, p_ * V2);
+                  acc[1] = r_fma(hU, p_ + q_, acc[1]);
+                  acc[1] = r_fma(hT, r_fma(a2, Y2, r_fma(a1, Y1, X1)), acc[1]);
+                  const real Z1 = r_fma(r_, V1, t_ * V2), Z2 = r_fma(t_, V1, r_ * V2);
+                  acc[2] = r_fma(hU, r_ + t_, acc[2]);
+                  acc[2] = r_fma(hT, r_fma(a1, Z2, r_fma(a2, Z1, X2)), acc[2]);
+                  acc[NV - 1] = r_fma(hT, r_fma((real(2) + bT) * ss, U, T * W), acc[NV - 1]);
                 }
               }
             }
@@ -350,7 +360,7 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
           }
           if (lane < TRI_CAP && chan) {
             const int a = tab.ch[pb + c0 + ia];
-            const real c3h = tab.c3[pb + c0 + ia] * real(0.5);
+            const real c3h = tab.c3[pb + c0 + ia] * real(MODE == 2 ? 0.25 : 0.5);
             if constexpr (MODE == 0) {
               my_out[a] += acc[0] * c3h;
             } else if constexpr (MODE == 1) {
