@@ -28,10 +28,10 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # scaled by what the same counters read for a copy kernel of known size; None where no such run was made.
 TRAFFIC = {
     # (FETCH_SIZE KiB x 2.0 + WRITE_SIZE KiB x 1.0) x 1024, averaged over the two per-species launches of a step;
-    # factors from a 256 MiB device copy in the same runs (profiles/force3_kernel_water768_f32_hbm_counters.txt,
-    # profiles/gradforce3_kernel_water768_f64_hbm_counters.txt)
-    ("force3_kernel", "water768_f32"): 39.9e6,
-    ("gradforce3_kernel", "water768_f64"): 77.8e6,
+    # factors from the 1 GiB device copies of this script in the same runs
+    # (profiles/force3_kernel_water768_f32_hbm_counters.txt, profiles/gradforce3_kernel_water768_f64_hbm_counters.txt)
+    ("force3_kernel", "water768_f32"): 38.1e6,
+    ("gradforce3_kernel", "water768_f64"): 78.9e6,
 }
 
 
@@ -126,8 +126,6 @@ def main():
     ap.add_argument("--workload", default="water768_f32")
     ap.add_argument("--mode", default=None, choices=[None, "fwd_force", "full_step"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
-                    help="also run a plain device copy of this size three times (reference point for HBM counters)")
     ap.add_argument("--streams", type=int, default=2, choices=[1, 2],
                     help="2: the per-species op chains (independent until the forces are summed) are issued on one "
                          "HIP stream per species; 1: everything on one stream")
@@ -250,7 +248,8 @@ def main():
             Ftot = Ftot + f
         return Ftot
 
-    # what a plain device copy reaches on this GPU (bytes read + bytes written per second): second roofline denominator
+    # what a plain device copy reaches on this GPU (bytes read + bytes written per second): second roofline denominator;
+    # the six 1 GiB copies (__amd_rocclr_copyBuffer) are also the reference point of the HBM traffic counters
     src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
     dst = torch.empty_like(src)
     dst.copy_(src)
@@ -262,14 +261,6 @@ def main():
     torch.cuda.synchronize()
     copy_gbs = 5 * 2 * src.numel() * 4 / (ev[0].elapsed_time(ev[1]) * 1e-3) / 1e9
     del src, dst
-
-    if args.calibrate_copy:
-        src = torch.ones(args.calibrate_copy * (1 << 20) // 4, dtype=torch.float32, device=dev)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
 
     # One step = one replay of a HIP graph that holds the whole op sequence (the ops run on the stream they are
     # called on, so stream capture records their kernels; scratch is grown by the eager warm-up steps first).
