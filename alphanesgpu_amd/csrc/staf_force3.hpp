@@ -29,9 +29,29 @@
 
 namespace staf {
 
-// register-to-register inclusive prefix sum over the 64 lanes (same tree as wave_sum_to_last)
+// register-to-register inclusive prefix sums over the 64 lanes of four values at once (same tree as
+// wave_sum_to_last; the four chains are interleaved step by step, so that the wait states a lane move needs after
+// the instruction that wrote its source are filled by the other chains)
 template <typename T>
-__device__ inline T wave_scan(T v) { return wave_sum_to_last(v); }
+__device__ inline void wave_scan4(T (&v)[4]) {
+  T s[4];
+#pragma unroll
+  for (int c = 0; c < 4; c++) s[c] = v[c] + dpp_get<0x111, 0xf>(v[c]);
+#pragma unroll
+  for (int c = 0; c < 4; c++) s[c] += dpp_get<0x112, 0xf>(v[c]);
+#pragma unroll
+  for (int c = 0; c < 4; c++) s[c] += dpp_get<0x113, 0xf>(v[c]);
+#pragma unroll
+  for (int c = 0; c < 4; c++) s[c] += dpp_get<0x114, 0xf>(s[c]);
+#pragma unroll
+  for (int c = 0; c < 4; c++) s[c] += dpp_get<0x118, 0xf>(s[c]);
+#pragma unroll
+  for (int c = 0; c < 4; c++) s[c] += dpp_get<0x142, 0xa>(s[c]);   // lane 15 of a row -> every lane of the next row
+#pragma unroll
+  for (int c = 0; c < 4; c++) s[c] += dpp_get<0x143, 0xc>(s[c]);   // lane 31 -> rows 2 and 3
+#pragma unroll
+  for (int c = 0; c < 4; c++) v[c] = s[c];
+}
 
 template <typename real>
 struct Force3Cfg {
@@ -339,27 +359,27 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
       // slot j: the lanes of a row are contiguous.  Row sum = prefix at the row's last lane minus prefix
       // before its first lane of this pass.
       __builtin_amdgcn_wave_barrier();
+      wave_scan4(vj);
 #pragma unroll
-      for (int c = 0; c < 4; c++) {
-        vj[c] = wave_scan(vj[c]);
-        myx[c * WAVE + lane] = vj[c];
-      }
+      for (int c = 0; c < 4; c++) myx[c * WAVE + lane] = vj[c];
       __builtin_amdgcn_wave_barrier();
       const int jn = __shfl_down(valid ? j : -1, 1, WAVE);
       const bool row_end = valid && (lane == WAVE - 1 || jn != j);
       if (row_end) {
         const int first = lane - (k - j - 1);   // lane of the row's first triplet (not positive: starts earlier)
+        const int before = first > 0 ? first - 1 : 0;
         real sj[4];
 #pragma unroll
         for (int c = 0; c < 4; c++) {
-          sj[c] = vj[c];
-          if (first > 0) sj[c] -= myx[c * WAVE + first - 1];
+          const real pre = myx[c * WAVE + before];
+          sj[c] = vj[c] - (first > 0 ? pre : real(0));
         }
         real4 t = accJ[j];
         t.x += sj[0]; t.y += sj[1]; t.z += sj[2]; t.w += sj[3];
         accJ[j] = t;
       }
-      // slot k: row by row (the k of one row are distinct)
+      // slot k: row by row (the k of one row are distinct).  LDS floating-point adds instead of this loop were
+      // measured: much slower in fp32 (1.6x the kernel), a few percent faster in fp64.
       const int jlo = __builtin_amdgcn_readfirstlane(j);
       const int llast = (ntri - 1 - nn0) < (WAVE - 1) ? (ntri - 1 - nn0) : (WAVE - 1);
       const int jhi = __builtin_amdgcn_readlane(j, llast);
