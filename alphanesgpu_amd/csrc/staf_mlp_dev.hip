@@ -13,6 +13,7 @@ namespace staf {
 
 constexpr int MLP_TA = 4;        // atoms per workgroup
 constexpr int MLP_BLOCK = 256;
+static_assert(MLP_TA <= MLP_BLOCK / WAVE, "the output neuron is summed by one wave per atom");
 
 template <typename T>
 struct MlpArgs {
@@ -58,11 +59,28 @@ __global__ __launch_bounds__(MLP_BLOCK) void mlp_kernel(MlpArgs<T> A) {
   for (int l = 0; l < A.nl; l++) {
     const int in_f = A.in_f[l], out_f = A.out_f[l];
     const int off_out = off_in + in_f;
+    if (out_f == 1) {
+      // the output neuron of the stack: wave t sums atom t's products over the lanes (fixed order)
+      const int t = tid / WAVE, lane = tid & (WAVE - 1);
+      if (t < MLP_TA) {
+        T part = 0;
+        for (int i = lane; i < in_f; i += WAVE) part += buf[t * A.tot + off_in + i] * A.W[l][i];
+        part = wave_sum(part);
+        if (lane == 0) {
+          T y = part + A.b[l][0];
+          if (A.act[l] == 1) y = m_tanh(y);
+          else if (A.act[l] == 2) y = y > T(0) ? y : T(0);
+          buf[t * A.tot + off_out] = y;
+        }
+      }
+    } else
     for (int j = tid; j < out_f; j += MLP_BLOCK) {
       T acc[MLP_TA];
       const T bj = A.b[l][j];
 #pragma unroll
       for (int t = 0; t < MLP_TA; t++) acc[t] = bj;
+      // the weight reads of twenty steps are in flight together (the loop is bound by their latency otherwise)
+#pragma unroll 20
       for (int i = 0; i < in_f; i++) {
         const T w = A.W[l][(size_t)i * out_f + j];
 #pragma unroll
@@ -103,6 +121,7 @@ __global__ __launch_bounds__(MLP_BLOCK) void mlp_kernel(MlpArgs<T> A) {
       T acc[MLP_TA];
 #pragma unroll
       for (int t = 0; t < MLP_TA; t++) acc[t] = 0;
+#pragma unroll 20
       for (int j = 0; j < out_f; j++) {
         const T w = A.Wt[l][(size_t)j * in_f + i];
 #pragma unroll
