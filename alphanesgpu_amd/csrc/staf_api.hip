@@ -49,6 +49,22 @@ __global__ void add_into_kernel(double* dst, const double* src, int n) {
   if (e < n) dst[e] += src[e];
 }
 
+// dst[e] = sum over the nb op outputs src[b*n + e], b ascending (fixed order); the same for the 3x3 virials
+__global__ void combine_kernel(double* dst, const double* src, int n, int nb, double* vdst, const double* vsrc) {
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e < n) {
+    double s = 0;
+    for (int b = 0; b < nb; b++) s += src[(size_t)b * n + e];
+    dst[e] = s;
+  }
+  if (e < 9) {
+    double s = 0;
+    if (vsrc)
+      for (int b = 0; b < nb; b++) s += vsrc[b * 9 + e];
+    vdst[e] = s;
+  }
+}
+
 bool read_numbers(const std::string& path, std::vector<double>& out, int* rows) {
   FILE* f = fopen(path.c_str(), "r");
   if (!f) return false;
@@ -84,7 +100,10 @@ struct StafModel {
   std::vector<int> Ar, Aa;
   std::vector<DevBuf<double>> alpha2b, alpha3b, emb2b, emb3b;
   staf::DescConfig<double> cfg;
-  hipStream_t stream = nullptr;
+  hipStream_t stream = nullptr;            // the call's stream (descriptors, copies, final sum)
+  std::vector<hipStream_t> sstream;        // one per centre species: their op chains are independent
+  hipEvent_t ev_fork = nullptr;
+  std::vector<hipEvent_t> ev_join;
   // device buffers
   DevBuf<double> pos, box, force, force_op, virial_op, af2, af3, g2, g3, e_atom, virial_acc;
   // device-resident MLP (default); false: the host evaluation of staf_mlp.cpp between the kernels
@@ -180,6 +199,13 @@ int staf_cuda_set_device(int device_id) {
 
 void staf_free(StafModel* m) {
   if (!m) return;
+  if (m->stream) (void)hipStreamSynchronize(m->stream);
+  for (hipStream_t s : m->sstream)
+    if (s) { (void)hipStreamSynchronize(s); (void)hipStreamDestroy(s); }
+  for (hipEvent_t e : m->ev_join)
+    if (e) (void)hipEventDestroy(e);
+  if (m->ev_fork) (void)hipEventDestroy(m->ev_fork);
+  if (m->stream) (void)hipStreamDestroy(m->stream);
   if (m->mlp) staf_mlp_destroy(m->mlp);
   for (auto& n : m->dnets) staf::dev_mlp_free(&n);
   for (auto* v : {&m->alpha2b, &m->alpha3b, &m->emb2b, &m->emb3b})
@@ -242,6 +268,19 @@ StafModel* staf_load(const char* model_dir, const StafOptions* opt) {
     }
   }
   if (staf::desc_configure<double>(m->cfg, m->Rc, m->nr, m->na, m->Rs, m->Ra) != STAF_OK) {
+    staf_free(m);
+    return NULL;
+  }
+  // Streams of the model (default priority; non-blocking: no implicit ordering with the legacy default stream).
+  bool ok = hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking) == hipSuccess &&
+            hipEventCreateWithFlags(&m->ev_fork, hipEventDisableTiming) == hipSuccess;
+  m->sstream.assign(m->nt, nullptr);
+  m->ev_join.assign(m->nt, nullptr);
+  for (int k = 0; k < m->nt && ok; k++)
+    ok = hipStreamCreateWithFlags(&m->sstream[k], hipStreamNonBlocking) == hipSuccess &&
+         hipEventCreateWithFlags(&m->ev_join[k], hipEventDisableTiming) == hipSuccess;
+  if (!ok) {
+    fprintf(stderr, "staf_load: cannot create the model's streams\n");
     staf_free(m);
     return NULL;
   }
@@ -322,7 +361,7 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
   int amax2 = 0, amax3 = 0;
   for (int k = 0; k < nt; k++) { amax2 = m->Ar[k] > amax2 ? m->Ar[k] : amax2; amax3 = m->Aa[k] > amax3 ? m->Aa[k] : amax3; }
   bool ok = m->pos.reserve((size_t)nall * 3) && m->box.reserve(6) && m->force.reserve((size_t)nall * 3) &&
-            m->force_op.reserve((size_t)nall * 3) && m->virial_op.reserve(9) && m->af2.reserve(L * amax2) &&
+            m->force_op.reserve((size_t)nall * 3 * 2 * nt) && m->virial_op.reserve((size_t)9 * 2 * nt) && m->af2.reserve(L * amax2) &&
             m->af3.reserve(L * amax3) && m->g2.reserve(L * amax2) && m->g3.reserve(L * amax3) &&
             m->e_atom.reserve(L) && m->virial_acc.reserve(9) &&
             m->raddescr.reserve(L * nr) && m->angdescr.reserve(L * na) && m->des3bsupp.reserve(L * nr) &&
@@ -343,15 +382,14 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
     STAF_HIP_OK(hipMemcpyAsync(m->how.p, m->how_h.data(), L * sizeof(int), hipMemcpyHostToDevice, st));
     STAF_HIP_OK(hipMemcpyAsync(m->with.p, m->with_h.data(), L * nr * sizeof(int), hipMemcpyHostToDevice, st));
   }
-  STAF_HIP_OK(hipStreamSynchronize(st));   // the host vectors above may be reused by the next call
+  // No synchronisation here: every host buffer above outlives the call's final synchronisation.
+  staf::DeferStatus defer;   // conditions the kernels detect are read once, after the last kernel
 
   // ---- descriptors (own minimum-image list, or the caller's list with explicit images)
   int rc = staf::desc_launch<double>(m->cfg, m->pos.p, m->box.p, 1, nlocal, nall, ext ? m->how.p : nullptr,
                                      ext ? m->with.p : nullptr, ext ? 1 : 0, m->raddescr.p, m->angdescr.p,
                                      m->des3bsupp.p, m->intmap2b.p, m->intmap3b.p, m->der2b.p, m->der3b.p,
                                      m->der3bsupp.p, m->numtriplet.p, st);
-  if (rc == STAF_OK && !staf::sync_errors_enabled()) rc = staf_ops_poll_status(st);
-  if (rc == STAF_E_RADIAL_OVERFLOW) return -10;
   if (rc != STAF_OK) return -20;
 
   double energy = 0.0;
@@ -359,49 +397,57 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
   const int n3 = nall * 3;
   staf_op_force_set_skip_pbc(ext ? 1 : 0);
   if (m->dev_mlp) {
-    // ---- everything stays on the device: per species fingerprints -> MLP -> forces; one synchronisation at the end
-    staf::launch_fill_zero<double>(m->force.p, n3, st);
-    staf::launch_fill_zero<double>(m->virial_acc.p, 9, st);
+    // ---- everything stays on the device: per species fingerprints -> MLP -> forces, one stream per species (the
+    // chains meet only in the sum of the forces); one synchronisation at the end of the call
+    const bool want_w = virial != nullptr;
+    STAF_HIP_OK(hipEventRecord(m->ev_fork, st));
+    int nops = 0;
     int shift = 0;
     for (int k = 0; k < nt; shift += tipos[k], k++) {
       const int Nl = tipos[k], Ar = m->Ar[k], Aa = m->Aa[k];
       if (Nl == 0) continue;
+      hipStream_t sk = m->sstream[k];
+      STAF_HIP_OK(hipStreamWaitEvent(sk, m->ev_fork, 0));
       const size_t o = (size_t)shift;
-      rc = staf_op_radial_afs_f64(m->raddescr.p + o * nr, nr, m->alpha2b[k].p, Ar, m->af2.p, 1, Nl,
-                                  m->intmap2b.p + o * (nr + 1), m->emb2b[k].p, m->type_map.p, nt, nlocal, st);
+      double* af2 = m->af2.p + o * amax2;
+      double* af3 = m->af3.p + o * amax3;
+      double* g2 = m->g2.p + o * amax2;
+      double* g3 = m->g3.p + o * amax3;
+      rc = staf_op_radial_afs_f64(m->raddescr.p + o * nr, nr, m->alpha2b[k].p, Ar, af2, 1, Nl,
+                                  m->intmap2b.p + o * (nr + 1), m->emb2b[k].p, m->type_map.p, nt, nlocal, sk);
       if (rc == STAF_OK)
-        rc = staf_op_angular_afs_f64(m->des3bsupp.p + o * nr, m->angdescr.p + o * na, nr, na, m->af3.p, 1, Nl,
+        rc = staf_op_angular_afs_f64(m->des3bsupp.p + o * nr, m->angdescr.p + o * na, nr, na, af3, 1, Nl,
                                      m->intmap3b.p + o * 2 * na, m->intmap2b.p + o * (nr + 1), m->alpha3b[k].p, Aa,
-                                     m->emb3b[k].p, m->type_map.p, m->numtriplet.p + o, nt, nlocal, st);
+                                     m->emb3b[k].p, m->type_map.p, m->numtriplet.p + o, nt, nlocal, sk);
       if (rc == STAF_OK)
-        rc = staf::dev_mlp_eval(m->dnets[k], m->af2.p, Ar, m->af3.p, Aa, Nl, m->e_atom.p + o, m->g2.p, m->g3.p, st);
+        rc = staf::dev_mlp_eval(m->dnets[k], af2, Ar, af3, Aa, Nl, m->e_atom.p + o, g2, g3, sk);
       if (rc != STAF_OK) return -20;
-      for (int body = 2; body <= 3; body++) {
+      for (int body = 2; body <= 3; body++, nops++) {
+        double* fo = m->force_op.p + (size_t)nops * n3;
+        double* wo = want_w ? m->virial_op.p + nops * 9 : nullptr;
+        const double* px = want_w ? m->pos.p : nullptr;
+        const double* bx = want_w ? m->box.p : nullptr;
         if (body == 2)
-          rc = staf_op_force_doublets_f64(m->g2.p, m->raddescr.p + o * nr, m->der2b.p + o * 3 * nr,
+          rc = staf_op_force_doublets_f64(g2, m->raddescr.p + o * nr, m->der2b.p + o * 3 * nr,
                                           m->intmap2b.p + o * (nr + 1), nr, nall, 1, Ar, m->alpha2b[k].p,
-                                          m->emb2b[k].p, nt, m->tipos.p, m->actual_type.p + k, m->force_op.p,
-                                          m->type_map.p, Nl, m->virial_op.p, m->pos.p, m->box.p, nlocal, st);
+                                          m->emb2b[k].p, nt, m->tipos.p, m->actual_type.p + k, fo, m->type_map.p, Nl,
+                                          wo, px, bx, nlocal, sk);
         else
-          rc = staf_op_force_tripl_f64(m->g3.p, m->des3bsupp.p + o * nr, m->angdescr.p + o * na,
+          rc = staf_op_force_tripl_f64(g3, m->des3bsupp.p + o * nr, m->angdescr.p + o * na,
                                        m->der3bsupp.p + o * 3 * nr, m->der3b.p + o * 6 * na,
                                        m->intmap2b.p + o * (nr + 1), m->intmap3b.p + o * 2 * na, nr, na, nall, 1, Aa,
-                                       m->emb3b[k].p, nt, m->tipos.p, m->actual_type.p + k, m->force_op.p,
-                                       m->numtriplet.p + o, m->alpha3b[k].p, m->type_map.p, Nl, m->virial_op.p,
-                                       m->pos.p, m->box.p, nlocal, st);
+                                       m->emb3b[k].p, nt, m->tipos.p, m->actual_type.p + k, fo, m->numtriplet.p + o,
+                                       m->alpha3b[k].p, m->type_map.p, Nl, wo, px, bx, nlocal, sk);
         if (rc != STAF_OK) return -20;
-        hipLaunchKernelGGL(add_into_kernel, dim3((n3 + 255) / 256), dim3(256), 0, st, m->force.p, m->force_op.p, n3);
-        hipLaunchKernelGGL(add_into_kernel, dim3(1), dim3(64), 0, st, m->virial_acc.p, m->virial_op.p, 9);
       }
+      STAF_HIP_OK(hipEventRecord(m->ev_join[k], sk));
+      STAF_HIP_OK(hipStreamWaitEvent(st, m->ev_join[k], 0));
     }
+    hipLaunchKernelGGL(combine_kernel, dim3((n3 + 255) / 256), dim3(256), 0, st, m->force.p, m->force_op.p, n3, nops,
+                       m->virial_acc.p, want_w ? m->virial_op.p : nullptr);
     m->e_atom_h.resize(nlocal);
     STAF_HIP_OK(hipMemcpyAsync(m->e_atom_h.data(), m->e_atom.p, L * sizeof(double), hipMemcpyDeviceToHost, st));
     STAF_HIP_OK(hipMemcpyAsync(W, m->virial_acc.p, 9 * sizeof(double), hipMemcpyDeviceToHost, st));
-    STAF_HIP_OK(hipStreamSynchronize(st));
-    for (int a = 0; a < nlocal; a++) energy += m->e_atom_h[a];   // slot order: fixed
-    energy *= 0.5;
-    if (!isfinite(energy))
-      fprintf(stderr, "staf_compute: non-finite energy=%g nlocal=%d nghost=%d\n", energy, nlocal, nghost);
   } else {
     // ---- fingerprints of every species, packed rows [Ar+Aa] for the MLP
     size_t total = 0;
@@ -506,7 +552,16 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
   }
   m->force_h.resize((size_t)n3);
   STAF_HIP_OK(hipMemcpyAsync(m->force_h.data(), m->force.p, (size_t)n3 * sizeof(double), hipMemcpyDeviceToHost, st));
-  STAF_HIP_OK(hipStreamSynchronize(st));
+  // the call's synchronisation: results are on the host, and so is what the kernels reported
+  rc = staf_ops_poll_status(st);
+  if (rc == STAF_E_RADIAL_OVERFLOW) return -10;
+  if (rc != STAF_OK) return -20;
+  if (m->dev_mlp) {
+    for (int a = 0; a < nlocal; a++) energy += m->e_atom_h[a];   // slot order: fixed
+    energy *= 0.5;
+    if (!isfinite(energy))
+      fprintf(stderr, "staf_compute: non-finite energy=%g nlocal=%d nghost=%d\n", energy, nlocal, nghost);
+  }
 
   if (e_rank) *e_rank = energy;
   if (f)

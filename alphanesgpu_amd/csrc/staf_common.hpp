@@ -210,6 +210,10 @@ void* scratch_reserve(DeviceState* st, hipStream_t stream, size_t bytes);   // g
 int* bucket_reserve(DeviceState* st, size_t n_counters, size_t n_entries, hipStream_t stream, int** entries);
 int finish_op(DeviceState* st, hipStream_t stream);            // launch check (+ optional sync & status fetch)
 bool sync_errors_enabled();
+struct DeferStatus {   // while one is alive, the calling thread's ops do not synchronise to report device conditions
+  DeferStatus();
+  ~DeferStatus();
+};
 
 // Optional timing of single kernels with HIP events on the stream they are launched on (off by default; switched on
 // with staf_ops_kernel_timing).  A KernelTimer brackets one launch; the pairs are summed by staf_ops_kernel_time.

@@ -1,5 +1,6 @@
 // Library-owned per-device state: status word, scratch and scatter buckets.
 #include "staf_common.hpp"
+#include "staf_reduce.hpp"
 
 #include <mutex>
 #include <unordered_map>
@@ -14,8 +15,13 @@ namespace staf {
 static std::mutex g_mu;
 static std::unordered_map<int, std::unique_ptr<DeviceState>> g_state;
 static int g_sync_errors = 1;
+// Calls made by this thread leave their device-detected conditions in the status word (no synchronisation per op)
+// while the count is positive: the MD entry runs its whole op sequence this way and reads the word once at the end.
+static thread_local int tl_defer_status = 0;
+DeferStatus::DeferStatus() { ++tl_defer_status; }
+DeferStatus::~DeferStatus() { --tl_defer_status; }
 
-bool sync_errors_enabled() { return g_sync_errors != 0; }
+bool sync_errors_enabled() { return g_sync_errors != 0 && tl_defer_status == 0; }
 
 static int g_kernel_timing = 0;
 static std::unordered_map<std::string, std::vector<std::pair<hipEvent_t, hipEvent_t>>> g_kernel_events;
@@ -34,7 +40,8 @@ DeviceState* device_state() {
   auto st = std::unique_ptr<DeviceState>(new DeviceState());
   st->device = dev;
   if (hipMalloc((void**)&st->status_d, sizeof(int)) != hipSuccess) return nullptr;
-  if (hipMemset(st->status_d, 0, sizeof(int)) != hipSuccess) return nullptr;
+  // the clear runs on the legacy default stream: wait for it, callers' streams need not be ordered after that one
+  if (hipMemset(st->status_d, 0, sizeof(int)) != hipSuccess || hipDeviceSynchronize() != hipSuccess) return nullptr;
   if (hipHostMalloc((void**)&st->status_h, sizeof(int), hipHostMallocDefault) != hipSuccess) return nullptr;
   *st->status_h = 0;
   DeviceState* raw = st.get();
@@ -76,7 +83,10 @@ int* bucket_reserve(DeviceState* st, size_t n_counters, size_t n_entries, hipStr
     size_t ent = n_entries + n_entries / 4;
     size_t want = (cnt + ent) * sizeof(int);
     if (hipMalloc(&w->buckets.buf, want) != hipSuccess) return nullptr;
-    if (hipMemset(w->buckets.buf, 0, cnt * sizeof(int)) != hipSuccess) return nullptr;
+    // cleared on the caller's stream, ahead of the kernels that count into it (a clear on the default stream is
+    // not ordered before work on a non-blocking stream)
+    launch_fill_zero<int>((int*)w->buckets.buf, (int)cnt, stream);
+    if (hipGetLastError() != hipSuccess) return nullptr;
     w->buckets.bytes = want;
     w->bucket_counters = cnt;
     w->bucket_entries = ent;
@@ -105,7 +115,7 @@ static int fetch_status(DeviceState* st, hipStream_t stream) {
 
 int finish_op(DeviceState* st, hipStream_t stream) {
   if (hipGetLastError() != hipSuccess) return STAF_E_HIP;
-  if (!g_sync_errors) return STAF_OK;
+  if (!sync_errors_enabled()) return STAF_OK;
   return fetch_status(st, stream);
 }
 
