@@ -72,9 +72,10 @@ class StafModel:
         if not self._h:
             raise RuntimeError(f"staf_load failed for {model_dir}")
 
-    def compute(self, x, box, types=None, nlocal=None, howmany=None, neigh=None):
+    def compute(self, x, box, types=None, nlocal=None, howmany=None, neigh=None, want_virial=True):
         """x [nall,3] float64, box [6] = (Lx, xy, xz, Ly, yz, Lz), types [nall] int32 (0-based).
-        Returns (energy of the owned atoms, forces [nall,3], virial [6] = xx yy zz xy xz yz)."""
+        Returns (energy of the owned atoms, forces [nall,3], virial [6] = xx yy zz xy xz yz); want_virial=False
+        passes a null virial pointer (the virial kernels are skipped) and returns None for it."""
         x = np.ascontiguousarray(x, np.float64).reshape(-1, 3)
         box = np.ascontiguousarray(box, np.float64).reshape(6)
         nall = x.shape[0]
@@ -88,7 +89,7 @@ class StafModel:
             w = np.ascontiguousarray(neigh, np.int32).reshape(nlocal, -1)
             maxneigh = w.shape[1]
         f = np.zeros((nall, 3), np.float64)
-        vir = np.zeros(6, np.float64)
+        vir = np.zeros(6, np.float64) if want_virial else None
         e = C.c_double(0.0)
         p = lambda a: None if a is None else a.ctypes.data_as(C.c_void_p)
         rc = self._L.staf_compute(self._h, nlocal, nghost, p(x), p(box), p(tp), p(hm), p(w), maxneigh, C.byref(e),

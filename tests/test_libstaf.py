@@ -245,6 +245,19 @@ def test_device_mlp_matches_host_mlp(prec, tol):
 
 
 @pytest.mark.gpu
+def test_compute_without_virial_gives_the_same_energy_and_forces():
+    """A null virial pointer skips the virial kernels; energy and forces keep their bits."""
+    from alphanesgpu_amd import libstaf
+    pos, box, tp, type_map = load_frame_mbpol(np.float64)
+    m = libstaf.StafModel(os.path.join(GOLDEN, "model_double"), precision=1)
+    e, f, vir = m.compute(pos.reshape(-1, 3), box[0], type_map)
+    e2, f2, vir2 = m.compute(pos.reshape(-1, 3), box[0], type_map, want_virial=False)
+    assert vir2 is None and np.all(np.isfinite(vir))
+    assert e2 == e and np.array_equal(f2, f)
+    m.close()
+
+
+@pytest.mark.gpu
 def test_compute_return_codes():
     """Validation order and codes of libstaf/src/staf_api.cpp:196-337."""
     from alphanesgpu_amd import libstaf
