@@ -278,7 +278,8 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
   real* ang = A.angdescr + atom * na;
   int2* im3 = (int2*)A.intmap3b + atom * na;
   real2* d3 = (real2*)A.der3b + atom * 3 * na;
-  for (int nn = tid; nn < na; nn += blockDim.x) {
+  const int nend = A.zero_padding ? na : ntr;   // the reference writes nothing beyond an atom's triplets
+  for (int nn = tid; nn < nend; nn += blockDim.x) {
     if (nn < ntr) {
       int j, k;
       tri_decode(nn, m, j, k);
@@ -305,10 +306,10 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
       o.x = aj * (uk2 - cs * uj2) + hk * rj[6];
       o.y = ak * (uj2 - cs * uk2) + hj * rk[6];
       d3[2 * na + nn] = o;
-    } else {
+    } else if (A.zero_padding) {
       ang[nn] = 0;
       im3[nn] = make_int2(0, 0);
-      if (A.zero_padding) {
+      {
         real2 z;
         z.x = 0;
         z.y = 0;

@@ -83,8 +83,9 @@ int staf_op_construct_descriptors_light_f64(double radial_cutoff, int radial_buf
 
 /* Options of the descriptor op (apply to both precisions; call after construct).
  *   dist2_fma     0: dist2 = (x*x+y*y)+z*z uncontracted (default); 1: fma(z,z,fma(y,y,x*x))
- *   zero_padding  0: padded slots of der3b are left untouched like the reference (default);
- *                 1: they are written as 0.  (All other outputs are always fully written.) */
+ *   zero_padding  0: slots of angdescr, intmap3b and der3b beyond an atom's triplets are left untouched like the
+ *                    reference, which never writes any padding (default);
+ *                 1: they are written as 0.  (The nr-wide outputs are always fully written, padding as 0.) */
 int staf_op_descriptor_options(int dist2_fma, int zero_padding);
 
 /* Reads back {A, B, C, pow_alpha, pow_beta} computed by construct. */
