@@ -41,6 +41,8 @@ __device__ inline float r_pow(float x, float n) { return powf(x, n); }
 __device__ inline double r_pow(double x, double n) { return pow(x, n); }
 __device__ inline float r_rint(float x) { return rintf(x); }
 __device__ inline double r_rint(double x) { return rint(x); }
+__device__ inline float r_floor(float x) { return floorf(x); }
+__device__ inline double r_floor(double x) { return floor(x); }
 __device__ inline float r_fma(float a, float b, float c) { return fmaf(a, b, c); }
 __device__ inline double r_fma(double a, double b, double c) { return fma(a, b, c); }
 

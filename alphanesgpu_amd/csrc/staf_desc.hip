@@ -35,6 +35,11 @@ struct DescArgs {
   int skip_pbc;            // no minimum-image wrap (neighbours carry their periodic image)
   real Rc, Ra, Rs, cA, cB, cC, pa, pb;
   int dist2_fma, zero_padding;
+  // cell list of the frame (null: every atom is a candidate): atoms grouped by cell, see cell_build_kernel
+  const int* cell_dims;    // [nf, 4] cells along a, b, c (1: the axis is not divided), number of cells
+  const int* cell_start;   // [nf, CELL_MAX + 1]
+  const int* cell_atoms;   // [nf, N]
+  const int* cell_of;      // [nf, N] cell of every atom
   real* raddescr;
   real* angdescr;
   real* des3bsupp;
@@ -93,6 +98,121 @@ __device__ inline real norm_plain(const real* d) {
   return r_sqrt((d[0] * d[0] + d[1] * d[1]) + d[2] * d[2]);
 }
 
+// ---------------------------------------------------------------------------
+// Cell list for large frames (replaces the binning kernels of celle_gpu.cu.cc:11-101; the grid rule is this
+// library's own).  The box is cut into nx x ny x nz cells in fractional coordinates with every cell at least Rc
+// wide measured perpendicular to its faces, so that all atoms within Rc of a centre (minimum image by rounding the
+// fractional difference, as the scan does) lie in the centre's cell or one of its 26 neighbours.  An axis with
+// fewer than three such cells is not divided (its two neighbours would coincide).  One workgroup per frame.
+// The order of the atoms inside a cell is arbitrary: the neighbour search sorts what it finds.
+// ---------------------------------------------------------------------------
+constexpr int CELL_MAX = 4096;
+constexpr int CELL_THREADS = 1024;   // one workgroup bins a whole frame: as wide as a workgroup gets
+
+template <typename real>
+__global__ __launch_bounds__(CELL_THREADS) void cell_build_kernel(const real* __restrict__ pos, const real* __restrict__ boxes,
+                                                         int N, real Rc, int* __restrict__ cell_dims,
+                                                         int* __restrict__ cell_start, int* __restrict__ cell_atoms,
+                                                         int* __restrict__ cell_of) {
+  __shared__ int cnt[CELL_MAX];
+  __shared__ int dims[4];
+  __shared__ int carry;
+  const int tid = threadIdx.x, b = blockIdx.x;
+  real box[6], inv[6];
+#pragma unroll
+  for (int c = 0; c < 6; c++) box[c] = boxes[b * 6 + c];
+  inverse_box(box, inv);
+  if (tid == 0) {
+    // lattice vectors a = (b0,0,0), b = (b1,b3,0), c = (b2,b4,b5); heights = volume / area of the opposite face
+    const double ax = box[0], bx = box[1], by = box[3], cx = box[2], cy = box[4], cz = box[5];
+    const double vol = fabs(ax * by * cz);
+    const double bcx = by * cz, bcy = -bx * cz, bcz = bx * cy - by * cx;   // b x c
+    const double cax = 0.0, cay = cz * ax, caz = -cy * ax;                 // c x a
+    const double ha = vol / sqrt(bcx * bcx + bcy * bcy + bcz * bcz);
+    const double hb = vol / sqrt(cax * cax + cay * cay + caz * caz);
+    const double hc = vol / fabs(ax * by);
+    int n[3] = {(int)(ha / (double)Rc), (int)(hb / (double)Rc), (int)(hc / (double)Rc)};
+    for (int c = 0; c < 3; c++) n[c] = n[c] < 3 ? 1 : n[c];
+    while ((long long)n[0] * n[1] * n[2] > CELL_MAX) {   // coarser cells only widen the search
+      int big = n[0] >= n[1] && n[0] >= n[2] ? 0 : (n[1] >= n[2] ? 1 : 2);
+      n[big] = n[big] - 1 < 3 ? 1 : n[big] - 1;
+    }
+    dims[0] = n[0]; dims[1] = n[1]; dims[2] = n[2]; dims[3] = n[0] * n[1] * n[2];
+    for (int c = 0; c < 4; c++) cell_dims[b * 4 + c] = dims[c];
+    carry = 0;
+  }
+  __syncthreads();
+  const int nx = dims[0], ny = dims[1], nz = dims[2], ncell = dims[3];
+  for (int c = tid; c < ncell; c += CELL_THREADS) cnt[c] = 0;
+  __syncthreads();
+  const real* pf = pos + (size_t)b * N * 3;
+  int* of = cell_of + (size_t)b * N;
+  // eight atoms per thread at a time: their position reads are in flight together
+  for (int a0 = tid; a0 < N; a0 += 8 * CELL_THREADS) {
+    real px[8], py[8], pz[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      const int a = a0 + u * CELL_THREADS < N ? a0 + u * CELL_THREADS : N - 1;
+      px[u] = pf[3 * a]; py[u] = pf[3 * a + 1]; pz[u] = pf[3 * a + 2];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      const int a = a0 + u * CELL_THREADS;
+      if (a >= N) break;
+      real s[3];
+      to_frac(inv, px[u], py[u], pz[u], s);
+      int c3[3];
+      const int nn[3] = {nx, ny, nz};
+#pragma unroll
+      for (int c = 0; c < 3; c++) {
+        const real f = s[c] - r_floor(s[c]);   // [0, 1]
+        int q = (int)(f * (real)nn[c]);
+        c3[c] = q < 0 ? 0 : (q >= nn[c] ? nn[c] - 1 : q);
+      }
+      const int cell = (c3[0] * ny + c3[1]) * nz + c3[2];
+      of[a] = cell;
+      atomicAdd(&cnt[cell], 1);
+    }
+  }
+  __syncthreads();
+  // exclusive prefix over the cells, one block of threads at a time
+  int* start = cell_start + (size_t)b * (CELL_MAX + 1);
+  for (int c0 = 0; c0 < ncell; c0 += CELL_THREADS) {
+    const int c = c0 + tid;
+    const int v = c < ncell ? cnt[c] : 0;
+    // inclusive scan of v over the threads through LDS
+    __shared__ int sc[CELL_THREADS];
+    sc[tid] = v;
+    __syncthreads();
+    for (int o = 1; o < CELL_THREADS; o <<= 1) {
+      const int t = tid >= o ? sc[tid - o] : 0;
+      __syncthreads();
+      sc[tid] += t;
+      __syncthreads();
+    }
+    const int base = carry;
+    if (c < ncell) {
+      start[c] = base + sc[tid] - v;
+      cnt[c] = base + sc[tid] - v;   // becomes the fill cursor
+    }
+    __syncthreads();
+    if (tid == CELL_THREADS - 1) carry = base + sc[CELL_THREADS - 1];
+    __syncthreads();
+  }
+  if (tid == 0) start[ncell] = carry;
+  int* atoms = cell_atoms + (size_t)b * N;
+  for (int a0 = tid; a0 < N; a0 += 8 * CELL_THREADS) {
+    int cl[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) cl[u] = of[a0 + u * CELL_THREADS < N ? a0 + u * CELL_THREADS : N - 1];
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      const int a = a0 + u * CELL_THREADS;
+      if (a < N) atoms[atomicAdd(&cnt[cl[u]], 1)] = a;
+    }
+  }
+}
+
 template <typename real>
 __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
   using real2 = typename Vec2<real>::type;
@@ -129,7 +249,55 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
 
   // 1. candidate scan -- or the caller's list (already cut off and sorted by distance)
   const bool injected = A.inj_howmany != nullptr;
-  if (!injected) {
+  if (!injected && A.cell_start) {
+    // candidates = the atoms of the centre's cell and its neighbours (every atom appears once: an axis has one
+    // cell or at least three)
+    __shared__ int nb_start[27], nb_off[28];
+    const int* dm = A.cell_dims + b * 4;
+    const int nx = dm[0], ny = dm[1], nz = dm[2];
+    const int* cstart = A.cell_start + (size_t)b * (CELL_MAX + 1);
+    const int* catoms = A.cell_atoms + (size_t)b * N;
+    if (tid < 27) {
+      const int ci = A.cell_of[(size_t)b * N + i];
+      const int cz = ci % nz, cy = (ci / nz) % ny, cx = ci / (nz * ny);
+      const int dx = tid / 9 - 1, dy = (tid / 3) % 3 - 1, dz = tid % 3 - 1;
+      int cnt = 0, st0 = 0;
+      if ((nx > 1 || dx == 0) && (ny > 1 || dy == 0) && (nz > 1 || dz == 0)) {
+        const int x = (cx + dx + nx) % nx, y = (cy + dy + ny) % ny, z = (cz + dz + nz) % nz;
+        const int c = (x * ny + y) * nz + z;
+        st0 = cstart[c];
+        cnt = cstart[c + 1] - st0;
+      }
+      nb_start[tid] = st0;
+      nb_off[tid + 1] = cnt;
+    }
+    __syncthreads();
+    if (tid == 0) {
+      nb_off[0] = 0;
+      for (int c = 0; c < 27; c++) nb_off[c + 1] += nb_off[c];
+    }
+    __syncthreads();
+    const int total = nb_off[27];
+    for (int q = tid; q < total; q += 256) {
+      int c = 0;
+      while (q >= nb_off[c + 1]) c++;
+      const int j = catoms[nb_start[c] + q - nb_off[c]];
+      if (j == i) continue;
+      real sj[3], d[3];
+      to_frac(inv, pf[3 * j], pf[3 * j + 1], pf[3 * j + 2], sj);
+      const real d2 = mic_delta(box, sj, si, A.dist2_fma, A.skip_pbc, d);
+      if (d2 < rc2) {
+        const int slot = atomicAdd(&cnt_all, 1);
+        if (slot < nr) {
+          c_j[slot] = j;
+          c_d2[slot] = d2;
+          c_d[3 * slot] = d[0];
+          c_d[3 * slot + 1] = d[1];
+          c_d[3 * slot + 2] = d[2];
+        }
+      }
+    }
+  } else if (!injected) {
     // the position reads of four candidates per thread are issued together
     for (int j0 = tid; j0 < A.Npos; j0 += 4 * 256) {
       real px[4], py[4], pz[4];
@@ -329,6 +497,7 @@ size_t desc_lds_bytes(int nr) {
 // ---- host side -------------------------------------------------------------
 
 static std::mutex g_cfg_mu;
+static int g_cell_threshold = 2048;   // frames of at least this many atoms search through a cell list
 static DescConfig<float> g_cfg_f;
 static DescConfig<double> g_cfg_d;
 template <typename real> DescConfig<real>& cfg();
@@ -415,6 +584,23 @@ int desc_launch(const DescConfig<real>& c, const real* pos, const real* box, int
   A.raddescr = raddescr; A.angdescr = angdescr; A.des3bsupp = des3bsupp; A.intmap2b = intmap2b;
   A.intmap3b = intmap3b; A.der2b = der2b; A.der3b = der3b; A.der3bsupp = der3bsupp; A.numtriplet = numtriplet;
   A.status = st->status_d;
+  A.cell_dims = A.cell_start = A.cell_atoms = A.cell_of = nullptr;
+  const int cell_from = g_cell_threshold;
+  if (!inj_howmany && cell_from > 0 && N >= cell_from) {
+    const size_t ints = (size_t)nf * (4 + (CELL_MAX + 1) + 2 * (size_t)N);
+    int* w = (int*)scratch_reserve(st, stream, ints * sizeof(int));
+    if (!w) return STAF_E_HIP;
+    int* dims = w;
+    int* start = dims + (size_t)nf * 4;
+    int* atoms = start + (size_t)nf * (CELL_MAX + 1);
+    int* of = atoms + (size_t)nf * N;
+    {
+      KernelTimer kt_("cell_build_kernel", stream);
+      hipLaunchKernelGGL(cell_build_kernel<real>, dim3(nf), dim3(CELL_THREADS), 0, stream, pos, box, N, c.Rc, dims, start,
+                         atoms, of);
+    }
+    A.cell_dims = dims; A.cell_start = start; A.cell_atoms = atoms; A.cell_of = of;
+  }
   size_t lds = desc_lds_bytes<real>(c.nr);
   if (lds > 60 * 1024) return STAF_E_LIMIT;
   {
@@ -466,6 +652,12 @@ int staf_op_construct_descriptors_light_f32(float rc, int nr, int na, int numpar
 int staf_op_construct_descriptors_light_f64(double rc, int nr, int na, int numpar, double rs, double ra,
                                             int max_batch, const char* path) {
   return staf::construct<double>(rc, nr, na, numpar, rs, ra, max_batch, path);
+}
+
+int staf_op_descriptor_cell_threshold(int n_atoms) {
+  std::lock_guard<std::mutex> lock(staf::g_cfg_mu);
+  staf::g_cell_threshold = n_atoms;
+  return STAF_OK;
 }
 
 int staf_op_descriptor_options(int dist2_fma, int zero_padding) {

@@ -270,9 +270,15 @@ def main():
         step()
     ops.poll_status()
     if not args.no_graph:
+        # the library keeps its scratch per stream and cannot grow it while a stream is captured: the step runs
+        # once eagerly on the very streams the capture uses
+        cap = torch.cuda.Stream()
+        with torch.cuda.stream(cap):
+            step()
+        ops.poll_status()
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
+        with torch.cuda.graph(graph, stream=cap):
             graph_out = step()
         run = graph.replay
     for _ in range(args.warmup):

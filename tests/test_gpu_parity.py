@@ -345,6 +345,41 @@ def test_angular_buffer_smaller_than_triplet_count(oracle, dtype):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_cell_list_gives_the_same_descriptors(dtype):
+    """Large frames find their neighbours through a cell list, small ones test every atom: every output of the
+    descriptor op must have the same bits either way.  768 atoms (4 x 4 x 4 cells at Rc = 4.5), an orthorhombic and
+    a sheared box, some atoms moved by whole lattice vectors (positions outside the box)."""
+    import torch
+    from alphanesgpu_amd import ops, synth
+    b = _synth("water768_f32")
+    N, nf = b["N"], 2
+    pos0 = b["pos"][:nf].astype(dtype).reshape(nf, N, 3)
+    L = float(b["box"][0][0])
+    tdt = torch.float64 if dtype == np.float64 else torch.float32
+    rng = np.random.default_rng(5)
+    try:
+        for box6 in ([L, 0, 0, L, 0, L], [L, 0.3 * L, -0.2 * L, L, 0.25 * L, L]):
+            a, bv, c = np.array([box6[0], 0, 0]), np.array([box6[1], box6[3], 0]), np.array([box6[2], box6[4], box6[5]])
+            pos = pos0.copy()
+            k = rng.integers(-2, 3, size=(nf, N, 3))
+            moved = rng.random((nf, N)) < 0.2
+            pos += (moved[..., None] * (k[..., :1] * a + k[..., 1:2] * bv + k[..., 2:] * c)).astype(dtype)
+            box = np.tile(np.array(box6, dtype), (nf, 1))
+            tp, tb = torch.as_tensor(pos.reshape(nf, -1)).cuda(), torch.as_tensor(box).cuda()
+            ops.construct_descriptors_light(synth.RC, 80, NA, N, tb, synth.RS, synth.RA, nf, dtype=tdt)
+            ops.descriptor_options(dist2_fma=False, zero_padding=True)
+            ops.descriptor_cell_threshold(0)
+            every = [x.clone() for x in ops.compute_descriptors_light(tp, tb)]
+            ops.descriptor_cell_threshold(1)
+            cells = ops.compute_descriptors_light(tp, tb)
+            assert int(every[3][..., 0].min()) > 10      # intmap2b counts: a real neighbourhood everywhere
+            for x, y in zip(every, cells):
+                assert torch.equal(x, y)
+    finally:
+        ops.descriptor_cell_threshold(2048)
+
+
 def test_hip_graph_replay_with_two_streams_matches_eager():
     """The whole op sequence captured once in a HIP graph, the two per-species chains forked onto their own streams
     (per-stream scratch inside the library): every replay, with eager calls and synchronisations in between, gives
