@@ -376,6 +376,24 @@ def test_cell_list_gives_the_same_descriptors(dtype):
             assert int(every[3][..., 0].min()) > 10      # intmap2b counts: a real neighbourhood everywhere
             for x, y in zip(every, cells):
                 assert torch.equal(x, y)
+        # a box too small to be divided (9.86 / 4.5 < 3: one cell per axis) and one divided along one axis only
+        b96 = _synth("water96")
+        p96 = b96["pos"][:1].astype(dtype)
+        L9 = float(b96["box"][0][0])
+        for box6, reps in (([L9, 0, 0, L9, 0, L9], 1), ([L9, 0, 0, L9, 0, 2 * L9], 2)):
+            pos = p96.reshape(1, -1, 3)
+            if reps == 2:
+                pos = np.concatenate([pos, pos + np.array([0, 0, L9], dtype)], axis=1)
+            n96 = pos.shape[1]
+            box = np.array([box6], dtype)
+            tp, tb = torch.as_tensor(np.ascontiguousarray(pos.reshape(1, -1))).cuda(), torch.as_tensor(box).cuda()
+            ops.construct_descriptors_light(synth.RC, 80, NA, n96, tb, synth.RS, synth.RA, 1, dtype=tdt)
+            ops.descriptor_cell_threshold(0)
+            every = [x.clone() for x in ops.compute_descriptors_light(tp, tb)]
+            ops.descriptor_cell_threshold(1)
+            cells = ops.compute_descriptors_light(tp, tb)
+            for x, y in zip(every, cells):
+                assert torch.equal(x, y)
     finally:
         ops.descriptor_cell_threshold(2048)
 
