@@ -103,19 +103,27 @@ def cpu_baseline(batch, params, up, mode, nr, na, max_frames=2, threads=16):
                                    type_map, tipos, k, c(d["numtriplet"]))
 
     nfs = min(max_frames, batch["nf"])
-    t0 = time.perf_counter()
-    frames(0, nfs)
-    el = time.perf_counter() - t0
+    reps = 3 if mode == "full_step" else 5
+
+    def median_time(fn):
+        fn()   # warm-up
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return float(np.median(ts))
+
+    el = median_time(lambda: frames(0, nfs))
     threads = max(1, min(threads, os.cpu_count() or 1))
     nfr = batch["nf"]
-    t0 = time.perf_counter()
     with ThreadPoolExecutor(threads) as ex:
-        list(ex.map(lambda i: frames(i % nfr, i % nfr + 1), range(threads)))
-    elm = time.perf_counter() - t0
+        elm = median_time(lambda: list(ex.map(lambda i: frames(i % nfr, i % nfr + 1), range(threads))))
     return dict(value=nfs / el, unit="frames/s", cores=1, kind="port",
-                sample=f"{nfs} frame(s) of the same batch, same ops, scalar C++ oracle (-O2 -ffp-contract=off), 1 thread",
+                sample=f"{nfs} frame(s) of the same batch, same ops, scalar C++ oracle (-O2 -ffp-contract=off), 1 thread, "
+                       f"median of {reps} after a warm-up",
                 multicore=dict(value=threads / elm, unit="frames/s", cores=threads,
-                               sample=f"{threads} frames, one per thread, same oracle"))
+                               sample=f"{threads} frames, one per thread, same oracle, median of {reps}"))
 
 
 def main():
@@ -334,6 +342,15 @@ def main():
             kern[name] = dict(ms_per_step=ms / nprof, launches_per_step=n // nprof, avg_launch_ms=ms / n)
     per_step = {k: op_ms[k] * calls[k] for k in op_ms}
     step_bytes = sum(ab[k] for k in kern if k in ab)
+    # the same byte count over the active slots only (pairs and triplets that exist), reported beside the padded one
+    d_ = ops.compute_descriptors_light(pos, box, out=dbuf)
+    torch.cuda.synchronize()
+    cnt2 = d_[3][..., 0].clamp(max=nr).double()
+    mtr = d_[8].double()
+    nr_act = float(cnt2.mean())
+    na_act = float(torch.clamp(mtr * (mtr - 1) / 2, max=na).mean())
+    ab_act = algorithmic_bytes(N, tipos, nr_act, na_act, Ar, Aa, nt, s)
+    step_bytes_act = sum(ab_act[k] for k in kern if k in ab_act)
     # the kernel the step spends most of its time in, priced against HBM with the bytes its op signature moves
     dom = max((k for k in kern if k in ab), key=lambda k: kern[k]["ms_per_step"])
     dom_bytes_per_launch = ab[dom] * nf / kern[dom]["launches_per_step"]
@@ -366,6 +383,8 @@ def main():
         "kernel_ms_per_step": {k: v["ms_per_step"] for k, v in kern.items()},
         "whole_step_hbm_frac": step_bytes * nf / (el / args.steps) / 1e9 / HBM_PEAK_GBS,
         "whole_step_frac_of_measured_copy": step_bytes * nf / (el / args.steps) / 1e9 / copy_gbs,
+        "whole_step_hbm_frac_active_slots": step_bytes_act * nf / (el / args.steps) / 1e9 / HBM_PEAK_GBS,
+        "active_slots": {"pairs_per_atom": nr_act, "triplets_per_atom": na_act},
         "op_ms_per_step": per_step,
         "ms_per_frame": el / args.steps * 1e3 / nf,
         "single_stream": {"value": nf * args.steps / el1, "ms_per_step": el1 / args.steps * 1e3},
