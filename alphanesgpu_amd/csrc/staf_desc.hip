@@ -233,6 +233,7 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
   const int tid = threadIdx.x;
   const int b = blockIdx.x / N;
   const int i = blockIdx.x - b * N;
+  PHASE_CLOCK_BEGIN();
   if (tid == 0) { cnt_all = 0; cnt_ang = 0; }
   for (int e = tid; e < nr; e += blockDim.x) s_rank[e] = 0;
   if (tid < 6) sbox[tid] = A.box[b * 6 + tid];
@@ -342,6 +343,7 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
     }
   }
   __syncthreads();
+  PHASE_MARK(0);
   const int hm = cnt_all;
   const int n = hm < nr ? hm : nr;
   if (hm > nr && tid == 0) atomicOr(A.status, 1);
@@ -371,6 +373,7 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
     }
     __syncthreads();
   }
+  PHASE_MARK(1);
   // 3. radial fill
   const bool same_cut = A.Ra == A.Rc;
   const bool std_pow = A.pa == real(1) && A.pb == real(-30);   // the exponents fill_repulsion uses
@@ -433,7 +436,9 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
       }
     }
   }
+  PHASE_MARK(2);
   __syncthreads();
+  PHASE_MARK(3);
   const int m = cnt_ang;
   if (tid == 0) {
     im[0] = hm;
@@ -446,6 +451,9 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
   real* ang = A.angdescr + atom * na;
   int2* im3 = (int2*)A.intmap3b + atom * na;
   real2* d3 = (real2*)A.der3b + atom * 3 * na;
+  // Consecutive lanes take consecutive triplets: the stores of a wave are whole cache lines.  (Four consecutive
+  // triplets per thread with one index decode was measured: fewer instructions, but the strided stores made the
+  // kernel a third slower.)
   const int nend = A.zero_padding ? na : ntr;   // the reference writes nothing beyond an atom's triplets
   for (int nn = tid; nn < nend; nn += blockDim.x) {
     if (nn < ntr) {
@@ -487,6 +495,8 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
       }
     }
   }
+  PHASE_MARK(4);
+  PHASE_CLOCK_END();
 }
 
 template <typename real>
@@ -642,6 +652,7 @@ static int compute(const real* pos, const real* box, int nf, int N, real* raddes
 }
 
 }  // namespace staf
+PHASE_CLOCK_READER(staf_debug_phase_clock_desc)
 
 extern "C" {
 
