@@ -17,9 +17,12 @@
 //     so every thread accumulates its own channel privately with its
 //     parameters in registers, and table reads are contiguous in the channel.
 //     The four subsets of a wave are combined with two cross-lane adds and
-//     added into per-wave accumulators in LDS; the waves are summed once per
-//     atom in a fixed order (bit-reproducible).  No barrier per class for the
-//     reduction.
+//     added into per-wave fingerprint accumulators in LDS, which are summed once
+//     per atom in a fixed order.  The parameter-gradient sums of a pass go through
+//     a small per-wave exchange buffer and are added, waves in ascending order, to
+//     the workgroup's single accumulator set by the first 16 threads after the next
+//     barrier the kernel needs anyway (bit-reproducible, no barrier of its own; one
+//     set instead of one per wave keeps the LDS footprint at four workgroups per CU).
 //   * triplets are staged in LDS in blocks (table row offsets, T, and for
 //     MODE 2 the contraction U of der3b with dL/dF), so tensors laid out by
 //     the storage index nn are read exactly once.
@@ -33,7 +36,13 @@ constexpr int TRI_WAVES = TRI_BLOCK / WAVE;
 constexpr int TRI_CAP = 16;    // channels tabulated per pass = lanes of a subset
 constexpr int TRI_CAPP = TRI_CAP + 1;   // table row pitch: the entry after a row's channels holds (D, V) of its slot
 constexpr int TRI_SUBS = TRI_BLOCK / TRI_CAP;
-constexpr int TRI_QB = 512;    // triplets staged per block
+template <typename real, int MODE>
+struct TriCfg {
+  static constexpr int QB = 512;   // triplets staged per block
+  // waves per SIMD the register allocation is held to: the double-precision force gradient would otherwise come
+  // out two registers above the 128 that let four workgroups share a CU
+  static constexpr int MIN_WAVES = (MODE == 2 && sizeof(real) == 8) ? 4 : 1;
+};
 constexpr int TRI_GRID_MAX = 2048;  // workgroups of the persistent gradient modes (one partial row each)
 
 // Exponential of the hot loops.
@@ -107,29 +116,32 @@ struct TriArgs {
 template <typename real, int MODE>
 struct TriLds {
   static constexpr int NV = (MODE == 0) ? 1 : (MODE == 1 ? 3 : 4);
+  static constexpr int QB = TriCfg<real, MODE>::QB;
   __host__ __device__ static size_t n_reals(int nr, int Aa, int nt) {
     const int nsig = 2 * nt - 1;
     size_t r = (size_t)nr * TRI_CAPP * 2;                   // pair tables (real2 per (row, channel)), + (D, V) per row
     r += nr;                                                // sD
     r += Aa;                                                // sP
     r += (size_t)TRI_WAVES * Aa;                            // per-wave channel sums
-    if (MODE != 0) r += (size_t)TRI_WAVES * nsig * Aa * 3;  // per-wave parameter-gradient sums
+    if (MODE != 0) r += (size_t)nsig * Aa * 3;              // parameter-gradient sums of the workgroup
+    if (MODE != 0) r += (size_t)TRI_WAVES * TRI_CAP * 3;    // exchange buffer of a pass
     if (MODE == 2) r += (size_t)4 * nr;                     // sV, sQ
-    r += (size_t)TRI_QB * (MODE == 2 ? 2 : 1);              // staged T (and U)
+    r += (size_t)QB * (MODE == 2 ? 2 : 1);                  // staged T (and U)
     return r;
   }
   __host__ __device__ static size_t bytes(int nr, int Aa, int nt) {
     size_t b = chan_table_bytes<real>(2 * nt - 1, Aa) + n_reals(nr, Aa, nt) * sizeof(real);
-    b += (size_t)(2 * TRI_QB + 2 * nr + NT_MAX + 1) * sizeof(int);
+    b += (size_t)2 * QB * sizeof(unsigned short) + (size_t)(2 * nr + NT_MAX + 1) * sizeof(int);
     return (b + 15) & ~(size_t)15;
   }
 };
 
 template <typename real, int MODE>
-__global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) {
+__global__ __launch_bounds__(TRI_BLOCK, (TriCfg<real, MODE>::MIN_WAVES)) void tri_reduce_kernel(TriArgs<real> A) {
   using real2 = typename Vec2<real>::type;
   using HE = HotExp<real>;
   constexpr int NV = TriLds<real, MODE>::NV;
+  constexpr int TRI_QB = TriCfg<real, MODE>::QB;
   extern __shared__ __align__(16) unsigned char smem[];
   const int nr = A.nr, na = A.na, Aa = A.Aa, nt = A.nt;
   const int nsig = 2 * nt - 1;
@@ -141,15 +153,16 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
   real* sD = rp; rp += nr;
   real* sP = rp; rp += Aa;
   real* outw = rp; rp += (size_t)TRI_WAVES * Aa;
-  real* accw = rp; if (MODE != 0) rp += (size_t)TRI_WAVES * nacc;
+  real* accw = rp; if (MODE != 0) rp += (size_t)nacc;
+  real* xch = rp; if (MODE != 0) rp += (size_t)TRI_WAVES * TRI_CAP * 3;
   real* sV = rp;
   real* sQ = rp + nr;
   if (MODE == 2) rp += (size_t)4 * nr;
   real* sT = rp; rp += TRI_QB;
   real* sU = rp; if (MODE == 2) rp += TRI_QB;
-  int* offA = (int*)rp;          // [TRI_QB] first table row of the staged triplet, times TRI_CAPP
-  int* offB = offA + TRI_QB;     // [TRI_QB] second
-  int* lst = offB + TRI_QB;
+  unsigned short* offA = (unsigned short*)rp;   // [TRI_QB] first table row of the staged triplet, times TRI_CAPP
+  unsigned short* offB = offA + TRI_QB;         // [TRI_QB] second
+  int* lst = (int*)(offB + TRI_QB);
   int* stp = lst + nr;
   int* off = stp + nr;
 
@@ -158,14 +171,30 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
   const int ia = tid & (TRI_CAP - 1), sub = tid / TRI_CAP;
   tab.build(A.alpha3b, A.emb3b);
   if (MODE != 0)
-    for (int q = tid; q < TRI_WAVES * nacc; q += TRI_BLOCK) accw[q] = 0;
+    for (int q = tid; q < nacc; q += TRI_BLOCK) accw[q] = 0;
   int shift = 0;
   if (MODE == 2) {
     const int at = A.actual_type[0];
     for (int y = 0; y < at; y++) shift += A.tipos[y];
   }
   real* my_out = outw + wave * Aa;
-  real* my_acc = accw + (size_t)wave * nacc;
+  real* my_xch = xch + (size_t)wave * TRI_CAP * 3;
+  // Parameter-gradient sums of the last pass: thread ia < 16 of the workgroup adds the four waves' values of its
+  // channel to accumulator row `pending` (-1: nothing to add).  Called right after a barrier that follows the pass
+  // and before the next one, so that the exchange buffer is complete and not yet rewritten.
+  int pending = -1;
+  auto flush_pass = [&]() {
+    if (MODE != 0 && tid < TRI_CAP && pending >= 0) {
+#pragma unroll
+      for (int v = 0; v < 3; v++) {
+        real s = xch[ia * 3 + v];
+#pragma unroll
+        for (int w = 1; w < TRI_WAVES; w++) s += xch[(w * TRI_CAP + ia) * 3 + v];
+        accw[pending + v] += s;
+      }
+    }
+    pending = -1;
+  };
   __syncthreads();
 
   const int total = A.nf * A.Nl;
@@ -233,7 +262,10 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
           real a1 = 0, a2 = 0, be = 0;
           if (chan) { a1 = tab.a1[pb + c0 + ia]; a2 = tab.a2[pb + c0 + ia]; be = tab.be[pb + c0 + ia]; }
           const real a1s = HE::scale(a1), a2s = HE::scale(a2), bes = HE::scale(be);
-          if (!first) __syncthreads();   // tables and staged block of the previous pass fully consumed
+          if (!first) {
+            __syncthreads();   // tables and staged block of the previous pass fully consumed
+            flush_pass();
+          }
           first = false;
           // ---- tables of the class: E[row][ia] = (exp(a1 D), exp(a2 D)), D (and V) by row
           for (int row = sub; row < nrows; row += TRI_SUBS) {
@@ -278,8 +310,8 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
               const int j = s1 < s2 ? s1 : s2, k = s1 < s2 ? s2 : s1;
               const int nn = tri_rowstart(j, m) + k - j - 1;
               const bool ok = nn < na;
-              offA[qq] = x * TRI_CAPP;
-              offB[qq] = (rowB0 + y) * TRI_CAPP;
+              offA[qq] = (unsigned short)(x * TRI_CAPP);
+              offB[qq] = (unsigned short)((rowB0 + y) * TRI_CAPP);
               real T = 0;
               if (ok) T = Trow[nn];
               sT[qq] = T;
@@ -366,18 +398,20 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
             } else if constexpr (MODE == 1) {
               const real f = c3h * sP[a];
 #pragma unroll
-              for (int v = 0; v < 3; v++) my_acc[(sg * Aa + a) * 3 + v] += acc[v] * f;
+              for (int v = 0; v < 3; v++) my_xch[ia * 3 + v] = acc[v] * f;
             } else {
               my_out[a] += acc[0] * c3h;
               const real f = c3h * sP[a];
 #pragma unroll
-              for (int v = 0; v < 3; v++) my_acc[(sg * Aa + a) * 3 + v] += acc[v + 1] * f;
+              for (int v = 0; v < 3; v++) my_xch[ia * 3 + v] = acc[v + 1] * f;
             }
+            if (MODE != 0) pending = (sg * Aa + a) * 3;
           }
         }
       }
     }
     __syncthreads();
+    flush_pass();
     if (MODE != 1)
       for (int a = tid; a < Aa; a += TRI_BLOCK) {
         real s = 0;
@@ -388,12 +422,7 @@ __global__ __launch_bounds__(TRI_BLOCK) void tri_reduce_kernel(TriArgs<real> A) 
     __syncthreads();
   }
   if (MODE != 0) {
-    for (int q = tid; q < nacc; q += TRI_BLOCK) {
-      real s = 0;
-#pragma unroll
-      for (int w = 0; w < TRI_WAVES; w++) s += accw[(size_t)w * nacc + q];
-      A.partial[(size_t)blockIdx.x * nacc + q] = s;
-    }
+    for (int q = tid; q < nacc; q += TRI_BLOCK) A.partial[(size_t)blockIdx.x * nacc + q] = accw[q];
   }
 }
 
