@@ -31,7 +31,7 @@ TRAFFIC = {
     # factors from the 1 GiB device copies of this script in the same runs
     # (profiles/force3_kernel_water768_f32_hbm_counters.txt, profiles/gradforce3_kernel_water768_f64_hbm_counters.txt)
     ("force3_kernel", "water768_f32"): 38.1e6,
-    ("gradforce3_kernel", "water768_f64"): 78.9e6,
+    ("gradforce3_kernel", "water768_f64"): 95.2e6,
 }
 
 
