@@ -134,3 +134,24 @@ def test_autograd_through_the_layers_matches_finite_differences_of_the_oracle(or
     # finite differences with h = 1e-5 on a smooth function of O(1) curvature: ~1e-9 absolute
     assert np.all(np.abs(got - want) <= 2e-7 * scale), (got, want)
     assert np.count_nonzero(np.abs(want) > 1e-6 * scale) >= len(want) - 4
+
+
+def test_layer_classes_have_the_reference_signatures():
+    """Names and argument lists of STAF/source_routine/*.py (descriptor_builder.py:16,31, physics_layer_mod.py:10,33,
+    55,59, force_layer_mod.py:9,25-27,78,90-92)."""
+    import inspect
+    from alphanesgpu_amd import layers
+    sig = lambda f: [p for p in inspect.signature(f).parameters if p != "self"]
+    assert sig(layers.descriptor_layer.__init__)[:8] == ["rc", "rad_buff", "rc_ang", "ang_buff", "N", "box_example",
+                                                         "Rs", "maxbatch"]
+    assert sig(layers.descriptor_layer.forward) == ["pos", "box"]
+    assert sig(layers.physics_layer.__init__) == ["init_alpha2b", "init_alpha3b", "initial_type_emb"]
+    assert sig(layers.physics_layer.forward) == ["x2b", "x3bsupp", "intmap2b", "x3b", "intmap3b", "numtriplet",
+                                                 "type_map"]
+    assert sig(layers.lognorm_layer.__init__) == ["mu"] and sig(layers.lognorm_layer.forward) == ["restot"]
+    call = ["net_der_r", "x2b", "intder2b", "int2b", "alpha2b", "net_der_a", "x3b", "x3bsupp", "intder3b",
+            "intder3bsupp", "int3b", "numtriplet", "alpha3b", "type_emb_2b", "type_emb_3b", "type_map", "tipos",
+            "type_now"]
+    assert sig(layers.force_layer.__init__) == ["radbuff", "angbuff"] and sig(layers.force_layer.forward) == call
+    assert sig(layers.force_virial_layer.__init__) == ["radbuff", "angbuff", "with_grad"]
+    assert sig(layers.force_virial_layer.forward) == call + ["pos", "box"]
