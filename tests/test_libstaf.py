@@ -282,3 +282,48 @@ def test_compute_return_codes():
     m.close()
     with pytest.raises(RuntimeError):
         libstaf.StafModel("/nonexistent_model_dir")
+
+
+# ----------------------------------------------------------------------------- a caller written in C
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+MD_STEP = os.path.join(ROOT, "tests", "c_consumer", "md_step")
+
+
+def test_headers_are_plain_c_and_the_c_caller_is_built():
+    """include/*.h compile as C99 and as C++11 with -pedantic (they are what a C or C++ host includes), and the C
+    caller built against include/staf.h alone links the library and reports a usage error without touching a GPU."""
+    import subprocess
+    for h in ("staf.h", "staf_mlp.h", "staf_ops.h"):
+        path = os.path.join(ROOT, "include", h)
+        for cc, std, lang in (("gcc", "-std=c99", "c"), ("g++", "-std=c++11", "c++")):
+            r = subprocess.run([cc, std, "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-x", lang, path],
+                               capture_output=True, text=True)
+            assert r.returncode == 0, (h, cc, r.stderr)
+    assert os.path.exists(MD_STEP), "run __graft_entry__.build() first"
+    r = subprocess.run([MD_STEP], capture_output=True, text=True)
+    assert r.returncode == 100 and "usage" in r.stderr
+
+
+@pytest.mark.gpu
+def test_c_caller_reproduces_recorded_energy():
+    """The plain-C program (tests/c_consumer/md_step.c: staf_load, staf_compute with the library's own neighbour
+    list, staf_free) on the reference's 768-atom frame with its float32 model: E and rms(F) recorded by the
+    reference (test/test-lammps-STAF-inference-STAF-comp/results/frames.csv:2); a second step on rigidly shifted
+    coordinates gives the same energy and forces to rounding."""
+    import subprocess
+    d = os.path.join(GOLDEN, "frame_mbpol")
+    r = subprocess.run([MD_STEP, os.path.join(GOLDEN, "model_float"), os.path.join(d, "pos_0"),
+                        os.path.join(d, "box_0"), os.path.join(d, "type.dat"), "0", "2"],
+                       capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, (r.stdout, r.stderr)
+    lines = [l.split() for l in r.stdout.splitlines() if l.startswith("step")]
+    assert len(lines) == 2 and all(l[3] == "0" for l in lines)
+    e = [float(l[5]) for l in lines]
+    rms = [float(l[7]) for l in lines]
+    ka = KNOWN["frame0_model_float"]
+    assert abs(e[0] - ka["E_lammps"]) < 1.5e-4 and abs(rms[0] - ka["rms_F_python"]) < 5e-6
+    # float32 network: the shifted coordinates round differently (same bounds as the permutation check above)
+    assert abs(e[1] - e[0]) < 1e-5 * abs(e[0]) and abs(rms[1] - rms[0]) < 2e-5
+    vir = [float(x) for x in lines[0][9:15]]
+    assert vir[3] == vir[4] == vir[5] == 0.0 and all(v != 0.0 for v in vir[:3])
