@@ -62,3 +62,19 @@ def test_construct_coefficients_and_cutoff_curve(tmp_path, oracle):
         ulp6 = lambda v: 10.0 ** (np.floor(np.log10(np.maximum(np.abs(v), 1e-300))) - 5)
         assert mine.shape == (1000, 2)
         assert np.all(np.abs(mine - ref) <= 1.6 * ulp6(ref) + 1e-12)
+
+
+def test_library_depends_on_the_hip_runtime_only():
+    """The boundary carries no framework types and the library no framework dependency: its dynamic section names
+    the HIP runtime and the C/C++ runtimes, nothing of torch (a C or C++ host links it as it is), and it exports no
+    oracle symbol."""
+    import subprocess
+    from alphanesgpu_amd import _lib
+    dyn = subprocess.run(["readelf", "-d", _lib.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    needed = re.findall(r"\(NEEDED\)\s+Shared library: \[([^\]]+)\]", dyn)
+    assert any(n.startswith("libamdhip64") for n in needed)
+    allowed = ("libamdhip64", "libstdc++", "libm.", "libgcc_s", "libc.", "ld-linux", "libpthread", "libdl", "librt")
+    assert all(n.startswith(allowed) for n in needed), needed
+    syms = subprocess.run(["nm", "-D", "--defined-only", _lib.LIB_PATH], capture_output=True, text=True,
+                          check=True).stdout
+    assert "oracle" not in syms.lower()
