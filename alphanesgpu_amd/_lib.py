@@ -38,6 +38,13 @@ def lib():
             raise RuntimeError(
                 f"{LIB_PATH} not found: build it with `python -m alphanesgpu_amd.build` "
                 "(there is no CPU or PyTorch fallback for the STAF kernels)")
+        # One process holds one HIP runtime.  PyTorch ships its own copy of it under the same library name: when
+        # PyTorch is going to be used in this process its copy has to be the one loaded first (this library then
+        # binds to it); loaded in the other order, PyTorch finds no GPU.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         _lib = C.CDLL(LIB_PATH)
         _lib.staf_ops_version.restype = C.c_char_p
     return _lib

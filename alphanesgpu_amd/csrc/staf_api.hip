@@ -44,6 +44,29 @@ struct DevBuf {
   }
 };
 
+// Pinned host staging (allocated pinned, never registered): one block for everything a call sends, one for what it
+// brings back, so that a call makes one copy each way.
+template <typename T>
+struct PinBuf {
+  T* p = nullptr;
+  size_t n = 0;
+  bool reserve(size_t want) {
+    if (want <= n) return true;
+    if (p) (void)hipHostFree(p);
+    p = nullptr;
+    n = 0;
+    want += want / 4;
+    if (hipHostMalloc((void**)&p, want * sizeof(T), hipHostMallocDefault) != hipSuccess) return false;
+    n = want;
+    return true;
+  }
+  void release() {
+    if (p) (void)hipHostFree(p);
+    p = nullptr;
+    n = 0;
+  }
+};
+
 __global__ void add_into_kernel(double* dst, const double* src, int n) {
   const int e = blockIdx.x * blockDim.x + threadIdx.x;
   if (e < n) dst[e] += src[e];
@@ -105,17 +128,41 @@ struct StafModel {
   hipEvent_t ev_fork = nullptr;
   std::vector<hipEvent_t> ev_join;
   // device buffers
-  DevBuf<double> pos, box, force, force_op, virial_op, af2, af3, g2, g3, e_atom, virial_acc;
+  // in_d  = [pos nall*3 | box 6 | howmany nlocal ints | with nlocal*nr ints]   (mirror of in_h, one copy per call)
+  // out_d = [force nall*3 | virial 9 | atomic energies nlocal]                 (mirror of out_h, one copy per call)
+  DevBuf<double> in_d, out_d, force_op, virial_op, af2, af3, g2, g3;
+  PinBuf<double> in_h, out_h;
+  std::vector<int> type_map_up, tipos_up;   // what the device copies of type_map and tipos hold
+  bool actual_type_up = false;
+  // The kernel sequence of a call (descriptors .. sum of the forces), recorded as a HIP graph once a configuration
+  // of the same shape has been evaluated eagerly (which also sizes every scratch buffer), then replayed: an MD run
+  // repeats one shape for many steps, and issuing ~27 launches costs the host more than the GPU needs to run them.
+  struct Replay {
+    int state = 0;             // 0: nothing, 1: shape seen once (eagerly), 2: graph ready
+    int nlocal = 0, nall = 0, ext = 0, want_w = 0;
+    std::vector<int> tipos;
+    const void* in_d = nullptr;
+    const void* out_d = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    void drop() {
+      if (exec) (void)hipGraphExecDestroy(exec);
+      if (graph) (void)hipGraphDestroy(graph);
+      exec = nullptr;
+      graph = nullptr;
+      state = 0;
+    }
+  } replay;
+  bool use_graph = true;
   // device-resident MLP (default); false: the host evaluation of staf_mlp.cpp between the kernels
   bool dev_mlp = false;
   std::vector<staf::DevMlpNet> dnets;
-  std::vector<double> e_atom_h;
   DevBuf<double> raddescr, angdescr, des3bsupp, der2b, der3b, der3bsupp;
-  DevBuf<int> intmap2b, intmap3b, numtriplet, type_map, tipos, actual_type, how, with;
+  DevBuf<int> intmap2b, intmap3b, numtriplet, type_map, tipos, actual_type;
   // host staging
-  std::vector<double> pos_h, force_h, af_h, gr_h, tmp2, tmp3;
+  std::vector<double> af_h, gr_h, tmp2, tmp3;
   std::vector<float> af_f, gr_f;
-  std::vector<int> order_to_slot, slot_to_order, type_map_h, how_h, with_h;
+  std::vector<int> order_to_slot, slot_to_order, type_map_h;
 };
 
 static bool load_species_params(StafModel* m) {
@@ -200,6 +247,7 @@ int staf_cuda_set_device(int device_id) {
 void staf_free(StafModel* m) {
   if (!m) return;
   if (m->stream) (void)hipStreamSynchronize(m->stream);
+  m->replay.drop();
   for (hipStream_t s : m->sstream)
     if (s) { (void)hipStreamSynchronize(s); (void)hipStreamDestroy(s); }
   for (hipEvent_t e : m->ev_join)
@@ -210,12 +258,12 @@ void staf_free(StafModel* m) {
   for (auto& n : m->dnets) staf::dev_mlp_free(&n);
   for (auto* v : {&m->alpha2b, &m->alpha3b, &m->emb2b, &m->emb3b})
     for (auto& b : *v) b.release();
-  for (DevBuf<double>* b : {&m->pos, &m->box, &m->force, &m->force_op, &m->virial_op, &m->af2, &m->af3, &m->g2, &m->g3, &m->e_atom,
-                            &m->virial_acc,
+  m->in_h.release();
+  m->out_h.release();
+  for (DevBuf<double>* b : {&m->in_d, &m->out_d, &m->force_op, &m->virial_op, &m->af2, &m->af3, &m->g2, &m->g3,
                             &m->raddescr, &m->angdescr, &m->des3bsupp, &m->der2b, &m->der3b, &m->der3bsupp})
     b->release();
-  for (DevBuf<int>* b : {&m->intmap2b, &m->intmap3b, &m->numtriplet, &m->type_map, &m->tipos, &m->actual_type, &m->how,
-                         &m->with})
+  for (DevBuf<int>* b : {&m->intmap2b, &m->intmap3b, &m->numtriplet, &m->type_map, &m->tipos, &m->actual_type})
     b->release();
   delete m;
 }
@@ -255,6 +303,9 @@ StafModel* staf_load(const char* model_dir, const StafOptions* opt) {
       staf_free(m);
       return NULL;
     }
+  // The kernel sequence of a repeated shape is replayed as a HIP graph unless the caller asks for eager launches
+  // (StafOptions.reserved bit 2, or STAF_MD_EAGER=1 in the environment).
+  m->use_graph = !(m->opt.reserved & 4) && !getenv("STAF_MD_EAGER");
   // The MLP runs on the GPU between the fingerprint and the force kernels unless the caller asks for the host
   // evaluation (StafOptions.reserved bit 1, or STAF_MLP_HOST=1 in the environment).
   if (!(m->opt.reserved & 2) && !getenv("STAF_MLP_HOST")) {
@@ -328,127 +379,202 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
     m->slot_to_order[i] = i;
     m->type_map_h[i] = sp;
   }
+  // ---- the call's input block, written straight into pinned memory
+  const size_t L = (size_t)nlocal;
+  const size_t n_in_d = (size_t)nall * 3 + 6;                                 // doubles
+  const size_t n_in_i = ext ? L + L * nr : 0;                                 // ints behind them
+  const size_t n_in = n_in_d + (n_in_i + 1) / 2;
+  const size_t n_out = (size_t)nall * 3 + 9 + L;
+  if (!m->in_h.reserve(n_in) || !m->out_h.reserve(n_out)) return -1;
+  double* pos_h = m->in_h.p;
+  int* how_h = (int*)(m->in_h.p + n_in_d);
+  int* with_h = how_h + L;
   if (ext) {
-    m->how_h.assign(nlocal, 0);
-    m->with_h.assign((size_t)nlocal * nr, 0);
+    memset(how_h, 0, n_in_i * sizeof(int));
     for (int i = 0; i < nlocal; i++) {
       const int slot = m->order_to_slot[i];
       int nn = howmany[i];
       if (nn < 0) nn = 0;
       if (nn > nr) nn = nr;   // truncated like the reference (staf_api.cpp:321-323)
       if (nn > maxneigh) nn = maxneigh;
-      m->how_h[slot] = nn;
+      how_h[slot] = nn;
       for (int k = 0; k < nn; k++) {
         const int j = with[(size_t)i * maxneigh + k];
         if (j < 0 || j >= nall) {
           fprintf(stderr, "staf_compute: neighbor index %d out of range [0,%d)\n", j, nall);
           return -9;
         }
-        m->with_h[(size_t)slot * nr + k] = m->order_to_slot[j];
+        with_h[(size_t)slot * nr + k] = m->order_to_slot[j];
       }
     }
   }
-  m->pos_h.resize((size_t)nall * 3);
   for (int i = 0; i < nall; i++) {
     const int s = m->order_to_slot[i];
-    m->pos_h[3 * s] = x[3 * i];
-    m->pos_h[3 * s + 1] = x[3 * i + 1];
-    m->pos_h[3 * s + 2] = x[3 * i + 2];
+    pos_h[3 * s] = x[3 * i];
+    pos_h[3 * s + 1] = x[3 * i + 1];
+    pos_h[3 * s + 2] = x[3 * i + 2];
   }
+  memcpy(pos_h + (size_t)nall * 3, box, 6 * sizeof(double));
 
   // ---- device buffers
-  const size_t L = (size_t)nlocal;
   int amax2 = 0, amax3 = 0;
   for (int k = 0; k < nt; k++) { amax2 = m->Ar[k] > amax2 ? m->Ar[k] : amax2; amax3 = m->Aa[k] > amax3 ? m->Aa[k] : amax3; }
-  bool ok = m->pos.reserve((size_t)nall * 3) && m->box.reserve(6) && m->force.reserve((size_t)nall * 3) &&
+  const int* type_map_before = m->type_map.p;
+  bool ok = m->in_d.reserve(n_in) && m->out_d.reserve(n_out) &&
             m->force_op.reserve((size_t)nall * 3 * 2 * nt) && m->virial_op.reserve((size_t)9 * 2 * nt) && m->af2.reserve(L * amax2) &&
             m->af3.reserve(L * amax3) && m->g2.reserve(L * amax2) && m->g3.reserve(L * amax3) &&
-            m->e_atom.reserve(L) && m->virial_acc.reserve(9) &&
             m->raddescr.reserve(L * nr) && m->angdescr.reserve(L * na) && m->des3bsupp.reserve(L * nr) &&
             m->der2b.reserve(L * 3 * nr) && m->der3b.reserve(L * 6 * na) && m->der3bsupp.reserve(L * 3 * nr) &&
             m->intmap2b.reserve(L * (nr + 1)) && m->intmap3b.reserve(L * 2 * na) && m->numtriplet.reserve(L) &&
-            m->type_map.reserve(nall) && m->tipos.reserve(nt) && m->actual_type.reserve(nt) &&
-            (!ext || (m->how.reserve(L) && m->with.reserve(L * nr)));
+            m->type_map.reserve(nall) && m->tipos.reserve(nt) && m->actual_type.reserve(nt);
   if (!ok) return -1;
+  if (m->type_map.p != type_map_before) m->type_map_up.clear();   // a new block holds nothing yet
   hipStream_t st = m->stream;
-  STAF_HIP_OK(hipMemcpyAsync(m->pos.p, m->pos_h.data(), (size_t)nall * 3 * sizeof(double), hipMemcpyHostToDevice, st));
-  STAF_HIP_OK(hipMemcpyAsync(m->box.p, box, 6 * sizeof(double), hipMemcpyHostToDevice, st));
-  STAF_HIP_OK(hipMemcpyAsync(m->type_map.p, m->type_map_h.data(), (size_t)nall * sizeof(int), hipMemcpyHostToDevice, st));
-  STAF_HIP_OK(hipMemcpyAsync(m->tipos.p, tipos.data(), nt * sizeof(int), hipMemcpyHostToDevice, st));
-  std::vector<int> ats(nt);
-  for (int k = 0; k < nt; k++) ats[k] = k;
-  STAF_HIP_OK(hipMemcpyAsync(m->actual_type.p, ats.data(), nt * sizeof(int), hipMemcpyHostToDevice, st));
-  if (ext) {
-    STAF_HIP_OK(hipMemcpyAsync(m->how.p, m->how_h.data(), L * sizeof(int), hipMemcpyHostToDevice, st));
-    STAF_HIP_OK(hipMemcpyAsync(m->with.p, m->with_h.data(), L * nr * sizeof(int), hipMemcpyHostToDevice, st));
+  double* const d_pos = m->in_d.p;
+  double* const d_box = d_pos + (size_t)nall * 3;
+  int* const d_how = (int*)(m->in_d.p + n_in_d);
+  int* const d_with = d_how + L;
+  double* const d_force = m->out_d.p;
+  double* const d_W = d_force + (size_t)nall * 3;
+  double* const d_e = d_W + 9;
+  STAF_HIP_OK(hipMemcpyAsync(m->in_d.p, m->in_h.p, n_in * sizeof(double), hipMemcpyHostToDevice, st));
+  // species of the slots and atoms per species: sent when they differ from what the device holds (in MD they change
+  // when atoms migrate, not every step); the blocking copies read host vectors that the next lines may replace
+  if (m->type_map_up != m->type_map_h) {
+    STAF_HIP_OK(hipMemcpy(m->type_map.p, m->type_map_h.data(), (size_t)nall * sizeof(int), hipMemcpyHostToDevice));
+    m->type_map_up = m->type_map_h;
   }
-  // No synchronisation here: every host buffer above outlives the call's final synchronisation.
+  if (m->tipos_up != tipos) {
+    STAF_HIP_OK(hipMemcpy(m->tipos.p, tipos.data(), nt * sizeof(int), hipMemcpyHostToDevice));
+    m->tipos_up = tipos;
+  }
+  if (!m->actual_type_up) {
+    std::vector<int> ats(nt);
+    for (int k = 0; k < nt; k++) ats[k] = k;
+    STAF_HIP_OK(hipMemcpy(m->actual_type.p, ats.data(), nt * sizeof(int), hipMemcpyHostToDevice));
+    m->actual_type_up = true;
+  }
+  // No synchronisation here: the pinned input block outlives the call's final synchronisation.
   staf::DeferStatus defer;   // conditions the kernels detect are read once, after the last kernel
 
   // ---- descriptors (own minimum-image list, or the caller's list with explicit images)
-  int rc = staf::desc_launch<double>(m->cfg, m->pos.p, m->box.p, 1, nlocal, nall, ext ? m->how.p : nullptr,
-                                     ext ? m->with.p : nullptr, ext ? 1 : 0, m->raddescr.p, m->angdescr.p,
+  auto descriptors = [&]() -> int {
+    return staf::desc_launch<double>(m->cfg, d_pos, d_box, 1, nlocal, nall, ext ? d_how : nullptr,
+                                     ext ? d_with : nullptr, ext ? 1 : 0, m->raddescr.p, m->angdescr.p,
                                      m->des3bsupp.p, m->intmap2b.p, m->intmap3b.p, m->der2b.p, m->der3b.p,
-                                     m->der3bsupp.p, m->numtriplet.p, st);
-  if (rc != STAF_OK) return -20;
-
+                                     m->der3bsupp.p, m->numtriplet.p, st) == STAF_OK ? 0 : -20;
+  };
+  int rc = 0;
   double energy = 0.0;
   double W[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
   const int n3 = nall * 3;
+  const bool want_w = virial != nullptr;
   staf_op_force_set_skip_pbc(ext ? 1 : 0);
-  if (m->dev_mlp) {
-    // ---- everything stays on the device: per species fingerprints -> MLP -> forces, one stream per species (the
-    // chains meet only in the sum of the forces); one synchronisation at the end of the call
-    const bool want_w = virial != nullptr;
+  // ---- everything stays on the device: per species fingerprints -> MLP -> forces, one stream per species (the
+  // chains meet only in the sum of the forces); one synchronisation at the end of the call
+  auto device_sequence = [&]() -> int {
+    if (descriptors() != 0) return -20;
+    // every species stream branches off right behind the descriptors, and the call's stream waits for all of
+    // them only after the last chain has been issued: a recorded graph then holds independent branches
     STAF_HIP_OK(hipEventRecord(m->ev_fork, st));
+    for (int k = 0; k < nt; k++)
+      if (tipos[k] > 0) STAF_HIP_OK(hipStreamWaitEvent(m->sstream[k], m->ev_fork, 0));
+    // The chains are issued step by step across the species (all fingerprint ops, then all networks, ...): the host
+    // -- also when it replays a recorded graph -- submits launches one after the other, and a chain issued as a
+    // whole would have run before the next one is even submitted.
     int nops = 0;
-    int shift = 0;
-    for (int k = 0; k < nt; shift += tipos[k], k++) {
-      const int Nl = tipos[k], Ar = m->Ar[k], Aa = m->Aa[k];
-      if (Nl == 0) continue;
-      hipStream_t sk = m->sstream[k];
-      STAF_HIP_OK(hipStreamWaitEvent(sk, m->ev_fork, 0));
-      const size_t o = (size_t)shift;
-      double* af2 = m->af2.p + o * amax2;
-      double* af3 = m->af3.p + o * amax3;
-      double* g2 = m->g2.p + o * amax2;
-      double* g3 = m->g3.p + o * amax3;
-      rc = staf_op_radial_afs_f64(m->raddescr.p + o * nr, nr, m->alpha2b[k].p, Ar, af2, 1, Nl,
-                                  m->intmap2b.p + o * (nr + 1), m->emb2b[k].p, m->type_map.p, nt, nlocal, sk);
-      if (rc == STAF_OK)
-        rc = staf_op_angular_afs_f64(m->des3bsupp.p + o * nr, m->angdescr.p + o * na, nr, na, af3, 1, Nl,
-                                     m->intmap3b.p + o * 2 * na, m->intmap2b.p + o * (nr + 1), m->alpha3b[k].p, Aa,
-                                     m->emb3b[k].p, m->type_map.p, m->numtriplet.p + o, nt, nlocal, sk);
-      if (rc == STAF_OK)
-        rc = staf::dev_mlp_eval(m->dnets[k], af2, Ar, af3, Aa, Nl, m->e_atom.p + o, g2, g3, sk);
-      if (rc != STAF_OK) return -20;
-      for (int body = 2; body <= 3; body++, nops++) {
-        double* fo = m->force_op.p + (size_t)nops * n3;
-        double* wo = want_w ? m->virial_op.p + nops * 9 : nullptr;
-        const double* px = want_w ? m->pos.p : nullptr;
-        const double* bx = want_w ? m->box.p : nullptr;
-        if (body == 2)
-          rc = staf_op_force_doublets_f64(g2, m->raddescr.p + o * nr, m->der2b.p + o * 3 * nr,
-                                          m->intmap2b.p + o * (nr + 1), nr, nall, 1, Ar, m->alpha2b[k].p,
-                                          m->emb2b[k].p, nt, m->tipos.p, m->actual_type.p + k, fo, m->type_map.p, Nl,
-                                          wo, px, bx, nlocal, sk);
-        else
-          rc = staf_op_force_tripl_f64(g3, m->des3bsupp.p + o * nr, m->angdescr.p + o * na,
-                                       m->der3bsupp.p + o * 3 * nr, m->der3b.p + o * 6 * na,
-                                       m->intmap2b.p + o * (nr + 1), m->intmap3b.p + o * 2 * na, nr, na, nall, 1, Aa,
-                                       m->emb3b[k].p, nt, m->tipos.p, m->actual_type.p + k, fo, m->numtriplet.p + o,
-                                       m->alpha3b[k].p, m->type_map.p, Nl, wo, px, bx, nlocal, sk);
+    for (int step = 0; step < 5; step++) {
+      int shift = 0, slot = 0;
+      for (int k = 0; k < nt; shift += tipos[k], k++) {
+        const int Nl = tipos[k], Ar = m->Ar[k], Aa = m->Aa[k];
+        if (Nl == 0) continue;
+        hipStream_t sk = m->sstream[k];
+        const size_t o = (size_t)shift;
+        double* af2 = m->af2.p + o * amax2;
+        double* af3 = m->af3.p + o * amax3;
+        double* g2 = m->g2.p + o * amax2;
+        double* g3 = m->g3.p + o * amax3;
+        const int op = 2 * slot + (step - 3);          // output slot of the force ops (steps 3 and 4)
+        slot++;
+        double* fo = m->force_op.p + (size_t)(op < 0 ? 0 : op) * n3;
+        double* wo = want_w ? m->virial_op.p + (op < 0 ? 0 : op) * 9 : nullptr;
+        const double* px = want_w ? d_pos : nullptr;
+        const double* bx = want_w ? d_box : nullptr;
+        switch (step) {
+          case 0:
+            rc = staf_op_radial_afs_f64(m->raddescr.p + o * nr, nr, m->alpha2b[k].p, Ar, af2, 1, Nl,
+                                        m->intmap2b.p + o * (nr + 1), m->emb2b[k].p, m->type_map.p, nt, nlocal, sk);
+            break;
+          case 1:
+            rc = staf_op_angular_afs_f64(m->des3bsupp.p + o * nr, m->angdescr.p + o * na, nr, na, af3, 1, Nl,
+                                         m->intmap3b.p + o * 2 * na, m->intmap2b.p + o * (nr + 1), m->alpha3b[k].p,
+                                         Aa, m->emb3b[k].p, m->type_map.p, m->numtriplet.p + o, nt, nlocal, sk);
+            break;
+          case 2:
+            rc = staf::dev_mlp_eval(m->dnets[k], af2, Ar, af3, Aa, Nl, d_e + o, g2, g3, sk);
+            break;
+          case 3:
+            rc = staf_op_force_doublets_f64(g2, m->raddescr.p + o * nr, m->der2b.p + o * 3 * nr,
+                                            m->intmap2b.p + o * (nr + 1), nr, nall, 1, Ar, m->alpha2b[k].p,
+                                            m->emb2b[k].p, nt, m->tipos.p, m->actual_type.p + k, fo, m->type_map.p,
+                                            Nl, wo, px, bx, nlocal, sk);
+            break;
+          default:
+            rc = staf_op_force_tripl_f64(g3, m->des3bsupp.p + o * nr, m->angdescr.p + o * na,
+                                         m->der3bsupp.p + o * 3 * nr, m->der3b.p + o * 6 * na,
+                                         m->intmap2b.p + o * (nr + 1), m->intmap3b.p + o * 2 * na, nr, na, nall, 1,
+                                         Aa, m->emb3b[k].p, nt, m->tipos.p, m->actual_type.p + k, fo,
+                                         m->numtriplet.p + o, m->alpha3b[k].p, m->type_map.p, Nl, wo, px, bx, nlocal,
+                                         sk);
+            STAF_HIP_OK(hipEventRecord(m->ev_join[k], sk));
+            break;
+        }
         if (rc != STAF_OK) return -20;
+        if (step >= 3) nops = op + 1 > nops ? op + 1 : nops;
       }
-      STAF_HIP_OK(hipEventRecord(m->ev_join[k], sk));
-      STAF_HIP_OK(hipStreamWaitEvent(st, m->ev_join[k], 0));
     }
-    hipLaunchKernelGGL(combine_kernel, dim3((n3 + 255) / 256), dim3(256), 0, st, m->force.p, m->force_op.p, n3, nops,
-                       m->virial_acc.p, want_w ? m->virial_op.p : nullptr);
-    m->e_atom_h.resize(nlocal);
-    STAF_HIP_OK(hipMemcpyAsync(m->e_atom_h.data(), m->e_atom.p, L * sizeof(double), hipMemcpyDeviceToHost, st));
-    STAF_HIP_OK(hipMemcpyAsync(W, m->virial_acc.p, 9 * sizeof(double), hipMemcpyDeviceToHost, st));
+    for (int k = 0; k < nt; k++)
+      if (tipos[k] > 0) STAF_HIP_OK(hipStreamWaitEvent(st, m->ev_join[k], 0));
+    hipLaunchKernelGGL(combine_kernel, dim3((n3 + 255) / 256), dim3(256), 0, st, d_force, m->force_op.p, n3, nops,
+                       d_W, want_w ? m->virial_op.p : nullptr);
+    return hipGetLastError() == hipSuccess ? 0 : -20;
+  };
+  if (m->dev_mlp) {
+    StafModel::Replay& rp = m->replay;
+    const bool same = rp.state > 0 && rp.nlocal == nlocal && rp.nall == nall && rp.ext == (int)ext &&
+                      rp.want_w == (int)want_w && rp.tipos == tipos && rp.in_d == m->in_d.p && rp.out_d == m->out_d.p;
+    if (!m->use_graph || !same) {
+      rp.drop();
+      if (device_sequence() != 0) return -20;
+      if (m->use_graph) {
+        rp.state = 1;
+        rp.nlocal = nlocal; rp.nall = nall; rp.ext = ext; rp.want_w = want_w; rp.tipos = tipos;
+        rp.in_d = m->in_d.p; rp.out_d = m->out_d.p;
+      }
+    } else {
+      if (rp.state == 1) {
+        // second call of this shape: every buffer and scratch block has its final size, record the sequence
+        STAF_HIP_OK(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+        const int issued = device_sequence();
+        hipGraph_t g = nullptr;
+        const hipError_t ended = hipStreamEndCapture(st, &g);
+        if (issued != 0 || ended != hipSuccess || !g) {
+          if (g) (void)hipGraphDestroy(g);
+          (void)hipGetLastError();
+          rp.drop();
+          return -20;
+        }
+        rp.graph = g;
+        if (hipGraphInstantiate(&rp.exec, rp.graph, nullptr, nullptr, 0) != hipSuccess) {
+          rp.drop();
+          return -20;
+        }
+        rp.state = 2;
+      }
+      STAF_HIP_OK(hipGraphLaunch(rp.exec, st));
+    }
   } else {
+    if (descriptors() != 0) return -20;
     // ---- fingerprints of every species, packed rows [Ar+Aa] for the MLP
     size_t total = 0;
     for (int k = 0; k < nt; k++) total += (size_t)tipos[k] * (m->Ar[k] + m->Aa[k]);
@@ -510,7 +636,7 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
       fprintf(stderr, "staf_compute: non-finite energy=%g nlocal=%d nghost=%d\n", energy, nlocal, nghost);
 
     // ---- forces: 2-body + 3-body of every centre species, with the virial
-    staf::launch_fill_zero<double>(m->force.p, nall * 3, st);
+    staf::launch_fill_zero<double>(d_force, nall * 3, st);
     double Wk[9];
     off = 0;
     shift = 0;
@@ -534,30 +660,34 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
           rc = staf_op_force_doublets_f64(m->g2.p, m->raddescr.p + o * nr, m->der2b.p + o * 3 * nr,
                                           m->intmap2b.p + o * (nr + 1), nr, nall, 1, Ar, m->alpha2b[k].p, m->emb2b[k].p,
                                           nt, m->tipos.p, m->actual_type.p + k, m->force_op.p, m->type_map.p, Nl,
-                                          m->virial_op.p, m->pos.p, m->box.p, nlocal, st);
+                                          m->virial_op.p, d_pos, d_box, nlocal, st);
         else
           rc = staf_op_force_tripl_f64(m->g3.p, m->des3bsupp.p + o * nr, m->angdescr.p + o * na,
                                        m->der3bsupp.p + o * 3 * nr, m->der3b.p + o * 6 * na,
                                        m->intmap2b.p + o * (nr + 1), m->intmap3b.p + o * 2 * na, nr, na, nall, 1, Aa,
                                        m->emb3b[k].p, nt, m->tipos.p, m->actual_type.p + k, m->force_op.p,
                                        m->numtriplet.p + o, m->alpha3b[k].p, m->type_map.p, Nl, m->virial_op.p,
-                                       m->pos.p, m->box.p, nlocal, st);
+                                       d_pos, d_box, nlocal, st);
         if (rc != STAF_OK) return -20;
-        hipLaunchKernelGGL(add_into_kernel, dim3((n3 + 255) / 256), dim3(256), 0, st, m->force.p, m->force_op.p, n3);
+        hipLaunchKernelGGL(add_into_kernel, dim3((n3 + 255) / 256), dim3(256), 0, st, d_force, m->force_op.p, n3);
         STAF_HIP_OK(hipMemcpyAsync(Wk, m->virial_op.p, 9 * sizeof(double), hipMemcpyDeviceToHost, st));
         STAF_HIP_OK(hipStreamSynchronize(st));
         for (int c = 0; c < 9; c++) W[c] += Wk[c];
       }
     }
   }
-  m->force_h.resize((size_t)n3);
-  STAF_HIP_OK(hipMemcpyAsync(m->force_h.data(), m->force.p, (size_t)n3 * sizeof(double), hipMemcpyDeviceToHost, st));
+  // forces, and on the device path the virial and the atomic energies behind them, in one copy
+  const size_t n_back = m->dev_mlp ? n_out : (size_t)n3;
+  STAF_HIP_OK(hipMemcpyAsync(m->out_h.p, m->out_d.p, n_back * sizeof(double), hipMemcpyDeviceToHost, st));
+  const double* force_h = m->out_h.p;
   // the call's synchronisation: results are on the host, and so is what the kernels reported
   rc = staf_ops_poll_status(st);
   if (rc == STAF_E_RADIAL_OVERFLOW) return -10;
   if (rc != STAF_OK) return -20;
   if (m->dev_mlp) {
-    for (int a = 0; a < nlocal; a++) energy += m->e_atom_h[a];   // slot order: fixed
+    const double* e_atom_h = m->out_h.p + (size_t)n3 + 9;
+    for (int c = 0; c < 9; c++) W[c] = m->out_h.p[(size_t)n3 + c];
+    for (int a = 0; a < nlocal; a++) energy += e_atom_h[a];   // slot order: fixed
     energy *= 0.5;
     if (!isfinite(energy))
       fprintf(stderr, "staf_compute: non-finite energy=%g nlocal=%d nghost=%d\n", energy, nlocal, nghost);
@@ -567,9 +697,9 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
   if (f)
     for (int s = 0; s < nall; s++) {
       const int i = m->slot_to_order[s];
-      f[3 * i] = m->force_h[3 * s];
-      f[3 * i + 1] = m->force_h[3 * s + 1];
-      f[3 * i + 2] = m->force_h[3 * s + 2];
+      f[3 * i] = force_h[3 * s];
+      f[3 * i + 1] = force_h[3 * s + 1];
+      f[3 * i + 2] = force_h[3 * s + 2];
     }
   if (virial) {
     virial[0] = W[0];

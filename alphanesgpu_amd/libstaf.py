@@ -61,12 +61,13 @@ def options_default():
 
 class StafModel:
     def __init__(self, model_dir, precision=0, device_id=0, mlp_backend=STAF_MLP_NATIVE, full_virial=False,
-                 host_mlp=False):
+                 host_mlp=False, eager=False):
         L = _bind()
         o = options_default()
         o.mlp_backend, o.device_id, o.precision = mlp_backend, device_id, precision
-        # reserved bit 0: all six virial components; bit 1: evaluate the MLP on the host instead of on the GPU
-        o.reserved = (1 if full_virial else 0) | (2 if host_mlp else 0)
+        # reserved bit 0: all six virial components; bit 1: evaluate the MLP on the host instead of on the GPU;
+        # bit 2: launch every call's kernels eagerly instead of replaying a recorded HIP graph
+        o.reserved = (1 if full_virial else 0) | (2 if host_mlp else 0) | (4 if eager else 0)
         self._L = L
         self._h = L.staf_load(str(model_dir).encode(), C.byref(o))
         if not self._h:
