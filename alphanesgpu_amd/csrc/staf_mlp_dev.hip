@@ -8,6 +8,7 @@
 // transposed copy serves the backward pass); each weight read serves the TA atoms of the workgroup.
 #include "staf_mlp_dev.hpp"
 
+#include <stdlib.h>
 #include <vector>
 
 namespace staf {
@@ -212,6 +213,189 @@ __global__ __launch_bounds__(MLP_BLOCK) void mlp_kernel(MlpArgs<T> A) {
   PHASE_CLOCK_END();
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Matrix-core form of the same evaluation.  The Dense layers are small dense matrix products ([atoms, in] x
+// [in, out]), the one place on this path where the matrix cores fit: a workgroup takes 16 atoms (the rows of a
+// 16x16x4 MFMA tile), so the weight matrices stream through a CU once per 16 atoms instead of once per 2-4, which is
+// what bounds the vector kernel above.  Activations live in LDS as X[feature][16 atoms]; a unit of work is (tile of
+// 16 output columns, slice of the inner dimension) with up to MM_STEPS weight reads in flight per lane; units are
+// dealt round-robin to the 16 waves; slice sums meet in LDS and are added in ascending slice order (fixed order).
+constexpr int MM_TA = 16;
+constexpr int MM_BLOCK = 1024;
+constexpr int MM_WAVES = MM_BLOCK / WAVE;
+constexpr int MM_STEPS = 12;      // MFMA steps (4 rows of the inner dimension each) per batch of weight reads
+constexpr int MM_SLICES = 4;      // at most this many slices of the inner dimension
+
+template <typename T> struct MfmaOp;
+template <> struct MfmaOp<double> {
+  typedef double acc_t __attribute__((ext_vector_type(4)));
+  __device__ static acc_t run(double a, double b, acc_t c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
+  __device__ static int acc_row(int lane, int v) { return lane / 16 + 4 * v; }
+};
+template <> struct MfmaOp<float> {
+  typedef float acc_t __attribute__((ext_vector_type(4)));
+  __device__ static acc_t run(float a, float b, acc_t c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+  __device__ static int acc_row(int lane, int v) { return 4 * (lane / 16) + v; }
+};
+// operand layout of the 16x16x4 tiles: A[row = lane % 16][k = lane / 16], B[k = lane / 16][col = lane % 16];
+// accumulator element v of a lane: col = lane % 16, row = acc_row(lane, v) (the two precisions differ)
+
+__host__ __device__ inline int mm_slices(int K) {
+  const int nstep = (K + 3) / 4;
+  const int s = (nstep + MM_STEPS - 1) / MM_STEPS;
+  return s < 1 ? 1 : (s > MM_SLICES ? MM_SLICES : s);
+}
+
+// part[slice][j][atom] = sum over the slice's rows k of X[k][atom] * M[k][j];  M [K, J] row-major in global memory,
+// X [K][MM_TA] in LDS.  Returns the number of slices.
+template <typename T>
+__device__ inline int mm_products(const T* __restrict__ M, int K, int J, const T* X, T* part) {
+  typedef typename MfmaOp<T>::acc_t acc_t;
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  const int ntile = (J + 15) / 16;
+  const int nstep = (K + 3) / 4;
+  const int nsl = mm_slices(K);
+  const int per = (nstep + nsl - 1) / nsl;
+  const int kq = lane / 16, c16 = lane % 16;
+  for (int u = wave; u < ntile * nsl; u += MM_WAVES) {
+    const int tile = u % ntile, sl = u / ntile;
+    const int s0 = sl * per;
+    const int s1 = (s0 + per) < nstep ? (s0 + per) : nstep;
+    const int col = tile * 16 + c16;
+    const int colc = col < J ? col : J - 1;
+    acc_t acc = {0, 0, 0, 0};
+    for (int sb = s0; sb < s1; sb += MM_STEPS) {
+      T b[MM_STEPS], a[MM_STEPS];
+      // rows beyond the slice or the matrix are read at the last row (inside the matrix) and enter as zeros
+#pragma unroll
+      for (int q = 0; q < MM_STEPS; q++) {
+        const int k = 4 * (sb + q) + kq;
+        const int kc = k < K ? k : K - 1;
+        b[q] = M[(size_t)kc * J + colc];
+      }
+#pragma unroll
+      for (int q = 0; q < MM_STEPS; q++) {
+        const int k = 4 * (sb + q) + kq;
+        const int kc = k < K ? k : K - 1;
+        a[q] = X[kc * MM_TA + c16];
+      }
+#pragma unroll
+      for (int q = 0; q < MM_STEPS; q++) {
+        const int k = 4 * (sb + q) + kq;
+        const bool in = (sb + q) < s1 && k < K;
+        acc = MfmaOp<T>::run(in ? a[q] : T(0), (in && col < J) ? b[q] : T(0), acc);
+      }
+    }
+    if (col < J) {
+#pragma unroll
+      for (int v = 0; v < 4; v++) part[((size_t)sl * J + col) * MM_TA + MfmaOp<T>::acc_row(lane, v)] = acc[v];
+    }
+  }
+  return nsl;
+}
+
+template <typename T>
+__global__ __launch_bounds__(MM_BLOCK) void mlp_matrix_kernel(MlpArgs<T> A) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  T* X = (T*)smem;                            // [tot][MM_TA]: input and every layer's output
+  T* dl = X + (size_t)A.tot * MM_TA;          // [maxw][MM_TA]: back-propagated deltas
+  T* part = dl + (size_t)A.maxw * MM_TA;      // [slices][width][MM_TA]
+  const int tid = threadIdx.x;
+  const int a0 = blockIdx.x * MM_TA;
+  const int n_af = A.n_af;
+  PHASE_CLOCK_BEGIN();
+  for (int q = tid; q < MM_TA * n_af; q += MM_BLOCK) {
+    const int t = q / n_af, i = q - t * n_af;
+    const int atom = a0 + t;
+    T v = 0;
+    if (atom < A.Nl) {
+      const T afv = (T)(i < A.Ar ? A.af2[(size_t)atom * A.Ar + i] : A.af3[(size_t)atom * A.Aa + (i - A.Ar)]);
+      v = m_log(afv + T(1e-3)) - A.mu[i];
+    }
+    X[i * MM_TA + t] = v;
+  }
+  __syncthreads();
+  PHASE_MARK(0);
+  // ---- forward
+  int off_in = 0;
+  for (int l = 0; l < A.nl; l++) {
+    const int in_f = A.in_f[l], out_f = A.out_f[l];
+    const int off_out = off_in + in_f;
+    const int nsl = mm_products<T>(A.W[l], in_f, out_f, X + (size_t)off_in * MM_TA, part);
+    __syncthreads();
+    PHASE_MARK(1);
+    for (int q = tid; q < out_f * MM_TA; q += MM_BLOCK) {
+      const int j = q / MM_TA;
+      T y = A.b[l][j];
+      for (int sl = 0; sl < nsl; sl++) y += part[(size_t)sl * out_f * MM_TA + q];
+      if (A.act[l] == 1) y = m_tanh(y);
+      else if (A.act[l] == 2) y = y > T(0) ? y : T(0);
+      X[(size_t)off_out * MM_TA + q] = y;
+    }
+    __syncthreads();
+    PHASE_MARK(2);
+    off_in = off_out;
+  }
+  // off_in is now the offset of the last layer's output (one value per atom)
+  if (tid < MM_TA && a0 + tid < A.Nl) A.e_atom[a0 + tid] = (double)X[(size_t)off_in * MM_TA + tid];
+  // ---- backward: delta of the summed atomic energy
+  for (int q = tid; q < MM_TA; q += MM_BLOCK) dl[q] = T(1);
+  __syncthreads();
+  int off_out = off_in;
+  for (int l = A.nl - 1; l >= 0; l--) {
+    const int in_f = A.in_f[l], out_f = A.out_f[l];
+    const int off_i = off_out - in_f;
+    // delta times the activation derivative, in place
+    for (int q = tid; q < out_f * MM_TA; q += MM_BLOCK) {
+      const T y = X[(size_t)off_out * MM_TA + q];
+      T g = dl[q];
+      if (A.act[l] == 1) g *= (T(1) - y * y);
+      else if (A.act[l] == 2 && y <= T(0)) g = T(0);
+      dl[q] = g;
+    }
+    __syncthreads();
+    // delta of the layer's input: Wt [out, in] is the matrix, the deltas [out][atoms] the vectors
+    PHASE_MARK(3);
+    const int nsl = mm_products<T>(A.Wt[l], out_f, in_f, dl, part);
+    __syncthreads();
+    PHASE_MARK(4);
+    for (int q = tid; q < in_f * MM_TA; q += MM_BLOCK) {
+      T g = 0;
+      for (int sl = 0; sl < nsl; sl++) g += part[(size_t)sl * in_f * MM_TA + q];
+      dl[q] = g;
+    }
+    __syncthreads();
+    PHASE_MARK(5);
+    off_out = off_i;
+  }
+  // ---- d sum(atomic) / d af = delta / (af + 1e-3)
+  for (int q = tid; q < MM_TA * n_af; q += MM_BLOCK) {
+    const int t = q / n_af, i = q - t * n_af;
+    const int atom = a0 + t;
+    if (atom >= A.Nl) continue;
+    const bool two = i < A.Ar;
+    const T afv = (T)(two ? A.af2[(size_t)atom * A.Ar + i] : A.af3[(size_t)atom * A.Aa + (i - A.Ar)]);
+    const double g = (double)(dl[i * MM_TA + t] / (afv + T(1e-3)));
+    if (two) A.g2[(size_t)atom * A.Ar + i] = g;
+    else A.g3[(size_t)atom * A.Aa + (i - A.Ar)] = g;
+  }
+  PHASE_MARK(6);
+  PHASE_CLOCK_END();
+}
+
+// LDS of a workgroup of the matrix kernel: activations, deltas, slice sums of the widest product
+template <typename T>
+static size_t mm_lds_bytes(const DevMlpNet& net) {
+  size_t npart = 0;
+  for (int l = 0; l < net.nl; l++) {
+    const size_t f = (size_t)mm_slices(net.in_f[l]) * net.out_f[l];
+    const size_t b = (size_t)mm_slices(net.out_f[l]) * net.in_f[l];
+    npart = f > npart ? f : npart;
+    npart = b > npart ? b : npart;
+  }
+  return ((size_t)net.tot + net.maxw + npart) * MM_TA * sizeof(T);
+}
+
 // LDS of one workgroup of ta atoms: activations, deltas, and slice sums (slices * ta * width <= ta * max(MLP_BLOCK,
 // rounded width))
 template <typename T>
@@ -229,9 +413,17 @@ static bool upload_net(const StafMlp* mlp, int type, DevMlpNet* net) {
   net->n_af = staf_mlp_n_af(mlp, type);
   net->tot = net->n_af;
   net->maxw = net->n_af;
-  if (hipMalloc(&net->mu, net->n_af * sizeof(T)) != hipSuccess) return false;
-  if (hipMemcpy(net->mu, staf_mlp_internal_mu(mlp, type), net->n_af * sizeof(T), hipMemcpyHostToDevice) != hipSuccess)
-    return false;
+  // every parameter of the stack in one block (one upload, neighbouring pages): [mu | per layer W, Wt, b], each part
+  // on a 256-byte boundary
+  std::vector<T> host;
+  auto place = [&](const T* src, size_t n) {
+    const size_t at = (host.size() + 31) & ~(size_t)31;
+    host.resize(at + n, T(0));
+    for (size_t i = 0; i < n; i++) host[at + i] = src[i];
+    return at;
+  };
+  const size_t at_mu = place((const T*)staf_mlp_internal_mu(mlp, type), net->n_af);
+  size_t at_W[DEV_MLP_MAX_LAYERS], at_Wt[DEV_MLP_MAX_LAYERS], at_b[DEV_MLP_MAX_LAYERS];
   for (int l = 0; l < nl; l++) {
     const void *W, *b;
     if (staf_mlp_internal_layer(mlp, type, l, &net->act[l], &net->in_f[l], &net->out_f[l], &W, &b) != 0) return false;
@@ -242,17 +434,36 @@ static bool upload_net(const StafMlp* mlp, int type, DevMlpNet* net) {
     const T* w = (const T*)W;
     for (int i = 0; i < in_f; i++)
       for (int j = 0; j < out_f; j++) wt[(size_t)j * in_f + i] = w[(size_t)i * out_f + j];
-    const size_t nb = (size_t)in_f * out_f * sizeof(T);
-    if (hipMalloc(&net->W[l], nb) != hipSuccess || hipMalloc(&net->Wt[l], nb) != hipSuccess ||
-        hipMalloc(&net->b[l], out_f * sizeof(T)) != hipSuccess)
-      return false;
-    if (hipMemcpy(net->W[l], W, nb, hipMemcpyHostToDevice) != hipSuccess ||
-        hipMemcpy(net->Wt[l], wt.data(), nb, hipMemcpyHostToDevice) != hipSuccess ||
-        hipMemcpy(net->b[l], b, out_f * sizeof(T), hipMemcpyHostToDevice) != hipSuccess)
-      return false;
+    at_W[l] = place(w, (size_t)in_f * out_f);
+    at_Wt[l] = place(wt.data(), (size_t)in_f * out_f);
+    at_b[l] = place((const T*)b, out_f);
   }
-  // a stack too wide for the kernel's LDS is left to the host evaluation
-  return net->out_f[nl - 1] == 1 && net->in_f[0] == net->n_af && mlp_lds_bytes<T>(*net, MLP_TA_MAX) <= 64 * 1024;
+  T* block = nullptr;
+  if (hipMalloc((void**)&block, host.size() * sizeof(T)) != hipSuccess) return false;
+  net->mu = block;   // the block's address: freed through it
+  if (hipMemcpy(block, host.data(), host.size() * sizeof(T), hipMemcpyHostToDevice) != hipSuccess) return false;
+  (void)at_mu;       // 0: mu leads the block
+  for (int l = 0; l < nl; l++) {
+    net->W[l] = block + at_W[l];
+    net->Wt[l] = block + at_Wt[l];
+    net->b[l] = block + at_b[l];
+  }
+  if (net->out_f[nl - 1] != 1 || net->in_f[0] != net->n_af) return false;
+  // The matrix kernel needs more LDS than the 64 KB a kernel gets by default (160 KB per CU exist): ask once.
+  // (the attribute is per kernel, not per launch: it is kept at the largest request seen)
+  static size_t granted = 64 * 1024;
+  const size_t mm = mm_lds_bytes<T>(*net);
+  if (mm <= granted) {
+    net->matrix_path = true;
+  } else if (mm <= 152 * 1024 &&
+             hipFuncSetAttribute((const void*)mlp_matrix_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                 (int)mm) == hipSuccess) {
+    granted = mm;
+    net->matrix_path = true;
+  }
+  (void)hipGetLastError();
+  // a stack too wide for either kernel's LDS is left to the host evaluation
+  return net->matrix_path || mlp_lds_bytes<T>(*net, MLP_TA_MAX) <= 64 * 1024;
 }
 
 bool dev_mlp_upload(const StafMlp* mlp, int type, DevMlpNet* net) {
@@ -262,12 +473,7 @@ bool dev_mlp_upload(const StafMlp* mlp, int type, DevMlpNet* net) {
 }
 
 void dev_mlp_free(DevMlpNet* net) {
-  if (net->mu) (void)hipFree(net->mu);
-  for (int l = 0; l < DEV_MLP_MAX_LAYERS; l++) {
-    if (net->W[l]) (void)hipFree(net->W[l]);
-    if (net->Wt[l]) (void)hipFree(net->Wt[l]);
-    if (net->b[l]) (void)hipFree(net->b[l]);
-  }
+  if (net->mu) (void)hipFree(net->mu);   // one block holds mu and every layer
   *net = DevMlpNet();
 }
 
@@ -282,6 +488,17 @@ static int eval_net(const DevMlpNet& net, const double* af2, int Ar, const doubl
   }
   A.mu = (const T*)net.mu;
   A.af2 = af2; A.af3 = af3; A.e_atom = e_atom; A.g2 = g2; A.g3 = g3;
+  // Which kernel: one workgroup of either takes 25-35 us for the reference's 60-140-140-1 stack whatever its atom
+  // count (the weight matrices stream through its CU layer by layer), so the vector kernel (2-4 atoms a workgroup)
+  // serves up to ~1000 atoms in one round of workgroups and the matrix kernel (16 atoms) sixteen times as many; in
+  // single precision the matrix kernel is the faster one throughout.  STAF_MLP_VECTOR / STAF_MLP_MATRIX in the
+  // environment force one of them (tests).
+  const bool prefer_matrix = sizeof(T) == 4 || Nl > 1024 || getenv("STAF_MLP_MATRIX");
+  if (net.matrix_path && prefer_matrix && !getenv("STAF_MLP_VECTOR")) {
+    hipLaunchKernelGGL((mlp_matrix_kernel<T>), dim3((Nl + MM_TA - 1) / MM_TA), dim3(MM_BLOCK), mm_lds_bytes<T>(net),
+                       stream, A);
+    return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
+  }
   const int ta = Nl <= 2 * 256 ? 2 : 4;   // up to 256 workgroups (one per CU) take 2 atoms each
   const size_t lds = mlp_lds_bytes<T>(net, ta);
   if (lds > 64 * 1024) return STAF_E_LIMIT;

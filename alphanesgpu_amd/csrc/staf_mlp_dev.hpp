@@ -15,6 +15,7 @@ struct DevMlpNet {
   void* Wt[DEV_MLP_MAX_LAYERS] = {nullptr};
   void* b[DEV_MLP_MAX_LAYERS] = {nullptr};
   void* mu = nullptr;
+  bool matrix_path = false;   // the matrix-core kernel can hold this stack (LDS), else the vector kernel runs
 };
 
 bool dev_mlp_upload(const StafMlp* mlp, int type, DevMlpNet* net);   // false: not representable (fall back to host)

@@ -233,15 +233,53 @@ def test_device_mlp_matches_host_mlp(prec, tol):
     pos, box, types = load_water_smoke(np.float64)
     pos = pos.reshape(-1, 3)
     p = 1 if prec == "double" else 0
-    dev = libstaf.StafModel(os.path.join(GOLDEN, f"model_{prec}"), precision=p, full_virial=True)
     host = libstaf.StafModel(os.path.join(GOLDEN, f"model_{prec}"), precision=p, full_virial=True, host_mlp=True)
     e0, f0, v0 = host.compute(pos, box[0], types)
-    e1, f1, v1 = dev.compute(pos, box[0], types)
-    assert abs(e1 - e0) <= max(tol, 1e-6 if p == 0 else 0) * abs(e0)
-    assert nerr(f1, f0) <= tol
-    assert nerr(v1, v0) <= tol
-    dev.close()
     host.close()
+    # the kernel the library picks by itself, then each of its two device kernels (a handle of its own each: a
+    # handle replays what its first calls recorded)
+    for force in (None, "STAF_MLP_MATRIX", "STAF_MLP_VECTOR"):
+        if force:
+            os.environ[force] = "1"
+        try:
+            dev = libstaf.StafModel(os.path.join(GOLDEN, f"model_{prec}"), precision=p, full_virial=True)
+            e1, f1, v1 = dev.compute(pos, box[0], types)
+            dev.close()
+        finally:
+            if force:
+                os.environ.pop(force, None)
+        assert abs(e1 - e0) <= max(tol, 1e-6 if p == 0 else 0) * abs(e0), force
+        assert nerr(f1, f0) <= tol, force
+        assert nerr(v1, v0) <= tol, force
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("prec,tol", [("double", 1e-11), ("float", 2e-5)])
+def test_device_mlp_kernels_on_small_widths_and_ragged_atom_counts(tmp_path, prec, tol):
+    """Both device kernels of the network (the matrix-core one, 16 atoms per workgroup, and the vector one) against
+    the host evaluation on a written three-species model whose widths (fingerprints 9/7/11, hidden 20) are no
+    multiples of the tile sizes and whose atom counts (7, 9, 3) leave every workgroup partly empty: a wrong row
+    layout of the matrix tiles or a padding row entering a sum shows here, not on the 256/512-atom frames."""
+    from alphanesgpu_amd import libstaf, model_dir
+    from test_oracle_pins import cluster, small_model
+    ps = small_model(3, (5, 4, 6), (4, 3, 5, 3, 4, 3), seed=5, hidden=20, dense=True)
+    pos, box, tipos, type_map = cluster([7, 9, 3], seed=9)
+    model_dir.write_model_dir(str(tmp_path), ps, rc=4.5, rc_ang=3.2, rs=1.6, radial_buffer=24, angular_buffer=276,
+                              tipos=tipos, precision=prec)
+    p = 1 if prec == "double" else 0
+    host = libstaf.StafModel(str(tmp_path), precision=p, full_virial=True, host_mlp=True)
+    e0, f0, v0 = host.compute(pos.reshape(-1, 3), box[0], type_map)
+    host.close()
+    for force in ("STAF_MLP_MATRIX", "STAF_MLP_VECTOR"):      # the library picks by size and precision otherwise
+        os.environ[force] = "1"
+        try:
+            dev = libstaf.StafModel(str(tmp_path), precision=p, full_virial=True)
+            e1, f1, v1 = dev.compute(pos.reshape(-1, 3), box[0], type_map)
+            dev.close()
+        finally:
+            os.environ.pop(force, None)
+        assert abs(e1 - e0) <= max(tol, 1e-6 if p == 0 else 0) * abs(e0), force
+        assert nerr(f1, f0) <= tol and nerr(v1, v0) <= tol, force
 
 
 @pytest.mark.gpu
