@@ -481,3 +481,44 @@ def test_hip_graph_replay_with_two_streams_matches_eager():
     finally:
         ops.set_sync_errors(True)
 
+
+
+@pytest.mark.gpu
+def test_random_configurations(oracle):
+    """Twelve seeded random configurations through every op: 1-3 species with 1-13 atoms each (parameter rows and
+    classes of every shape), 1-3 frames, orthorhombic and triclinic boxes with the cluster shifted far outside the
+    cell, random cutoffs Rs < Ra <= Rc, channel counts 1-6 per block, an angular buffer anywhere between the atom
+    count and the full triangle (truncated triplet lists included), either precision, block or dense embeddings."""
+    rng = np.random.default_rng(20240611)
+    for case in range(12):
+        nt = int(rng.integers(1, 4))
+        tip = [int(x) for x in rng.integers(1, 14, nt)]
+        n = sum(tip)
+        nf = int(rng.integers(1, 4))
+        L = float(rng.uniform(9.5, 16.0))
+        spread = float(rng.uniform(2.2, 4.5))
+        tric = float(rng.random() < 0.5)
+        pos, box = np.zeros((nf, 3 * n)), np.zeros((nf, 6))
+        for b in range(nf):
+            pts = []
+            while len(pts) < n:
+                c = rng.uniform(-spread, spread, 3)
+                if all(np.linalg.norm(c - q) > 0.85 for q in pts):
+                    pts.append(c)
+            pos[b] = (np.array(pts) + rng.uniform(-30, 30, 3)).reshape(-1)
+            box[b] = [L, 0.6 * tric, -0.3 * tric, L + 0.7, 0.4 * tric, L + 1.3]
+        rc = float(rng.uniform(3.0, 4.6))
+        ra = float(rng.uniform(2.0, rc))
+        rs = float(rng.uniform(0.9, 0.5 * rc))
+        nr = n + 2
+        na = int(rng.integers(max(3, n), nr * (nr - 1) // 2 + 1))
+        ar = tuple(int(x) for x in rng.integers(1, 7, nt))
+        aa = tuple(int(x) for x in rng.integers(1, 7, nt * (nt + 1) // 2))
+        dtype = np.float64 if rng.random() < 0.6 else np.float32
+        dense = bool(rng.random() < 0.5)
+        try:
+            _generic_case(oracle, pos, box, tip, dtype, nr=nr, na=na, rc=rc, ra=ra, rs=rs, nt=nt, seed=case + 1,
+                          dense=dense, maps=(ar, aa))
+        except AssertionError as e:
+            raise AssertionError(f"case {case}: nt={nt} tipos={tip} nf={nf} rc={rc:.2f} ra={ra:.2f} rs={rs:.2f} "
+                                 f"nr={nr} na={na} ar={ar} aa={aa} {np.dtype(dtype).name} dense={dense}: {e}") from e
