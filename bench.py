@@ -33,6 +33,13 @@ TRAFFIC = {
     ("force3_kernel", "water768_f32"): 38.1e6,
     ("gradforce3_kernel", "water768_f64"): 95.2e6,
 }
+# Share of the GPU's vector-issue slots that the same kernel fills when launched alone (SQ_INSTS_VALU x 4 cycles over
+# duration x 1024 SIMDs x 2.4 GHz, time-weighted over the two per-species launches; profiles/*_sq_counters.txt):
+# the roofline these kernels actually run against, reported beside the HBM one
+VALU_ISSUE = {
+    ("force3_kernel", "water768_f32"): 0.53,
+    ("gradforce3_kernel", "water768_f64"): 0.55,
+}
 
 
 def algorithmic_bytes(N, tipos, nr, na, Ar, Aa, nt, s):
@@ -374,6 +381,7 @@ def main():
                    "species_streams": args.streams, "launch": "python per op" if graph is None else "hip graph replay"},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": TRAFFIC.get((dom, args.workload)),
+                     "valu_issue_share": VALU_ISSUE.get((dom, args.workload)),
                      "measured_copy_GBs": copy_gbs, "frac_of_measured_copy": achieved / copy_gbs,
                      "algorithmic_bytes_per_launch": dom_bytes_per_launch,
                      "avg_launch_ms": kern[dom]["avg_launch_ms"],
