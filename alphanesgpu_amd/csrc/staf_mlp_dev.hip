@@ -450,16 +450,18 @@ static bool upload_net(const StafMlp* mlp, int type, DevMlpNet* net) {
   }
   if (net->out_f[nl - 1] != 1 || net->in_f[0] != net->n_af) return false;
   // The matrix kernel needs more LDS than the 64 KB a kernel gets by default (160 KB per CU exist): ask once.
-  // (the attribute is per kernel, not per launch: it is kept at the largest request seen)
-  static size_t granted = 64 * 1024;
+  // (the attribute is per kernel, not per launch: it is set to the largest request seen, on the device in use)
+  static size_t largest = 0;
   const size_t mm = mm_lds_bytes<T>(*net);
-  if (mm <= granted) {
+  if (mm <= 64 * 1024) {
     net->matrix_path = true;
-  } else if (mm <= 152 * 1024 &&
-             hipFuncSetAttribute((const void*)mlp_matrix_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                 (int)mm) == hipSuccess) {
-    granted = mm;
-    net->matrix_path = true;
+  } else if (mm <= 152 * 1024) {
+    const size_t want = mm > largest ? mm : largest;
+    if (hipFuncSetAttribute((const void*)mlp_matrix_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)want) == hipSuccess) {
+      largest = want;
+      net->matrix_path = true;
+    }
   }
   (void)hipGetLastError();
   // a stack too wide for either kernel's LDS is left to the host evaluation
