@@ -95,6 +95,23 @@ int* bucket_reserve(DeviceState* st, size_t n_counters, size_t n_entries, hipStr
   return (int*)w->buckets.buf;
 }
 
+template <typename real>
+__global__ void add_n_kernel(real* dst, const real* a, const real* b, const real* c, const real* d, int n) {
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= n) return;
+  real s = a[e] + b[e];
+  if (c) s += c[e];
+  if (d) s += d[e];
+  dst[e] = s;
+}
+
+template <typename real>
+static int add_n(real* dst, const real* a, const real* b, const real* c, const real* d, int n, void* stream) {
+  if (!dst || !a || !b || n <= 0 || (d && !c)) return STAF_E_BAD_ARG;
+  hipLaunchKernelGGL(add_n_kernel<real>, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream, dst, a, b, c, d, n);
+  return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
+}
+
 static int decode_status(int bits) {
   if (bits & 1) return STAF_E_RADIAL_OVERFLOW;
   if (bits & 2) return STAF_E_SCATTER_OVERFLOW;
@@ -168,6 +185,15 @@ void staf_ops_release(void) {
   if (st->status_d) (void)hipFree(st->status_d);
   if (st->status_h) (void)hipHostFree(st->status_h);
   staf::g_state.erase(it);
+}
+
+int staf_op_add_n_f32(float* dst, const float* a, const float* b, const float* c, const float* d, int n,
+                      void* stream) {
+  return staf::add_n<float>(dst, a, b, c, d, n, stream);
+}
+int staf_op_add_n_f64(double* dst, const double* a, const double* b, const double* c, const double* d, int n,
+                      void* stream) {
+  return staf::add_n<double>(dst, a, b, c, d, n, stream);
 }
 
 int staf_op_init_force_radial(int buffdim) { return buffdim > 0 ? STAF_OK : STAF_E_BAD_ARG; }

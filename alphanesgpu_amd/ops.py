@@ -131,6 +131,25 @@ def descriptor_cell_threshold(n_atoms=2048):
     call("staf_op_descriptor_cell_threshold", _I(int(n_atoms)))
 
 
+def add_n(tensors, out=None):
+    """Sum of same-shaped tensors in one launch per four inputs, ((a + b) + c) + d in that order: the callers' sum of
+    the per-op force arrays (force_radial + force_angular, tf.math.add_n over the species)."""
+    ts = [_dense(t) for t in tensors]
+    if len(ts) == 1:
+        return ts[0].clone() if out is None else out.copy_(ts[0])
+    s, _ = sfx(ts[0].dtype)
+    out = torch.empty_like(ts[0]) if out is None else out
+    acc = None
+    while ts:
+        group = ([acc] if acc is not None else []) + ts[:4 - (acc is not None)]
+        ts = ts[4 - (acc is not None):]
+        group += [None] * (4 - len(group))
+        call(f"staf_op_add_n_{s}", ptr(out), ptr(group[0]), ptr(group[1]), ptr(group[2]), ptr(group[3]),
+             _I(out.numel()), _stream())
+        acc = out
+    return out
+
+
 def descriptor_coefficients(dtype=torch.float64):
     s, ct = sfx(dtype)
     out = (ct * 5)()

@@ -239,12 +239,12 @@ def main():
             timed("gradforce3", lambda: ops.compute_force_tripl_grad(Q, G3[k], supk, angk, d3sk, d3k, im2k, im3k,
                                                                      p["alpha3b"], p["emb3b"], tm, tp, at[k],
                                                                      ntrk), record)
-        return f2 + f3
+        return [f2, f3]
 
     def step(record=False, streams=side):
         d = timed("descriptor", lambda: ops.compute_descriptors_light(pos, box, out=dbuf), record)
         if streams is None:
-            parts = [species_chain(k, s, d, record) for k, s in enumerate(slices)]
+            parts = [f for k, s in enumerate(slices) for f in species_chain(k, s, d, record)]
         else:
             main_stream = torch.cuda.current_stream()   # the capture stream while a graph is recorded
             ready = main_stream.record_event()
@@ -252,16 +252,15 @@ def main():
             for k, s in enumerate(slices):
                 with torch.cuda.stream(streams[k]):
                     streams[k].wait_event(ready)
-                    f = species_chain(k, s, d, record)
-                    f.record_stream(main_stream)
-                    parts.append(f)
+                    for f in species_chain(k, s, d, record):
+                        f.record_stream(main_stream)
+                        parts.append(f)
                     done.append(streams[k].record_event())
             for ev in done:
                 main_stream.wait_event(ev)
-        Ftot = parts[0]
-        for f in parts[1:]:
-            Ftot = Ftot + f
-        return Ftot
+        # total force = sum of the per-op force arrays (the reference's force_radial + force_angular and add_n over
+        # the species), one launch
+        return ops.add_n(parts)
 
     # what a plain device copy reaches on this GPU (bytes read + bytes written per second): second roofline denominator;
     # the six 1 GiB copies (__amd_rocclr_copyBuffer) are also the reference point of the HBM traffic counters

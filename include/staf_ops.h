@@ -256,6 +256,15 @@ int staf_op_gradforce_tripl_f64(const double* prevgrad, const double* netderiv, 
                                 double* grad_emb3b, const double* prevgrad_virial, const double* pos,
                                 const double* box, int ld_atoms, void* stream);
 
+/* Sum of up to four arrays of n elements, dst[e] = ((a[e] + b[e]) + c[e]) + d[e] (c, d may be null), in one launch:
+ * what the callers do with the per-op force arrays (force_radial + force_angular in
+ * STAF/source_routine/force_layer_mod.py:43, tf.math.add_n over the species in
+ * STAF/staf_models/staf_model.py:210).  dst may be one of the inputs.  No counterpart among the reference's ops. */
+int staf_op_add_n_f32(float* dst, const float* a, const float* b, const float* c, const float* d, int n,
+                      void* stream);
+int staf_op_add_n_f64(double* dst, const double* a, const double* b, const double* c, const double* d, int n,
+                      void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -522,3 +522,23 @@ def test_random_configurations(oracle):
         except AssertionError as e:
             raise AssertionError(f"case {case}: nt={nt} tipos={tip} nf={nf} rc={rc:.2f} ra={ra:.2f} rs={rs:.2f} "
                                  f"nr={nr} na={na} ar={ar} aa={aa} {np.dtype(dtype).name} dense={dense}: {e}") from e
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_add_n_is_the_sequential_sum(dtype):
+    """ops.add_n (the callers' sum of per-op force arrays) against adding the arrays one after the other: same
+    order, same bits, for 1 to 9 inputs, also in place."""
+    import torch
+    from alphanesgpu_amd import ops
+    tdt = torch.float32 if dtype == np.float32 else torch.float64
+    g = torch.Generator(device="cpu").manual_seed(3)
+    xs = [torch.randn(2, 3001, generator=g, dtype=tdt).cuda() for _ in range(9)]
+    for n in range(1, 10):
+        want = xs[0].clone()
+        for x in xs[1:n]:
+            want = want + x
+        assert torch.equal(ops.add_n(xs[:n]), want), n
+    acc = xs[0].clone()
+    ops.add_n([acc, xs[1], xs[2]], out=acc)
+    assert torch.equal(acc, (xs[0] + xs[1]) + xs[2])
