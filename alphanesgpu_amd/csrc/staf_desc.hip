@@ -221,8 +221,10 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
   // LDS carve-up
   real* c_d2 = (real*)smem;            // [nr] candidate dist2
   real* c_d = c_d2 + nr;               // [3*nr] candidate delta (neighbour - centre)
-  // [nr][8] per sorted neighbour: unit vector centre - neighbour (3), 1/r, grad of fc wrt d (3), fc -- one record,
-  // so the angular fill reads a neighbour with two (fp32) or four (fp64) 16-byte LDS reads
+  // [8][nr] per sorted neighbour: unit vector centre - neighbour (3), 1/r, grad of fc wrt d (3), fc.  Component-
+  // major: the lanes of a wave hold consecutive triplets, i.e. one j and consecutive k, so a component of the k
+  // records is read from consecutive words (no bank conflict) and of the j record as a broadcast (records of 8
+  // components side by side cost 2-4 conflict cycles per read)
   real* s_rec = c_d + 3 * nr;
   int* c_j = (int*)(s_rec + 8 * nr);   // [nr] candidate index
   int* s_j = c_j + nr;                 // [nr] sorted neighbour index
@@ -415,15 +417,15 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
       A.des3bsupp[row + rank] = fc;
       im[1 + rank] = j;
       s_j[rank] = j;
-      s_rec[8 * rank + 3] = invr;
-      s_rec[8 * rank + 7] = fc;
+      s_rec[3 * nr + rank] = invr;
+      s_rec[7 * nr + rank] = fc;
 #pragma unroll
       for (int c = 0; c < 3; c++) {
         const real u = d[c] * invr;
         A.der2b[row3 + c * nr + rank] = dD * u;
         A.der3bsupp[row3 + c * nr + rank] = dfc * u;
-        s_rec[8 * rank + c] = u;
-        s_rec[8 * rank + 4 + c] = dfc * u;
+        s_rec[c * nr + rank] = u;
+        s_rec[(4 + c) * nr + rank] = dfc * u;
       }
     } else {
       A.raddescr[row + e] = 0;
@@ -461,7 +463,7 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
       tri_decode(nn, m, j, k);
       real rj[8], rk[8];
 #pragma unroll
-      for (int c = 0; c < 8; c++) { rj[c] = s_rec[8 * j + c]; rk[c] = s_rec[8 * k + c]; }
+      for (int c = 0; c < 8; c++) { rj[c] = s_rec[c * nr + j]; rk[c] = s_rec[c * nr + k]; }
       const real uj0 = rj[0], uj1 = rj[1], uj2 = rj[2];
       const real uk0 = rk[0], uk1 = rk[1], uk2 = rk[2];
       const real cs = uj0 * uk0 + uj1 * uk1 + uj2 * uk2;
