@@ -138,7 +138,11 @@ struct StafModel {
   // of the same shape has been evaluated eagerly (which also sizes every scratch buffer), then replayed: an MD run
   // repeats one shape for many steps, and issuing ~27 launches costs the host more than the GPU needs to run them.
   struct Replay {
-    int state = 0;             // 0: nothing, 1: shape seen once (eagerly), 2: graph ready
+    int state = 0;             // 0: nothing, 1: shape seen (eagerly), 2: graph ready
+    // Recording costs about as much as six replays save.  A shape is recorded when it has come `need` times in a
+    // row; a graph that was dropped young (the shape changed after few replays, as when atoms migrate between
+    // ranks every few steps) doubles `need`, one that lived long resets it.
+    int seen = 0, replays = 0, need = 2;
     int nlocal = 0, nall = 0, ext = 0, want_w = 0;
     std::vector<int> tipos;
     const void* in_d = nullptr;
@@ -544,16 +548,21 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
     const bool same = rp.state > 0 && rp.nlocal == nlocal && rp.nall == nall && rp.ext == (int)ext &&
                       rp.want_w == (int)want_w && rp.tipos == tipos && rp.in_d == m->in_d.p && rp.out_d == m->out_d.p;
     if (!m->use_graph || !same) {
+      if (rp.state == 2) rp.need = rp.replays < 12 ? (rp.need < 64 ? 2 * rp.need : 64) : 2;
       rp.drop();
       if (device_sequence() != 0) return -20;
       if (m->use_graph) {
         rp.state = 1;
+        rp.seen = 1;
+        rp.replays = 0;
         rp.nlocal = nlocal; rp.nall = nall; rp.ext = ext; rp.want_w = want_w; rp.tipos = tipos;
         rp.in_d = m->in_d.p; rp.out_d = m->out_d.p;
       }
+    } else if (rp.state == 1 && ++rp.seen < rp.need) {
+      if (device_sequence() != 0) return -20;
     } else {
       if (rp.state == 1) {
-        // second call of this shape: every buffer and scratch block has its final size, record the sequence
+        // the shape keeps coming and every buffer and scratch block has its final size: record the sequence
         STAF_HIP_OK(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
         const int issued = device_sequence();
         hipGraph_t g = nullptr;
@@ -572,6 +581,7 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
         rp.state = 2;
       }
       STAF_HIP_OK(hipGraphLaunch(rp.exec, st));
+      rp.replays++;
     }
   } else {
     if (descriptors() != 0) return -20;

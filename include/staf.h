@@ -27,9 +27,9 @@ typedef struct StafOptions {
   int precision;  /* 0 = the MLP runs in float32, 1 = float64 (descriptors, fingerprints, forces: always float64) */
   int reserved;   /* bit 0 set: fill all six virial components (reference: diagonal only, off-diagonals 0);
                    * bit 1 set: evaluate the MLP on the host between the kernels (default: on the GPU);
-                   * bit 2 set: launch every kernel of every call eagerly (default: from the second call of a shape
-                   *            -- same atom counts per species, same list mode -- the call's kernel sequence is
-                   *            recorded as a HIP graph and replayed) */
+                   * bit 2 set: launch every kernel of every call eagerly (default: once a shape -- same atom counts
+                   *            per species, same list mode -- has come twice in a row, more often if shapes change
+                   *            every few calls, the call's kernel sequence is recorded as a HIP graph and replayed) */
 } StafOptions;
 
 /* Defaults of the reference (libstaf/src/staf_api.cpp:39-45): ORT backend, device 0, float32 MLP. */

@@ -308,7 +308,9 @@ def test_replayed_calls_give_the_bits_of_eager_calls_and_follow_shape_changes():
     posA, boxA, _, tmA = load_frame_mbpol(np.float64)
     posB, boxB, typB = load_water_smoke(np.float64)
     rng = np.random.default_rng(17)
-    plan = [("A", True)] * 4 + [("B", True)] * 3 + [("A", True)] * 3 + [("A", False)] * 3 + [("B", False)] * 2
+    # (a shape is recorded after 2 calls in a row at first, after 4 and 8 once graphs have been dropped young: the
+    # runs below are long enough to be recorded and replayed each time)
+    plan = [("A", True)] * 4 + [("B", True)] * 3 + [("A", True)] * 7 + [("A", False)] * 10 + [("B", False)] * 2
     first = {}
     for step, (which, want_w) in enumerate(plan):
         pos, box, types = (posA, boxA[0], tmA) if which == "A" else (posB, boxB[0], typB)
