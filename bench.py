@@ -141,9 +141,10 @@ def main():
     ap.add_argument("--workload", default="water768_f32")
     ap.add_argument("--mode", default=None, choices=[None, "fwd_force", "full_step"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--streams", type=int, default=2, choices=[1, 2],
+    ap.add_argument("--streams", type=int, default=3, choices=[1, 2, 3],
                     help="2: the per-species op chains (independent until the forces are summed) are issued on one "
-                         "HIP stream per species; 1: everything on one stream")
+                         "HIP stream per species; 3: in addition the 2-body ops of the species with the most centres "
+                         "run on the step's own stream beside its 3-body ops; 1: everything on one stream")
     ap.add_argument("--no-graph", action="store_true",
                     help="launch every op of every step from Python instead of replaying one captured HIP graph")
     ap.add_argument("--contiguous-splits", action="store_true",
@@ -217,64 +218,104 @@ def main():
 
     side = [torch.cuda.Stream() for _ in range(nt)] if args.streams > 1 else None
 
-    def species_chain(k, s, d, record):
-        rad, ang, sup, im2, im3, d2, d3, d3s, ntr = d
-        p = P[k]
-        v = [sl(x, s) for x in (rad, ang, sup, im2, im3, d2, d3, d3s, ntr)]
+    # The ops of one centre species, by body order (2 / 3) and phase: 0 fingerprints, 1 forces, 2 parameter gradient
+    # of the energy branch, 3 gradient of the force op.  In a real step the network sits between phase 0 and 1
+    # and the loss between 1 and 2, so an op of a phase depends on both ops of the species' previous phase.
+    n_phase = 4 if mode == "full_step" else 2
+
+    def species_views(k, d):
+        return [sl(x, slices[k]) for x in d]
+
+    def body_op(k, v, body, phase, record):
         radk, angk, supk, im2k, im3k, d2k, d3k, d3sk, ntrk = v
-        timed("af2", lambda: ops.compute_sort_proj(radk, im2k, p["alpha2b"], p["emb2b"], tm), record)
-        timed("af3", lambda: ops.compute_sort_proj3body(angk, supk, im3k, im2k, p["alpha3b"], p["emb3b"], tm, ntrk,
-                                                        nt=nt), record)
-        f2 = timed("force2", lambda: ops.compute_force_radial(G2[k], d2k, im2k, radk, p["alpha2b"], p["emb2b"], tm,
-                                                              tp, at[k]), record)
-        f3 = timed("force3", lambda: ops.compute_force_tripl(G3[k], supk, angk, d3sk, d3k, im2k, im3k, p["alpha3b"],
-                                                             p["emb3b"], tm, tp, at[k], ntrk), record)
-        if mode == "full_step":
-            timed("grad2", lambda: ops.compute_two_body_par_grad(P2[k], radk, im2k, p["alpha2b"], p["emb2b"], tm),
-                  record)
-            timed("grad3", lambda: ops.compute_sort_proj3body_grad(P3[k], angk, supk, im3k, im2k, p["alpha3b"],
-                                                                   p["emb3b"], tm, ntrk, nt=nt), record)
-            timed("gradforce2", lambda: ops.compute_force_radial_grad(Q, G2[k], d2k, im2k, radk, p["alpha2b"],
-                                                                      p["emb2b"], tm, tp, at[k]), record)
-            timed("gradforce3", lambda: ops.compute_force_tripl_grad(Q, G3[k], supk, angk, d3sk, d3k, im2k, im3k,
-                                                                     p["alpha3b"], p["emb3b"], tm, tp, at[k],
-                                                                     ntrk), record)
-        return [f2, f3]
+        p = P[k]
+        if body == 2:
+            if phase == 0:
+                return timed("af2", lambda: ops.compute_sort_proj(radk, im2k, p["alpha2b"], p["emb2b"], tm), record)
+            if phase == 1:
+                return timed("force2", lambda: ops.compute_force_radial(G2[k], d2k, im2k, radk, p["alpha2b"],
+                                                                        p["emb2b"], tm, tp, at[k]), record)
+            if phase == 2:
+                return timed("grad2", lambda: ops.compute_two_body_par_grad(P2[k], radk, im2k, p["alpha2b"],
+                                                                            p["emb2b"], tm), record)
+            return timed("gradforce2", lambda: ops.compute_force_radial_grad(Q, G2[k], d2k, im2k, radk, p["alpha2b"],
+                                                                             p["emb2b"], tm, tp, at[k]), record)
+        if phase == 0:
+            return timed("af3", lambda: ops.compute_sort_proj3body(angk, supk, im3k, im2k, p["alpha3b"], p["emb3b"],
+                                                                   tm, ntrk, nt=nt), record)
+        if phase == 1:
+            return timed("force3", lambda: ops.compute_force_tripl(G3[k], supk, angk, d3sk, d3k, im2k, im3k,
+                                                                   p["alpha3b"], p["emb3b"], tm, tp, at[k], ntrk),
+                         record)
+        if phase == 2:
+            return timed("grad3", lambda: ops.compute_sort_proj3body_grad(P3[k], angk, supk, im3k, im2k,
+                                                                          p["alpha3b"], p["emb3b"], tm, ntrk, nt=nt),
+                         record)
+        return timed("gradforce3", lambda: ops.compute_force_tripl_grad(Q, G3[k], supk, angk, d3sk, d3k, im2k, im3k,
+                                                                        p["alpha3b"], p["emb3b"], tm, tp, at[k],
+                                                                        ntrk), record)
+
+    def species_chain(k, d, record, forces):
+        """af2, af3, force2, force3, (grad2, grad3, gradforce2, gradforce3) of species k on the current stream."""
+        v = species_views(k, d)
+        for phase in range(n_phase):
+            for body in (2, 3):
+                out = body_op(k, v, body, phase, record)
+                if phase == 1:
+                    forces[(k, body)] = out
+
+    big = int(np.argmax(tipos))   # the species with the most centres: its 3-body chain is the longest in the step
 
     def step(record=False, streams=side):
         d = timed("descriptor", lambda: ops.compute_descriptors_light(pos, box, out=dbuf), record)
+        forces = {}
         if streams is None:
-            parts = [f for k, s in enumerate(slices) for f in species_chain(k, s, d, record)]
+            for k in range(nt):
+                species_chain(k, d, record, forces)
         else:
             main_stream = torch.cuda.current_stream()   # the capture stream while a graph is recorded
             ready = main_stream.record_event()
-            parts, done = [], []
-            for k, s in enumerate(slices):
+            done = []
+            for k in range(nt):
+                if k == big and args.streams == 3:
+                    continue
                 with torch.cuda.stream(streams[k]):
                     streams[k].wait_event(ready)
-                    for f in species_chain(k, s, d, record):
-                        f.record_stream(main_stream)
-                        parts.append(f)
+                    species_chain(k, d, record, forces)
                     done.append(streams[k].record_event())
+            if args.streams == 3:
+                # The largest species in two chains: its 3-body ops on its own stream, its 2-body ops on the
+                # step's stream (idle otherwise until the forces are summed).  Phase by phase each chain waits for
+                # the other's previous op, which is the dependency the network and the loss create in a real step.
+                sb = streams[big]
+                v = species_views(big, d)
+                with torch.cuda.stream(sb):
+                    sb.wait_event(ready)
+                for phase in range(2):
+                    out2 = body_op(big, v, 2, phase, record)
+                    e2 = main_stream.record_event()
+                    with torch.cuda.stream(sb):
+                        out3 = body_op(big, v, 3, phase, record)
+                        e3 = sb.record_event()
+                    if phase == 1:
+                        forces[(big, 2)], forces[(big, 3)] = out2, out3
+                    if phase + 1 < n_phase:
+                        main_stream.wait_event(e3)
+                        sb.wait_event(e2)
+                # (the gradient ops all hang on the loss, not on each other: no wait between them)
+                for phase in range(2, n_phase):
+                    body_op(big, v, 2, phase, record)
+                with torch.cuda.stream(sb):
+                    for phase in range(2, n_phase):
+                        body_op(big, v, 3, phase, record)
+                done.append(sb.record_event())
             for ev in done:
                 main_stream.wait_event(ev)
+            for f in forces.values():
+                f.record_stream(main_stream)
         # total force = sum of the per-op force arrays (the reference's force_radial + force_angular and add_n over
-        # the species), one launch
-        return ops.add_n(parts)
-
-    # what a plain device copy reaches on this GPU (bytes read + bytes written per second): second roofline denominator;
-    # the six 1 GiB copies (__amd_rocclr_copyBuffer) are also the reference point of the HBM traffic counters
-    src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
-    dst = torch.empty_like(src)
-    dst.copy_(src)
-    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
-    ev[0].record()
-    for _ in range(5):
-        dst.copy_(src)
-    ev[1].record()
-    torch.cuda.synchronize()
-    copy_gbs = 5 * 2 * src.numel() * 4 / (ev[0].elapsed_time(ev[1]) * 1e-3) / 1e9
-    del src, dst
+        # the species), one launch, always in the same order
+        return ops.add_n([forces[(k, body)] for k in range(nt) for body in (2, 3)])
 
     # One step = one replay of a HIP graph that holds the whole op sequence (the ops run on the stream they are
     # called on, so stream capture records their kernels; scratch is grown by the eager warm-up steps first).
@@ -334,6 +375,21 @@ def main():
     op_ms = {k: float(np.mean([a.elapsed_time(b) for a, b in v])) for k, v in timers.items()}
     calls = {k: len(v) // nprof for k, v in timers.items()}
 
+    # what a plain device copy reaches on this GPU (bytes read + bytes written per second): second roofline denominator
+    # (measured after the timed steps: six GiB of copies just before them would not leave the GPU as it was);
+    # the six 1 GiB copies (__amd_rocclr_copyBuffer) are also the reference point of the HBM traffic counters
+    src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    ev[0].record()
+    for _ in range(5):
+        dst.copy_(src)
+    ev[1].record()
+    torch.cuda.synchronize()
+    copy_gbs = 5 * 2 * src.numel() * 4 / (ev[0].elapsed_time(ev[1]) * 1e-3) / 1e9
+    del src, dst
+
     # per-kernel GPU time from the library's own HIP events, recorded on the stream each kernel is launched on
     ops.kernel_timing(True)
     for _ in range(nprof):
@@ -377,7 +433,11 @@ def main():
         "config": {"workload": args.workload, "mode": mode, "atoms": N, "frames_per_step": nf, "Rc": synth.RC,
                    "radial_buffer": nr, "angular_buffer": na, "Ar": Ar, "Aa": Aa,
                    "species_tensors": "contiguous copies" if args.contiguous_splits else "views",
-                   "species_streams": args.streams, "launch": "python per op" if graph is None else "hip graph replay"},
+                   "species_streams": args.streams,
+                   "schedule": {1: "one stream", 2: "one stream per species",
+                                3: "one stream per species, 2-body ops of the largest species on the step's stream"
+                                }[args.streams],
+                   "launch": "python per op" if graph is None else "hip graph replay"},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": TRAFFIC.get((dom, args.workload)),
                      "valu_issue_share": VALU_ISSUE.get((dom, args.workload)),
