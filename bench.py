@@ -36,6 +36,7 @@ TRAFFIC = {
 # Share of the GPU's vector-issue slots that the same kernel fills when launched alone (SQ_INSTS_VALU x 4 cycles over
 # duration x 1024 SIMDs x 2.4 GHz, time-weighted over the two per-species launches; profiles/*_sq_counters.txt):
 # the roofline these kernels actually run against, reported beside the HBM one
+SETTLE_STEPS = 300   # untimed graph replays of the set-up, see main()
 VALU_ISSUE = {
     ("force3_kernel", "water768_f32"): 0.53,
     ("gradforce3_kernel", "water768_f64"): 0.55,
@@ -136,7 +137,7 @@ def cpu_baseline(batch, params, up, mode, nr, na, max_frames=2, threads=16):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="water768_f32")
     ap.add_argument("--mode", default=None, choices=[None, "fwd_force", "full_step"])
@@ -336,6 +337,11 @@ def main():
         with torch.cuda.graph(graph, stream=cap):
             graph_out = step()
         run = graph.replay
+    # A fresh process finds the GPU at idle clocks, and a few steps of 0.15-0.5 ms do not bring it to its working
+    # clocks (the first fifty steps run 4-5 % slower than the steady state a training run is in): part of the set-up
+    # is a run of untimed steps, beside the caller's own warm-up steps.
+    for _ in range(SETTLE_STEPS if graph is not None else 20):
+        run()
     for _ in range(args.warmup):
         run()
     ops.poll_status()
