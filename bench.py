@@ -277,39 +277,47 @@ def main():
             main_stream = torch.cuda.current_stream()   # the capture stream while a graph is recorded
             ready = main_stream.record_event()
             done = []
-            for k in range(nt):
-                if k == big and args.streams == 3:
-                    continue
-                with torch.cuda.stream(streams[k]):
-                    streams[k].wait_event(ready)
-                    species_chain(k, d, record, forces)
-                    done.append(streams[k].record_event())
+
+            def small_species():
+                for k in sorted(range(nt), key=lambda k: -tipos[k]):
+                    if k == big and args.streams == 3:
+                        continue
+                    with torch.cuda.stream(streams[k]):
+                        streams[k].wait_event(ready)
+                        species_chain(k, d, record, forces)
+                        done.append(streams[k].record_event())
+
             if args.streams == 3:
                 # The largest species in two chains: its 3-body ops on its own stream, its 2-body ops on the
-                # step's stream (idle otherwise until the forces are summed).  Phase by phase each chain waits for
-                # the other's previous op, which is the dependency the network and the loss create in a real step.
+                # step's stream (idle otherwise until the forces are summed).  Each chain's force op waits for the
+                # other's fingerprint op, the dependency the network creates in a real step.  (The gradient ops take
+                # their upstream gradients as given, here as in the per-species chains: no wait between them.)
+                # Issue order = the order in which a graph replay submits the chains: the longest one (the 3-body ops
+                # of the largest species) goes first, so that it starts right behind the descriptors, the other
+                # species' chains last (issued between the two, they held back the large species' 2-body ops
+                # until they were through).
                 sb = streams[big]
                 v = species_views(big, d)
-                with torch.cuda.stream(sb):
-                    sb.wait_event(ready)
                 for phase in range(2):
-                    out2 = body_op(big, v, 2, phase, record)
-                    e2 = main_stream.record_event()
                     with torch.cuda.stream(sb):
+                        if phase == 0:
+                            sb.wait_event(ready)
                         out3 = body_op(big, v, 3, phase, record)
                         e3 = sb.record_event()
-                    if phase == 1:
-                        forces[(big, 2)], forces[(big, 3)] = out2, out3
-                    if phase + 1 < n_phase:
+                    out2 = body_op(big, v, 2, phase, record)
+                    e2 = main_stream.record_event()
+                    if phase == 0:
                         main_stream.wait_event(e3)
                         sb.wait_event(e2)
-                # (the gradient ops all hang on the loss, not on each other: no wait between them)
-                for phase in range(2, n_phase):
-                    body_op(big, v, 2, phase, record)
+                    else:
+                        forces[(big, 2)], forces[(big, 3)] = out2, out3
                 with torch.cuda.stream(sb):
                     for phase in range(2, n_phase):
                         body_op(big, v, 3, phase, record)
-                done.append(sb.record_event())
+                    done.append(sb.record_event())
+                for phase in range(2, n_phase):
+                    body_op(big, v, 2, phase, record)
+            small_species()
             for ev in done:
                 main_stream.wait_event(ev)
             for f in forces.values():
