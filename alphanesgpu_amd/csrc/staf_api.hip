@@ -18,6 +18,7 @@
 #include <string.h>
 
 #include <string>
+#include <algorithm>
 #include <vector>
 
 extern "C" void staf_op_force_set_skip_pbc(int skip);
@@ -487,11 +488,18 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
     // -- also when it replays a recorded graph -- submits launches one after the other, and a chain issued as a
     // whole would have run before the next one is even submitted.
     int nops = 0;
+    // Within a step the species with the most atoms comes first: launches (and the nodes of a replayed graph) are
+    // submitted in issue order, and the longest chain should not be the one that starts last.
+    std::vector<int> first_atom(nt, 0), op_slot(nt, 0), by_size;
+    for (int k = 0, at = 0, sl = 0; k < nt; at += tipos[k], k++) {
+      first_atom[k] = at;
+      if (tipos[k] > 0) { op_slot[k] = sl++; by_size.push_back(k); }
+    }
+    std::stable_sort(by_size.begin(), by_size.end(), [&](int a, int b) { return tipos[a] > tipos[b]; });
     for (int step = 0; step < 5; step++) {
-      int shift = 0, slot = 0;
-      for (int k = 0; k < nt; shift += tipos[k], k++) {
+      for (int k : by_size) {
         const int Nl = tipos[k], Ar = m->Ar[k], Aa = m->Aa[k];
-        if (Nl == 0) continue;
+        const int shift = first_atom[k], slot = op_slot[k];
         hipStream_t sk = m->sstream[k];
         const size_t o = (size_t)shift;
         double* af2 = m->af2.p + o * amax2;
@@ -499,7 +507,6 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
         double* g2 = m->g2.p + o * amax2;
         double* g3 = m->g3.p + o * amax3;
         const int op = 2 * slot + (step - 3);          // output slot of the force ops (steps 3 and 4)
-        slot++;
         double* fo = m->force_op.p + (size_t)(op < 0 ? 0 : op) * n3;
         double* wo = want_w ? m->virial_op.p + (op < 0 ? 0 : op) * 9 : nullptr;
         const double* px = want_w ? d_pos : nullptr;
