@@ -163,6 +163,7 @@ static inline int grad_blocks(int atoms) {
 template <typename real>
 static int radial_afs(const real* D, int nr, const real* alpha2b, int Ar, real* out, int nf, int Nl, const int* im2,
                       const real* emb2b, const int* type_map, int nt, int ld, void* stream_) {
+  if (Nl == 0 && nf > 0 && Ar > 0) return STAF_OK;   // a species without atoms in these frames: nothing to write
   if (!D || !alpha2b || !out || !im2 || !emb2b || !type_map || nr <= 0 || Ar <= 0 || nf <= 0 || Nl <= 0 || nt <= 0)
     return STAF_E_BAD_ARG;
   if (nt > NT_MAX) return STAF_E_LIMIT;
@@ -182,6 +183,12 @@ template <typename real>
 static int alpha_dist_grad(const real* D, int nr, const real* alpha2b, int Ar, real* g_alpha, int nf, int Nl,
                            const int* im2, const real* P, const real* emb2b, const int* type_map, real* g_emb, int nt,
                            int ld, void* stream_) {
+  if (Nl == 0 && nf > 0 && Ar > 0 && nt > 0 && g_alpha && g_emb) {
+    // a species without atoms in these frames: its sums are empty
+    launch_fill_zero<real>(g_alpha, nt * Ar, (hipStream_t)stream_);
+    launch_fill_zero<real>(g_emb, nt * Ar, (hipStream_t)stream_);
+    return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
+  }
   if (!D || !alpha2b || !g_alpha || !g_emb || !im2 || !P || !emb2b || !type_map || nr <= 0 || Ar <= 0 || nf <= 0 ||
       Nl <= 0 || nt <= 0)
     return STAF_E_BAD_ARG;
@@ -212,6 +219,7 @@ static int angular_afs(const real* Dsup, const real* Tang, int nr, int na, real*
                        const int* im2, const real* alpha3b, int Aa, const real* emb3b, const int* type_map,
                        const int* numtriplet, int nt, int ld, void* stream_) {
   (void)im3;
+  if (Nl == 0 && nf > 0 && Aa > 0) return STAF_OK;   // a species without atoms in these frames: nothing to write
   if (!Dsup || !Tang || !out || !im2 || !alpha3b || !emb3b || !type_map || !numtriplet || nr <= 0 || na <= 0 ||
       Aa <= 0 || nf <= 0 || Nl <= 0 || nt <= 0)
     return STAF_E_BAD_ARG;
@@ -236,6 +244,12 @@ static int alphagrad_ang(const real* Dsup, const real* Tang, int nr, int na, con
                          const real* emb3b, const int* type_map, real* g_emb, const int* numtriplet, int ntc, int nt,
                          int ld, void* stream_) {
   (void)im3;
+  if (Nl == 0 && nf > 0 && Aa > 0 && nt > 0 && ntc >= 2 * nt - 1 && g_alpha && g_emb) {
+    // a species without atoms in these frames: its sums are empty
+    launch_fill_zero<real>(g_alpha, ntc * Aa * 3, (hipStream_t)stream_);
+    launch_fill_zero<real>(g_emb, ntc * Aa, (hipStream_t)stream_);
+    return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
+  }
   if (!Dsup || !Tang || !P || !im2 || !alpha3b || !g_alpha || !g_emb || !emb3b || !type_map || !numtriplet ||
       nr <= 0 || na <= 0 || Aa <= 0 || nf <= 0 || Nl <= 0 || nt <= 0 || ntc < 2 * nt - 1)
     return STAF_E_BAD_ARG;

@@ -407,15 +407,32 @@ static int launch_gather(DeviceState* st, const ForceScratch& fs, const int* tip
   return finish_op(st, stream);
 }
 
+// A species without atoms in these frames contributes no force (and no virial): the op still fills its outputs.
+template <typename real>
+static int empty_species_force(real* force, real* virial, int nf, int N, void* stream_) {
+  launch_fill_zero<real>(force, nf * 3 * N, (hipStream_t)stream_);
+  if (virial) launch_fill_zero<real>(virial, nf * 9, (hipStream_t)stream_);
+  return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
+}
+
+// The same for the gradient of a force op: no centre, so the sums over centres are empty and gradnet has no rows.
+template <typename real>
+static int empty_species_grad(real* g_alpha, int n_alpha, real* g_emb, int n_emb, void* stream_) {
+  launch_fill_zero<real>(g_alpha, n_alpha, (hipStream_t)stream_);
+  launch_fill_zero<real>(g_emb, n_emb, (hipStream_t)stream_);
+  return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
+}
+
 template <typename real>
 static int force_doublets(const real* G, const real* D, const real* dD, const int* im2, int nr, int N, int nf, int Ar,
                           const real* alpha2b, const real* emb2b, int nt, const int* tipos, const int* actual_type,
                           real* force, const int* type_map, int Nl, real* virial, const real* pos, const real* box,
                           int ld, void* stream_) {
+  if ((virial || pos || box) && !(virial && pos && box)) return STAF_E_BAD_ARG;
+  if (Nl == 0 && nf > 0 && N > 0 && force) return empty_species_force<real>(force, virial, nf, N, stream_);
   if (!G || !D || !dD || !im2 || !alpha2b || !emb2b || !tipos || !actual_type || !force || !type_map || nr <= 0 ||
       N <= 0 || nf <= 0 || Ar <= 0 || nt <= 0 || Nl <= 0 || Nl > N)
     return STAF_E_BAD_ARG;
-  if ((virial || pos || box) && !(virial && pos && box)) return STAF_E_BAD_ARG;
   if (nt > NT_MAX) return STAF_E_LIMIT;
   if (ld <= 0) ld = Nl;
   DeviceState* st = device_state();
@@ -445,10 +462,11 @@ static int force_tripl(const real* G, const real* Dsup, const real* Tang, const 
                        const real* alpha3b, const int* type_map, int Nl, real* virial, const real* pos,
                        const real* box, int ld, void* stream_) {
   (void)im3;
+  if ((virial || pos || box) && !(virial && pos && box)) return STAF_E_BAD_ARG;
+  if (Nl == 0 && nf > 0 && N > 0 && force) return empty_species_force<real>(force, virial, nf, N, stream_);
   if (!G || !Dsup || !Tang || !dDsup || !d3b || !im2 || !emb3b || !tipos || !actual_type || !force || !numtriplet ||
       !alpha3b || !type_map || nr <= 0 || na <= 0 || N <= 0 || nf <= 0 || Aa <= 0 || nt <= 0 || Nl <= 0 || Nl > N)
     return STAF_E_BAD_ARG;
-  if ((virial || pos || box) && !(virial && pos && box)) return STAF_E_BAD_ARG;
   if (nt > NT_MAX) return STAF_E_LIMIT;
   if (ld <= 0) ld = Nl;
   DeviceState* st = device_state();
@@ -481,10 +499,12 @@ static int gradforce_2b(const real* Q, const real* D, int nr, const real* alpha2
                         const int* im2, int nf, int N, int Nl, const real* G, const real* emb2b, int nt,
                         const int* type_map, const int* tipos, const int* actual_type, real* gnet, real* g_alpha,
                         real* g_emb, const real* Qvir, const real* pos, const real* box, int ld, void* stream_) {
+  if ((Qvir || pos || box) && !(Qvir && pos && box)) return STAF_E_BAD_ARG;
+  if (Nl == 0 && nf > 0 && Ar > 0 && nt > 0 && g_alpha && g_emb)
+    return empty_species_grad<real>(g_alpha, nt * Ar, g_emb, nt * Ar, stream_);
   if (!Q || !D || !alpha2b || !dD || !im2 || !G || !emb2b || !type_map || !tipos || !actual_type || !gnet ||
       !g_alpha || !g_emb || nr <= 0 || Ar <= 0 || nf <= 0 || N <= 0 || Nl <= 0 || Nl > N || nt <= 0)
     return STAF_E_BAD_ARG;
-  if ((Qvir || pos || box) && !(Qvir && pos && box)) return STAF_E_BAD_ARG;
   if (nt > NT_MAX) return STAF_E_LIMIT;
   if (ld <= 0) ld = Nl;
   DeviceState* st = device_state();
@@ -515,11 +535,15 @@ static int gradforce_tripl(const real* Q, const real* G, const real* Dsup, const
                            const real* alpha3b, const int* type_map, int Nl, real* gnet, real* g_alpha, real* g_emb,
                            const real* Qvir, const real* pos, const real* box, int ld, void* stream_) {
   (void)im3;
+  if ((Qvir || pos || box) && !(Qvir && pos && box)) return STAF_E_BAD_ARG;
+  if (Nl == 0 && nf > 0 && Aa > 0 && nt > 0 && g_alpha && g_emb) {
+    const int ntc = nt * (nt + 1) / 2;
+    return empty_species_grad<real>(g_alpha, ntc * Aa * 3, g_emb, ntc * Aa, stream_);
+  }
   if (!Q || !G || !Dsup || !Tang || !dDsup || !d3b || !im2 || !emb3b || !tipos || !actual_type || !numtriplet ||
       !alpha3b || !type_map || !gnet || !g_alpha || !g_emb || nr <= 0 || na <= 0 || N <= 0 || nf <= 0 || Aa <= 0 ||
       nt <= 0 || Nl <= 0 || Nl > N)
     return STAF_E_BAD_ARG;
-  if ((Qvir || pos || box) && !(Qvir && pos && box)) return STAF_E_BAD_ARG;
   if (nt > NT_MAX) return STAF_E_LIMIT;
   if (ld <= 0) ld = Nl;
   DeviceState* st = device_state();

@@ -26,6 +26,10 @@
  *     pointers, as the reference ops receive them.
  *   - type-embedding arguments are the SQUARED embeddings (the reference's
  *     Python layers square them before the op call).
+ *   - N_local = 0 (a species with no atom in these frames) is a valid call of
+ *     the per-species ops: fingerprint ops write nothing, force ops fill force
+ *     (and virial) with zeros, gradient ops fill the parameter gradients with
+ *     zeros; the other pointers are not read.
  *   - state is per device and not re-entrant: calls on one device must be
  *     ordered on one stream at a time.
  */

@@ -542,3 +542,26 @@ def test_add_n_is_the_sequential_sum(dtype):
     acc = xs[0].clone()
     ops.add_n([acc, xs[1], xs[2]], out=acc)
     assert torch.equal(acc, (xs[0] + xs[1]) + xs[2])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_species_without_atoms(oracle, dtype):
+    """A three-species parameter set on frames that hold no atom of the middle species: its ops are called with an
+    empty centre range, write nothing (fingerprints), zeros (forces, virial, parameter gradients), and the other
+    species' results are those of the oracle."""
+    import torch
+    from alphanesgpu_amd import ops
+    rng = np.random.default_rng(8)
+    tip = [6, 0, 7]
+    n = sum(tip)
+    pts = []
+    while len(pts) < n:
+        c = rng.uniform(-3.0, 3.0, 3)
+        if all(np.linalg.norm(c - q) > 0.9 for q in pts):
+            pts.append(c)
+    pos = np.array(pts).reshape(1, -1)
+    box = np.array([[13.0, 0, 0, 14.0, 0, 15.0]])
+    errs, ref = _generic_case(oracle, pos, box, tip, dtype, nr=16, na=60, rc=4.5, ra=3.5, rs=1.5, nt=3, dense=True,
+                              maps=((3, 2, 4), (2, 3, 2, 2, 3, 2)))
+    assert ref["af2"][1].shape[1] == 0 and not ref["f2"][1].any() and not ref["gf3"][1][1].any()
