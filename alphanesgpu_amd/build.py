@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libstaf_hip.so")
 SOURCES = ["staf_runtime.hip", "staf_desc.hip", "staf_af.hip", "staf_force.hip", "staf_api.hip", "staf_mlp_dev.hip", "staf_mlp.cpp"]
-HEADERS = ["staf_common.hpp", "staf_tile.hpp", "staf_reduce.hpp", "staf_tri.hpp", "staf_force3.hpp", "staf_mlp_dev.hpp", "staf_mlp_internal.h", os.path.join("..", "..", "include", "staf_ops.h"),
+HEADERS = ["staf_common.hpp", "staf_tile.hpp", "staf_reduce.hpp", "staf_tri.hpp", "staf_force3.hpp", "staf_transpose.hpp", "staf_mlp_dev.hpp", "staf_mlp_internal.h", os.path.join("..", "..", "include", "staf_ops.h"),
            os.path.join("..", "..", "include", "staf.h"), os.path.join("..", "..", "include", "staf_mlp.h")]
 ARCH = "gfx950"
 # packed-fp32 instructions are switched off for all device code

@@ -194,14 +194,14 @@ static int alpha_dist_grad(const real* D, int nr, const real* alpha2b, int Ar, r
     return STAF_E_BAD_ARG;
   if (nt > NT_MAX) return STAF_E_LIMIT;
   if (ld <= 0) ld = Nl;
-  DeviceState* st = device_state();
-  if (!st) return STAF_E_HIP;
+  DeviceState* st = device_state((hipStream_t)stream_);
+  if (!st) return reserve_failure((hipStream_t)stream_);
   hipStream_t stream = (hipStream_t)stream_;
   const int nout = 2 * nt * Ar;
   const int nb = grad_blocks(nf * Nl);
   real* partial = (real*)scratch_reserve(st, stream, ((size_t)nb + RED_SLICES) * nout * sizeof(real));
   real* red_tmp = partial ? partial + (size_t)nb * nout : nullptr;
-  if (!partial) return STAF_E_HIP;
+  if (!partial) return reserve_failure(stream);
   size_t lds = (size_t)(2 * nt * Ar + AF_WAVES * nout + AF_WAVES * nr) * sizeof(real) +
                (size_t)AF_WAVES * (2 * nr + NT_MAX + 1) * sizeof(int);
   if (lds > 64 * 1024) return STAF_E_LIMIT;
@@ -255,15 +255,15 @@ static int alphagrad_ang(const real* Dsup, const real* Tang, int nr, int na, con
     return STAF_E_BAD_ARG;
   if (nt > NT_MAX) return STAF_E_LIMIT;
   if (ld <= 0) ld = Nl;
-  DeviceState* st = device_state();
-  if (!st) return STAF_E_HIP;
+  DeviceState* st = device_state((hipStream_t)stream_);
+  if (!st) return reserve_failure((hipStream_t)stream_);
   hipStream_t stream = (hipStream_t)stream_;
   const int nsig = 2 * nt - 1;
   const int nout = nsig * Aa * 3;
   const int nb = nf * Nl < TRI_GRID_MAX ? nf * Nl : TRI_GRID_MAX;
   real* partial = (real*)scratch_reserve(st, stream, ((size_t)nb + RED_SLICES) * nout * sizeof(real));
   real* red_tmp = partial ? partial + (size_t)nb * nout : nullptr;
-  if (!partial) return STAF_E_HIP;
+  if (!partial) return reserve_failure(stream);
   size_t lds = TriLds<real, 1>::bytes(nr, Aa, nt);
   if (lds > 64 * 1024) return STAF_E_LIMIT;
   // rows sigma >= nsig of the outputs receive no contribution

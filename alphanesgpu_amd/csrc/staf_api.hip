@@ -21,8 +21,6 @@
 #include <algorithm>
 #include <vector>
 
-extern "C" void staf_op_force_set_skip_pbc(int skip);
-
 namespace {
 
 template <typename T>
@@ -474,7 +472,7 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
   double W[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
   const int n3 = nall * 3;
   const bool want_w = virial != nullptr;
-  staf_op_force_set_skip_pbc(ext ? 1 : 0);
+  const int skip_pbc = ext ? 1 : 0;   // the caller's neighbours are explicit periodic images
   // ---- everything stays on the device: per species fingerprints -> MLP -> forces, one stream per species (the
   // chains meet only in the sum of the forces); one synchronisation at the end of the call
   auto device_sequence = [&]() -> int {
@@ -525,18 +523,18 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
             rc = staf::dev_mlp_eval(m->dnets[k], af2, Ar, af3, Aa, Nl, d_e + o, g2, g3, sk);
             break;
           case 3:
-            rc = staf_op_force_doublets_f64(g2, m->raddescr.p + o * nr, m->der2b.p + o * 3 * nr,
-                                            m->intmap2b.p + o * (nr + 1), nr, nall, 1, Ar, m->alpha2b[k].p,
-                                            m->emb2b[k].p, nt, m->tipos.p, m->actual_type.p + k, fo, m->type_map.p,
-                                            Nl, wo, px, bx, nlocal, sk);
+            rc = staf::force_doublets<double>(g2, m->raddescr.p + o * nr, m->der2b.p + o * 3 * nr,
+                                              m->intmap2b.p + o * (nr + 1), nr, nall, 1, Ar, m->alpha2b[k].p,
+                                              m->emb2b[k].p, nt, m->tipos.p, m->actual_type.p + k, fo, m->type_map.p,
+                                              Nl, wo, px, bx, nlocal, skip_pbc, sk);
             break;
           default:
-            rc = staf_op_force_tripl_f64(g3, m->des3bsupp.p + o * nr, m->angdescr.p + o * na,
-                                         m->der3bsupp.p + o * 3 * nr, m->der3b.p + o * 6 * na,
-                                         m->intmap2b.p + o * (nr + 1), m->intmap3b.p + o * 2 * na, nr, na, nall, 1,
-                                         Aa, m->emb3b[k].p, nt, m->tipos.p, m->actual_type.p + k, fo,
-                                         m->numtriplet.p + o, m->alpha3b[k].p, m->type_map.p, Nl, wo, px, bx, nlocal,
-                                         sk);
+            rc = staf::force_tripl<double>(g3, m->des3bsupp.p + o * nr, m->angdescr.p + o * na,
+                                           m->der3bsupp.p + o * 3 * nr, m->der3b.p + o * 6 * na,
+                                           m->intmap2b.p + o * (nr + 1), m->intmap3b.p + o * 2 * na, nr, na, nall, 1,
+                                           Aa, m->emb3b[k].p, nt, m->tipos.p, m->actual_type.p + k, fo,
+                                           m->numtriplet.p + o, m->alpha3b[k].p, m->type_map.p, Nl, wo, px, bx, nlocal,
+                                           skip_pbc, sk);
             STAF_HIP_OK(hipEventRecord(m->ev_join[k], sk));
             break;
         }
@@ -674,17 +672,17 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
       STAF_HIP_OK(hipStreamSynchronize(st));
       for (int body = 2; body <= 3; body++) {
         if (body == 2)
-          rc = staf_op_force_doublets_f64(m->g2.p, m->raddescr.p + o * nr, m->der2b.p + o * 3 * nr,
-                                          m->intmap2b.p + o * (nr + 1), nr, nall, 1, Ar, m->alpha2b[k].p, m->emb2b[k].p,
-                                          nt, m->tipos.p, m->actual_type.p + k, m->force_op.p, m->type_map.p, Nl,
-                                          m->virial_op.p, d_pos, d_box, nlocal, st);
+          rc = staf::force_doublets<double>(m->g2.p, m->raddescr.p + o * nr, m->der2b.p + o * 3 * nr,
+                                            m->intmap2b.p + o * (nr + 1), nr, nall, 1, Ar, m->alpha2b[k].p,
+                                            m->emb2b[k].p, nt, m->tipos.p, m->actual_type.p + k, m->force_op.p,
+                                            m->type_map.p, Nl, m->virial_op.p, d_pos, d_box, nlocal, skip_pbc, st);
         else
-          rc = staf_op_force_tripl_f64(m->g3.p, m->des3bsupp.p + o * nr, m->angdescr.p + o * na,
-                                       m->der3bsupp.p + o * 3 * nr, m->der3b.p + o * 6 * na,
-                                       m->intmap2b.p + o * (nr + 1), m->intmap3b.p + o * 2 * na, nr, na, nall, 1, Aa,
-                                       m->emb3b[k].p, nt, m->tipos.p, m->actual_type.p + k, m->force_op.p,
-                                       m->numtriplet.p + o, m->alpha3b[k].p, m->type_map.p, Nl, m->virial_op.p,
-                                       d_pos, d_box, nlocal, st);
+          rc = staf::force_tripl<double>(m->g3.p, m->des3bsupp.p + o * nr, m->angdescr.p + o * na,
+                                         m->der3bsupp.p + o * 3 * nr, m->der3b.p + o * 6 * na,
+                                         m->intmap2b.p + o * (nr + 1), m->intmap3b.p + o * 2 * na, nr, na, nall, 1, Aa,
+                                         m->emb3b[k].p, nt, m->tipos.p, m->actual_type.p + k, m->force_op.p,
+                                         m->numtriplet.p + o, m->alpha3b[k].p, m->type_map.p, Nl, m->virial_op.p,
+                                         d_pos, d_box, nlocal, skip_pbc, st);
         if (rc != STAF_OK) return -20;
         hipLaunchKernelGGL(add_into_kernel, dim3((n3 + 255) / 256), dim3(256), 0, st, d_force, m->force_op.p, n3);
         STAF_HIP_OK(hipMemcpyAsync(Wk, m->virial_op.p, 9 * sizeof(double), hipMemcpyDeviceToHost, st));

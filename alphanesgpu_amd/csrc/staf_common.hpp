@@ -9,6 +9,7 @@
 #include <stdint.h>
 
 #include <unordered_map>
+#include <vector>
 
 #include "../../include/staf_ops.h"
 
@@ -195,22 +196,64 @@ struct Workspace {
 // which do not depend on each other) never share scratch, so they may run concurrently.
 struct StreamWork {
   Workspace scratch;         // per-slot partial forces / partial sums
-  Workspace buckets;         // transpose buckets (counters + entries), kept zeroed between calls
-  size_t bucket_counters = 0;    // capacity, in ints, of the counter part
-  size_t bucket_entries = 0;     // capacity, in ints, of the entry part
+  Workspace buckets;         // transpose a force op builds for itself: build counters, counts, keys
+  size_t bucket_counters = 0;    // capacity, in ints, of each of the two counter parts
+  size_t bucket_entries = 0;     // capacity, in ints, of the key part
 };
+
+// What a kernel needs of a transpose (receiver -> sorted (centre, slot) keys, see staf_transpose.hpp).
+struct TransposeRef {
+  int* build_cnt = nullptr;  // [nf * Nrecv] fill cursors of a build, all zero between builds
+  int* cnt = nullptr;        // [nf * Nrecv] keys per receiving atom
+  int* keys = nullptr;       // [nf * Nrecv, cap]
+  int cap = 0;
+  int key_shift = 0;         // centre number of row 0 of the map the force op was handed
+};
+
+// Transpose the descriptor op keeps beside an intmap2b tensor it has written.
+struct Transpose {
+  const int* im2 = nullptr;  // the intmap2b tensor [nf, N, nr+1] it was built from
+  int nf = 0, N = 0, Nrecv = 0, nr = 0;
+  TransposeRef ref;
+  Workspace buf;
+  size_t cap_recv = 0, cap_keys = 0;   // capacities of buf, in ints, of a counter part and of the key part
+  unsigned long long stamp = 0;        // last use, for replacement
+};
+constexpr int TRANSPOSE_SLOTS = 8;     // descriptor output tensors whose transposes are kept at a time
 
 struct DeviceState {
   int device = -1;
-  int* status_d = nullptr;   // device word, error bits OR-ed in by kernels
+  // One word per device, shared by every stream and model that uses the device: kernels OR their error bits into it,
+  // and a poll (or the synchronising return of an op) reports and clears whatever any of them raised.
+  int* status_d = nullptr;
   int* status_h = nullptr;   // pinned host mirror
   std::unordered_map<hipStream_t, StreamWork> work;
+  Transpose transposes[TRANSPOSE_SLOTS];
+  std::vector<void*> retired;   // outgrown blocks, freed by staf_ops_release
+  unsigned long long transpose_clock = 0;
 };
 
-DeviceState* device_state();                                   // for the current device, created on demand
-void* scratch_reserve(DeviceState* st, hipStream_t stream, size_t bytes);   // grows, never shrinks
-int* bucket_reserve(DeviceState* st, size_t n_counters, size_t n_entries, hipStream_t stream, int** entries);
+// For the current device, created on the first call (which allocates and synchronises: refused with null while
+// `stream` is being captured).
+DeviceState* device_state(hipStream_t stream);
+// True while `stream` is being captured into a graph: memory may then neither be freed nor allocated, and a fill
+// launched to initialise a fresh block would become part of the graph.
+bool stream_is_capturing(hipStream_t stream);
+// Both grow on demand and never shrink; under capture a request that does not fit what the stream already holds
+// returns null (the caller reports STAF_E_CAPTURE) instead of freeing and allocating.
+void* scratch_reserve(DeviceState* st, hipStream_t stream, size_t bytes);
+// Transpose a force op builds for itself (n_recv receiving atoms, cap keys each), in the stream's own work area.
+bool bucket_reserve(DeviceState* st, size_t n_recv, int cap, hipStream_t stream, TransposeRef* out);
+// Transpose kept beside the intmap2b tensor `im2` the descriptor op is about to write (nf frames, N centres, Nrecv
+// receiving atoms, cap keys per receiver).  Null block -> false.
+bool transpose_for_descriptor(DeviceState* st, const int* im2, int nf, int N, int Nrecv, int nr, int cap,
+                              hipStream_t stream, TransposeRef* out);
+// The transpose that covers the map view a force op was handed (pointer into a descriptor output, frame stride ld),
+// if the library holds one.
+bool transpose_find(DeviceState* st, const int* im2_view, int nf, int Nrecv, int Nl, int ld, int nr, TransposeRef* out);
 int finish_op(DeviceState* st, hipStream_t stream);            // launch check (+ optional sync & status fetch)
+// STAF_E_CAPTURE when the stream is being captured, else STAF_E_HIP: the code for a work area that could not be had
+int reserve_failure(hipStream_t stream);
 bool sync_errors_enabled();
 struct DeferStatus {   // while one is alive, the calling thread's ops do not synchronise to report device conditions
   DeferStatus();
@@ -257,5 +300,21 @@ int desc_launch(const DescConfig<real>& c, const real* pos, const real* box, int
                 const int* inj_howmany, const int* inj_with, int skip_pbc, real* raddescr, real* angdescr,
                 real* des3bsupp, int* intmap2b, int* intmap3b, real* der2b, real* der3b, real* der3bsupp,
                 int* numtriplet, hipStream_t stream);
+
+
+// Force ops with the wrap switch of the virial forms given per call (skip_pbc = 1: neighbour positions already are
+// periodic images; the extern "C" entry points pass the process-wide setting of staf_op_force_set_skip_pbc, the MD
+// entry its own per call).  Argument lists as in include/staf_ops.h.
+template <typename real>
+int force_doublets(const real* G, const real* D, const real* dD, const int* im2, int nr, int N, int nf, int Ar,
+                   const real* alpha2b, const real* emb2b, int nt, const int* tipos, const int* actual_type,
+                   real* force, const int* type_map, int Nl, real* virial, const real* pos, const real* box, int ld,
+                   int skip_pbc, void* stream);
+template <typename real>
+int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* dDsup, const real* d3b,
+                const int* im2, const int* im3, int nr, int na, int N, int nf, int Aa, const real* emb3b, int nt,
+                const int* tipos, const int* actual_type, real* force, const int* numtriplet, const real* alpha3b,
+                const int* type_map, int Nl, real* virial, const real* pos, const real* box, int ld, int skip_pbc,
+                void* stream);
 
 }  // namespace staf

@@ -16,8 +16,14 @@
 //      owning consecutive triplet indices so that angdescr / intmap3b / der3b
 //      rows are written as contiguous vectors.
 // The neighbour list never touches HBM; the only HBM traffic is the position
-// read and the nine op outputs, each written exactly once (padding included).
+// read and the nine op outputs.  Every output element is written exactly once,
+// padding as 0 -- the reference zeroes angdescr, intmap2b, intmap3b and
+// numtriplet before its kernels run (reforce.cc:357-358,375-376,385-386,420-421)
+// -- with one exception: der3b beyond an atom's triplets, which the reference
+// leaves uninitialised too, is only written when the zero_padding option is set.
 #include "staf_common.hpp"
+#include "staf_reduce.hpp"
+#include "staf_transpose.hpp"
 
 #include <math.h>
 #include <stdio.h>
@@ -50,6 +56,7 @@ struct DescArgs {
   real* der3bsupp;
   int* numtriplet;
   int* status;
+  TransposeRef tr;         // transposed neighbour map kept beside intmap2b (receiving atoms: the Npos positions)
 };
 
 // Everything that decides an integer output (which atoms are neighbours, their
@@ -376,6 +383,13 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
     __syncthreads();
   }
   PHASE_MARK(1);
+  // Every slot registers with the atom it points at (the transposed map the force ops gather through).  The second
+  // wave does it while the first one fills the radial rows: the atomics' round trip is off the critical path.
+  if (tid >= WAVE && tid < 2 * WAVE) {
+    for (int e = tid - WAVE; e < n; e += WAVE)
+      transpose_push(A.tr.build_cnt, A.tr.keys, A.tr.cap, (size_t)b * A.Npos + c_j[e], i, injected ? e : s_rank[e],
+                     A.status);
+  }
   // 3. radial fill
   const bool same_cut = A.Ra == A.Rc;
   const bool std_pow = A.pa == real(1) && A.pb == real(-30);   // the exponents fill_repulsion uses
@@ -456,8 +470,9 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
   // Consecutive lanes take consecutive triplets: the stores of a wave are whole cache lines.  (Four consecutive
   // triplets per thread with one index decode was measured: fewer instructions, but the strided stores made the
   // kernel a third slower.)
-  const int nend = A.zero_padding ? na : ntr;   // the reference writes nothing beyond an atom's triplets
-  for (int nn = tid; nn < nend; nn += blockDim.x) {
+  // angdescr and intmap3b are written over the whole row (the reference zeroes both tensors before its kernels
+  // run, STAF/src/descriptor_builder/reforce.cc:357-358,385-386); der3b beyond the triplets only on request
+  for (int nn = tid; nn < na; nn += blockDim.x) {
     if (nn < ntr) {
       int j, k;
       tri_decode(nn, m, j, k);
@@ -484,10 +499,10 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
       o.x = aj * (uk2 - cs * uj2) + hk * rj[6];
       o.y = ak * (uj2 - cs * uk2) + hj * rk[6];
       d3[2 * na + nn] = o;
-    } else if (A.zero_padding) {
+    } else {
       ang[nn] = 0;
       im3[nn] = make_int2(0, 0);
-      {
+      if (A.zero_padding) {
         real2 z;
         z.x = 0;
         z.y = 0;
@@ -510,11 +525,30 @@ size_t desc_lds_bytes(int nr) {
 
 static std::mutex g_cfg_mu;
 static int g_cell_threshold = 2048;   // frames of at least this many atoms search through a cell list
-static DescConfig<float> g_cfg_f;
-static DescConfig<double> g_cfg_d;
-template <typename real> DescConfig<real>& cfg();
-template <> DescConfig<float>& cfg<float>() { return g_cfg_f; }
-template <> DescConfig<double>& cfg<double>() { return g_cfg_d; }
+// Geometry set by construct: one configuration per device and precision.  construct() stores it for the device
+// that is current and as the process default, which serves devices construct() was never called on (the
+// reference keeps one process-wide configuration, STAF/src/descriptor_builder/reforce.cc:97-158).
+template <typename real>
+struct CfgStore {
+  DescConfig<real> dflt;
+  std::unordered_map<int, DescConfig<real>> dev;
+  DescConfig<real>& current() {   // g_cfg_mu held
+    int d = 0;
+    if (hipGetDevice(&d) != hipSuccess) return dflt;
+    auto it = dev.find(d);
+    return it == dev.end() ? dflt : it->second;
+  }
+  void store(const DescConfig<real>& c) {   // g_cfg_mu held
+    int d = 0;
+    if (hipGetDevice(&d) == hipSuccess) dev[d] = c;
+    dflt = c;
+  }
+};
+static CfgStore<float> g_cfg_f;
+static CfgStore<double> g_cfg_d;
+template <typename real> CfgStore<real>& cfg();
+template <> CfgStore<float>& cfg<float>() { return g_cfg_f; }
+template <> CfgStore<double>& cfg<double>() { return g_cfg_d; }
 
 // Short-range coefficients of D(r) = A/r^alpha + B/r^beta + C matching value,
 // slope and curvature of the cosine cutoff at rs; evaluated in `real` like
@@ -571,9 +605,7 @@ static int construct(real Rc, int nr, int na, int numpar, real Rs, real Ra, int 
     fclose(f);
   }
   std::lock_guard<std::mutex> lock(g_cfg_mu);
-  c.dist2_fma = cfg<real>().dist2_fma;
-  c.zero_padding = cfg<real>().zero_padding;
-  cfg<real>() = c;
+  cfg<real>().store(c);   // the options go back to their defaults: a mode set for an earlier geometry does not linger
   return STAF_OK;
 }
 
@@ -586,8 +618,8 @@ int desc_launch(const DescConfig<real>& c, const real* pos, const real* box, int
   if (!pos || !box || !raddescr || !angdescr || !des3bsupp || !intmap2b || !intmap3b || !der2b || !der3b ||
       !der3bsupp || !numtriplet || nf <= 0 || N <= 0 || Npos < N || (inj_howmany && !inj_with))
     return STAF_E_BAD_ARG;
-  DeviceState* st = device_state();
-  if (!st) return STAF_E_HIP;
+  DeviceState* st = device_state(stream);
+  if (!st) return reserve_failure(stream);
   DescArgs<real> A;
   A.pos = pos; A.box = box; A.nf = nf; A.N = N; A.Npos = Npos; A.nr = c.nr; A.na = c.na;
   A.inj_howmany = inj_howmany; A.inj_with = inj_with; A.skip_pbc = skip_pbc;
@@ -596,12 +628,17 @@ int desc_launch(const DescConfig<real>& c, const real* pos, const real* box, int
   A.raddescr = raddescr; A.angdescr = angdescr; A.des3bsupp = des3bsupp; A.intmap2b = intmap2b;
   A.intmap3b = intmap3b; A.der2b = der2b; A.der3b = der3b; A.der3bsupp = der3bsupp; A.numtriplet = numtriplet;
   A.status = st->status_d;
+  if (N >= (1 << (31 - KEY_SLOT_BITS))) return STAF_E_LIMIT;
+  // own lists are symmetric (an atom is listed by exactly its own neighbours, at most nr); a caller's list may name
+  // a ghost atom from more centres than that
+  const int cap = inj_howmany ? 4 * c.nr : c.nr;
+  if (!transpose_for_descriptor(st, intmap2b, nf, N, Npos, c.nr, cap, stream, &A.tr)) return reserve_failure(stream);
   A.cell_dims = A.cell_start = A.cell_atoms = A.cell_of = nullptr;
   const int cell_from = g_cell_threshold;
   if (!inj_howmany && cell_from > 0 && N >= cell_from) {
     const size_t ints = (size_t)nf * (4 + (CELL_MAX + 1) + 2 * (size_t)N);
     int* w = (int*)scratch_reserve(st, stream, ints * sizeof(int));
-    if (!w) return STAF_E_HIP;
+    if (!w) return reserve_failure(stream);
     int* dims = w;
     int* start = dims + (size_t)nf * 4;
     int* atoms = start + (size_t)nf * (CELL_MAX + 1);
@@ -618,6 +655,10 @@ int desc_launch(const DescConfig<real>& c, const real* pos, const real* box, int
   {
     KernelTimer kt_("desc_kernel", stream);
     hipLaunchKernelGGL(desc_kernel<real>, dim3((unsigned)(nf * N)), dim3(256), lds, stream, A);
+  }
+  {
+    KernelTimer kt_("transpose_sort_kernel", stream);
+    launch_transpose_sort(A.tr, nf * Npos, stream);
   }
   return finish_op(st, stream);
 }
@@ -647,7 +688,7 @@ static int compute(const real* pos, const real* box, int nf, int N, real* raddes
   DescConfig<real> c;
   {
     std::lock_guard<std::mutex> lock(g_cfg_mu);
-    c = cfg<real>();
+    c = cfg<real>().current();
   }
   return desc_launch<real>(c, pos, box, nf, N, N, nullptr, nullptr, 0, raddescr, angdescr, des3bsupp, intmap2b,
                            intmap3b, der2b, der3b, der3bsupp, numtriplet, (hipStream_t)stream_);
@@ -675,23 +716,26 @@ int staf_op_descriptor_cell_threshold(int n_atoms) {
 
 int staf_op_descriptor_options(int dist2_fma, int zero_padding) {
   std::lock_guard<std::mutex> lock(staf::g_cfg_mu);
-  staf::g_cfg_f.dist2_fma = staf::g_cfg_d.dist2_fma = dist2_fma ? 1 : 0;
-  staf::g_cfg_f.zero_padding = staf::g_cfg_d.zero_padding = zero_padding ? 1 : 0;
+  auto set = [&](auto& c) { c.dist2_fma = dist2_fma ? 1 : 0; c.zero_padding = zero_padding ? 1 : 0; };
+  set(staf::g_cfg_f.current()); set(staf::g_cfg_d.current());
+  set(staf::g_cfg_f.dflt); set(staf::g_cfg_d.dflt);
   return STAF_OK;
 }
 
 int staf_op_descriptor_coefficients_f32(float* o) {
   std::lock_guard<std::mutex> lock(staf::g_cfg_mu);
-  if (!staf::g_cfg_f.ready) return STAF_E_NOT_CONSTRUCTED;
+  const staf::DescConfig<float>& c = staf::g_cfg_f.current();
+  if (!c.ready) return STAF_E_NOT_CONSTRUCTED;
   if (!o) return STAF_E_BAD_ARG;
-  o[0] = staf::g_cfg_f.cA; o[1] = staf::g_cfg_f.cB; o[2] = staf::g_cfg_f.cC; o[3] = staf::g_cfg_f.pa; o[4] = staf::g_cfg_f.pb;
+  o[0] = c.cA; o[1] = c.cB; o[2] = c.cC; o[3] = c.pa; o[4] = c.pb;
   return STAF_OK;
 }
 int staf_op_descriptor_coefficients_f64(double* o) {
   std::lock_guard<std::mutex> lock(staf::g_cfg_mu);
-  if (!staf::g_cfg_d.ready) return STAF_E_NOT_CONSTRUCTED;
+  const staf::DescConfig<double>& c = staf::g_cfg_d.current();
+  if (!c.ready) return STAF_E_NOT_CONSTRUCTED;
   if (!o) return STAF_E_BAD_ARG;
-  o[0] = staf::g_cfg_d.cA; o[1] = staf::g_cfg_d.cB; o[2] = staf::g_cfg_d.cC; o[3] = staf::g_cfg_d.pa; o[4] = staf::g_cfg_d.pb;
+  o[0] = c.cA; o[1] = c.cB; o[2] = c.cC; o[3] = c.pa; o[4] = c.pb;
   return STAF_OK;
 }
 

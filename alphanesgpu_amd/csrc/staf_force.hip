@@ -3,18 +3,19 @@
 // back_prop_grad_force2b_kernel and gradforce_tripl_kernel
 // (STAF/src/force/{rad,ang}/reforce.cu.cc, STAF/src/grad_force/{rad,ang}/reforce.cu.cc).
 //
-// Force scatter is owner-computes and deterministic:
-//   pass A  (per centre i)   pair force of every neighbour slot -> scratch
-//                            gslot[b,i,s,3], centre's own force -> self[b,i,3];
-//                            each slot is also registered in the bucket of the
-//                            atom that receives it (integer atomics only);
-//   pass B  (per receiver a) the bucket is put in canonical (centre, slot)
-//                            order and summed with a fixed tree.
+// Force scatter is owner-computes and deterministic: every atom collects the pair forces of the slots that point
+// at it through the transposed neighbour map (staf_transpose.hpp; built once per descriptor call), in ascending
+// (centre, slot) order and with a fixed tree -- no floating-point atomics.
+//   2-body op  one kernel, one wave per atom of the frame: it evaluates the pair force of each of its own slots
+//              (as a centre of the op's species) and of each slot that lists it (read from that centre's rows).
+//   3-body op  pass A (per centre) slot forces -> scratch gslot[b,i,s,3], centre's own force -> self[b,i,3];
+//              pass B (per receiving atom) gathers them.
 // The 120x re-read of der3b by the reference's gradient kernel (one pass per
 // channel and species pair) is gone: der3b is contracted once per triplet with
 // dL/dF into three scalars, and all channels are evaluated from those.
 #include "staf_tile.hpp"
 #include "staf_reduce.hpp"
+#include "staf_transpose.hpp"
 #include "staf_tri.hpp"
 
 namespace staf {
@@ -35,76 +36,117 @@ __device__ inline int species_shift(const int* tipos, const int* actual_type) {
   return s;
 }
 
-// register slot (key) with the receiving atom `recv` of frame b
-__device__ inline void bucket_push(int* bcnt, int* bent, int cap, size_t recv, int key, int* status) {
-  const int pos = atomicAdd(&bcnt[recv], 1);
-  if (pos < cap) bent[recv * cap + pos] = key;
-  else atomicOr(status, 2);
-}
-
 }  // namespace staf
 #include "staf_force3.hpp"
 namespace staf {
 
 // ---------------------------------------------------------------------------
-// 2-body force, pass A.  One wave per centre, lane <-> slot.
-//   g_s = 1/2 sum_a G[a] c2[t_s,a] e^{alpha D}(1 + alpha D) * grad D_s
+// 2-body force.  One wave per atom a of the frame, lane <-> slot.
+//   g(i,s) = 1/2 sum_ch G[i,ch] c2[t,ch] e^{alpha[t,ch] D}(1 + alpha[t,ch] D) * grad D(i,s),  t = species of the
+//   neighbour in slot s of centre i
+//   F_a = - sum_s g(a,s)  [a is a centre of the op's species]  + sum_{(i,s) listing a} g(i,s)
+// The second sum runs over the keys of a in the transposed map whose centre belongs to the op's rows.  VIRIAL: the
+// wave also leaves its centre's 3x3 sum - sum_s g(a,s) (x) r(a,s) in vpart.
 // ---------------------------------------------------------------------------
 template <typename real>
-__global__ __launch_bounds__(F_BLOCK) void force2_kernel(const real* __restrict__ G, const real* __restrict__ D,
-                                                         const real* __restrict__ dD, const int* __restrict__ im2,
-                                                         const real* __restrict__ alpha2b,
-                                                         const real* __restrict__ emb2b,
-                                                         const int* __restrict__ type_map, real* __restrict__ gslot,
-                                                         real* __restrict__ self, int* bcnt, int* bent, int cap,
-                                                         int* status, int nf, int N, int Nl, int ld, int nr, int Ar,
-                                                         int nt) {
+struct Force2Args {
+  const real* G;         // [nf, Nl, Ar]
+  const real* D;         // raddescr [nf, ld, nr]
+  const real* dD;        // der2b [nf, ld, 3, nr]
+  const int* im2;        // [nf, ld, nr+1]
+  const real* alpha2b;
+  const real* emb2b;
+  const int* type_map;
+  const int* tipos;
+  const int* actual_type;
+  real* force;           // [nf, 3N]
+  real* vpart;           // VIRIAL: [nf, Nl, 9]
+  const real* pos;
+  const real* box;
+  TransposeRef tr;
+  int* status;
+  int skip_pbc, nf, N, Nl, ld, nr, Ar, nt;
+};
+
+template <typename real, bool VIRIAL>
+__global__ __launch_bounds__(F_BLOCK) void force2_kernel(Force2Args<real> A) {
   using HE = HotExp<real>;
   extern __shared__ __align__(16) unsigned char smem[];
+  const int Ar = A.Ar, nt = A.nt, nr = A.nr, Nl = A.Nl;
   real* p_al = (real*)smem;      // [nt*Ar]
   real* p_c2 = p_al + nt * Ar;   // [nt*Ar]
-  real* w_G = p_c2 + nt * Ar;    // [F_WAVES][Ar]
-  for (int q = threadIdx.x; q < nt * Ar; q += blockDim.x) { p_al[q] = alpha2b[q]; p_c2[q] = emb2b[q]; }
-  const int wave = threadIdx.x / WAVE, lane = lane_id();
-  real* myG = w_G + wave * Ar;
-  const int atom = blockIdx.x * F_WAVES + wave;
-  const bool live = atom < nf * Nl;
-  int b = 0, p = 0;
-  size_t rowAtom = 0;
-  if (live) {
-    b = atom / Nl; p = atom - b * Nl;
-    rowAtom = (size_t)b * ld + p;
-    for (int a = lane; a < Ar; a += WAVE) myG[a] = G[(size_t)atom * Ar + a];
-  }
+  for (int q = threadIdx.x; q < nt * Ar; q += blockDim.x) { p_al[q] = A.alpha2b[q]; p_c2[q] = A.emb2b[q]; }
   __syncthreads();
-  if (!live) return;
-  const int* im = im2 + rowAtom * (nr + 1);
-  int cnt = im[0];
-  if (cnt > nr) cnt = nr;
-  real sf[3] = {0, 0, 0};
-  const size_t rowScr = (size_t)atom;
-  for (int s = lane; s < cnt; s += WAVE) {
-    const int nj = im[1 + s];
-    const int t = type_map[nj];
-    const real d = D[rowAtom * nr + s];
-    real w = 0;
-    for (int a = 0; a < Ar; a++) {
-      const real ad = p_al[t * Ar + a] * d;
-      w += myG[a] * (p_c2[t * Ar + a] * HE::eval(HE::scale(ad)) * (real(1) + ad));
-    }
-    w *= real(0.5);
+  const int wave = threadIdx.x / WAVE, lane = lane_id();
+  const int recv = blockIdx.x * F_WAVES + wave;
+  if (recv >= A.nf * A.N) return;
+  const int b = recv / A.N, a = recv - b * A.N;
+  const int shift = species_shift(A.tipos, A.actual_type);
+  const int pl = a - shift;
+  real f[3] = {0, 0, 0};
+  real v[9];
 #pragma unroll
-    for (int c = 0; c < 3; c++) {
-      const real g = w * dD[rowAtom * 3 * nr + c * nr + s];
-      gslot[(rowScr * nr + s) * 3 + c] = g;
-      sf[c] -= g;
+  for (int c = 0; c < 9; c++) v[c] = 0;
+  // weight of the pair force of slot s of centre row `row` (row of G: gr), neighbour species t
+  auto pair_weight = [&](size_t row, size_t gr, int s, int t) -> real {
+    const real d = A.D[row * nr + s];
+    const real* g = A.G + gr * Ar;
+    real w = 0;
+    for (int ch = 0; ch < Ar; ch++) {
+      const real ad = p_al[t * Ar + ch] * d;
+      w += g[ch] * (p_c2[t * Ar + ch] * HE::eval(HE::scale(ad)) * (real(1) + ad));
     }
-    bucket_push(bcnt, bent, cap, (size_t)b * N + nj, p * nr + s, status);
+    return w * real(0.5);
+  };
+  if (pl >= 0 && pl < Nl) {
+    // own slots
+    const size_t row = (size_t)b * A.ld + pl;
+    const int* im = A.im2 + row * (nr + 1);
+    int cnt = im[0];
+    if (cnt > nr) cnt = nr;
+    for (int s = lane; s < cnt; s += WAVE) {
+      const int nj = im[1 + s];
+      const real w = pair_weight(row, (size_t)b * Nl + pl, s, A.type_map[nj]);
+      real g[3];
+#pragma unroll
+      for (int c = 0; c < 3; c++) {
+        g[c] = w * A.dD[row * 3 * nr + c * nr + s];
+        f[c] -= g[c];
+      }
+      if (VIRIAL) {
+        real r[3];
+        mic_cart_from_cart(A.pos + ((size_t)b * A.N + a) * 3, A.pos + ((size_t)b * A.N + nj) * 3,
+                           A.box + (size_t)b * 6, A.skip_pbc, r);
+#pragma unroll
+        for (int c = 0; c < 3; c++)
+#pragma unroll
+          for (int e = 0; e < 3; e++) v[c * 3 + e] -= g[c] * r[e];
+      }
+    }
+  }
+  // slots of the op's centres that list this atom
+  const int L = A.tr.cnt[recv];
+  const int* keys = A.tr.keys + (size_t)recv * A.tr.cap;
+  const int ta = A.type_map[a];
+  for (int e = lane; e < L; e += WAVE) {
+    const int key = keys[e];
+    const int p = key_centre(key) - A.tr.key_shift, s = key_slot(key);
+    if (p < 0 || p >= Nl) continue;
+    const size_t row = (size_t)b * A.ld + p;
+    if (A.im2[row * (nr + 1) + 1 + s] != a) { atomicOr(A.status, 4); continue; }   // the map is not the one transposed
+    const real w = pair_weight(row, (size_t)b * Nl + p, s, ta);
+#pragma unroll
+    for (int c = 0; c < 3; c++) f[c] += w * A.dD[row * 3 * nr + c * nr + s];
   }
 #pragma unroll
-  for (int c = 0; c < 3; c++) {
-    const real tot = wave_sum(sf[c]);
-    if (lane == 0) self[rowScr * 3 + c] = tot;
+  for (int c = 0; c < 3; c++) f[c] = wave_sum(f[c]);
+  if (lane < 3) A.force[((size_t)b * A.N + a) * 3 + lane] = lane == 0 ? f[0] : (lane == 1 ? f[1] : f[2]);
+  if (VIRIAL && pl >= 0 && pl < Nl) {
+#pragma unroll
+    for (int c = 0; c < 9; c++) {
+      const real t = wave_sum(v[c]);
+      if (lane == 0) A.vpart[((size_t)b * Nl + pl) * 9 + c] = t;
+    }
   }
 }
 
@@ -178,51 +220,35 @@ __global__ __launch_bounds__(F_BLOCK) void virial_frame_kernel(const real* __res
 }
 
 // ---------------------------------------------------------------------------
-// pass B: one wave per receiving atom.  Bucket entries (keys p*nr+s of the
-// centre slots that point at this atom) are ranked, the slot forces are placed
-// in rank order and summed with a fixed tree; the centre's own force is added
-// when the receiver belongs to the centre species.  Clears the bucket counter.
+// 3-body force, pass B: one wave per receiving atom.  The keys of the atom in the transposed map are in ascending
+// (centre, slot) order; lane e takes keys e, e + 64, ... whose centre is one of the op's rows, and the lanes are
+// added with a fixed tree.  The centre's own force is added when the receiver belongs to the centre species.
 // ---------------------------------------------------------------------------
 template <typename real>
 __global__ __launch_bounds__(F_BLOCK) void gather_kernel(const real* __restrict__ gslot,
-                                                         const real* __restrict__ self, int* bcnt,
-                                                         const int* __restrict__ bent, int cap,
+                                                         const real* __restrict__ self,
+                                                         const int* __restrict__ im2, TransposeRef tr,
                                                          const int* __restrict__ tipos,
                                                          const int* __restrict__ actual_type,
-                                                         real* __restrict__ force, int nf, int N, int Nl, int nr) {
-  extern __shared__ __align__(16) unsigned char smem[];
-  real* w_val = (real*)smem;                      // [F_WAVES][3*cap]
-  int* w_key = (int*)(w_val + F_WAVES * 3 * cap);  // [F_WAVES][cap]
+                                                         real* __restrict__ force, int* status, int nf, int N,
+                                                         int Nl, int ld, int nr) {
   const int wave = threadIdx.x / WAVE, lane = lane_id();
-  real* val = w_val + wave * 3 * cap;
-  int* key = w_key + wave * cap;
   const int recv = blockIdx.x * F_WAVES + wave;
   if (recv >= nf * N) return;
   const int b = recv / N, a = recv - b * N;
   const int shift = species_shift(tipos, actual_type);
-  int L = bcnt[recv];
-  L = __builtin_amdgcn_readfirstlane(L);
-  if (L > cap) L = cap;
-  for (int e = lane; e < L; e += WAVE) key[e] = bent[(size_t)recv * cap + e];
-  __builtin_amdgcn_wave_barrier();
-  __threadfence_block();
-  if (lane == 0 && L > 0) bcnt[recv] = 0;
-  for (int e = lane; e < L; e += WAVE) {
-    const int ke = key[e];
-    int rank = 0;
-    for (int o = 0; o < L; o++) rank += (key[o] < ke) ? 1 : 0;
-    const size_t src = ((size_t)b * Nl * nr + ke) * 3;
-    val[3 * rank] = gslot[src];
-    val[3 * rank + 1] = gslot[src + 1];
-    val[3 * rank + 2] = gslot[src + 2];
-  }
-  __builtin_amdgcn_wave_barrier();
-  __threadfence_block();
+  const int L = tr.cnt[recv];
+  const int* keys = tr.keys + (size_t)recv * tr.cap;
   real f[3] = {0, 0, 0};
   for (int e = lane; e < L; e += WAVE) {
-    f[0] += val[3 * e];
-    f[1] += val[3 * e + 1];
-    f[2] += val[3 * e + 2];
+    const int key = keys[e];
+    const int p = key_centre(key) - tr.key_shift, s = key_slot(key);
+    if (p < 0 || p >= Nl) continue;
+    if (im2[((size_t)b * ld + p) * (nr + 1) + 1 + s] != a) { atomicOr(status, 4); continue; }
+    const real* g = gslot + (((size_t)b * Nl + p) * nr + s) * 3;
+    f[0] += g[0];
+    f[1] += g[1];
+    f[2] += g[2];
   }
 #pragma unroll
   for (int c = 0; c < 3; c++) f[c] = wave_sum(f[c]);
@@ -357,54 +383,19 @@ static inline int grad_blocks_f(int atoms) {
   return nb < GRAD_MAX_BLOCKS_F ? nb : GRAD_MAX_BLOCKS_F;
 }
 
-struct ForceScratch {
-  void* gslot;
-  void* self;
-  void* vpart;
-  int* bcnt;
-  int* bent;
-  int cap;
-};
-
-template <typename real>
-static int force_scratch(DeviceState* st, int nf, int N, int Nl, int nr, hipStream_t stream, ForceScratch* fs) {
-  const size_t ng = (size_t)nf * Nl * nr * 3, ns = (size_t)nf * Nl * 3, nv = (size_t)nf * Nl * 9;
-  real* base = (real*)scratch_reserve(st, stream, (ng + ns + nv) * sizeof(real));
-  if (!base) return STAF_E_HIP;
-  fs->gslot = base;
-  fs->self = base + ng;
-  fs->vpart = base + ng + ns;
-  fs->cap = 4 * nr;
-  fs->bcnt = bucket_reserve(st, (size_t)nf * N, (size_t)nf * N * fs->cap, stream, &fs->bent);
-  if (!fs->bcnt) return STAF_E_HIP;
-  return STAF_OK;
-}
-
-template <typename real>
-static void launch_virial(const ForceScratch& fs, const int* im2, const int* counts, const real* pos, const real* box,
-                          const int* tipos, const int* actual_type, real* virial, int nf, int N, int Nl, int ld,
-                          int nr, hipStream_t stream) {
-  const int atoms = nf * Nl;
-  hipLaunchKernelGGL(virial_centre_kernel<real>, dim3((atoms + F_WAVES - 1) / F_WAVES), dim3(F_BLOCK), 0, stream,
-                     (const real*)fs.gslot, im2, counts, pos, box, tipos, actual_type, (real*)fs.vpart, nf, N, Nl,
-                     ld, nr, g_force_skip_pbc);
-  hipLaunchKernelGGL(virial_frame_kernel<real>, dim3(nf), dim3(F_BLOCK), 0, stream, (const real*)fs.vpart, virial,
-                     Nl);
-}
-
-template <typename real>
-static int launch_gather(DeviceState* st, const ForceScratch& fs, const int* tipos, const int* actual_type,
-                         real* force, int nf, int N, int Nl, int nr, hipStream_t stream) {
-  size_t lds = (size_t)F_WAVES * fs.cap * (3 * sizeof(real) + sizeof(int));
-  if (lds > 64 * 1024) return STAF_E_LIMIT;
-  const int recv = nf * N;
-  {
-    KernelTimer kt_("gather_kernel", stream);
-    hipLaunchKernelGGL(gather_kernel<real>, dim3((recv + F_WAVES - 1) / F_WAVES), dim3(F_BLOCK), lds, stream,
-                       (const real*)fs.gslot, (const real*)fs.self, fs.bcnt, (const int*)fs.bent, fs.cap, tipos,
-                       actual_type, force, nf, N, Nl, nr);
-  }
-  return finish_op(st, stream);
+// The transposed neighbour map for a force op: the one the descriptor op left beside the tensor `im2` points into,
+// or, for any other copy of the map, one built here in the stream's work area (push + sort launches).
+static int force_transpose(DeviceState* st, const int* im2, int nf, int N, int Nl, int ld, int nr, hipStream_t stream,
+                           TransposeRef* tr) {
+  if (transpose_find(st, im2, nf, N, Nl, ld, nr, tr)) return STAF_OK;
+  const int cap = 4 * nr;
+  if ((size_t)TR_WAVES * cap * sizeof(int) > 64 * 1024) return STAF_E_LIMIT;
+  if (!bucket_reserve(st, (size_t)nf * N, cap, stream, tr)) return reserve_failure(stream);
+  const int total = nf * Nl * nr;
+  hipLaunchKernelGGL(transpose_push_kernel, dim3((total + TR_BLOCK - 1) / TR_BLOCK), dim3(TR_BLOCK), 0, stream, im2,
+                     tr->build_cnt, tr->keys, tr->cap, st->status_d, nf, N, Nl, ld, nr);
+  launch_transpose_sort(*tr, nf * N, stream);
+  return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }
 
 // A species without atoms in these frames contributes no force (and no virial): the op still fills its outputs.
@@ -424,43 +415,55 @@ static int empty_species_grad(real* g_alpha, int n_alpha, real* g_emb, int n_emb
 }
 
 template <typename real>
-static int force_doublets(const real* G, const real* D, const real* dD, const int* im2, int nr, int N, int nf, int Ar,
-                          const real* alpha2b, const real* emb2b, int nt, const int* tipos, const int* actual_type,
-                          real* force, const int* type_map, int Nl, real* virial, const real* pos, const real* box,
-                          int ld, void* stream_) {
+int force_doublets(const real* G, const real* D, const real* dD, const int* im2, int nr, int N, int nf, int Ar,
+                   const real* alpha2b, const real* emb2b, int nt, const int* tipos, const int* actual_type,
+                   real* force, const int* type_map, int Nl, real* virial, const real* pos, const real* box, int ld,
+                   int skip_pbc, void* stream_) {
   if ((virial || pos || box) && !(virial && pos && box)) return STAF_E_BAD_ARG;
   if (Nl == 0 && nf > 0 && N > 0 && force) return empty_species_force<real>(force, virial, nf, N, stream_);
   if (!G || !D || !dD || !im2 || !alpha2b || !emb2b || !tipos || !actual_type || !force || !type_map || nr <= 0 ||
       N <= 0 || nf <= 0 || Ar <= 0 || nt <= 0 || Nl <= 0 || Nl > N)
     return STAF_E_BAD_ARG;
-  if (nt > NT_MAX) return STAF_E_LIMIT;
+  if (nt > NT_MAX || nr > (1 << KEY_SLOT_BITS) || N >= (1 << (31 - KEY_SLOT_BITS))) return STAF_E_LIMIT;
   if (ld <= 0) ld = Nl;
-  DeviceState* st = device_state();
-  if (!st) return STAF_E_HIP;
+  DeviceState* st = device_state((hipStream_t)stream_);
+  if (!st) return reserve_failure((hipStream_t)stream_);
   hipStream_t stream = (hipStream_t)stream_;
-  ForceScratch fs;
-  int rc = force_scratch<real>(st, nf, N, Nl, nr, stream, &fs);
+  Force2Args<real> A;
+  int rc = force_transpose(st, im2, nf, N, Nl, ld, nr, stream, &A.tr);
   if (rc) return rc;
-  size_t lds = (size_t)(2 * nt * Ar + F_WAVES * Ar) * sizeof(real);
+  A.G = G; A.D = D; A.dD = dD; A.im2 = im2; A.alpha2b = alpha2b; A.emb2b = emb2b; A.type_map = type_map;
+  A.tipos = tipos; A.actual_type = actual_type; A.force = force; A.vpart = nullptr; A.pos = pos; A.box = box;
+  A.status = st->status_d; A.skip_pbc = skip_pbc;
+  A.nf = nf; A.N = N; A.Nl = Nl; A.ld = ld; A.nr = nr; A.Ar = Ar; A.nt = nt;
+  if (virial) {
+    A.vpart = (real*)scratch_reserve(st, stream, (size_t)nf * Nl * 9 * sizeof(real));
+    if (!A.vpart) return reserve_failure(stream);
+  }
+  const size_t lds = (size_t)2 * nt * Ar * sizeof(real);
   if (lds > 64 * 1024) return STAF_E_LIMIT;
-  const int atoms = nf * Nl;
+  const int atoms = nf * N;
   {
     KernelTimer kt_("force2_kernel", stream);
-    hipLaunchKernelGGL(force2_kernel<real>, dim3((atoms + F_WAVES - 1) / F_WAVES), dim3(F_BLOCK), lds, stream, G, D, dD,
-                       im2, alpha2b, emb2b, type_map, (real*)fs.gslot, (real*)fs.self, fs.bcnt, fs.bent, fs.cap,
-                       st->status_d, nf, N, Nl, ld, nr, Ar, nt);
+    if (virial)
+      hipLaunchKernelGGL((force2_kernel<real, true>), dim3((atoms + F_WAVES - 1) / F_WAVES), dim3(F_BLOCK), lds,
+                         stream, A);
+    else
+      hipLaunchKernelGGL((force2_kernel<real, false>), dim3((atoms + F_WAVES - 1) / F_WAVES), dim3(F_BLOCK), lds,
+                         stream, A);
   }
   if (virial)
-    launch_virial<real>(fs, im2, (const int*)nullptr, pos, box, tipos, actual_type, virial, nf, N, Nl, ld, nr, stream);
-  return launch_gather<real>(st, fs, tipos, actual_type, force, nf, N, Nl, nr, stream);
+    hipLaunchKernelGGL(virial_frame_kernel<real>, dim3(nf), dim3(F_BLOCK), 0, stream, (const real*)A.vpart, virial,
+                       Nl);
+  return finish_op(st, stream);
 }
 
 template <typename real>
-static int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* dDsup, const real* d3b,
-                       const int* im2, const int* im3, int nr, int na, int N, int nf, int Aa, const real* emb3b,
-                       int nt, const int* tipos, const int* actual_type, real* force, const int* numtriplet,
-                       const real* alpha3b, const int* type_map, int Nl, real* virial, const real* pos,
-                       const real* box, int ld, void* stream_) {
+int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* dDsup, const real* d3b,
+                const int* im2, const int* im3, int nr, int na, int N, int nf, int Aa, const real* emb3b, int nt,
+                const int* tipos, const int* actual_type, real* force, const int* numtriplet, const real* alpha3b,
+                const int* type_map, int Nl, real* virial, const real* pos, const real* box, int ld, int skip_pbc,
+                void* stream_) {
   (void)im3;
   if ((virial || pos || box) && !(virial && pos && box)) return STAF_E_BAD_ARG;
   if (Nl == 0 && nf > 0 && N > 0 && force) return empty_species_force<real>(force, virial, nf, N, stream_);
@@ -469,13 +472,18 @@ static int force_tripl(const real* G, const real* Dsup, const real* Tang, const 
     return STAF_E_BAD_ARG;
   if (nt > NT_MAX) return STAF_E_LIMIT;
   if (ld <= 0) ld = Nl;
-  DeviceState* st = device_state();
-  if (!st) return STAF_E_HIP;
+  DeviceState* st = device_state((hipStream_t)stream_);
+  if (!st) return reserve_failure((hipStream_t)stream_);
   hipStream_t stream = (hipStream_t)stream_;
-  ForceScratch fs;
-  int rc = force_scratch<real>(st, nf, N, Nl, nr, stream, &fs);
+  if (!Force3Cfg<real>::fits(nr, nt) || N >= (1 << (31 - KEY_SLOT_BITS))) return STAF_E_LIMIT;
+  TransposeRef tr;
+  int rc = force_transpose(st, im2, nf, N, Nl, ld, nr, stream, &tr);
   if (rc) return rc;
-  if (!Force3Cfg<real>::fits(nr, nt)) return STAF_E_LIMIT;
+  const size_t ng = (size_t)nf * Nl * nr * 3, ns = (size_t)nf * Nl * 3, nv = virial ? (size_t)nf * Nl * 9 : 0;
+  real* gslot = (real*)scratch_reserve(st, stream, (ng + ns + nv) * sizeof(real));
+  if (!gslot) return reserve_failure(stream);
+  real* self = gslot + ng;
+  real* vpart = self + ns;
   const size_t lds = Force3Cfg<real>::bytes(nr, Aa, nt);
   if (lds > 64 * 1024) {
     if (lds > 160 * 1024 ||
@@ -486,19 +494,40 @@ static int force_tripl(const real* G, const real* Dsup, const real* Tang, const 
   {
     KernelTimer kt_("force3_kernel", stream);
     hipLaunchKernelGGL(force3_kernel<real>, dim3(nf * Nl), dim3(Force3Cfg<real>::THREADS), lds, stream, G, Dsup, Tang,
-                       dDsup, d3b, im2, alpha3b, emb3b, type_map, numtriplet, (real*)fs.gslot, (real*)fs.self, fs.bcnt,
-                       fs.bent, fs.cap, st->status_d, nf, N, Nl, ld, nr, na, Aa, nt);
+                       dDsup, d3b, im2, alpha3b, emb3b, type_map, numtriplet, gslot, self, nf, N, Nl, ld, nr, na, Aa,
+                       nt);
   }
-  if (virial)
-    launch_virial<real>(fs, im2, numtriplet, pos, box, tipos, actual_type, virial, nf, N, Nl, ld, nr, stream);
-  return launch_gather<real>(st, fs, tipos, actual_type, force, nf, N, Nl, nr, stream);
+  if (virial) {
+    const int atoms = nf * Nl;
+    hipLaunchKernelGGL(virial_centre_kernel<real>, dim3((atoms + F_WAVES - 1) / F_WAVES), dim3(F_BLOCK), 0, stream,
+                       (const real*)gslot, im2, numtriplet, pos, box, tipos, actual_type, vpart, nf, N, Nl, ld, nr,
+                       skip_pbc);
+    hipLaunchKernelGGL(virial_frame_kernel<real>, dim3(nf), dim3(F_BLOCK), 0, stream, (const real*)vpart, virial, Nl);
+  }
+  {
+    KernelTimer kt_("gather_kernel", stream);
+    const int recv = nf * N;
+    hipLaunchKernelGGL(gather_kernel<real>, dim3((recv + F_WAVES - 1) / F_WAVES), dim3(F_BLOCK), 0, stream,
+                       (const real*)gslot, (const real*)self, im2, tr, tipos, actual_type, force, st->status_d, nf, N,
+                       Nl, ld, nr);
+  }
+  return finish_op(st, stream);
 }
+
+template int force_doublets<double>(const double*, const double*, const double*, const int*, int, int, int, int,
+                                    const double*, const double*, int, const int*, const int*, double*, const int*,
+                                    int, double*, const double*, const double*, int, int, void*);
+template int force_tripl<double>(const double*, const double*, const double*, const double*, const double*,
+                                 const int*, const int*, int, int, int, int, int, const double*, int, const int*,
+                                 const int*, double*, const int*, const double*, const int*, int, double*,
+                                 const double*, const double*, int, int, void*);
 
 template <typename real>
 static int gradforce_2b(const real* Q, const real* D, int nr, const real* alpha2b, int Ar, const real* dD,
                         const int* im2, int nf, int N, int Nl, const real* G, const real* emb2b, int nt,
                         const int* type_map, const int* tipos, const int* actual_type, real* gnet, real* g_alpha,
-                        real* g_emb, const real* Qvir, const real* pos, const real* box, int ld, void* stream_) {
+                        real* g_emb, const real* Qvir, const real* pos, const real* box, int ld, int skip_pbc,
+                        void* stream_) {
   if ((Qvir || pos || box) && !(Qvir && pos && box)) return STAF_E_BAD_ARG;
   if (Nl == 0 && nf > 0 && Ar > 0 && nt > 0 && g_alpha && g_emb)
     return empty_species_grad<real>(g_alpha, nt * Ar, g_emb, nt * Ar, stream_);
@@ -507,21 +536,21 @@ static int gradforce_2b(const real* Q, const real* D, int nr, const real* alpha2
     return STAF_E_BAD_ARG;
   if (nt > NT_MAX) return STAF_E_LIMIT;
   if (ld <= 0) ld = Nl;
-  DeviceState* st = device_state();
-  if (!st) return STAF_E_HIP;
+  DeviceState* st = device_state((hipStream_t)stream_);
+  if (!st) return reserve_failure((hipStream_t)stream_);
   hipStream_t stream = (hipStream_t)stream_;
   const int nout = 2 * nt * Ar;
   const int nb = grad_blocks_f(nf * Nl);
   real* partial = (real*)scratch_reserve(st, stream, ((size_t)nb + RED_SLICES) * nout * sizeof(real));
   real* red_tmp = partial ? partial + (size_t)nb * nout : nullptr;
-  if (!partial) return STAF_E_HIP;
+  if (!partial) return reserve_failure(stream);
   size_t lds = (size_t)(2 * nt * Ar + F_WAVES * nout + 2 * F_WAVES * nr) * sizeof(real) +
                (size_t)F_WAVES * (2 * nr + NT_MAX + 1) * sizeof(int);
   if (lds > 64 * 1024) return STAF_E_LIMIT;
   {
     KernelTimer kt_("gradforce2_kernel", stream);
     hipLaunchKernelGGL(gradforce2_kernel<real>, dim3(nb), dim3(F_BLOCK), lds, stream, Q, G, D, dD, im2, alpha2b, emb2b,
-                       type_map, tipos, actual_type, gnet, partial, Qvir, pos, box, g_force_skip_pbc, nf, N, Nl, ld, nr,
+                       type_map, tipos, actual_type, gnet, partial, Qvir, pos, box, skip_pbc, nf, N, Nl, ld, nr,
                        Ar, nt);
   }
   launch_reduce_partials<real>(partial, nb, nout, g_alpha, nt * Ar, nt * Ar, g_emb, nt * Ar, nt * Ar, red_tmp, stream);
@@ -533,7 +562,7 @@ static int gradforce_tripl(const real* Q, const real* G, const real* Dsup, const
                            const real* d3b, const int* im2, const int* im3, int nr, int na, int N, int nf, int Aa,
                            const real* emb3b, int nt, const int* tipos, const int* actual_type, const int* numtriplet,
                            const real* alpha3b, const int* type_map, int Nl, real* gnet, real* g_alpha, real* g_emb,
-                           const real* Qvir, const real* pos, const real* box, int ld, void* stream_) {
+                           const real* Qvir, const real* pos, const real* box, int ld, int skip_pbc, void* stream_) {
   (void)im3;
   if ((Qvir || pos || box) && !(Qvir && pos && box)) return STAF_E_BAD_ARG;
   if (Nl == 0 && nf > 0 && Aa > 0 && nt > 0 && g_alpha && g_emb) {
@@ -546,8 +575,8 @@ static int gradforce_tripl(const real* Q, const real* G, const real* Dsup, const
     return STAF_E_BAD_ARG;
   if (nt > NT_MAX) return STAF_E_LIMIT;
   if (ld <= 0) ld = Nl;
-  DeviceState* st = device_state();
-  if (!st) return STAF_E_HIP;
+  DeviceState* st = device_state((hipStream_t)stream_);
+  if (!st) return reserve_failure((hipStream_t)stream_);
   hipStream_t stream = (hipStream_t)stream_;
   const int ntc = nt * (nt + 1) / 2;
   const int nsig = 2 * nt - 1;
@@ -555,7 +584,7 @@ static int gradforce_tripl(const real* Q, const real* G, const real* Dsup, const
   const int nb = nf * Nl < TRI_GRID_MAX ? nf * Nl : TRI_GRID_MAX;
   real* partial = (real*)scratch_reserve(st, stream, ((size_t)nb + RED_SLICES) * nout * sizeof(real));
   real* red_tmp = partial ? partial + (size_t)nb * nout : nullptr;
-  if (!partial) return STAF_E_HIP;
+  if (!partial) return reserve_failure(stream);
   size_t lds = TriLds<real, 2>::bytes(nr, Aa, nt);
   if (lds > 64 * 1024) return STAF_E_LIMIT;
   const int nall = ntc * Aa * 3;
@@ -563,7 +592,7 @@ static int gradforce_tripl(const real* Q, const real* G, const real* Dsup, const
   A.Dsup = Dsup; A.Tang = Tang; A.im2 = im2; A.alpha3b = alpha3b; A.emb3b = emb3b; A.type_map = type_map;
   A.numtriplet = numtriplet; A.P = G; A.Q = Q; A.dDsup = dDsup; A.d3b = d3b; A.tipos = tipos;
   A.actual_type = actual_type; A.out = gnet; A.partial = partial; A.Qvir = Qvir; A.pos = pos; A.box = box;
-  A.skip_pbc = g_force_skip_pbc;
+  A.skip_pbc = skip_pbc;
   A.nf = nf; A.N = N; A.Nl = Nl; A.ld = ld; A.nr = nr; A.na = na; A.Aa = Aa; A.nt = nt;
   {
     KernelTimer kt_("gradforce3_kernel", stream);
@@ -588,7 +617,7 @@ void staf_op_force_set_skip_pbc(int skip) { staf::g_force_skip_pbc = skip ? 1 : 
                                    real* virial, const real* pos, const real* box, int ld_atoms, void* stream) {       \
     return staf::force_doublets<real>(netderiv, des_r, intderiv_r, intmap_r, nr, N, dimbat, num_alpha_radiale,         \
                                       alpha_radiale, type_emb2b, nt, tipos, actual_type, forces2b, type_map, N_local,  \
-                                      virial, pos, box, ld_atoms, stream);                                             \
+                                      virial, pos, box, ld_atoms, staf::g_force_skip_pbc, stream);                     \
   }                                                                                                                    \
   int staf_op_force_tripl_##SFX(const real* netderiv, const real* desr, const real* desa, const real* intderiv_r,      \
                                 const real* intderiv_a, const int* intmap_r, const int* intmap_a, int nr, int na,      \
@@ -598,7 +627,8 @@ void staf_op_force_set_skip_pbc(int skip) { staf::g_force_skip_pbc = skip ? 1 : 
                                 int ld_atoms, void* stream) {                                                          \
     return staf::force_tripl<real>(netderiv, desr, desa, intderiv_r, intderiv_a, intmap_r, intmap_a, nr, na, N,        \
                                    dimbat, num_finger, type_emb3b, nt, tipos, actual_type, forces3b, num_triplets,     \
-                                   smooth_a, type_map, N_local, virial, pos, box, ld_atoms, stream);                   \
+                                   smooth_a, type_map, N_local, virial, pos, box, ld_atoms, staf::g_force_skip_pbc,    \
+                                   stream);                                                                            \
   }                                                                                                                    \
   int staf_op_gradforce_2b_##SFX(const real* prevgrad, const real* radiale, int nr, const real* alpha_radiale,         \
                                  int num_finger, const real* desder, const int* intmap_r, int dimbat, int N,           \
@@ -608,7 +638,8 @@ void staf_op_force_set_skip_pbc(int skip) { staf::g_force_skip_pbc = skip ? 1 : 
                                  const real* box, int ld_atoms, void* stream) {                                        \
     return staf::gradforce_2b<real>(prevgrad, radiale, nr, alpha_radiale, num_finger, desder, intmap_r, dimbat, N,     \
                                     N_local, netderiv, type_emb2b, nt, type_map, tipos, actual_type, grad_net,         \
-                                    grad_alpha2b, grad_emb2b, prevgrad_virial, pos, box, ld_atoms, stream);            \
+                                    grad_alpha2b, grad_emb2b, prevgrad_virial, pos, box, ld_atoms,                     \
+                                    staf::g_force_skip_pbc, stream);                                                   \
   }                                                                                                                    \
   int staf_op_gradforce_tripl_##SFX(const real* prevgrad, const real* netderiv, const real* desr, const real* desa,    \
                                     const real* intderiv_r, const real* intderiv_a, const int* intmap_r,               \
@@ -621,7 +652,7 @@ void staf_op_force_set_skip_pbc(int skip) { staf::g_force_skip_pbc = skip ? 1 : 
     return staf::gradforce_tripl<real>(prevgrad, netderiv, desr, desa, intderiv_r, intderiv_a, intmap_r, intmap_a, nr, \
                                        na, N, dimbat, num_finger, type_emb3b, nt, tipos, actual_type, num_triplets,    \
                                        smooth_a, type_map, N_local, gradnet_3b, grad_alpha3b, grad_emb3b,              \
-                                       prevgrad_virial, pos, box, ld_atoms, stream);                                   \
+                                       prevgrad_virial, pos, box, ld_atoms, staf::g_force_skip_pbc, stream);           \
   }
 
 STAF_FORCE_ENTRY(float, f32)

@@ -22,6 +22,8 @@
 //     slot k are added to the wave's own LDS accumulators row by row (inside a row the k are distinct).  The
 //     four waves' accumulators are added in a fixed order: results are bit-reproducible.
 //     F_s = sum_p Sd(s,p) dT/dd_s(s,p) + (sum_p SB_s(s,p)) grad fc_s
+// The slot forces go to scratch (gslot, and the centre's own force to self); the atoms that receive them collect
+// them in gather_kernel through the transposed neighbour map.
 #pragma once
 #include <type_traits>
 
@@ -81,8 +83,8 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
     const real* __restrict__ G, const real* __restrict__ Dsup, const real* __restrict__ Tang,
     const real* __restrict__ dDsup, const real* __restrict__ d3b, const int* __restrict__ im2,
     const real* __restrict__ alpha3b, const real* __restrict__ emb3b, const int* __restrict__ type_map,
-    const int* __restrict__ numtriplet, real* __restrict__ gslot, real* __restrict__ self, int* bcnt, int* bent,
-    int cap, int* status, int nf, int N, int Nl, int ld, int nr, int na, int Aa, int nt) {
+    const int* __restrict__ numtriplet, real* __restrict__ gslot, real* __restrict__ self, int nf, int N, int Nl,
+    int ld, int nr, int na, int Aa, int nt) {
   using real2 = typename Vec2<real>::type;
   using real4 = typename Vec4<real>::type;
   using HE = HotExp<real>;
@@ -186,7 +188,6 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
     for (int c = 0; c < 3; c++) sg[c * nr + tid] = g_s[c];
   }
   if (slot) stp[tid] = t_s;
-  int bpos = 0;   // place in the receiving atom's bucket (see below)
   __syncthreads();
   PHASE_MARK(0);
   int maxact = 0;
@@ -255,10 +256,6 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
       }
       __syncthreads();
       PHASE_MARK(2);
-      // The slot registers with its receiving atom: an integer atomic whose return is only needed for a store at
-      // the very end.  Issued here, ahead of the longest stretch without global reads, its latency is covered by
-      // the channel loop; the next wait on the (in-order) memory counter is the one for the der3b rows.
-      if (w0 == 0 && c0 == 0 && slot) bpos = atomicAdd(&bcnt[(size_t)b * N + nj], 1);
       // One copy of the loop per number of passes, so that no branch separates the (triplet, channel) items and
       // the LDS reads of the next items are in flight while the current ones are computed.
       auto channels = [&](auto npass_c) {
@@ -394,10 +391,6 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
     }
     PHASE_MARK(4);
   }
-  if (ntri <= 0 && slot) bpos = atomicAdd(&bcnt[(size_t)b * N + nj], 1);   // no triplet: not registered yet
-  // The atomic's return is taken here, while no store is in flight: the memory counter is in order, so waiting for
-  // it after the stores below would wait for them as well.
-  asm volatile("" : "+v"(bpos));
   __syncthreads();
   PHASE_MARK(5);
 
@@ -421,7 +414,9 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
   }
   __syncthreads();
   // global stores after the last barrier: nothing waits for them
-  if (slot) {
+  // every slot of the row is written: the atoms that gather see all slots of the neighbour map, also those beyond
+  // the angular cutoff, which carry no 3-body force (f3 = 0 there)
+  if (tid < nr) {
 #pragma unroll
     for (int c = 0; c < 3; c++) gslot[((size_t)atom * nr + tid) * 3 + c] = f3[c];
   }
@@ -430,10 +425,6 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
 #pragma unroll
     for (int w = 0; w < NW; w++) a += xch[w * 4 + tid];
     self[(size_t)atom * 3 + tid] = -a;
-  }
-  if (slot) {   // the slot's place in the bucket of its receiving atom
-    if (bpos < cap) bent[((size_t)b * N + nj) * cap + bpos] = p_ * nr + tid;
-    else atomicOr(status, 2);
   }
   PHASE_MARK(6);
   PHASE_CLOCK_END();

@@ -31,12 +31,14 @@ void kernel_timing_record(const char* kernel, hipEvent_t a, hipEvent_t b) {
   g_kernel_events[kernel].emplace_back(a, b);
 }
 
-DeviceState* device_state() {
+DeviceState* device_state(hipStream_t stream) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return nullptr;
   std::lock_guard<std::mutex> lock(g_mu);
   auto it = g_state.find(dev);
   if (it != g_state.end()) return it->second.get();
+  // the first call on a device allocates and synchronises: not while the caller's stream is being captured
+  if (stream_is_capturing(stream)) return nullptr;
   auto st = std::unique_ptr<DeviceState>(new DeviceState());
   st->device = dev;
   if (hipMalloc((void**)&st->status_d, sizeof(int)) != hipSuccess) return nullptr;
@@ -54,45 +56,120 @@ static StreamWork* stream_work(DeviceState* st, hipStream_t stream) {
   return &st->work[stream];   // references into an unordered_map stay valid when it grows
 }
 
+bool stream_is_capturing(hipStream_t stream) {
+  hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &cs) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return cs != hipStreamCaptureStatusNone;
+}
+
+int reserve_failure(hipStream_t stream) { return stream_is_capturing(stream) ? STAF_E_CAPTURE : STAF_E_HIP; }
+
+// A block that has become too small is not freed but retired until staf_ops_release: kernels in flight, and graphs
+// instantiated while it was current, may still address it.  Blocks grow by half, so the retired ones of a work area
+// add up to less than twice its final size.
+static bool grow(DeviceState* st, Workspace* w, size_t bytes, hipStream_t stream) {
+  if (stream_is_capturing(stream)) return false;
+  void* fresh = nullptr;
+  const size_t want = bytes + bytes / 2;
+  if (hipMalloc(&fresh, want) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  if (w->buf) st->retired.push_back(w->buf);
+  w->buf = fresh;
+  w->bytes = want;
+  return true;
+}
+
 void* scratch_reserve(DeviceState* st, hipStream_t stream, size_t bytes) {
   StreamWork* w = stream_work(st, stream);
   if (bytes <= w->scratch.bytes) return w->scratch.buf;
-  if (w->scratch.buf) {
-    // hipFree waits for in-flight work that may still read the old block
-    if (hipFree(w->scratch.buf) != hipSuccess) return nullptr;
-    w->scratch.buf = nullptr;
-    w->scratch.bytes = 0;
-  }
-  size_t want = bytes + bytes / 4;
-  if (hipMalloc(&w->scratch.buf, want) != hipSuccess) return nullptr;
-  w->scratch.bytes = want;
-  return w->scratch.buf;
+  std::lock_guard<std::mutex> lock(g_mu);
+  return grow(st, &w->scratch, bytes, stream) ? w->scratch.buf : nullptr;
 }
 
-// Scatter buckets: n_counters ints (kept all-zero between calls: the gather
-// kernel clears every counter it consumes) followed by n_entries ints.
-int* bucket_reserve(DeviceState* st, size_t n_counters, size_t n_entries, hipStream_t stream, int** entries) {
-  StreamWork* w = stream_work(st, stream);
-  if (n_counters > w->bucket_counters || n_entries > w->bucket_entries) {
-    if (w->buckets.buf) {
-      if (hipFree(w->buckets.buf) != hipSuccess) return nullptr;
-      w->buckets.buf = nullptr;
-      w->buckets.bytes = 0;
-    }
-    size_t cnt = n_counters + n_counters / 4;
-    size_t ent = n_entries + n_entries / 4;
-    size_t want = (cnt + ent) * sizeof(int);
-    if (hipMalloc(&w->buckets.buf, want) != hipSuccess) return nullptr;
-    // cleared on the caller's stream, ahead of the kernels that count into it (a clear on the default stream is
-    // not ordered before work on a non-blocking stream)
-    launch_fill_zero<int>((int*)w->buckets.buf, (int)cnt, stream);
-    if (hipGetLastError() != hipSuccess) return nullptr;
-    w->buckets.bytes = want;
-    w->bucket_counters = cnt;
-    w->bucket_entries = ent;
+// Layout of a transpose block: [build counters | counts | keys].  The build counters must read zero when a build
+// starts: a fresh block is cleared once, on the caller's stream (a clear on the default stream is not ordered
+// before work on a non-blocking stream), and every build's sort pass leaves them at zero again.
+static bool transpose_block(DeviceState* st, Workspace* buf, size_t* cap_recv, size_t* cap_keys, size_t n_recv,
+                            size_t n_keys, hipStream_t stream) {
+  if (n_recv > *cap_recv || n_keys > *cap_keys) {
+    const size_t r = n_recv > *cap_recv ? n_recv : *cap_recv;
+    const size_t k = n_keys > *cap_keys ? n_keys : *cap_keys;
+    if (!grow(st, buf, (2 * r + k) * sizeof(int), stream)) return false;
+    // the whole grown block is handed out in the same proportions
+    const size_t have = buf->bytes / sizeof(int);
+    *cap_recv = r + (have - (2 * r + k)) / 4;
+    *cap_keys = have - 2 * *cap_recv;
+    launch_fill_zero<int>((int*)buf->buf, (int)*cap_recv, stream);
+    if (hipGetLastError() != hipSuccess) return false;
   }
-  *entries = (int*)w->buckets.buf + w->bucket_counters;
-  return (int*)w->buckets.buf;
+  return true;
+}
+
+bool bucket_reserve(DeviceState* st, size_t n_recv, int cap, hipStream_t stream, TransposeRef* out) {
+  StreamWork* w = stream_work(st, stream);
+  std::lock_guard<std::mutex> lock(g_mu);
+  if (!transpose_block(st, &w->buckets, &w->bucket_counters, &w->bucket_entries, n_recv, n_recv * cap, stream))
+    return false;
+  out->build_cnt = (int*)w->buckets.buf;
+  out->cnt = out->build_cnt + w->bucket_counters;
+  out->keys = out->cnt + w->bucket_counters;
+  out->cap = cap;
+  out->key_shift = 0;
+  return true;
+}
+
+bool transpose_for_descriptor(DeviceState* st, const int* im2, int nf, int N, int Nrecv, int nr, int cap,
+                              hipStream_t stream, TransposeRef* out) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  const size_t want_recv = (size_t)nf * Nrecv, want_keys = want_recv * cap;
+  Transpose* t = nullptr;
+  for (auto& e : st->transposes)
+    if (e.im2 == im2) { t = &e; break; }
+  if (!t) {
+    // A tensor not seen before takes the place that has not been used for the longest time.  Under capture nothing
+    // can be allocated, so only places whose block is already large enough qualify (a graph recorded earlier with
+    // such a place rebuilds the transpose in it on every replay, before it reads it).
+    const bool capturing = stream_is_capturing(stream);
+    for (auto& e : st->transposes) {
+      if (capturing && (e.cap_recv < want_recv || e.cap_keys < want_keys)) continue;
+      if (!t || e.stamp < t->stamp) t = &e;
+    }
+    if (!t) return false;
+  }
+  const size_t n_recv = (size_t)nf * Nrecv;
+  if (!transpose_block(st, &t->buf, &t->cap_recv, &t->cap_keys, n_recv, n_recv * cap, stream)) return false;
+  t->im2 = im2; t->nf = nf; t->N = N; t->Nrecv = Nrecv; t->nr = nr;
+  t->ref.build_cnt = (int*)t->buf.buf;
+  t->ref.cnt = t->ref.build_cnt + t->cap_recv;
+  t->ref.keys = t->ref.cnt + t->cap_recv;
+  t->ref.cap = cap;
+  t->ref.key_shift = 0;
+  t->stamp = ++st->transpose_clock;
+  *out = t->ref;
+  return true;
+}
+
+bool transpose_find(DeviceState* st, const int* im2_view, int nf, int Nrecv, int Nl, int ld, int nr,
+                    TransposeRef* out) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  for (auto& e : st->transposes) {
+    if (!e.im2 || e.nr != nr || e.nf != nf || e.Nrecv != Nrecv || e.N != ld) continue;
+    if (im2_view < e.im2) continue;
+    const size_t off = (size_t)(im2_view - e.im2);
+    if (off % (size_t)(nr + 1)) continue;
+    const size_t first = off / (size_t)(nr + 1);
+    if (first + (size_t)Nl > (size_t)e.N) continue;
+    e.stamp = ++st->transpose_clock;
+    *out = e.ref;
+    out->key_shift = (int)first;
+    return true;
+  }
+  return false;
 }
 
 template <typename real>
@@ -115,6 +192,7 @@ static int add_n(real* dst, const real* a, const real* b, const real* c, const r
 static int decode_status(int bits) {
   if (bits & 1) return STAF_E_RADIAL_OVERFLOW;
   if (bits & 2) return STAF_E_SCATTER_OVERFLOW;
+  if (bits & 4) return STAF_E_STALE_MAP;
   return STAF_OK;
 }
 
@@ -145,8 +223,8 @@ const char* staf_ops_version(void) { return "0.1"; }
 void staf_ops_set_sync_errors(int mode) { staf::g_sync_errors = mode ? 1 : 0; }
 
 int staf_ops_poll_status(void* stream) {
-  staf::DeviceState* st = staf::device_state();
-  if (!st) return STAF_E_HIP;
+  staf::DeviceState* st = staf::device_state((hipStream_t)stream);
+  if (!st) return staf::reserve_failure((hipStream_t)stream);
   return staf::fetch_status(st, (hipStream_t)stream);
 }
 
@@ -182,6 +260,9 @@ void staf_ops_release(void) {
     if (kv.second.scratch.buf) (void)hipFree(kv.second.scratch.buf);
     if (kv.second.buckets.buf) (void)hipFree(kv.second.buckets.buf);
   }
+  for (auto& t : st->transposes)
+    if (t.buf.buf) (void)hipFree(t.buf.buf);
+  for (void* p : st->retired) (void)hipFree(p);
   if (st->status_d) (void)hipFree(st->status_d);
   if (st->status_h) (void)hipHostFree(st->status_h);
   staf::g_state.erase(it);

@@ -46,10 +46,14 @@ def _view_ptr(t, ld_ref=None):
         if st[0] % row:
             raise ValueError("bad frame stride")
         ld = st[0] // row
+        if ld_ref is not None and ld != ld_ref:
+            raise ValueError("per-centre tensors of one call must share the frame stride")
     else:
-        ld = ld_ref if ld_ref is not None else t.shape[1]
-    if ld_ref is not None and ld != ld_ref:
-        raise ValueError("per-centre tensors of one call must share the frame stride")
+        # one frame: the stride is never used to step, but it still tells whether the tensor is a slice of a
+        # descriptor output [1, N, ...] (frame stride N), which lets the library find what it keeps for that tensor
+        ld = st[0] // row if (st[0] % row == 0 and st[0] // row >= t.shape[1]) else t.shape[1]
+        if ld_ref is not None:
+            ld = ld_ref
     return C.c_void_p(t.data_ptr()), ld
 
 

@@ -37,35 +37,42 @@ def _rot(q):
 def water_frame(lattice, L, sigma, seed, jitter=0.5):
     """One frame: -> pos [3N] (all O then all H, unwrapped, centred on 0), box6.
     Molecule centres are stratified: one per lattice cell, uniform inside `jitter` x the cell edge around
-    the cell centre (0.5 = anywhere in its own cell), which gives the ~38 neighbours within 4.5 A of liquid water."""
+    the cell centre (0.5 = anywhere in its own cell), which gives the ~38 neighbours within 4.5 A of liquid water.
+    A molecule is accepted when none of its atoms is closer than MIN_INTER to an atom placed before it (minimum
+    image); otherwise its orientation and its place in the cell are drawn again, and after every 50 failures the
+    part of the cell it may fall in shrinks towards the cell centre, where a fitting orientation always exists."""
     rng = _rng(seed)
     nx, ny, nz = lattice
     nmol = nx * ny * nz
     half = np.deg2rad(HOH) / 2
     h_local = OH * np.array([[np.sin(half), 0.0, np.cos(half)], [-np.sin(half), 0.0, np.cos(half)]])
     sp = np.array([L / nx, L / ny, L / nz])
+    placed = np.zeros((3 * nmol, 3))
     O = np.zeros((nmol, 3))
     H = np.zeros((nmol, 2, 3))
-    placed = np.zeros((0, 3))
     m = 0
     for iz in range(nz):
         for iy in range(ny):
             for ix in range(nx):
-                c = (np.array([ix, iy, iz]) + 0.5) * sp + rng.uniform(-jitter, jitter, 3) * sp
-                for _ in range(200):
+                centre = (np.array([ix, iy, iz]) + 0.5) * sp
+                for attempt in range(4000):
+                    jit = jitter * 0.8 ** (attempt // 50)
+                    c = centre + rng.uniform(-jit, jit, 3) * sp
                     q = rng.standard_normal(4)
                     q /= np.linalg.norm(q)
                     hs = c + h_local @ _rot(q).T
                     mol = np.vstack([c[None], hs])
-                    if placed.shape[0]:
-                        d = mol[:, None, :] - placed[None, :, :]
+                    if m:
+                        d = mol[:, None, :] - placed[None, :3 * m, :]
                         d -= L * np.rint(d / L)
                         if np.min(np.einsum("abc,abc->ab", d, d)) < MIN_INTER ** 2:
                             continue
                     break
+                else:
+                    raise RuntimeError(f"water_frame: molecule {m} does not fit (seed {seed})")
                 O[m] = c
                 H[m] = hs
-                placed = np.vstack([placed, mol])
+                placed[3 * m:3 * m + 3] = mol
                 m += 1
     pos = np.vstack([O, H.reshape(-1, 3)])
     if sigma > 0:

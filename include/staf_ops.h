@@ -30,8 +30,24 @@
  *     the per-species ops: fingerprint ops write nothing, force ops fill force
  *     (and virial) with zeros, gradient ops fill the parameter gradients with
  *     zeros; the other pointers are not read.
- *   - state is per device and not re-entrant: calls on one device must be
- *     ordered on one stream at a time.
+ *   - state is per device.  Work areas are kept per stream, so calls issued on
+ *     different streams of a device may overlap; calls on one stream are ordered.
+ *     The error word of staf_ops_poll_status is one per device, shared by all
+ *     streams: a poll reports what any of them raised.
+ *   - the force ops gather through a transposed neighbour map that the
+ *     descriptor op builds and keeps beside the intmap2b tensor it writes
+ *     (the 8 most recently written tensors per device).  A force op whose
+ *     interaction_map_rad points into such a tensor (ld_atoms = N) uses that
+ *     transpose; the tensor must then still hold what the descriptor op wrote
+ *     (a slot that does not is reported as STAF_E_STALE_MAP).  Any other copy
+ *     of the map (tf.split output, ld_atoms = N_local) is transposed by the
+ *     force op itself, at the price of two more launches.
+ *   - graph capture: every entry point may be captured once the same call (same
+ *     shapes, same stream, same output tensors for the descriptor op) has run
+ *     eagerly, which sizes the library's work areas; a call that would have to
+ *     allocate under capture returns STAF_E_CAPTURE and allocates nothing.
+ *     Outgrown work areas stay allocated until staf_ops_release, so graphs
+ *     recorded earlier keep valid addresses.
  */
 #ifndef STAF_OPS_H
 #define STAF_OPS_H
@@ -47,6 +63,10 @@ extern "C" {
 #define STAF_E_RADIAL_OVERFLOW (-10) /* an atom has more than radial_buffer neighbours (reference: exit(0), reforce.cc:329-337) */
 #define STAF_E_SCATTER_OVERFLOW (-11)/* an atom is listed by more centres than the force scatter can hold (4*nr) */
 #define STAF_E_LIMIT (-12)           /* nt, channels or buffers beyond the kernels' compile-time limits */
+#define STAF_E_CAPTURE (-13)         /* the stream is being captured into a graph and the call would have to allocate:
+                                        run the same call once outside the capture first */
+#define STAF_E_STALE_MAP (-14)       /* a force op was handed a view of a descriptor output whose intmap2b no longer
+                                        holds what the descriptor op wrote there */
 
 /* ---- library state ------------------------------------------------------ */
 
@@ -85,11 +105,14 @@ int staf_op_construct_descriptors_light_f32(float radial_cutoff, int radial_buff
 int staf_op_construct_descriptors_light_f64(double radial_cutoff, int radial_buffer, int angular_buffer, int numpar,
                                             double rs, double ra, int max_batch, const char* cutoff_curve_path);
 
-/* Options of the descriptor op (apply to both precisions; call after construct).
+/* Options of the descriptor op (apply to both precisions on the current device; construct resets them to their
+ * defaults, so call this after construct).
  *   dist2_fma     0: dist2 = (x*x+y*y)+z*z uncontracted (default); 1: fma(z,z,fma(y,y,x*x))
- *   zero_padding  0: slots of angdescr, intmap3b and der3b beyond an atom's triplets are left untouched like the
- *                    reference, which never writes any padding (default);
- *                 1: they are written as 0.  (The nr-wide outputs are always fully written, padding as 0.) */
+ *   zero_padding  0: der3b beyond an atom's triplets is left untouched (default; the reference leaves it
+ *                    uninitialised as well); 1: it is written as 0.
+ * All other padding is always written as 0: angdescr, intmap2b, intmap3b and numtriplet are zeroed by the reference
+ * op before its kernels run (reforce.cc:357-358,375-376,385-386,420-421), and the padded slots of raddescr,
+ * des3bsupp, der2b and der3bsupp, which the reference leaves uninitialised, are written as 0 too. */
 int staf_op_descriptor_options(int dist2_fma, int zero_padding);
 
 /* Frames of at least n_atoms atoms find their neighbours through a cell list (the role of the binning kernels of
@@ -107,7 +130,8 @@ int staf_op_descriptor_coefficients_f64(double* out5);
  *   positions [nf, 3N] Cartesian, boxer [nf, 6] = [Lx, xy, xz, Ly, yz, Lz]
  *   raddescr [nf,N,nr]  angdescr [nf,N,na]  des3bsupp [nf,N,nr]  intmap2b [nf,N,nr+1]
  *   intmap3b [nf,N,2*na]  der2b [nf,N,3,nr]  der3b [nf,N,3,2*na]  der3bsupp [nf,N,3,nr]  numtriplet [nf,N]
- * Padded slots are written as 0 (der3b: see staf_op_descriptor_options). */
+ * Padded slots are written as 0 (der3b: see staf_op_descriptor_options).  Also builds the transposed neighbour map
+ * of intmap2b that the force ops use (kept by the library, keyed by the address of intmap2b). */
 int staf_op_compute_descriptors_light_f32(const float* positions, const float* boxer, int nf, int N, float* raddescr,
                                           float* angdescr, float* des3bsupp, int* intmap2b, int* intmap3b,
                                           float* der2b, float* der3b, float* der3bsupp, int* numtriplet,
@@ -157,14 +181,15 @@ int staf_op_init_grad_force_tripl(int buffdim);
 
 /* Virial forms only: 0 (default) = r_i - r_j is wrapped to the minimum image of the periodic box; 1 = no wrap, the
  * neighbour positions already are the periodic images (domain-decomposed MD with ghost atoms).  Process-wide, like
- * staf_force_skip_pbc of the reference (STAF/include/staf_force_pbc.cuh:5-10). */
+ * staf_force_skip_pbc of the reference (STAF/include/staf_force_pbc.cuh:5-10); read by the staf_op_* entry points of
+ * this header only (staf_compute of staf.h decides per call and neither reads nor changes it). */
 void staf_op_force_set_skip_pbc(int skip);
 
 /* computeforce_doublets_Launcher (ComputeForceRadial) -- STAF/src/force/rad/reforce.cc:39-57, reforce.cu.cc:45-172
  * and computeforce_doublets_virial_Launcher (ComputeForceRadialVirial) -- reforce.cc:124-146, reforce.cu.cc:174-314.
  *   forces2b [nf,3N] (all atoms; fully written).  virial [nf,9] row-major W_ab -= g_a r_b, pos [nf,3N]
  *   Cartesian, box [nf,6]; pass virial = pos = box = NULL for the plain op.
- * Deterministic: per-slot pair forces are reduced by an owner-computes gather, no float atomics. */
+ * Deterministic: every atom gathers the pair forces of the slots that list it, in a fixed order; no float atomics. */
 int staf_op_force_doublets_f32(const float* netderiv, const float* des_r, const float* intderiv_r,
                                const int* intmap_r, int nr, int N, int dimbat, int num_alpha_radiale,
                                const float* alpha_radiale, const float* type_emb2b, int nt, const int* tipos,

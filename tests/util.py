@@ -100,6 +100,22 @@ def nerr(a, b):
     return float(np.max(np.abs(a - b)) / (s if s > 0 else 1.0))
 
 
+def eerr(a, b, where=None):
+    """Element-wise error max_e |a_e - b_e| / (|b_e| + rms(b)): `eerr <= tol` is the statement
+    |a - b| <= tol |b| + tol rms(b) for every element, so small entries are held to the scale of the typical
+    entry and not to that of the largest one.  where: boolean mask of the elements that count (rms over them)."""
+    a = np.asarray(a, np.float64)
+    b = np.asarray(b, np.float64)
+    if where is not None:
+        a, b = a[where], b[where]
+    if b.size == 0:
+        return 0.0
+    rms = float(np.sqrt(np.mean(b * b)))
+    if rms == 0.0:
+        return float(np.max(np.abs(a - b)))
+    return float(np.max(np.abs(a - b) / (np.abs(b) + rms)))
+
+
 def radial_mask(intmap2b, nr):
     """[nf,N,nr] True on active neighbour slots."""
     return np.arange(nr)[None, None, :] < intmap2b[:, :, :1]
