@@ -12,6 +12,10 @@
 #include "staf_reduce.hpp"
 #include "staf_tri.hpp"
 
+#include <stdio.h>
+#include <mutex>
+#include <unordered_map>
+
 namespace staf {
 
 constexpr int AF_BLOCK = 256;
@@ -179,39 +183,122 @@ static int radial_afs(const real* D, int nr, const real* alpha2b, int Ar, real* 
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }
 
+// Work area of the 2-body parameter gradient: one row of 2*nt*Ar partial sums per workgroup of grad2_kernel, then
+// RED_SLICES rows for the first pass of the reduction.
+static inline size_t grad2_work_reals(int nf, int Nl, int nt, int Ar) {
+  return ((size_t)grad_blocks(nf * Nl) + RED_SLICES) * 2 * nt * Ar;
+}
+
 template <typename real>
-static int alpha_dist_grad(const real* D, int nr, const real* alpha2b, int Ar, real* g_alpha, int nf, int Nl,
-                           const int* im2, const real* P, const real* emb2b, const int* type_map, real* g_emb, int nt,
-                           int ld, void* stream_) {
-  if (Nl == 0 && nf > 0 && Ar > 0 && nt > 0 && g_alpha && g_emb) {
-    // a species without atoms in these frames: its sums are empty
-    launch_fill_zero<real>(g_alpha, nt * Ar, (hipStream_t)stream_);
-    launch_fill_zero<real>(g_emb, nt * Ar, (hipStream_t)stream_);
-    return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
-  }
+static int alpha_dist_grad_check(const real* D, int nr, const real* alpha2b, int Ar, real* g_alpha, int nf, int Nl,
+                                 const int* im2, const real* P, const real* emb2b, const int* type_map, real* g_emb,
+                                 int nt) {
   if (!D || !alpha2b || !g_alpha || !g_emb || !im2 || !P || !emb2b || !type_map || nr <= 0 || Ar <= 0 || nf <= 0 ||
       Nl <= 0 || nt <= 0)
     return STAF_E_BAD_ARG;
   if (nt > NT_MAX) return STAF_E_LIMIT;
-  if (ld <= 0) ld = Nl;
-  DeviceState* st = device_state((hipStream_t)stream_);
-  if (!st) return reserve_failure((hipStream_t)stream_);
-  hipStream_t stream = (hipStream_t)stream_;
+  const size_t lds = (size_t)(2 * nt * Ar + AF_WAVES * 2 * nt * Ar + AF_WAVES * nr) * sizeof(real) +
+                     (size_t)AF_WAVES * (2 * nr + NT_MAX + 1) * sizeof(int);
+  if (lds > 64 * 1024) return STAF_E_LIMIT;
+  return STAF_OK;
+}
+
+// Launches grad2_kernel and the fixed-order reduction on `work` (grad2_work_reals reals, every element written
+// before it is read: nothing has to be cleared).  timed: bracket the kernel with events when timing is switched on.
+template <typename real>
+static int alpha_dist_grad_launch(const real* D, int nr, const real* alpha2b, int Ar, real* g_alpha, int nf, int Nl,
+                                  const int* im2, const real* P, const real* emb2b, const int* type_map, real* g_emb,
+                                  int nt, int ld, real* work, bool timed, hipStream_t stream) {
   const int nout = 2 * nt * Ar;
   const int nb = grad_blocks(nf * Nl);
-  real* partial = (real*)scratch_reserve(st, stream, ((size_t)nb + RED_SLICES) * nout * sizeof(real));
-  real* red_tmp = partial ? partial + (size_t)nb * nout : nullptr;
-  if (!partial) return reserve_failure(stream);
-  size_t lds = (size_t)(2 * nt * Ar + AF_WAVES * nout + AF_WAVES * nr) * sizeof(real) +
-               (size_t)AF_WAVES * (2 * nr + NT_MAX + 1) * sizeof(int);
-  if (lds > 64 * 1024) return STAF_E_LIMIT;
-  {
+  real* partial = work;
+  real* red_tmp = work + (size_t)nb * nout;
+  const size_t lds = (size_t)(2 * nt * Ar + AF_WAVES * nout + AF_WAVES * nr) * sizeof(real) +
+                     (size_t)AF_WAVES * (2 * nr + NT_MAX + 1) * sizeof(int);
+  if (timed) {
     KernelTimer kt_("grad2_kernel", stream);
+    hipLaunchKernelGGL(grad2_kernel<real>, dim3(nb), dim3(AF_BLOCK), lds, stream, D, im2, alpha2b, emb2b, type_map, P,
+                       partial, nf, Nl, ld, nr, Ar, nt);
+  } else {
     hipLaunchKernelGGL(grad2_kernel<real>, dim3(nb), dim3(AF_BLOCK), lds, stream, D, im2, alpha2b, emb2b, type_map, P,
                        partial, nf, Nl, ld, nr, Ar, nt);
   }
   launch_reduce_partials<real>(partial, nb, nout, g_alpha, nt * Ar, nt * Ar, g_emb, nt * Ar, nt * Ar, red_tmp, stream);
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
+}
+
+template <typename real>
+static int alpha_dist_grad(const real* D, int nr, const real* alpha2b, int Ar, real* g_alpha, int nf, int Nl,
+                           const int* im2, const real* P, const real* emb2b, const int* type_map, real* g_emb, int nt,
+                           int ld, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (Nl == 0 && nf > 0 && Ar > 0 && nt > 0 && g_alpha && g_emb) {
+    // a species without atoms in these frames: its sums are empty
+    launch_fill_zero<real>(g_alpha, nt * Ar, stream);
+    launch_fill_zero<real>(g_emb, nt * Ar, stream);
+    return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
+  }
+  const int rc = alpha_dist_grad_check<real>(D, nr, alpha2b, Ar, g_alpha, nf, Nl, im2, P, emb2b, type_map, g_emb, nt);
+  if (rc) return rc;
+  if (ld <= 0) ld = Nl;
+  DeviceState* st = device_state((hipStream_t)stream_);
+  if (!st) return reserve_failure((hipStream_t)stream_);
+  real* work = (real*)scratch_reserve(st, stream, grad2_work_reals(nf, Nl, nt, Ar) * sizeof(real));
+  if (!work) return reserve_failure(stream);
+  return alpha_dist_grad_launch<real>(D, nr, alpha2b, Ar, g_alpha, nf, Nl, im2, P, emb2b, type_map, g_emb, nt, ld,
+                                      work, true, stream);
+}
+
+// ---- the same op for callers that cannot allocate -------------------------------------------------------------
+// Work area in the library's own image instead of hipMalloc'ed memory: each GPU the library is loaded on holds its
+// own copy of this array, at its own address, until the process ends.  The name below is a host-side handle only;
+// the device address is asked for once per device (noalloc_work) and that address is what kernels are given.
+constexpr size_t NOALLOC_WORK_BYTES = (size_t)1 << 20;
+static __device__ __align__(256) unsigned char scratch[NOALLOC_WORK_BYTES];
+
+static std::mutex g_noalloc_mu;
+static std::unordered_map<int, void*> g_noalloc_ptr;   // device ordinal -> device address of `scratch` there
+
+static void* noalloc_work() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+  std::lock_guard<std::mutex> lock(g_noalloc_mu);
+  auto it = g_noalloc_ptr.find(dev);
+  if (it != g_noalloc_ptr.end()) return it->second;
+  void* ptr = nullptr;
+  if (hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  g_noalloc_ptr.emplace(dev, ptr);
+  return ptr;
+}
+
+static int alpha_dist_grad_noalloc(const double* D, int nr, const double* alpha2b, int Ar, double* g_alpha, int nf,
+                                   int Nl, const int* im2, const double* P, const double* emb2b, const int* type_map,
+                                   double* g_emb, int nt, int ld, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (Nl == 0 && nf > 0 && Ar > 0 && nt > 0 && g_alpha && g_emb) {
+    launch_fill_zero<double>(g_alpha, nt * Ar, stream);
+    launch_fill_zero<double>(g_emb, nt * Ar, stream);
+    return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
+  }
+  const int rc = alpha_dist_grad_check<double>(D, nr, alpha2b, Ar, g_alpha, nf, Nl, im2, P, emb2b, type_map, g_emb, nt);
+  if (rc) return rc;
+  const size_t need = grad2_work_reals(nf, Nl, nt, Ar) * sizeof(double);
+  if (need > NOALLOC_WORK_BYTES) {
+    fprintf(stderr,
+            "staf_op_alpha_dist_grad_noalloc_f64: nt = %d, nalpha_r = %d need a work area of %zu bytes, the built-in "
+            "one holds %zu (nt * nalpha_r <= %zu); use staf_op_alpha_dist_grad_f64\n",
+            nt, Ar, need, NOALLOC_WORK_BYTES,
+            NOALLOC_WORK_BYTES / (sizeof(double) * 2 * ((size_t)GRAD_MAX_BLOCKS + RED_SLICES)));
+    return STAF_E_LIMIT;
+  }
+  if (ld <= 0) ld = Nl;
+  double* work = (double*)noalloc_work();
+  if (!work) return STAF_E_HIP;
+  return alpha_dist_grad_launch<double>(D, nr, alpha2b, Ar, g_alpha, nf, Nl, im2, P, emb2b, type_map, g_emb, nt, ld,
+                                        work, false, stream);
 }
 
 template <typename real>
@@ -315,6 +402,12 @@ int staf_op_alpha_dist_grad_f64(const double* D, int nr, const double* alpha2b, 
                                 int Nl, const int* im2, const double* P, const double* emb2b, const int* type_map,
                                 double* g_emb, int nt, int ld, void* stream) {
   return staf::alpha_dist_grad<double>(D, nr, alpha2b, Ar, g_alpha, nf, Nl, im2, P, emb2b, type_map, g_emb, nt, ld,
+                                       stream);
+}
+int staf_op_alpha_dist_grad_noalloc_f64(const double* D, int nr, const double* alpha2b, int Ar, double* g_alpha,
+                                        int nf, int Nl, const int* im2, const double* P, const double* emb2b,
+                                        const int* type_map, double* g_emb, int nt, int ld, void* stream) {
+  return staf::alpha_dist_grad_noalloc(D, nr, alpha2b, Ar, g_alpha, nf, Nl, im2, P, emb2b, type_map, g_emb, nt, ld,
                                        stream);
 }
 int staf_op_alphagrad_ang_f32(const float* Dsup, const float* Tang, int nr, int na, const float* P, int nf, int Nl,

@@ -231,6 +231,21 @@ int staf_op_alpha_dist_grad_f64(const double* radial_descriptor, int nr, const d
                                 const double* prevgrad, const double* type_emb2b, const int* type_map,
                                 double* nextgrad_emb2b, int nt, int ld_atoms, void* stream);
 
+/* The same op for callers that cannot allocate device memory (code under HIP graph capture that has not run the
+ * call eagerly before, serving loops and harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * Arguments and results as staf_op_alpha_dist_grad_f64, bit for bit; the work area (partial sums of the workgroups)
+ * is a 1 MiB array in the library's own device image instead of memory grown on demand, which limits the call to
+ * (min(ceil(dimbat * N_local / 4), 1024) + 32) * 2 * nt * nalpha_r * 8 bytes <= 1 MiB -- any batch with
+ * nt * nalpha_r <= 62 -- and returns STAF_E_LIMIT with a message on stderr beyond that.  The call allocates nothing and frees
+ * nothing.  All calls on one GPU share that array: calls that overlap on one GPU (different streams or threads)
+ * race.  The first call on a device looks up the array's device address (hipGetSymbolAddress): make it outside a
+ * capture. */
+int staf_op_alpha_dist_grad_noalloc_f64(const double* radial_descriptor, int nr, const double* alpha2b, int nalpha_r,
+                                        double* nextgrad_alpha2b, int dimbat, int N_local,
+                                        const int* interaction_map_rad, const double* prevgrad,
+                                        const double* type_emb2b, const int* type_map, double* nextgrad_emb2b, int nt,
+                                        int ld_atoms, void* stream);
+
 /* alphagrad_ang_Launcher (ComputeSortProj3bodyGrad) -- STAF/src/grad_finger/ang/reforce.cc:12-31, reforce.cu.cc:13-133.
  *   prevgrad [nf,Nl,nsmooth_a] = dL/dAF3 -> next_alpha3b_grad [nt_couple,3*nsmooth_a],
  *   next_emb3b_grad [nt_couple,nsmooth_a] (identically zero, as in the reference). */
