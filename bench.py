@@ -24,23 +24,79 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (see profiles/),
-# scaled by what the same counters read for a copy kernel of known size; None where no such run was made.
-TRAFFIC = {
-    # (FETCH_SIZE KiB x 2.0 + WRITE_SIZE KiB x 1.0) x 1024, averaged over the two per-species launches of a step;
-    # factors from the 1 GiB device copies of this script in the same runs
-    # (profiles/force3_kernel_water768_f32_hbm_counters.txt, profiles/gradforce3_kernel_water768_f64_hbm_counters.txt)
-    ("force3_kernel", "water768_f32"): 38.1e6,
-    ("gradforce3_kernel", "water768_f64"): 95.2e6,
+SETTLE_STEPS = 300   # untimed graph replays of the set-up, see run_workload()
+REPEATS = 5          # timed blocks of --steps steps each; the median block is reported
+
+PROFILES = os.path.join(ROOT, "profiles")
+# bench.py's kernel names (the library's timing names) -> the names the profiler prints
+PROFILED_NAME = {
+    ("force3_kernel", "f32"): "staf::force3_kernel<float>",
+    ("force3_kernel", "f64"): "staf::force3_kernel<double>",
+    ("gradforce3_kernel", "f32"): "staf::tri_reduce_kernel<float, 2>",
+    ("gradforce3_kernel", "f64"): "staf::tri_reduce_kernel<double, 2>",
+    ("af3_kernel", "f32"): "staf::tri_reduce_kernel<float, 0>",
+    ("af3_kernel", "f64"): "staf::tri_reduce_kernel<double, 0>",
+    ("grad3_kernel", "f32"): "staf::tri_reduce_kernel<float, 1>",
+    ("grad3_kernel", "f64"): "staf::tri_reduce_kernel<double, 1>",
+    ("desc_kernel", "f32"): "staf::desc_kernel<float>",
+    ("desc_kernel", "f64"): "staf::desc_kernel<double>",
 }
-# Share of the GPU's vector-issue slots that the same kernel fills when launched alone (SQ_INSTS_VALU x 4 cycles over
-# duration x 1024 SIMDs x 2.4 GHz, time-weighted over the two per-species launches; profiles/*_sq_counters.txt):
-# the roofline these kernels actually run against, reported beside the HBM one
-SETTLE_STEPS = 300   # untimed graph replays of the set-up, see main()
-VALU_ISSUE = {
-    ("force3_kernel", "water768_f32"): 0.53,
-    ("gradforce3_kernel", "water768_f64"): 0.55,
-}
+
+
+class ProfileMissing(RuntimeError):
+    pass
+
+
+def profile_traffic(kernel, workload, prec):
+    """HBM bytes per launch of `kernel` in `workload` from the committed rocprofv3 --pmc summary
+    profiles/<kernel>_<workload>_hbm_counters.txt: (FETCH_SIZE x f + WRITE_SIZE x w) KiB averaged over the kernel's
+    launches of a step, f and w = 1 GiB over what the same counter reads for the 1 GiB device copies of the same run.
+    Raises ProfileMissing when the file, the kernel or the calibration copy is not in it."""
+    import re
+    path = os.path.join(PROFILES, f"{kernel}_{workload}_hbm_counters.txt")
+    if not os.path.exists(path):
+        raise ProfileMissing(f"{path} not found: no measured HBM traffic for {kernel} in {workload}")
+    want = PROFILED_NAME[(kernel, prec)]
+    vals = {"FETCH_SIZE": {}, "WRITE_SIZE": {}}
+    copy = {}
+    for line in open(path):
+        m = re.match(r"^(.*?)\s+(\d+)\s+(FETCH_SIZE|WRITE_SIZE)=([0-9.eE+-]+)\(n=(\d+)\)\s*$", line)
+        if not m:
+            continue
+        name, grid, ctr, v, n = m.group(1), int(m.group(2)), m.group(3), float(m.group(4)), int(m.group(5))
+        if name.startswith("__amd_rocclr_copyBuffer") and v > 1e5:
+            copy[ctr] = v
+        elif want in name:
+            vals[ctr][grid] = (v, n)
+    if len(copy) != 2 or not vals["FETCH_SIZE"] or set(vals["FETCH_SIZE"]) != set(vals["WRITE_SIZE"]):
+        raise ProfileMissing(f"{path}: no rows for {want} (or no 1 GiB calibration copy) in both counters")
+    kib = 0.0
+    for grid, (f, _) in vals["FETCH_SIZE"].items():
+        w, _ = vals["WRITE_SIZE"][grid]
+        kib += f * (1048576.0 / copy["FETCH_SIZE"]) + w * (1048576.0 / copy["WRITE_SIZE"])
+    return kib / len(vals["FETCH_SIZE"]) * 1024.0, os.path.relpath(path, ROOT)
+
+
+def profile_valu_share(kernel, workload, mode, prec):
+    """Share of the GPU's vector-issue slots that `kernel` fills when launched alone (column `issue` of
+    profiles/step_<mode>_<workload>_sq_counters.txt, time-weighted over the kernel's launches of a step)."""
+    tag = {"fwd_force": "step_fwd_force", "full_step": "step_full"}[mode]
+    path = os.path.join(PROFILES, f"{tag}_{workload}_sq_counters.txt")
+    if not os.path.exists(path):
+        raise ProfileMissing(f"{path} not found: no SQ counters for {workload} ({mode})")
+    want = PROFILED_NAME[(kernel, prec)].replace("staf::", "")
+    num = den = 0.0
+    for line in open(path):
+        if not line.startswith(want):
+            continue
+        rest = line[len(want):].split()
+        # grid waves avg_us VALU LDS issue ...
+        us, issue = float(rest[2]), float(rest[5])
+        num += us * issue
+        den += us
+    if den == 0.0:
+        raise ProfileMissing(f"{path}: no row for {want}")
+    return num / den, os.path.relpath(path, ROOT)
 
 
 def algorithmic_bytes(N, tipos, nr, na, Ar, Aa, nt, s):
@@ -139,7 +195,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="water768_f32")
+    ap.add_argument("--workload", default=None,
+                    help="one workload only (water96, water768_f32, water768_f64, water768_train8, water6144); "
+                         "default: the headline water768_f32 fwd_force with the water768_f64 full_step record nested "
+                         "under \"also\"")
     ap.add_argument("--mode", default=None, choices=[None, "fwd_force", "full_step"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--streams", type=int, default=3, choices=[1, 2, 3],
@@ -155,18 +214,29 @@ def main():
         print("bench.py: this build measures one GPU only (frames are independent; see DESIGN.md for sharding); "
               "run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    if workload is not None:
+        out = run_workload(args, workload, args.mode)
+    else:
+        # The metric names both halves: fp32 descriptor fwd + force (the headline line) and the fp64 full step with
+        # the parameter-gradient ops, measured in the same process right behind it.
+        out = run_workload(args, "water768_f32", "fwd_force")
+        out["also"] = [run_workload(args, "water768_f64", "full_step")]
+    print(json.dumps(out))
 
+
+def run_workload(args, workload, mode):
     import torch
     from alphanesgpu_amd import ops, synth
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import pipeline
 
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        sys.exit(1)
     dev = torch.device("cuda:0")
-    batch = synth.water_batch(args.workload)
-    mode = args.mode or ("fwd_force" if args.workload in ("water768_f32", "water6144") else "full_step")
+    batch = synth.water_batch(workload)
+    mode = mode or ("fwd_force" if workload in ("water768_f32", "water6144") else "full_step")
     dtype = batch["dtype"]
     tdt = torch.float32 if dtype == np.float32 else torch.float64
     nr, na = synth.NR, synth.NA
@@ -320,8 +390,12 @@ def main():
             small_species()
             for ev in done:
                 main_stream.wait_event(ev)
-            for f in forces.values():
-                f.record_stream(main_stream)
+            # eager steps: the force arrays were allocated on the side streams and are consumed on this one.  Under
+            # capture the graph's private pool keeps them (and `forces` holds them until the sum is recorded): no
+            # allocator event is queued inside the captured region.
+            if not torch.cuda.is_current_stream_capturing():
+                for f in forces.values():
+                    f.record_stream(main_stream)
         # total force = sum of the per-op force arrays (the reference's force_radial + force_angular and add_n over
         # the species), one launch, always in the same order
         return ops.add_n([forces[(k, body)] for k in range(nt) for body in (2, 3)])
@@ -353,12 +427,17 @@ def main():
     for _ in range(args.warmup):
         run()
     ops.poll_status()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        run()
-    torch.cuda.synchronize()
-    el = time.perf_counter() - t0
+    # REPEATS blocks of exactly --steps steps, each between two device synchronisations; the median block is the
+    # figure reported (a single block of 20 steps lasts under 3 ms and picks up whatever else the host does)
+    block_s = []
+    for _ in range(REPEATS):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            run()
+        torch.cuda.synchronize()
+        block_s.append(time.perf_counter() - t0)
+    el = float(np.median(block_s))
     ops.poll_status()
     if graph is not None:
         # the replayed graph must reproduce the eager step bit for bit (all reductions have a fixed order)
@@ -412,7 +491,7 @@ def main():
     s = np.dtype(dtype).itemsize
     ab = algorithmic_bytes(N, tipos, nr, na, Ar, Aa, nt, s)
     kern = {}
-    for name in list(ab) + ["gather_kernel"]:
+    for name in list(ab) + ["gather_kernel", "transpose_sort_kernel", "cell_build_kernel"]:
         ms, n = ops.kernel_time(name)
         if n:
             kern[name] = dict(ms_per_step=ms / nprof, launches_per_step=n // nprof, avg_launch_ms=ms / n)
@@ -431,6 +510,22 @@ def main():
     dom = max((k for k in kern if k in ab), key=lambda k: kern[k]["ms_per_step"])
     dom_bytes_per_launch = ab[dom] * nf / kern[dom]["launches_per_step"]
     achieved = dom_bytes_per_launch / (kern[dom]["avg_launch_ms"] * 1e-3) / 1e9
+    prec = "f32" if dtype == np.float32 else "f64"
+    try:
+        traffic, traffic_src = profile_traffic(dom, workload, prec)
+    except ProfileMissing as e:
+        if workload in ("water768_f32", "water768_f64"):
+            raise SystemExit(f"bench.py: {e}")      # the configurations the metric is quoted on must be profiled
+        traffic, traffic_src = None, str(e)
+    try:
+        valu_share, valu_src = profile_valu_share(dom, workload, mode, prec)
+    except ProfileMissing as e:
+        if workload in ("water768_f32", "water768_f64"):
+            raise SystemExit(f"bench.py: {e}")
+        valu_share, valu_src = None, str(e)
+    # bytes desc_kernel really writes: the nr-wide tensors, angdescr and intmap3b over their whole rows (padding is
+    # written as 0 like the reference's memsets), der3b over the triplets that exist only
+    desc_written = N * (8 * nr + na) * s + N * (nr + 1 + 2 * na + 1) * 4 + N * 6 * na_act * s + (3 * N + 6) * s
     out = {
         "metric": "frames/s descriptor fwd+force/alpha bwd, 768-atom water fp32/fp64; % HBM roofline",
         "value": nf * args.steps / el,
@@ -442,25 +537,33 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32" if dtype == np.float32 else "f64",
+        "dtype": prec,
         "data": "synthetic",
-        "config": {"workload": args.workload, "mode": mode, "atoms": N, "frames_per_step": nf, "Rc": synth.RC,
+        "config": {"workload": workload, "mode": mode, "atoms": N, "frames_per_step": nf, "Rc": synth.RC,
                    "radial_buffer": nr, "angular_buffer": na, "Ar": Ar, "Aa": Aa,
+                   "descriptor_padding": "library default = the reference op's: angdescr, intmap2b, intmap3b, "
+                                         "numtriplet zero beyond the active slots; der3b padding left untouched",
                    "species_tensors": "contiguous copies" if args.contiguous_splits else "views",
                    "species_streams": args.streams,
                    "schedule": {1: "one stream", 2: "one stream per species",
                                 3: "one stream per species, 2-body ops of the largest species on the step's stream"
                                 }[args.streams],
-                   "launch": "python per op" if graph is None else "hip graph replay"},
+                   "launch": "python per op" if graph is None else "hip graph replay",
+                   "timing": f"median of {REPEATS} blocks of {args.steps} steps"},
+        "block_ms_per_step": [b / args.steps * 1e3 for b in block_s],
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": TRAFFIC.get((dom, args.workload)),
-                     "valu_issue_share": VALU_ISSUE.get((dom, args.workload)),
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                     "traffic_source": traffic_src,
+                     "valu_issue_share": valu_share, "valu_issue_share_source": valu_src,
                      "measured_copy_GBs": copy_gbs, "frac_of_measured_copy": achieved / copy_gbs,
                      "algorithmic_bytes_per_launch": dom_bytes_per_launch,
                      "avg_launch_ms": kern[dom]["avg_launch_ms"],
                      "launches_per_step": kern[dom]["launches_per_step"]},
         "kernel_hbm_frac": {k: ab[k] * nf / (kern[k]["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS
                             for k in kern if k in ab},
+        # desc_kernel against the bytes it writes (its signature's bytes include der3b padding it leaves alone)
+        "desc_kernel_hbm_frac_of_written_bytes": desc_written * nf / (kern["desc_kernel"]["ms_per_step"] * 1e-3) / 1e9
+                                                 / HBM_PEAK_GBS,
         "kernel_ms_per_step": {k: v["ms_per_step"] for k, v in kern.items()},
         "whole_step_hbm_frac": step_bytes * nf / (el / args.steps) / 1e9 / HBM_PEAK_GBS,
         "whole_step_frac_of_measured_copy": step_bytes * nf / (el / args.steps) / 1e9 / copy_gbs,
@@ -472,7 +575,9 @@ def main():
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(batch, params, up, mode, nr, na)
-    print(json.dumps(out))
+    # leave the device as the next workload of this process expects to find it
+    ops.set_sync_errors(True)
+    return out
 
 
 if __name__ == "__main__":

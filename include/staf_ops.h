@@ -86,7 +86,8 @@ int staf_ops_poll_status(void* stream);
 /* Measurement aid with no counterpart in the reference: when enabled, the library brackets its kernels with HIP
  * events on the stream they are launched on.  staf_ops_kernel_time waits for the device, returns the summed duration
  * and the number of launches of the named kernel ("desc_kernel", "af2_kernel", "af3_kernel", "force2_kernel",
- * "force3_kernel", "gather_kernel", "grad2_kernel", "grad3_kernel", "gradforce2_kernel", "gradforce3_kernel")
+ * "force3_kernel", "gather_kernel", "grad2_kernel", "grad3_kernel", "gradforce2_kernel", "gradforce3_kernel",
+ * "transpose_sort_kernel", "cell_build_kernel")
  * since the last call for that name, and forgets them. */
 void staf_ops_kernel_timing(int enable);
 int staf_ops_kernel_time(const char* kernel, double* total_ms, int* launches);
