@@ -301,29 +301,38 @@ static int alpha_dist_grad_noalloc(const double* D, int nr, const double* alpha2
                                         work, false, stream);
 }
 
+// unit != null (the MD entry): the fused kernel, which rebuilds the angular descriptor from the slots' unit vectors
+// instead of reading Tang (may be null then).
 template <typename real>
-static int angular_afs(const real* Dsup, const real* Tang, int nr, int na, real* out, int nf, int Nl, const int* im3,
-                       const int* im2, const real* alpha3b, int Aa, const real* emb3b, const int* type_map,
-                       const int* numtriplet, int nt, int ld, void* stream_) {
+int angular_afs(const real* Dsup, const real* Tang, const real* unit, int nr, int na, real* out, int nf, int Nl,
+                const int* im3, const int* im2, const real* alpha3b, int Aa, const real* emb3b, const int* type_map,
+                const int* numtriplet, int nt, int ld, void* stream_) {
   (void)im3;
   if (Nl == 0 && nf > 0 && Aa > 0) return STAF_OK;   // a species without atoms in these frames: nothing to write
-  if (!Dsup || !Tang || !out || !im2 || !alpha3b || !emb3b || !type_map || !numtriplet || nr <= 0 || na <= 0 ||
-      Aa <= 0 || nf <= 0 || Nl <= 0 || nt <= 0)
+  if (!Dsup || (!Tang && !unit) || !out || !im2 || !alpha3b || !emb3b || !type_map || !numtriplet || nr <= 0 ||
+      na <= 0 || Aa <= 0 || nf <= 0 || Nl <= 0 || nt <= 0)
     return STAF_E_BAD_ARG;
   if (nt > NT_MAX) return STAF_E_LIMIT;
   if (ld <= 0) ld = Nl;
-  size_t lds = TriLds<real, 0>::bytes(nr, Aa, nt);
+  size_t lds = TriLds<real, 0>::bytes(nr, Aa, nt, unit != nullptr);
   if (lds > 64 * 1024) return STAF_E_LIMIT;
   TriArgs<real> A = {};
-  A.Dsup = Dsup; A.Tang = Tang; A.im2 = im2; A.alpha3b = alpha3b; A.emb3b = emb3b; A.type_map = type_map;
-  A.numtriplet = numtriplet; A.out = out;
+  A.Dsup = Dsup; A.Tang = Tang; A.unit = unit; A.im2 = im2; A.alpha3b = alpha3b; A.emb3b = emb3b;
+  A.type_map = type_map; A.numtriplet = numtriplet; A.out = out;
   A.nf = nf; A.Nl = Nl; A.ld = ld; A.nr = nr; A.na = na; A.Aa = Aa; A.nt = nt;
   {
     KernelTimer kt_("af3_kernel", (hipStream_t)stream_);
-    hipLaunchKernelGGL((tri_reduce_kernel<real, 0>), dim3(nf * Nl), dim3(TRI_BLOCK), lds, (hipStream_t)stream_, A);
+    if (unit)
+      hipLaunchKernelGGL((tri_reduce_kernel<real, 0, true>), dim3(nf * Nl), dim3(TRI_BLOCK), lds,
+                         (hipStream_t)stream_, A);
+    else
+      hipLaunchKernelGGL((tri_reduce_kernel<real, 0>), dim3(nf * Nl), dim3(TRI_BLOCK), lds, (hipStream_t)stream_, A);
   }
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }
+template int angular_afs<double>(const double*, const double*, const double*, int, int, double*, int, int, const int*,
+                                 const int*, const double*, int, const double*, const int*, const int*, int, int,
+                                 void*);
 
 template <typename real>
 static int alphagrad_ang(const real* Dsup, const real* Tang, int nr, int na, const real* P, int nf, int Nl,
@@ -383,14 +392,14 @@ int staf_op_radial_afs_f64(const double* D, int nr, const double* alpha2b, int A
 int staf_op_angular_afs_f32(const float* Dsup, const float* Tang, int nr, int na, float* out, int nf, int Nl,
                             const int* im3, const int* im2, const float* alpha3b, int Aa, const float* emb3b,
                             const int* type_map, const int* numtriplet, int nt, int ld, void* stream) {
-  return staf::angular_afs<float>(Dsup, Tang, nr, na, out, nf, Nl, im3, im2, alpha3b, Aa, emb3b, type_map, numtriplet,
-                                  nt, ld, stream);
+  return staf::angular_afs<float>(Dsup, Tang, (const float*)nullptr, nr, na, out, nf, Nl, im3, im2, alpha3b, Aa, emb3b,
+                                  type_map, numtriplet, nt, ld, stream);
 }
 int staf_op_angular_afs_f64(const double* Dsup, const double* Tang, int nr, int na, double* out, int nf, int Nl,
                             const int* im3, const int* im2, const double* alpha3b, int Aa, const double* emb3b,
                             const int* type_map, const int* numtriplet, int nt, int ld, void* stream) {
-  return staf::angular_afs<double>(Dsup, Tang, nr, na, out, nf, Nl, im3, im2, alpha3b, Aa, emb3b, type_map,
-                                   numtriplet, nt, ld, stream);
+  return staf::angular_afs<double>(Dsup, Tang, (const double*)nullptr, nr, na, out, nf, Nl, im3, im2, alpha3b, Aa,
+                                   emb3b, type_map, numtriplet, nt, ld, stream);
 }
 int staf_op_alpha_dist_grad_f32(const float* D, int nr, const float* alpha2b, int Ar, float* g_alpha, int nf, int Nl,
                                 const int* im2, const float* P, const float* emb2b, const int* type_map,

@@ -4,8 +4,12 @@
 // the owned atoms, ghosts appended, neighbour-index remapping, un-packing of forces) and the step order of
 // calculateforces (libstaf/vendor/jmd/nn_nn_mlp.cu:838-889): neighbour list (own, or the caller's with no
 // periodic wrap) -> descriptors -> fingerprints of every species -> MLP -> 2-body + 3-body forces with virial.
-// Everything on the GPU runs in float64 through the same kernels as the training ops; the MLP is the per-species
-// Dense stack of staf_mlp.cpp evaluated on the host between the fingerprint and the force kernels.
+// Everything on the GPU runs in float64.  The path is fused in the sense that matters for memory: no tensor of the
+// angular buffer's width exists.  The descriptor kernel runs radial-only and leaves, per centre, its sorted
+// neighbour list with unit vectors, 1/r, cutoff values and their gradients (nr-wide rows); the 3-body fingerprint
+// and force kernels rebuild every triplet's angular descriptor and Jacobian from those rows in LDS.  HBM traffic of a
+// call is positions and types in, forces out, and those nr-wide rows.  The MLP is the per-species Dense stack,
+// evaluated on the GPU between the fingerprint and the force kernels (or on the host, staf_mlp.cpp, on request).
 #include "staf_common.hpp"
 #include "staf_reduce.hpp"
 #include "staf_mlp_dev.hpp"
@@ -160,8 +164,8 @@ struct StafModel {
   // device-resident MLP (default); false: the host evaluation of staf_mlp.cpp between the kernels
   bool dev_mlp = false;
   std::vector<staf::DevMlpNet> dnets;
-  DevBuf<double> raddescr, angdescr, des3bsupp, der2b, der3b, der3bsupp;
-  DevBuf<int> intmap2b, intmap3b, numtriplet, type_map, tipos, actual_type;
+  DevBuf<double> raddescr, des3bsupp, der2b, der3bsupp, unit;   // nr-wide rows per owned atom; unit = (u, 1/r)
+  DevBuf<int> intmap2b, numtriplet, type_map, tipos, actual_type;
   // host staging
   std::vector<double> af_h, gr_h, tmp2, tmp3;
   std::vector<float> af_f, gr_f;
@@ -264,9 +268,9 @@ void staf_free(StafModel* m) {
   m->in_h.release();
   m->out_h.release();
   for (DevBuf<double>* b : {&m->in_d, &m->out_d, &m->force_op, &m->virial_op, &m->af2, &m->af3, &m->g2, &m->g3,
-                            &m->raddescr, &m->angdescr, &m->des3bsupp, &m->der2b, &m->der3b, &m->der3bsupp})
+                            &m->raddescr, &m->des3bsupp, &m->der2b, &m->der3bsupp, &m->unit})
     b->release();
-  for (DevBuf<int>* b : {&m->intmap2b, &m->intmap3b, &m->numtriplet, &m->type_map, &m->tipos, &m->actual_type})
+  for (DevBuf<int>* b : {&m->intmap2b, &m->numtriplet, &m->type_map, &m->tipos, &m->actual_type})
     b->release();
   delete m;
 }
@@ -426,9 +430,9 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
   bool ok = m->in_d.reserve(n_in) && m->out_d.reserve(n_out) &&
             m->force_op.reserve((size_t)nall * 3 * 2 * nt) && m->virial_op.reserve((size_t)9 * 2 * nt) && m->af2.reserve(L * amax2) &&
             m->af3.reserve(L * amax3) && m->g2.reserve(L * amax2) && m->g3.reserve(L * amax3) &&
-            m->raddescr.reserve(L * nr) && m->angdescr.reserve(L * na) && m->des3bsupp.reserve(L * nr) &&
-            m->der2b.reserve(L * 3 * nr) && m->der3b.reserve(L * 6 * na) && m->der3bsupp.reserve(L * 3 * nr) &&
-            m->intmap2b.reserve(L * (nr + 1)) && m->intmap3b.reserve(L * 2 * na) && m->numtriplet.reserve(L) &&
+            m->raddescr.reserve(L * nr) && m->des3bsupp.reserve(L * nr) && m->der2b.reserve(L * 3 * nr) &&
+            m->der3bsupp.reserve(L * 3 * nr) && m->unit.reserve(L * 4 * nr) && m->intmap2b.reserve(L * (nr + 1)) &&
+            m->numtriplet.reserve(L) &&
             m->type_map.reserve(nall) && m->tipos.reserve(nt) && m->actual_type.reserve(nt);
   if (!ok) return -1;
   if (m->type_map.p != type_map_before) m->type_map_up.clear();   // a new block holds nothing yet
@@ -463,9 +467,9 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
   // ---- descriptors (own minimum-image list, or the caller's list with explicit images)
   auto descriptors = [&]() -> int {
     return staf::desc_launch<double>(m->cfg, d_pos, d_box, 1, nlocal, nall, ext ? d_how : nullptr,
-                                     ext ? d_with : nullptr, ext ? 1 : 0, m->raddescr.p, m->angdescr.p,
-                                     m->des3bsupp.p, m->intmap2b.p, m->intmap3b.p, m->der2b.p, m->der3b.p,
-                                     m->der3bsupp.p, m->numtriplet.p, st) == STAF_OK ? 0 : -20;
+                                     ext ? d_with : nullptr, ext ? 1 : 0, m->raddescr.p, nullptr, m->des3bsupp.p,
+                                     m->intmap2b.p, nullptr, m->der2b.p, nullptr, m->der3bsupp.p, m->numtriplet.p,
+                                     m->unit.p, st) == STAF_OK ? 0 : -20;
   };
   int rc = 0;
   double energy = 0.0;
@@ -515,9 +519,9 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
                                         m->intmap2b.p + o * (nr + 1), m->emb2b[k].p, m->type_map.p, nt, nlocal, sk);
             break;
           case 1:
-            rc = staf_op_angular_afs_f64(m->des3bsupp.p + o * nr, m->angdescr.p + o * na, nr, na, af3, 1, Nl,
-                                         m->intmap3b.p + o * 2 * na, m->intmap2b.p + o * (nr + 1), m->alpha3b[k].p,
-                                         Aa, m->emb3b[k].p, m->type_map.p, m->numtriplet.p + o, nt, nlocal, sk);
+            rc = staf::angular_afs<double>(m->des3bsupp.p + o * nr, nullptr, m->unit.p + o * 4 * nr, nr, na, af3, 1,
+                                           Nl, nullptr, m->intmap2b.p + o * (nr + 1), m->alpha3b[k].p, Aa,
+                                           m->emb3b[k].p, m->type_map.p, m->numtriplet.p + o, nt, nlocal, sk);
             break;
           case 2:
             rc = staf::dev_mlp_eval(m->dnets[k], af2, Ar, af3, Aa, Nl, d_e + o, g2, g3, sk);
@@ -529,10 +533,9 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
                                               Nl, wo, px, bx, nlocal, skip_pbc, sk);
             break;
           default:
-            rc = staf::force_tripl<double>(g3, m->des3bsupp.p + o * nr, m->angdescr.p + o * na,
-                                           m->der3bsupp.p + o * 3 * nr, m->der3b.p + o * 6 * na,
-                                           m->intmap2b.p + o * (nr + 1), m->intmap3b.p + o * 2 * na, nr, na, nall, 1,
-                                           Aa, m->emb3b[k].p, nt, m->tipos.p, m->actual_type.p + k, fo,
+            rc = staf::force_tripl<double>(g3, m->des3bsupp.p + o * nr, nullptr, m->der3bsupp.p + o * 3 * nr, nullptr,
+                                           m->unit.p + o * 4 * nr, m->intmap2b.p + o * (nr + 1), nullptr, nr, na, nall,
+                                           1, Aa, m->emb3b[k].p, nt, m->tipos.p, m->actual_type.p + k, fo,
                                            m->numtriplet.p + o, m->alpha3b[k].p, m->type_map.p, Nl, wo, px, bx, nlocal,
                                            skip_pbc, sk);
             STAF_HIP_OK(hipEventRecord(m->ev_join[k], sk));
@@ -604,9 +607,9 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
       rc = staf_op_radial_afs_f64(m->raddescr.p + o * nr, nr, m->alpha2b[k].p, Ar, m->af2.p, 1, Nl,
                                   m->intmap2b.p + o * (nr + 1), m->emb2b[k].p, m->type_map.p, nt, nlocal, st);
       if (rc == STAF_OK)
-        rc = staf_op_angular_afs_f64(m->des3bsupp.p + o * nr, m->angdescr.p + o * na, nr, na, m->af3.p, 1, Nl,
-                                     m->intmap3b.p + o * 2 * na, m->intmap2b.p + o * (nr + 1), m->alpha3b[k].p, Aa,
-                                     m->emb3b[k].p, m->type_map.p, m->numtriplet.p + o, nt, nlocal, st);
+        rc = staf::angular_afs<double>(m->des3bsupp.p + o * nr, nullptr, m->unit.p + o * 4 * nr, nr, na, m->af3.p, 1, Nl,
+                                       nullptr, m->intmap2b.p + o * (nr + 1), m->alpha3b[k].p, Aa, m->emb3b[k].p,
+                                       m->type_map.p, m->numtriplet.p + o, nt, nlocal, st);
       if (rc != STAF_OK) return -20;
       m->tmp2.resize((size_t)Nl * Ar);
       m->tmp3.resize((size_t)Nl * Aa);
@@ -677,10 +680,9 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
                                             m->emb2b[k].p, nt, m->tipos.p, m->actual_type.p + k, m->force_op.p,
                                             m->type_map.p, Nl, m->virial_op.p, d_pos, d_box, nlocal, skip_pbc, st);
         else
-          rc = staf::force_tripl<double>(m->g3.p, m->des3bsupp.p + o * nr, m->angdescr.p + o * na,
-                                         m->der3bsupp.p + o * 3 * nr, m->der3b.p + o * 6 * na,
-                                         m->intmap2b.p + o * (nr + 1), m->intmap3b.p + o * 2 * na, nr, na, nall, 1, Aa,
-                                         m->emb3b[k].p, nt, m->tipos.p, m->actual_type.p + k, m->force_op.p,
+          rc = staf::force_tripl<double>(m->g3.p, m->des3bsupp.p + o * nr, nullptr, m->der3bsupp.p + o * 3 * nr, nullptr,
+                                         m->unit.p + o * 4 * nr, m->intmap2b.p + o * (nr + 1), nullptr, nr, na, nall, 1,
+                                         Aa, m->emb3b[k].p, nt, m->tipos.p, m->actual_type.p + k, m->force_op.p,
                                          m->numtriplet.p + o, m->alpha3b[k].p, m->type_map.p, Nl, m->virial_op.p,
                                          d_pos, d_box, nlocal, skip_pbc, st);
         if (rc != STAF_OK) return -20;

@@ -293,13 +293,15 @@ struct DescConfig {
 
 // Internal launchers shared with the MD entry (staf_api): descriptor op with an explicit configuration, an
 // optional caller-supplied neighbour list (owned centres only, Npos >= N positions) and optional no-wrap mode.
+// unit != null: radial-only call -- no triplet tensor is written (angdescr, intmap3b, der3b may be null) and unit
+// [nf, N, 4, nr] receives the unit vectors centre - neighbour and 1/r of the sorted neighbours.
 template <typename real>
 int desc_configure(DescConfig<real>& c, real Rc, int nr, int na, real Rs, real Ra);
 template <typename real>
 int desc_launch(const DescConfig<real>& c, const real* pos, const real* box, int nf, int N, int Npos,
                 const int* inj_howmany, const int* inj_with, int skip_pbc, real* raddescr, real* angdescr,
                 real* des3bsupp, int* intmap2b, int* intmap3b, real* der2b, real* der3b, real* der3bsupp,
-                int* numtriplet, hipStream_t stream);
+                int* numtriplet, real* unit, hipStream_t stream);
 
 
 // Force ops with the wrap switch of the virial forms given per call (skip_pbc = 1: neighbour positions already are
@@ -310,9 +312,16 @@ int force_doublets(const real* G, const real* D, const real* dD, const int* im2,
                    const real* alpha2b, const real* emb2b, int nt, const int* tipos, const int* actual_type,
                    real* force, const int* type_map, int Nl, real* virial, const real* pos, const real* box, int ld,
                    int skip_pbc, void* stream);
+// unit != null: the fused forms of the MD entry (T and its Jacobian rebuilt from the radial-only descriptor call's
+// unit vectors; Tang, d3b, im3 are not read and may be null).
+template <typename real>
+int angular_afs(const real* Dsup, const real* Tang, const real* unit, int nr, int na, real* out, int nf, int Nl,
+                const int* im3, const int* im2, const real* alpha3b, int Aa, const real* emb3b, const int* type_map,
+                const int* numtriplet, int nt, int ld, void* stream);
 template <typename real>
 int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* dDsup, const real* d3b,
-                const int* im2, const int* im3, int nr, int na, int N, int nf, int Aa, const real* emb3b, int nt,
+                const real* unit, const int* im2, const int* im3, int nr, int na, int N, int nf, int Aa,
+                const real* emb3b, int nt,
                 const int* tipos, const int* actual_type, real* force, const int* numtriplet, const real* alpha3b,
                 const int* type_map, int Nl, real* virial, const real* pos, const real* box, int ld, int skip_pbc,
                 void* stream);

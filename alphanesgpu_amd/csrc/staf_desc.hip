@@ -55,6 +55,11 @@ struct DescArgs {
   real* der3b;
   real* der3bsupp;
   int* numtriplet;
+  // Radial-only mode of the MD entry: angular = 0 skips the triplet fill (angdescr, intmap3b, der3b are not touched
+  // and may be null) and unit receives, per sorted neighbour, the unit vector centre - neighbour and 1/r,
+  // [nf, N, 4, nr] -- with des3bsupp and der3bsupp all a 3-body kernel needs to rebuild T and its Jacobian itself.
+  real* unit;
+  int angular;
   int* status;
   TransposeRef tr;         // transposed neighbour map kept beside intmap2b (receiving atoms: the Npos positions)
 };
@@ -433,6 +438,7 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
       s_j[rank] = j;
       s_rec[3 * nr + rank] = invr;
       s_rec[7 * nr + rank] = fc;
+      if (A.unit) A.unit[(atom * 4 + 3) * nr + rank] = invr;
 #pragma unroll
       for (int c = 0; c < 3; c++) {
         const real u = d[c] * invr;
@@ -440,8 +446,13 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
         A.der3bsupp[row3 + c * nr + rank] = dfc * u;
         s_rec[c * nr + rank] = u;
         s_rec[(4 + c) * nr + rank] = dfc * u;
+        if (A.unit) A.unit[(atom * 4 + c) * nr + rank] = u;
       }
     } else {
+      if (A.unit) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) A.unit[(atom * 4 + c) * nr + e] = 0;
+      }
       A.raddescr[row + e] = 0;
       A.des3bsupp[row + e] = 0;
       im[1 + e] = 0;
@@ -461,6 +472,7 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
     A.numtriplet[atom] = m;
   }
 
+  if (!A.angular) return;
   // 4. angular fill: triplet nn <-> (j<k) over the first m sorted neighbours
   int ntr = (m * (m - 1)) / 2;
   if (ntr > na) ntr = na;
@@ -613,10 +625,11 @@ template <typename real>
 int desc_launch(const DescConfig<real>& c, const real* pos, const real* box, int nf, int N, int Npos,
                 const int* inj_howmany, const int* inj_with, int skip_pbc, real* raddescr, real* angdescr,
                 real* des3bsupp, int* intmap2b, int* intmap3b, real* der2b, real* der3b, real* der3bsupp,
-                int* numtriplet, hipStream_t stream) {
+                int* numtriplet, real* unit, hipStream_t stream) {
   if (!c.ready) return STAF_E_NOT_CONSTRUCTED;
-  if (!pos || !box || !raddescr || !angdescr || !des3bsupp || !intmap2b || !intmap3b || !der2b || !der3b ||
-      !der3bsupp || !numtriplet || nf <= 0 || N <= 0 || Npos < N || (inj_howmany && !inj_with))
+  const bool angular = unit == nullptr;   // with `unit` the call is radial-only
+  if (!pos || !box || !raddescr || !des3bsupp || !intmap2b || !der2b || !der3bsupp || !numtriplet || nf <= 0 ||
+      N <= 0 || Npos < N || (inj_howmany && !inj_with) || (angular && (!angdescr || !intmap3b || !der3b)))
     return STAF_E_BAD_ARG;
   DeviceState* st = device_state(stream);
   if (!st) return reserve_failure(stream);
@@ -627,6 +640,7 @@ int desc_launch(const DescConfig<real>& c, const real* pos, const real* box, int
   A.dist2_fma = c.dist2_fma; A.zero_padding = c.zero_padding;
   A.raddescr = raddescr; A.angdescr = angdescr; A.des3bsupp = des3bsupp; A.intmap2b = intmap2b;
   A.intmap3b = intmap3b; A.der2b = der2b; A.der3b = der3b; A.der3bsupp = der3bsupp; A.numtriplet = numtriplet;
+  A.unit = unit; A.angular = angular ? 1 : 0;
   A.status = st->status_d;
   if (N >= (1 << (31 - KEY_SLOT_BITS))) return STAF_E_LIMIT;
   // own lists are symmetric (an atom is listed by exactly its own neighbours, at most nr); a caller's list may name
@@ -664,10 +678,10 @@ int desc_launch(const DescConfig<real>& c, const real* pos, const real* box, int
 }
 template int desc_launch<float>(const DescConfig<float>&, const float*, const float*, int, int, int, const int*,
                                 const int*, int, float*, float*, float*, int*, int*, float*, float*, float*, int*,
-                                hipStream_t);
+                                float*, hipStream_t);
 template int desc_launch<double>(const DescConfig<double>&, const double*, const double*, int, int, int, const int*,
                                  const int*, int, double*, double*, double*, int*, int*, double*, double*, double*,
-                                 int*, hipStream_t);
+                                 int*, double*, hipStream_t);
 
 template <typename real>
 int desc_configure(DescConfig<real>& c, real Rc, int nr, int na, real Rs, real Ra) {
@@ -691,7 +705,7 @@ static int compute(const real* pos, const real* box, int nf, int N, real* raddes
     c = cfg<real>().current();
   }
   return desc_launch<real>(c, pos, box, nf, N, N, nullptr, nullptr, 0, raddescr, angdescr, des3bsupp, intmap2b,
-                           intmap3b, der2b, der3b, der3bsupp, numtriplet, (hipStream_t)stream_);
+                           intmap3b, der2b, der3b, der3bsupp, numtriplet, (real*)nullptr, (hipStream_t)stream_);
 }
 
 }  // namespace staf

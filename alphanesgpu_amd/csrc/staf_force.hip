@@ -65,6 +65,8 @@ struct Force2Args {
   const real* box;
   TransposeRef tr;
   int* status;
+  int host_shift;        // first atom of the centre species when the host knows it (a view of a descriptor output:
+                         // its offset in that tensor), else -1: taken from tipos / actual_type on the device
   int skip_pbc, nf, N, Nl, ld, nr, Ar, nt;
 };
 
@@ -81,7 +83,11 @@ __global__ __launch_bounds__(F_BLOCK) void force2_kernel(Force2Args<real> A) {
   const int recv = blockIdx.x * F_WAVES + wave;
   if (recv >= A.nf * A.N) return;
   const int b = recv / A.N, a = recv - b * A.N;
-  const int shift = species_shift(A.tipos, A.actual_type);
+  // The species' first atom: known on the host for a view of a descriptor output, which spares every wave two
+  // dependent reads ahead of all its other reads; the device's own figure is then only compared with it.
+  const int shift = A.host_shift >= 0 ? A.host_shift : species_shift(A.tipos, A.actual_type);
+  if (A.host_shift >= 0 && recv == 0 && lane == 0 && species_shift(A.tipos, A.actual_type) != A.host_shift)
+    atomicOr(A.status, 4);
   const int pl = a - shift;
   real f[3] = {0, 0, 0};
   real v[9];
@@ -104,8 +110,9 @@ __global__ __launch_bounds__(F_BLOCK) void force2_kernel(Force2Args<real> A) {
     const int* im = A.im2 + row * (nr + 1);
     int cnt = im[0];
     if (cnt > nr) cnt = nr;
-    for (int s = lane; s < cnt; s += WAVE) {
-      const int nj = im[1 + s];
+    for (int s = lane; s < nr; s += WAVE) {
+      const int nj = im[1 + s];   // read up to nr, not up to the count just requested: padded slots hold atom 0
+      if (s >= cnt) break;
       const real w = pair_weight(row, (size_t)b * Nl + pl, s, A.type_map[nj]);
       real g[3];
 #pragma unroll
@@ -230,13 +237,16 @@ __global__ __launch_bounds__(F_BLOCK) void gather_kernel(const real* __restrict_
                                                          const int* __restrict__ im2, TransposeRef tr,
                                                          const int* __restrict__ tipos,
                                                          const int* __restrict__ actual_type,
-                                                         real* __restrict__ force, int* status, int nf, int N,
-                                                         int Nl, int ld, int nr) {
+                                                         real* __restrict__ force, int* status, int host_shift,
+                                                         int nf, int N, int Nl, int ld, int nr) {
   const int wave = threadIdx.x / WAVE, lane = lane_id();
   const int recv = blockIdx.x * F_WAVES + wave;
   if (recv >= nf * N) return;
   const int b = recv / N, a = recv - b * N;
-  const int shift = species_shift(tipos, actual_type);
+  // the species' first atom: see force2_kernel
+  const int shift = host_shift >= 0 ? host_shift : species_shift(tipos, actual_type);
+  if (host_shift >= 0 && recv == 0 && lane == 0 && species_shift(tipos, actual_type) != host_shift)
+    atomicOr(status, 4);
   const int L = tr.cnt[recv];
   const int* keys = tr.keys + (size_t)recv * tr.cap;
   real f[3] = {0, 0, 0};
@@ -386,8 +396,9 @@ static inline int grad_blocks_f(int atoms) {
 // The transposed neighbour map for a force op: the one the descriptor op left beside the tensor `im2` points into,
 // or, for any other copy of the map, one built here in the stream's work area (push + sort launches).
 static int force_transpose(DeviceState* st, const int* im2, int nf, int N, int Nl, int ld, int nr, hipStream_t stream,
-                           TransposeRef* tr) {
-  if (transpose_find(st, im2, nf, N, Nl, ld, nr, tr)) return STAF_OK;
+                           TransposeRef* tr, bool* cached) {
+  *cached = transpose_find(st, im2, nf, N, Nl, ld, nr, tr);
+  if (*cached) return STAF_OK;
   const int cap = 4 * nr;
   if ((size_t)TR_WAVES * cap * sizeof(int) > 64 * 1024) return STAF_E_LIMIT;
   if (!bucket_reserve(st, (size_t)nf * N, cap, stream, tr)) return reserve_failure(stream);
@@ -430,11 +441,13 @@ int force_doublets(const real* G, const real* D, const real* dD, const int* im2,
   if (!st) return reserve_failure((hipStream_t)stream_);
   hipStream_t stream = (hipStream_t)stream_;
   Force2Args<real> A;
-  int rc = force_transpose(st, im2, nf, N, Nl, ld, nr, stream, &A.tr);
+  bool cached = false;
+  int rc = force_transpose(st, im2, nf, N, Nl, ld, nr, stream, &A.tr, &cached);
   if (rc) return rc;
   A.G = G; A.D = D; A.dD = dD; A.im2 = im2; A.alpha2b = alpha2b; A.emb2b = emb2b; A.type_map = type_map;
   A.tipos = tipos; A.actual_type = actual_type; A.force = force; A.vpart = nullptr; A.pos = pos; A.box = box;
   A.status = st->status_d; A.skip_pbc = skip_pbc;
+  A.host_shift = cached ? A.tr.key_shift : -1;
   A.nf = nf; A.N = N; A.Nl = Nl; A.ld = ld; A.nr = nr; A.Ar = Ar; A.nt = nt;
   if (virial) {
     A.vpart = (real*)scratch_reserve(st, stream, (size_t)nf * Nl * 9 * sizeof(real));
@@ -460,15 +473,17 @@ int force_doublets(const real* G, const real* D, const real* dD, const int* im2,
 
 template <typename real>
 int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* dDsup, const real* d3b,
-                const int* im2, const int* im3, int nr, int na, int N, int nf, int Aa, const real* emb3b, int nt,
+                const real* unit, const int* im2, const int* im3, int nr, int na, int N, int nf, int Aa,
+                const real* emb3b, int nt,
                 const int* tipos, const int* actual_type, real* force, const int* numtriplet, const real* alpha3b,
                 const int* type_map, int Nl, real* virial, const real* pos, const real* box, int ld, int skip_pbc,
                 void* stream_) {
   (void)im3;
   if ((virial || pos || box) && !(virial && pos && box)) return STAF_E_BAD_ARG;
   if (Nl == 0 && nf > 0 && N > 0 && force) return empty_species_force<real>(force, virial, nf, N, stream_);
-  if (!G || !Dsup || !Tang || !dDsup || !d3b || !im2 || !emb3b || !tipos || !actual_type || !force || !numtriplet ||
-      !alpha3b || !type_map || nr <= 0 || na <= 0 || N <= 0 || nf <= 0 || Aa <= 0 || nt <= 0 || Nl <= 0 || Nl > N)
+  if (!G || !Dsup || (!unit && (!Tang || !d3b)) || !dDsup || !im2 || !emb3b || !tipos || !actual_type || !force ||
+      !numtriplet || !alpha3b || !type_map || nr <= 0 || na <= 0 || N <= 0 || nf <= 0 || Aa <= 0 || nt <= 0 ||
+      Nl <= 0 || Nl > N)
     return STAF_E_BAD_ARG;
   if (nt > NT_MAX) return STAF_E_LIMIT;
   if (ld <= 0) ld = Nl;
@@ -477,25 +492,32 @@ int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* d
   hipStream_t stream = (hipStream_t)stream_;
   if (!Force3Cfg<real>::fits(nr, nt) || N >= (1 << (31 - KEY_SLOT_BITS))) return STAF_E_LIMIT;
   TransposeRef tr;
-  int rc = force_transpose(st, im2, nf, N, Nl, ld, nr, stream, &tr);
+  bool cached = false;
+  int rc = force_transpose(st, im2, nf, N, Nl, ld, nr, stream, &tr, &cached);
   if (rc) return rc;
   const size_t ng = (size_t)nf * Nl * nr * 3, ns = (size_t)nf * Nl * 3, nv = virial ? (size_t)nf * Nl * 9 : 0;
   real* gslot = (real*)scratch_reserve(st, stream, (ng + ns + nv) * sizeof(real));
   if (!gslot) return reserve_failure(stream);
   real* self = gslot + ng;
   real* vpart = self + ns;
-  const size_t lds = Force3Cfg<real>::bytes(nr, Aa, nt);
+  const bool fused = unit != nullptr;   // the MD entry: T and its Jacobian rebuilt from the unit vectors
+  const size_t lds = Force3Cfg<real>::bytes(nr, Aa, nt, fused);
+  const void* kern = fused ? (const void*)force3_kernel<real, true> : (const void*)force3_kernel<real, false>;
   if (lds > 64 * 1024) {
     if (lds > 160 * 1024 ||
-        hipFuncSetAttribute((const void*)force3_kernel<real>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
-            hipSuccess)
+        hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return STAF_E_LIMIT;
   }
   {
     KernelTimer kt_("force3_kernel", stream);
-    hipLaunchKernelGGL(force3_kernel<real>, dim3(nf * Nl), dim3(Force3Cfg<real>::THREADS), lds, stream, G, Dsup, Tang,
-                       dDsup, d3b, im2, alpha3b, emb3b, type_map, numtriplet, gslot, self, nf, N, Nl, ld, nr, na, Aa,
-                       nt);
+    if (fused)
+      hipLaunchKernelGGL((force3_kernel<real, true>), dim3(nf * Nl), dim3(Force3Cfg<real>::THREADS), lds, stream, G,
+                         Dsup, Tang, dDsup, d3b, unit, im2, alpha3b, emb3b, type_map, numtriplet, gslot, self, nf, N,
+                         Nl, ld, nr, na, Aa, nt);
+    else
+      hipLaunchKernelGGL((force3_kernel<real, false>), dim3(nf * Nl), dim3(Force3Cfg<real>::THREADS), lds, stream, G,
+                         Dsup, Tang, dDsup, d3b, unit, im2, alpha3b, emb3b, type_map, numtriplet, gslot, self, nf, N,
+                         Nl, ld, nr, na, Aa, nt);
   }
   if (virial) {
     const int atoms = nf * Nl;
@@ -508,8 +530,8 @@ int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* d
     KernelTimer kt_("gather_kernel", stream);
     const int recv = nf * N;
     hipLaunchKernelGGL(gather_kernel<real>, dim3((recv + F_WAVES - 1) / F_WAVES), dim3(F_BLOCK), 0, stream,
-                       (const real*)gslot, (const real*)self, im2, tr, tipos, actual_type, force, st->status_d, nf, N,
-                       Nl, ld, nr);
+                       (const real*)gslot, (const real*)self, im2, tr, tipos, actual_type, force, st->status_d,
+                       cached ? tr.key_shift : -1, nf, N, Nl, ld, nr);
   }
   return finish_op(st, stream);
 }
@@ -518,7 +540,8 @@ template int force_doublets<double>(const double*, const double*, const double*,
                                     const double*, const double*, int, const int*, const int*, double*, const int*,
                                     int, double*, const double*, const double*, int, int, void*);
 template int force_tripl<double>(const double*, const double*, const double*, const double*, const double*,
-                                 const int*, const int*, int, int, int, int, int, const double*, int, const int*,
+                                 const double*, const int*, const int*, int, int, int, int, int, const double*, int,
+                                 const int*,
                                  const int*, double*, const int*, const double*, const int*, int, double*,
                                  const double*, const double*, int, int, void*);
 
@@ -625,7 +648,8 @@ void staf_op_force_set_skip_pbc(int skip) { staf::g_force_skip_pbc = skip ? 1 : 
                                 const int* actual_type, real* forces3b, const int* num_triplets, const real* smooth_a, \
                                 const int* type_map, int N_local, real* virial, const real* pos, const real* box,      \
                                 int ld_atoms, void* stream) {                                                          \
-    return staf::force_tripl<real>(netderiv, desr, desa, intderiv_r, intderiv_a, intmap_r, intmap_a, nr, na, N,        \
+    return staf::force_tripl<real>(netderiv, desr, desa, intderiv_r, intderiv_a, (const real*)nullptr, intmap_r,      \
+                                   intmap_a, nr, na, N,                                                                \
                                    dimbat, num_finger, type_emb3b, nt, tipos, actual_type, forces3b, num_triplets,     \
                                    smooth_a, type_map, N_local, virial, pos, box, ld_atoms, staf::g_force_skip_pbc,    \
                                    stream);                                                                            \

@@ -67,21 +67,27 @@ struct Force3Cfg {
   static constexpr bool PREFETCH = false;
   __host__ __device__ static bool fits(int nr, int nt) { return nr <= 255 && nt <= NT_MAX; }   // slots packed in 8 bits
   __host__ __device__ static int pitch(int Aa) { return (Aa + 3) & ~3; }   // parameter row pitch (channels)
-  __host__ __device__ static size_t n_reals(int nr, int Aa, int nt) {
+  __host__ __device__ static size_t n_reals(int nr, int Aa, int nt, bool fused = false) {
     const int nsig = 2 * nt - 1;
     return (size_t)nsig * pitch(Aa) * 6 /*prm, prE*/ + (((size_t)CAPP * nt * nr + 1) & ~(size_t)1) * 2 /*E*/ +
            (size_t)NW * 8 * nr /*accJ, accK per wave*/ + nr /*D*/ + 3 * nr /*grad fc*/ +
-           (size_t)NW * 4 * WAVE /*scan exchange per wave*/;
+           (size_t)NW * 4 * WAVE /*scan exchange per wave*/ + (fused ? 4 * nr : 0) /*unit vectors, 1/r*/;
   }
-  __host__ __device__ static size_t bytes(int nr, int Aa, int nt) {
-    return n_reals(nr, Aa, nt) * sizeof(real) + (size_t)(16 + nr) * sizeof(int);
+  __host__ __device__ static size_t bytes(int nr, int Aa, int nt, bool fused = false) {
+    return n_reals(nr, Aa, nt, fused) * sizeof(real) + (size_t)(16 + nr) * sizeof(int);
   }
 };
 
-template <typename real>
+// FUSED (the MD entry): Tang and d3b are not read; a triplet's angular descriptor and its Jacobian are rebuilt from
+// the slots' unit vectors u, 1/r, cutoff values fc and their gradients (DescriptorsAngular_kernel,
+// STAF/src/descriptor_builder/reforce.cu.cc:195-228), with c = u_j . u_k, h = (c + 1)/2:
+//   T = h fc_j fc_k,   dT/dd_j = 1/2 fc_j fc_k / r_j (u_k - c u_j) + h fc_k grad fc_j,   j <-> k for dT/dd_k
+// `unit` is [nf, ld, 4, nr] = (u_x, u_y, u_z, 1/r) per sorted neighbour, written by the radial-only descriptor call.
+template <typename real, bool FUSED = false>
 __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
     const real* __restrict__ G, const real* __restrict__ Dsup, const real* __restrict__ Tang,
-    const real* __restrict__ dDsup, const real* __restrict__ d3b, const int* __restrict__ im2,
+    const real* __restrict__ dDsup, const real* __restrict__ d3b, const real* __restrict__ unit,
+    const int* __restrict__ im2,
     const real* __restrict__ alpha3b, const real* __restrict__ emb3b, const int* __restrict__ type_map,
     const int* __restrict__ numtriplet, real* __restrict__ gslot, real* __restrict__ self, int nf, int N, int Nl,
     int ld, int nr, int na, int Aa, int nt) {
@@ -101,7 +107,8 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
   real* sD = acc + (size_t)NW * 8 * nr;                    // [nr]
   real* sg = sD + nr;                                      // [3*nr] grad fc (der3bsupp)
   real* xch = sg + 3 * nr;                                 // [NW][4][64] prefix sums of a pass
-  int* nact = (int*)(xch + NW * 4 * WAVE);                 // [16] active channels per sigma (0 beyond nsig)
+  real* sU = xch + NW * 4 * WAVE;                          // FUSED: [4][nr] unit vector, 1/r
+  int* nact = (int*)(sU + (FUSED ? 4 * nr : 0));           // [16] active channels per sigma (0 beyond nsig)
   int* stp = nact + 16;                                    // [nr] species of every slot
   PHASE_CLOCK_BEGIN();
 
@@ -126,22 +133,28 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
   // needs only that index and overlaps the parameter rows.
   // Holding the der3b rows of the first sweep in registers from here on was measured and is slower.
   unsigned nj = 0;   // unsigned: no sign extension (and so no wait for the read) ahead of the reads that follow
-  real d_s = 0, g_s[3] = {0, 0, 0};
+  real d_s = 0, g_s[3] = {0, 0, 0}, u_s[4] = {0, 0, 0, 0};
   if (tid < nr) {
     nj = (unsigned)im[1 + tid];
     d_s = Dsup[rowAtom * nr + tid];
 #pragma unroll
     for (int c = 0; c < 3; c++) g_s[c] = dDsup[rowAtom * 3 * nr + c * nr + tid];
+    if constexpr (FUSED) {
+#pragma unroll
+      for (int c = 0; c < 4; c++) u_s[c] = unit[(rowAtom * 4 + c) * nr + tid];
+    }
   }
   // Reads of per-triplet rows are never predicated: a lane past the last triplet re-reads the last one (row element
   // 0 if there is none) and its value is masked where it is used.  With every read issued on every path the waits
   // can name how many later reads may stay in flight, which is what lets the prefetches below overlap.
   const int nlast = ntri > 0 ? ntri - 1 : 0;
   real Tn[NP];
+  if constexpr (!FUSED) {
 #pragma unroll
-  for (int p = 0; p < NP; p++) {
-    const int nn = (p * NW + wave) * WAVE + lane;
-    Tn[p] = Trow[nn < nlast ? nn : nlast];
+    for (int p = 0; p < NP; p++) {
+      const int nn = (p * NW + wave) * WAVE + lane;
+      Tn[p] = Trow[nn < nlast ? nn : nlast];
+    }
   }
   const bool slot = tid < m;
   int t_s = 0;
@@ -186,6 +199,10 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
     sD[tid] = d_s;
 #pragma unroll
     for (int c = 0; c < 3; c++) sg[c * nr + tid] = g_s[c];
+    if constexpr (FUSED) {
+#pragma unroll
+      for (int c = 0; c < 4; c++) sU[c * nr + tid] = u_s[c];
+    }
   }
   if (slot) stp[tid] = t_s;
   __syncthreads();
@@ -199,7 +216,7 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
   // set-up): all workgroups of a launch run in step, so reads issued only where they are needed arrive as one
   // burst with the vector units idle.
   real2 dn[NP][3];
-  if constexpr (L::PREFETCH) {
+  if constexpr (L::PREFETCH && !FUSED) {
 #pragma unroll
     for (int p = 0; p < NP; p++) {
       const int nn = (p * NW + wave) * WAVE + lane;
@@ -222,7 +239,12 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
       if (nn < ntri) {
         int j, k;
         tri_decode(nn, m, j, k);
-        T[p] = Tn[p];
+        if constexpr (FUSED) {
+          const real cs = sU[j] * sU[k] + sU[nr + j] * sU[nr + k] + sU[2 * nr + j] * sU[2 * nr + k];
+          T[p] = (real(0.5) * (cs + real(1))) * (sD[j] * sD[k]);
+        } else {
+          T[p] = Tn[p];
+        }
         const int tj = stp[j], tk = stp[k];
         rj[p] = (tk * nr + j) * CAPP;
         rk[p] = (tj * nr + k) * CAPP;
@@ -269,7 +291,11 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
           pk[p] = E + rk[p];
           po[p] = prm + rp[p] + c0 * 4;
         }
-        for (int ia = 0; ia < nch2; ia += 2) {
+        // fully unrolled with an early exit: every LDS address of the loop is a per-pass base plus an immediate
+        // offset, no pointer is stepped
+#pragma unroll
+        for (int ia = 0; ia < CAP; ia += 2) {
+          if (ia >= nch2) break;
 #pragma unroll
           for (int u = 0; u < 2; u++) {
             // the reads of one channel's items are in flight together; hoisting those of more channels would
@@ -306,7 +332,9 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
 
     // ---- contraction with der3b, slot sums of this wave.  Lanes past the last triplet hold T = 0 and finite sums
     // computed on row 0: their products are forced to 0.
-    if constexpr (!L::PREFETCH) {
+    if constexpr (FUSED) {
+      // nothing to load: a pass's Jacobian is rebuilt from the slot tile where it is used
+    } else if constexpr (!L::PREFETCH) {
 #pragma unroll
       for (int p = 0; p < NP; p++) {
         const int nn = w0 + (p * NW + wave) * WAVE + lane;
@@ -314,27 +342,50 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
         for (int c = 0; c < 3; c++) dn[p][c] = d3[c * na + (nn < nlast ? nn : nlast)];
       }
     }
+    // A pass's contributions to its slots j and k: (force x, y, z, radial factor).  The loaded rows are turned into
+    // products here, all passes at once, so that their registers are free again before the rows of the next sweep
+    // are requested; the fused form rebuilds a pass's Jacobian only where the pass is reduced (its tile reads are
+    // LDS reads, and holding all passes' products at once would cost half the resident waves in double precision).
     real vjs[NP][4], vks[NP][4];
-#pragma unroll
-    for (int p = 0; p < NP; p++) {
+    auto pass_products = [&](int p, real (&vj)[4], real (&vk)[4]) {
       const bool valid = w0 + (p * NW + wave) * WAVE + lane < ntri;
       const real sd = valid ? Sd[p] : real(0);
       const real hT = real(0.5) * T[p];
+      if constexpr (FUSED) {
+        // lanes past the last triplet hold j = k = 0: finite values, masked by sd = 0 and T = 0
+        const int j = jk[p] & 0xff, k = jk[p] >> 8;
+        const real uj[3] = {sU[j], sU[nr + j], sU[2 * nr + j]}, uk[3] = {sU[k], sU[nr + k], sU[2 * nr + k]};
+        const real cs = uj[0] * uk[0] + uj[1] * uk[1] + uj[2] * uk[2];
+        const real fj = sD[j], fk = sD[k];
+        const real half = real(0.5) * (cs + real(1)), ff = fj * fk;
+        const real aj = sd * (real(0.5) * sU[3 * nr + j] * ff), ak = sd * (real(0.5) * sU[3 * nr + k] * ff);
+        const real hk = sd * (half * fk), hj = sd * (half * fj);
 #pragma unroll
-      for (int c = 0; c < 3; c++) {
-        vjs[p][c] = sd * dn[p][c].x;
-        vks[p][c] = sd * dn[p][c].y;
+        for (int c = 0; c < 3; c++) {
+          vj[c] = aj * (uk[c] - cs * uj[c]) + hk * sg[c * nr + j];
+          vk[c] = ak * (uj[c] - cs * uk[c]) + hj * sg[c * nr + k];
+        }
+      } else {
+#pragma unroll
+        for (int c = 0; c < 3; c++) {
+          vj[c] = sd * dn[p][c].x;
+          vk[c] = sd * dn[p][c].y;
+        }
       }
-      vjs[p][3] = (U[p] + V[p]) * hT;
-      vks[p][3] = (U[p] - V[p]) * hT;
+      vj[3] = (U[p] + V[p]) * hT;
+      vk[3] = (U[p] - V[p]) * hT;
+    };
+    if constexpr (!FUSED) {
+#pragma unroll
+      for (int p = 0; p < NP; p++) pass_products(p, vjs[p], vks[p]);
     }
-    if (w0 + NW * NP * WAVE < ntri) {   // rows of the next sweep
+    if (!FUSED && w0 + NW * NP * WAVE < ntri) {   // rows of the next sweep
 #pragma unroll
       for (int p = 0; p < NP; p++) {
         const int nn = w0 + NW * NP * WAVE + (p * NW + wave) * WAVE + lane;
         Tn[p] = Trow[nn < nlast ? nn : nlast];
       }
-      if constexpr (L::PREFETCH) {
+      if constexpr (L::PREFETCH && !FUSED) {
 #pragma unroll
         for (int p = 0; p < NP; p++) {
           const int nn = w0 + NW * NP * WAVE + (p * NW + wave) * WAVE + lane;
@@ -351,8 +402,12 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
       const bool valid = nn < ntri;
       const int j = jk[p] & 0xff, k = jk[p] >> 8;
       real vj[4], vk[4];
+      if constexpr (FUSED) {
+        pass_products(p, vj, vk);
+      } else {
 #pragma unroll
-      for (int c = 0; c < 4; c++) { vj[c] = vjs[p][c]; vk[c] = vks[p][c]; }
+        for (int c = 0; c < 4; c++) { vj[c] = vjs[p][c]; vk[c] = vks[p][c]; }
+      }
       // slot j: the lanes of a row are contiguous.  Row sum = prefix at the row's last lane minus prefix
       // before its first lane of this pass.
       __builtin_amdgcn_wave_barrier();

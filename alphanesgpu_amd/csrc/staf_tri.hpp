@@ -92,7 +92,8 @@ __device__ inline int small_div(int q, int n, float inv_n) {
 template <typename real>
 struct TriArgs {
   const real* Dsup;       // des3bsupp  [nf, ld, nr]
-  const real* Tang;       // angdescr   [nf, ld, na]
+  const real* Tang;       // angdescr   [nf, ld, na] (not read by the FUSED kernel)
+  const real* unit;       // FUSED: unit vectors centre - neighbour and 1/r of the sorted neighbours [nf, ld, 4, nr]
   const int* im2;         // intmap2b   [nf, ld, nr+1]
   const real* alpha3b;    // [ntc, 3*Aa]
   const real* emb3b;      // [ntc, Aa]
@@ -117,9 +118,10 @@ template <typename real, int MODE>
 struct TriLds {
   static constexpr int NV = (MODE == 0) ? 1 : (MODE == 1 ? 3 : 4);
   static constexpr int QB = TriCfg<real, MODE>::QB;
-  __host__ __device__ static size_t n_reals(int nr, int Aa, int nt) {
+  __host__ __device__ static size_t n_reals(int nr, int Aa, int nt, bool fused = false) {
     const int nsig = 2 * nt - 1;
     size_t r = (size_t)nr * TRI_CAPP * 2;                   // pair tables (real2 per (row, channel)), + (D, V) per row
+    if (fused) r += (size_t)3 * nr;                         // unit vectors of the slots
     r += nr;                                                // sD
     r += Aa;                                                // sP
     r += (size_t)TRI_WAVES * Aa;                            // per-wave channel sums
@@ -129,15 +131,19 @@ struct TriLds {
     r += (size_t)QB * (MODE == 2 ? 2 : 1);                  // staged T (and U)
     return r;
   }
-  __host__ __device__ static size_t bytes(int nr, int Aa, int nt) {
-    size_t b = chan_table_bytes<real>(2 * nt - 1, Aa) + n_reals(nr, Aa, nt) * sizeof(real);
+  __host__ __device__ static size_t bytes(int nr, int Aa, int nt, bool fused = false) {
+    size_t b = chan_table_bytes<real>(2 * nt - 1, Aa) + n_reals(nr, Aa, nt, fused) * sizeof(real);
     b += (size_t)2 * QB * sizeof(unsigned short) + (size_t)(2 * nr + NT_MAX + 1) * sizeof(int);
     return (b + 15) & ~(size_t)15;
   }
 };
 
-template <typename real, int MODE>
+// FUSED (MODE 0 only, the MD entry): the angular descriptor of a triplet is not read from angdescr but rebuilt from
+// the slots' unit vectors and cutoff values, T = 1/2 (u_j . u_k + 1) fc_j fc_k
+// (DescriptorsAngular_kernel, STAF/src/descriptor_builder/reforce.cu.cc:195-212), so no na-wide tensor exists.
+template <typename real, int MODE, bool FUSED = false>
 __global__ __launch_bounds__(TRI_BLOCK, (TriCfg<real, MODE>::MIN_WAVES)) void tri_reduce_kernel(TriArgs<real> A) {
+  static_assert(!FUSED || MODE == 0, "only the fingerprint mode rebuilds T");
   using real2 = typename Vec2<real>::type;
   using HE = HotExp<real>;
   constexpr int NV = TriLds<real, MODE>::NV;
@@ -150,6 +156,7 @@ __global__ __launch_bounds__(TRI_BLOCK, (TriCfg<real, MODE>::MIN_WAVES)) void tr
   unsigned char* sp = tab.carve(smem, nsig, Aa);
   real* rp = (real*)sp;   // 16-byte aligned: the pair tables come first
   real2* tabE = (real2*)rp; rp += (size_t)nr * TRI_CAPP * 2;   // rows of both species of a class: at most m <= nr
+  real* sUn = rp; if (FUSED) rp += (size_t)3 * nr;             // [3][nr] unit vectors
   real* sD = rp; rp += nr;
   real* sP = rp; rp += Aa;
   real* outw = rp; rp += (size_t)TRI_WAVES * Aa;
@@ -209,6 +216,10 @@ __global__ __launch_bounds__(TRI_BLOCK, (TriCfg<real, MODE>::MIN_WAVES)) void tr
     // ---- per-atom slot data
     for (int s = tid; s < m; s += TRI_BLOCK) {
       sD[s] = A.Dsup[rowAtom * nr + s];
+      if (FUSED) {
+#pragma unroll
+        for (int c = 0; c < 3; c++) sUn[c * nr + s] = A.unit[(rowAtom * 4 + c) * nr + s];
+      }
       const int nj = im[1 + s];
       stp[s] = A.type_map[nj];
       if (MODE == 2) {
@@ -313,7 +324,14 @@ __global__ __launch_bounds__(TRI_BLOCK, (TriCfg<real, MODE>::MIN_WAVES)) void tr
               offA[qq] = (unsigned short)(x * TRI_CAPP);
               offB[qq] = (unsigned short)((rowB0 + y) * TRI_CAPP);
               real T = 0;
-              if (ok) T = Trow[nn];
+              if (ok) {
+                if constexpr (FUSED) {
+                  const real cs = sUn[j] * sUn[k] + sUn[nr + j] * sUn[nr + k] + sUn[2 * nr + j] * sUn[2 * nr + k];
+                  T = (real(0.5) * (cs + real(1))) * (sD[j] * sD[k]);
+                } else {
+                  T = Trow[nn];
+                }
+              }
               sT[qq] = T;
               if (MODE == 2) {
                 real U = 0;

@@ -66,7 +66,8 @@ extern "C" {
 #define STAF_E_CAPTURE (-13)         /* the stream is being captured into a graph and the call would have to allocate:
                                         run the same call once outside the capture first */
 #define STAF_E_STALE_MAP (-14)       /* a force op was handed a view of a descriptor output whose intmap2b no longer
-                                        holds what the descriptor op wrote there */
+                                        holds what the descriptor op wrote there, or whose first row is not the
+                                        first atom of the centre species (tipos, actual_type) */
 
 /* ---- library state ------------------------------------------------------ */
 

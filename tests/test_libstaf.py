@@ -162,6 +162,26 @@ def test_compute_matches_oracle_pipeline_fp64_model(oracle):
 
 
 @pytest.mark.gpu
+def test_compute_6144_atom_box_matches_oracle_pipeline(oracle):
+    """BASELINE config 5 through the MD entry: 2048 water molecules, one call, neighbour list rebuilt by the library
+    (cell list: 6144 >= 2048 atoms), no tensor of the angular buffer's width on the device; energy and forces against
+    the oracle ops wired in the reference's order (all-pairs neighbour search there), 1e-10."""
+    from alphanesgpu_amd import libstaf, synth
+    from test_oracle_pins import energy_and_forces
+    tipos, model = load_model("double")
+    b = synth.water_batch("water6144")
+    pos, box = b["pos"].astype(np.float64), b["box"].astype(np.float64)
+    E, F, W, _, _ = energy_and_forces(oracle, pos, box, b["tipos"], b["type_map"], _as64(model), virial=True)
+    m = libstaf.StafModel(os.path.join(GOLDEN, "model_double"), precision=1, full_virial=True)
+    e, f, vir = m.compute(pos.reshape(-1, 3), box[0], b["type_map"])
+    assert abs(e - float(E[0])) <= 1e-10 * abs(float(E[0]))
+    assert nerr(f.reshape(-1), F[0]) <= 1e-10
+    Wm = W[0].reshape(3, 3)
+    assert nerr(vir[:3], np.array([Wm[0, 0], Wm[1, 1], Wm[2, 2]])) <= 1e-10
+    m.close()
+
+
+@pytest.mark.gpu
 def test_compute_reproduces_recorded_energies_fp32_model(oracle):
     """float32 MLP (the reference's default build): E and rms(F) recorded by the reference for its 768-atom frame
     (test/test-lammps-STAF-inference-STAF-comp/results/frames.csv:2) and PE of data.water_smoke
