@@ -201,13 +201,20 @@ struct StreamWork {
   size_t bucket_entries = 0;     // capacity, in ints, of the key part
 };
 
-// What a kernel needs of a transpose (receiver -> sorted (centre, slot) keys, see staf_transpose.hpp).
+// What a force kernel needs to find the slots that list an atom (see staf_transpose.hpp).  Two forms:
+//   symmetric = 1  the map is one the library's own neighbour search wrote for all N atoms of the frames: i lists
+//                  j exactly when j lists i, so an atom's own row names the centres that list it, and the slot is
+//                  found by looking the atom up in that centre's row.  `full` is the whole tensor [nf, N, nr+1].
+//   symmetric = 0  a transposed map, receiver -> sorted (centre, slot) keys (caller-supplied lists, where ghost
+//                  atoms are listed without listing anybody; maps of unknown origin).
 struct TransposeRef {
+  int symmetric = 0;
+  const int* full = nullptr; // symmetric: the intmap2b tensor the view points into
   int* build_cnt = nullptr;  // [nf * Nrecv] fill cursors of a build, all zero between builds
   int* cnt = nullptr;        // [nf * Nrecv] keys per receiving atom
   int* keys = nullptr;       // [nf * Nrecv, cap]
   int cap = 0;
-  int key_shift = 0;         // centre number of row 0 of the map the force op was handed
+  int key_shift = 0;         // centre number (row in `full`) of row 0 of the map the force op was handed
 };
 
 // Transpose the descriptor op keeps beside an intmap2b tensor it has written.
@@ -244,10 +251,11 @@ bool stream_is_capturing(hipStream_t stream);
 void* scratch_reserve(DeviceState* st, hipStream_t stream, size_t bytes);
 // Transpose a force op builds for itself (n_recv receiving atoms, cap keys each), in the stream's own work area.
 bool bucket_reserve(DeviceState* st, size_t n_recv, int cap, hipStream_t stream, TransposeRef* out);
-// Transpose kept beside the intmap2b tensor `im2` the descriptor op is about to write (nf frames, N centres, Nrecv
-// receiving atoms, cap keys per receiver).  Null block -> false.
+// What the library keeps beside the intmap2b tensor `im2` the descriptor op is about to write (nf frames, N centres,
+// Nrecv receiving atoms): for its own neighbour search (symmetric) only the fact, for a caller's list a transposed
+// map of cap keys per receiver.  No block to be had -> false.
 bool transpose_for_descriptor(DeviceState* st, const int* im2, int nf, int N, int Nrecv, int nr, int cap,
-                              hipStream_t stream, TransposeRef* out);
+                              bool symmetric, hipStream_t stream, TransposeRef* out);
 // The transpose that covers the map view a force op was handed (pointer into a descriptor output, frame stride ld),
 // if the library holds one.
 bool transpose_find(DeviceState* st, const int* im2_view, int nf, int Nrecv, int Nl, int ld, int nr, TransposeRef* out);

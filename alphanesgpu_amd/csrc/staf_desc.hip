@@ -242,7 +242,6 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
   int* s_j = c_j + nr;                 // [nr] sorted neighbour index
   int* s_rank = s_j + nr;              // [nr] rank of every candidate
   __shared__ int cnt_all, cnt_ang;
-  __shared__ real sbox[6];
 
   const int tid = threadIdx.x;
   const int b = blockIdx.x / N;
@@ -250,16 +249,18 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
   PHASE_CLOCK_BEGIN();
   if (tid == 0) { cnt_all = 0; cnt_ang = 0; }
   for (int e = tid; e < nr; e += blockDim.x) s_rank[e] = 0;
-  if (tid < 6) sbox[tid] = A.box[b * 6 + tid];
-  __syncthreads();
-
+  // Box and centre position are the same for the whole workgroup: every thread reads them itself (reads of
+  // workgroup-uniform addresses), not one thread for all through LDS and a barrier.
+  const real* pf = A.pos + (size_t)b * A.Npos * 3;
   real box[6], inv[6];
 #pragma unroll
-  for (int c = 0; c < 6; c++) box[c] = sbox[c];
+  for (int c = 0; c < 6; c++) box[c] = A.box[b * 6 + c];
+  const real pix = pf[3 * i], piy = pf[3 * i + 1], piz = pf[3 * i + 2];
+  __syncthreads();
+
   inverse_box(box, inv);
-  const real* pf = A.pos + (size_t)b * A.Npos * 3;
   real si[3];
-  to_frac(inv, pf[3 * i], pf[3 * i + 1], pf[3 * i + 2], si);
+  to_frac(inv, pix, piy, piz, si);
   const real rc2 = A.Rc * A.Rc;
 
   // 1. candidate scan -- or the caller's list (already cut off and sorted by distance)
@@ -388,9 +389,10 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
     __syncthreads();
   }
   PHASE_MARK(1);
-  // Every slot registers with the atom it points at (the transposed map the force ops gather through).  The second
-  // wave does it while the first one fills the radial rows: the atomics' round trip is off the critical path.
-  if (tid >= WAVE && tid < 2 * WAVE) {
+  // A caller's list: every slot registers with the atom it points at (the transposed map the force ops gather
+  // through; the library's own lists are symmetric and need none).  The second wave does it while the first one
+  // fills the radial rows.
+  if (A.tr.keys && tid >= WAVE && tid < 2 * WAVE) {
     for (int e = tid - WAVE; e < n; e += WAVE)
       transpose_push(A.tr.build_cnt, A.tr.keys, A.tr.cap, (size_t)b * A.Npos + c_j[e], i, injected ? e : s_rank[e],
                      A.status);
@@ -643,10 +645,12 @@ int desc_launch(const DescConfig<real>& c, const real* pos, const real* box, int
   A.unit = unit; A.angular = angular ? 1 : 0;
   A.status = st->status_d;
   if (N >= (1 << (31 - KEY_SLOT_BITS))) return STAF_E_LIMIT;
-  // own lists are symmetric (an atom is listed by exactly its own neighbours, at most nr); a caller's list may name
-  // a ghost atom from more centres than that
-  const int cap = inj_howmany ? 4 * c.nr : c.nr;
-  if (!transpose_for_descriptor(st, intmap2b, nf, N, Npos, c.nr, cap, stream, &A.tr)) return reserve_failure(stream);
+  // The library's own search finds j from i exactly when it finds i from j (the squared distance is computed from
+  // the negated difference vector: same bits), so the map it writes needs no transposing; a caller's list may name
+  // ghost atoms, which list nobody, and from more centres than nr.
+  const bool symmetric = inj_howmany == nullptr;
+  if (!transpose_for_descriptor(st, intmap2b, nf, N, Npos, c.nr, 4 * c.nr, symmetric, stream, &A.tr))
+    return reserve_failure(stream);
   A.cell_dims = A.cell_start = A.cell_atoms = A.cell_of = nullptr;
   const int cell_from = g_cell_threshold;
   if (!inj_howmany && cell_from > 0 && N >= cell_from) {
@@ -670,7 +674,7 @@ int desc_launch(const DescConfig<real>& c, const real* pos, const real* box, int
     KernelTimer kt_("desc_kernel", stream);
     hipLaunchKernelGGL(desc_kernel<real>, dim3((unsigned)(nf * N)), dim3(256), lds, stream, A);
   }
-  {
+  if (!symmetric) {
     KernelTimer kt_("transpose_sort_kernel", stream);
     launch_transpose_sort(A.tr, nf * Npos, stream);
   }

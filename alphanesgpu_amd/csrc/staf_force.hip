@@ -4,8 +4,9 @@
 // (STAF/src/force/{rad,ang}/reforce.cu.cc, STAF/src/grad_force/{rad,ang}/reforce.cu.cc).
 //
 // Force scatter is owner-computes and deterministic: every atom collects the pair forces of the slots that point
-// at it through the transposed neighbour map (staf_transpose.hpp; built once per descriptor call), in ascending
-// (centre, slot) order and with a fixed tree -- no floating-point atomics.
+// at it, in a fixed order and with a fixed tree -- no floating-point atomics.  Which slots point at an atom comes
+// from the neighbour map itself when the library's own search wrote it (symmetric: the atom's own neighbours, the
+// slot looked up in the neighbour's row), else from a transposed map (staf_transpose.hpp).
 //   2-body op  one kernel, one wave per atom of the frame: it evaluates the pair force of each of its own slots
 //              (as a centre of the op's species) and of each slot that lists it (read from that centre's rows).
 //   3-body op  pass A (per centre) slot forces -> scratch gslot[b,i,s,3], centre's own force -> self[b,i,3];
@@ -132,18 +133,37 @@ __global__ __launch_bounds__(F_BLOCK) void force2_kernel(Force2Args<real> A) {
     }
   }
   // slots of the op's centres that list this atom
-  const int L = A.tr.cnt[recv];
-  const int* keys = A.tr.keys + (size_t)recv * A.tr.cap;
   const int ta = A.type_map[a];
-  for (int e = lane; e < L; e += WAVE) {
-    const int key = keys[e];
-    const int p = key_centre(key) - A.tr.key_shift, s = key_slot(key);
-    if (p < 0 || p >= Nl) continue;
-    const size_t row = (size_t)b * A.ld + p;
-    if (A.im2[row * (nr + 1) + 1 + s] != a) { atomicOr(A.status, 4); continue; }   // the map is not the one transposed
-    const real w = pair_weight(row, (size_t)b * Nl + p, s, ta);
+  if (A.tr.symmetric) {
+    // the centres that list a are a's own neighbours (row of a in the full map); lane <-> own slot
+    const int* mine = A.tr.full + ((size_t)b * A.N + a) * (nr + 1);
+    int cnt = mine[0];
+    if (cnt > nr) cnt = nr;
+    for (int t = lane; t < nr; t += WAVE) {
+      const int i = mine[1 + t];
+      if (t >= cnt) break;
+      const int p = i - A.tr.key_shift;
+      if (p < 0 || p >= Nl) continue;
+      const int s = slot_of(A.tr.full, b, A.N, nr, i, a);
+      if (s < 0) { atomicOr(A.status, 4); continue; }   // a lists i but i does not list a
+      const size_t row = (size_t)b * A.ld + p;
+      const real w = pair_weight(row, (size_t)b * Nl + p, s, ta);
 #pragma unroll
-    for (int c = 0; c < 3; c++) f[c] += w * A.dD[row * 3 * nr + c * nr + s];
+      for (int c = 0; c < 3; c++) f[c] += w * A.dD[row * 3 * nr + c * nr + s];
+    }
+  } else {
+    const int L = A.tr.cnt[recv];
+    const int* keys = A.tr.keys + (size_t)recv * A.tr.cap;
+    for (int e = lane; e < L; e += WAVE) {
+      const int key = keys[e];
+      const int p = key_centre(key) - A.tr.key_shift, s = key_slot(key);
+      if (p < 0 || p >= Nl) continue;
+      const size_t row = (size_t)b * A.ld + p;
+      if (A.im2[row * (nr + 1) + 1 + s] != a) { atomicOr(A.status, 4); continue; }   // the map is not the one transposed
+      const real w = pair_weight(row, (size_t)b * Nl + p, s, ta);
+#pragma unroll
+      for (int c = 0; c < 3; c++) f[c] += w * A.dD[row * 3 * nr + c * nr + s];
+    }
   }
 #pragma unroll
   for (int c = 0; c < 3; c++) f[c] = wave_sum(f[c]);
@@ -247,18 +267,37 @@ __global__ __launch_bounds__(F_BLOCK) void gather_kernel(const real* __restrict_
   const int shift = host_shift >= 0 ? host_shift : species_shift(tipos, actual_type);
   if (host_shift >= 0 && recv == 0 && lane == 0 && species_shift(tipos, actual_type) != host_shift)
     atomicOr(status, 4);
-  const int L = tr.cnt[recv];
-  const int* keys = tr.keys + (size_t)recv * tr.cap;
   real f[3] = {0, 0, 0};
-  for (int e = lane; e < L; e += WAVE) {
-    const int key = keys[e];
-    const int p = key_centre(key) - tr.key_shift, s = key_slot(key);
-    if (p < 0 || p >= Nl) continue;
-    if (im2[((size_t)b * ld + p) * (nr + 1) + 1 + s] != a) { atomicOr(status, 4); continue; }
-    const real* g = gslot + (((size_t)b * Nl + p) * nr + s) * 3;
-    f[0] += g[0];
-    f[1] += g[1];
-    f[2] += g[2];
+  if (tr.symmetric) {
+    // the centres that list a are a's own neighbours (row of a in the full map); lane <-> own slot
+    const int* mine = tr.full + ((size_t)b * N + a) * (nr + 1);
+    int cnt = mine[0];
+    if (cnt > nr) cnt = nr;
+    for (int t = lane; t < nr; t += WAVE) {
+      const int i = mine[1 + t];
+      if (t >= cnt) break;
+      const int p = i - tr.key_shift;
+      if (p < 0 || p >= Nl) continue;
+      const int s = slot_of(tr.full, b, N, nr, i, a);
+      if (s < 0) { atomicOr(status, 4); continue; }   // a lists i but i does not list a
+      const real* g = gslot + (((size_t)b * Nl + p) * nr + s) * 3;
+      f[0] += g[0];
+      f[1] += g[1];
+      f[2] += g[2];
+    }
+  } else {
+    const int L = tr.cnt[recv];
+    const int* keys = tr.keys + (size_t)recv * tr.cap;
+    for (int e = lane; e < L; e += WAVE) {
+      const int key = keys[e];
+      const int p = key_centre(key) - tr.key_shift, s = key_slot(key);
+      if (p < 0 || p >= Nl) continue;
+      if (im2[((size_t)b * ld + p) * (nr + 1) + 1 + s] != a) { atomicOr(status, 4); continue; }
+      const real* g = gslot + (((size_t)b * Nl + p) * nr + s) * 3;
+      f[0] += g[0];
+      f[1] += g[1];
+      f[2] += g[2];
+    }
   }
 #pragma unroll
   for (int c = 0; c < 3; c++) f[c] = wave_sum(f[c]);

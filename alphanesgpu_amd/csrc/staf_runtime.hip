@@ -115,6 +115,7 @@ bool bucket_reserve(DeviceState* st, size_t n_recv, int cap, hipStream_t stream,
   std::lock_guard<std::mutex> lock(g_mu);
   if (!transpose_block(st, &w->buckets, &w->bucket_counters, &w->bucket_entries, n_recv, n_recv * cap, stream))
     return false;
+  *out = TransposeRef();
   out->build_cnt = (int*)w->buckets.buf;
   out->cnt = out->build_cnt + w->bucket_counters;
   out->keys = out->cnt + w->bucket_counters;
@@ -124,9 +125,9 @@ bool bucket_reserve(DeviceState* st, size_t n_recv, int cap, hipStream_t stream,
 }
 
 bool transpose_for_descriptor(DeviceState* st, const int* im2, int nf, int N, int Nrecv, int nr, int cap,
-                              hipStream_t stream, TransposeRef* out) {
+                              bool symmetric, hipStream_t stream, TransposeRef* out) {
   std::lock_guard<std::mutex> lock(g_mu);
-  const size_t want_recv = (size_t)nf * Nrecv, want_keys = want_recv * cap;
+  const size_t want_recv = symmetric ? 0 : (size_t)nf * Nrecv, want_keys = want_recv * cap;
   Transpose* t = nullptr;
   for (auto& e : st->transposes)
     if (e.im2 == im2) { t = &e; break; }
@@ -141,14 +142,18 @@ bool transpose_for_descriptor(DeviceState* st, const int* im2, int nf, int N, in
     }
     if (!t) return false;
   }
-  const size_t n_recv = (size_t)nf * Nrecv;
-  if (!transpose_block(st, &t->buf, &t->cap_recv, &t->cap_keys, n_recv, n_recv * cap, stream)) return false;
+  if (!symmetric && !transpose_block(st, &t->buf, &t->cap_recv, &t->cap_keys, want_recv, want_keys, stream))
+    return false;
   t->im2 = im2; t->nf = nf; t->N = N; t->Nrecv = Nrecv; t->nr = nr;
-  t->ref.build_cnt = (int*)t->buf.buf;
-  t->ref.cnt = t->ref.build_cnt + t->cap_recv;
-  t->ref.keys = t->ref.cnt + t->cap_recv;
-  t->ref.cap = cap;
-  t->ref.key_shift = 0;
+  t->ref = TransposeRef();
+  t->ref.symmetric = symmetric ? 1 : 0;
+  t->ref.full = im2;
+  if (!symmetric) {
+    t->ref.build_cnt = (int*)t->buf.buf;
+    t->ref.cnt = t->ref.build_cnt + t->cap_recv;
+    t->ref.keys = t->ref.cnt + t->cap_recv;
+    t->ref.cap = cap;
+  }
   t->stamp = ++st->transpose_clock;
   *out = t->ref;
   return true;

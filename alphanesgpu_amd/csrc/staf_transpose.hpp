@@ -10,6 +10,10 @@
 //
 // Building uses integer atomics only (the arrival order they leave is removed by the sort); every list ends up in
 // ascending (centre, slot) order, so sums taken over it have a fixed order.
+//
+// None of this is needed for the maps the library's own neighbour search writes: those are symmetric, the centres
+// that list an atom are the atom's own neighbours, and the slot is found by looking the atom up in the centre's row
+// (slot_of below).  Sums then run in the order of the atom's own (distance-sorted) row.
 #pragma once
 #include "staf_common.hpp"
 
@@ -29,6 +33,41 @@ __device__ inline void transpose_push(int* build_cnt, int* keys, int cap, size_t
   const int pos = atomicAdd(&build_cnt[recv], 1);
   if (pos < cap) keys[recv * cap + pos] = key_make(centre, slot);
   else atomicOr(status, 2);
+}
+
+// Slot of atom `a` in the row of centre `i` of frame b of the symmetric map `full` [nf, N, nr+1], or -1 (the map is
+// not symmetric after all: reported by the caller).  The whole row is requested at once, sixteen entries per round
+// in four 16-byte reads (rows are only 4-byte aligned), and compared without an early exit: one round trip to
+// memory instead of one per entry.
+struct __attribute__((packed, aligned(4))) Int4U { int x, y, z, w; };
+__device__ inline int slot_of(const int* __restrict__ full, int b, int N, int nr, int i, int a) {
+  const int* r = full + ((size_t)b * N + i) * (nr + 1);
+  int cnt = r[0];
+  if (cnt > nr) cnt = nr;
+  const int* e = r + 1;
+  int found = -1;
+  int s0 = 0;
+  for (; s0 + 16 <= nr; s0 += 16) {
+    Int4U v[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) v[u] = *(const Int4U*)(e + s0 + 4 * u);
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      found = (v[u].x == a && s0 + 4 * u < cnt) ? s0 + 4 * u : found;
+      found = (v[u].y == a && s0 + 4 * u + 1 < cnt) ? s0 + 4 * u + 1 : found;
+      found = (v[u].z == a && s0 + 4 * u + 2 < cnt) ? s0 + 4 * u + 2 : found;
+      found = (v[u].w == a && s0 + 4 * u + 3 < cnt) ? s0 + 4 * u + 3 : found;
+    }
+  }
+  for (; s0 < nr; s0 += 4) {   // ragged end of the row, entry by entry (never beyond the row)
+    int v[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) v[u] = s0 + u < nr ? e[s0 + u] : -1;
+#pragma unroll
+    for (int u = 0; u < 4; u++) found = (v[u] == a && s0 + u < cnt) ? s0 + u : found;
+  }
+  // (padded entries hold 0, which is also an atom: only slots below the count are the centre's neighbours)
+  return found;
 }
 
 // One thread per (frame, centre, slot) of a map [nf, ld (Nl used), nr+1]: the push pass of a transpose built by a

@@ -218,8 +218,8 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
-    if workload is not None:
-        out = run_workload(args, workload, args.mode)
+    if args.workload is not None:
+        out = run_workload(args, args.workload, args.mode)
     else:
         # The metric names both halves: fp32 descriptor fwd + force (the headline line) and the fp64 full step with
         # the parameter-gradient ops, measured in the same process right behind it.

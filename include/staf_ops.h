@@ -34,14 +34,16 @@
  *     different streams of a device may overlap; calls on one stream are ordered.
  *     The error word of staf_ops_poll_status is one per device, shared by all
  *     streams: a poll reports what any of them raised.
- *   - the force ops gather through a transposed neighbour map that the
- *     descriptor op builds and keeps beside the intmap2b tensor it writes
- *     (the 8 most recently written tensors per device).  A force op whose
- *     interaction_map_rad points into such a tensor (ld_atoms = N) uses that
- *     transpose; the tensor must then still hold what the descriptor op wrote
- *     (a slot that does not is reported as STAF_E_STALE_MAP).  Any other copy
- *     of the map (tf.split output, ld_atoms = N_local) is transposed by the
- *     force op itself, at the price of two more launches.
+ *   - the force ops are owner-computes: every atom collects the pair forces of
+ *     the slots that list it.  The descriptor op remembers, by address, the
+ *     intmap2b tensors it has written (the 8 most recent per device); such a
+ *     map is symmetric (i lists j exactly when j lists i), so a force op whose
+ *     interaction_map_rad points into one (ld_atoms = N) finds the slots that
+ *     list an atom from the atom's own row.  The tensor must then still hold
+ *     what the descriptor op wrote (a broken pairing is reported as
+ *     STAF_E_STALE_MAP).  Any other copy of the map (tf.split output,
+ *     ld_atoms = N_local) is transposed by the force op itself, at the price of
+ *     two more launches.
  *   - graph capture: every entry point may be captured once the same call (same
  *     shapes, same stream, same output tensors for the descriptor op) has run
  *     eagerly, which sizes the library's work areas; a call that would have to
@@ -132,8 +134,8 @@ int staf_op_descriptor_coefficients_f64(double* out5);
  *   positions [nf, 3N] Cartesian, boxer [nf, 6] = [Lx, xy, xz, Ly, yz, Lz]
  *   raddescr [nf,N,nr]  angdescr [nf,N,na]  des3bsupp [nf,N,nr]  intmap2b [nf,N,nr+1]
  *   intmap3b [nf,N,2*na]  der2b [nf,N,3,nr]  der3b [nf,N,3,2*na]  der3bsupp [nf,N,3,nr]  numtriplet [nf,N]
- * Padded slots are written as 0 (der3b: see staf_op_descriptor_options).  Also builds the transposed neighbour map
- * of intmap2b that the force ops use (kept by the library, keyed by the address of intmap2b). */
+ * Padded slots are written as 0 (der3b: see staf_op_descriptor_options).  The library notes the address of intmap2b
+ * as that of a map of its own making (see the conventions above). */
 int staf_op_compute_descriptors_light_f32(const float* positions, const float* boxer, int nf, int N, float* raddescr,
                                           float* angdescr, float* des3bsupp, int* intmap2b, int* intmap3b,
                                           float* der2b, float* der3b, float* der3bsupp, int* numtriplet,
