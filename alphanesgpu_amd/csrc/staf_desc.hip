@@ -242,6 +242,7 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
   int* s_j = c_j + nr;                 // [nr] sorted neighbour index
   int* s_rank = s_j + nr;              // [nr] rank of every candidate
   __shared__ int cnt_all, cnt_ang;
+  __shared__ real sinv[6];
 
   const int tid = threadIdx.x;
   const int b = blockIdx.x / N;
@@ -250,15 +251,21 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
   if (tid == 0) { cnt_all = 0; cnt_ang = 0; }
   for (int e = tid; e < nr; e += blockDim.x) s_rank[e] = 0;
   // Box and centre position are the same for the whole workgroup: every thread reads them itself (reads of
-  // workgroup-uniform addresses), not one thread for all through LDS and a barrier.
+  // workgroup-uniform addresses).  The inverse box costs six divisions -- in double precision more instructions
+  // than a thread's whole share of the candidate scan -- so one wave computes it for all.
   const real* pf = A.pos + (size_t)b * A.Npos * 3;
   real box[6], inv[6];
 #pragma unroll
   for (int c = 0; c < 6; c++) box[c] = A.box[b * 6 + c];
   const real pix = pf[3 * i], piy = pf[3 * i + 1], piz = pf[3 * i + 2];
+  if (tid < WAVE) {
+    inverse_box(box, inv);
+    if (tid < 6) sinv[tid] = tid == 0 ? inv[0] : tid == 1 ? inv[1] : tid == 2 ? inv[2] : tid == 3 ? inv[3]
+                                                 : tid == 4 ? inv[4] : inv[5];
+  }
   __syncthreads();
-
-  inverse_box(box, inv);
+#pragma unroll
+  for (int c = 0; c < 6; c++) inv[c] = sinv[c];
   real si[3];
   to_frac(inv, pix, piy, piz, si);
   const real rc2 = A.Rc * A.Rc;
@@ -409,12 +416,12 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
       const real r = norm_plain(d);
       const real invr = real(1) / r;
       real sc, cc;
-      r_sincos(PI * r / A.Rc, &sc, &cc);
+      r_sincos_0pi(PI * r / A.Rc, &sc, &cc);   // r < Rc: the argument lies in [0, pi]
       real fc = 0, dfc = 0;
       if (r < A.Ra) {
         atomicAdd(&cnt_ang, 1);
         real sa = sc, ca = cc;
-        if (!same_cut) r_sincos(PI * r / A.Ra, &sa, &ca);
+        if (!same_cut) r_sincos_0pi(PI * r / A.Ra, &sa, &ca);   // r < Ra
         fc = real(0.5) * (ca + real(1));
         dfc = -real(0.5) * sa * PI / A.Ra;
       }
