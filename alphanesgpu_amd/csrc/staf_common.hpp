@@ -120,23 +120,38 @@ __device__ inline int wave_max(int v) {
   return v;
 }
 
+// Index arithmetic of the hot kernels uses the 24-bit multiplier (full rate; the 32-bit integer multiply takes
+// four times as long): operands here are slot, species and channel counts far below 2^23.
+__device__ inline int mul24(int a, int b) { return __mul24(a, b); }
+
 // First flat index of row j in the row-major upper triangle over m items
 // (pairs j<k): the reference's triplet numbering,
-// STAF/src/descriptor_builder/reforce.cu.cc:137-146.
-__device__ inline int tri_rowstart(int j, int m) { return j * m - (j * (j + 1)) / 2; }
+// STAF/src/descriptor_builder/reforce.cu.cc:137-146.  j m - j (j + 1) / 2 = j (2 m - 1 - j) / 2, m <= 2048.
+__device__ inline int tri_rowstart(int j, int m) { return mul24(j, 2 * m - 1 - j) >> 1; }
 
 // Inverse of the numbering: nn -> (j,k), 0 <= nn < m(m-1)/2, m <= 2048.  The hardware square root (1 ulp) puts
-// the row estimate within one of the exact row; the comparisons with the exact integer row starts settle it.
+// the row estimate within one of the exact row (two steps each way are taken); the row start follows the row in
+// steps of the row length m - 1 - j, so that the comparisons with the exact integer row starts cost no multiply.
 __device__ inline void tri_decode(int nn, int m, int& j, int& k) {
   const int t = 2 * m - 1;
-  int jj = (int)(((float)t - __builtin_amdgcn_sqrtf((float)(t * t - 8 * nn))) * 0.5f);
+  int jj = (int)(((float)t - __builtin_amdgcn_sqrtf((float)(mul24(t, t) - 8 * nn))) * 0.5f);
   jj = jj < 0 ? 0 : (jj > m - 2 ? m - 2 : jj);
-  if (jj > 0 && tri_rowstart(jj, m) > nn) --jj;
-  if (jj > 0 && tri_rowstart(jj, m) > nn) --jj;
-  if (jj < m - 2 && tri_rowstart(jj + 1, m) <= nn) ++jj;
-  if (jj < m - 2 && tri_rowstart(jj + 1, m) <= nn) ++jj;
+  int rs = mul24(jj, t - jj) >> 1;
+#pragma unroll
+  for (int it = 0; it < 2; it++) {   // row 0 starts at 0 <= nn: never stepped below
+    const bool down = rs > nn;
+    rs = down ? rs - (m - jj) : rs;
+    jj = down ? jj - 1 : jj;
+  }
+#pragma unroll
+  for (int it = 0; it < 2; it++) {   // the row after row m - 2 would start at m (m - 1) / 2 > nn: never stepped to
+    const int next = rs + (m - 1 - jj);
+    const bool up = next <= nn;
+    rs = up ? next : rs;
+    jj = up ? jj + 1 : jj;
+  }
   j = jj;
-  k = nn - tri_rowstart(jj, m) + jj + 1;
+  k = nn - rs + jj + 1;
 }
 
 // Minimum-image Cartesian separation r_i - r_j from Cartesian positions and

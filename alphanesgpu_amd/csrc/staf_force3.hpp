@@ -1,9 +1,9 @@
-// 3-body force, pass A: one 256-thread workgroup per centre atom, four barriers per centre.
+// 3-body force, pass A: one workgroup of four or eight waves per centre atom, four barriers per centre.
 // Replaces computeforce_tripl_kernel (STAF/src/force/ang/reforce.cu.cc:96-214).
 //
 // The kernel is bound by vector-ALU issue and by latency, so the layout keeps the per-(triplet, channel) work
 // minimal, keeps everything else out of the inner loop and avoids workgroup barriers:
-//   * lane <-> triplet in storage order (nn = 64*pass + lane, passes dealt round-robin to the four waves):
+//   * lane <-> triplet in storage order (nn = 64*pass + lane, passes dealt round-robin to the waves):
 //     angdescr and der3b are read coalesced, once; the triplets of a wave's NP passes (T, the three channel
 //     sums, packed indices) stay in registers from the first read to the slot sums.
 //   * exp(a1 D_s) and exp(a2 D_s) of every (channel ia, slot s, partner species tb) are tabulated in LDS once
@@ -18,9 +18,10 @@
 //     channel loop is unrolled, so that every LDS read of the loop is a per-triplet base address plus an
 //     immediate offset.
 //   * der3b contraction in the same lanes: the contributions to slot j of a pass form contiguous lane groups
-//     (rows of the triplet triangle) and are summed with one inclusive scan per value; the contributions to
-//     slot k are added to the wave's own LDS accumulators row by row (inside a row the k are distinct).  The
-//     four waves' accumulators are added in a fixed order: results are bit-reproducible.
+//     (rows of the triplet triangle) and are summed with one inclusive scan per value (the prefix before a row's
+//     first lane is taken with a lane read); the contributions to slot k are added to the wave's own LDS
+//     accumulators row by row (inside a row the k are distinct).  One accumulator per wave and slot takes both;
+//     the waves' accumulators are added in a fixed order: results are bit-reproducible.
 //     F_s = sum_p Sd(s,p) dT/dd_s(s,p) + (sum_p SB_s(s,p)) grad fc_s
 // The slot forces go to scratch (gslot, and the centre's own force to self); the atoms that receive them collect
 // them in gather_kernel through the transposed neighbour map.
@@ -55,23 +56,32 @@ __device__ inline void wave_scan4(T (&v)[4]) {
   for (int c = 0; c < 4; c++) v[c] = s[c];
 }
 
-template <typename real>
+// NW_: waves per workgroup, 4 or 8.  A sweep takes 16 passes of 64 triplets either way; with eight waves a wave holds
+// two of them, so that a centre's critical path and a wave's registers are about half of what they are with four.
+template <typename real, int NW_ = 4>
 struct Force3Cfg {
-  static constexpr int THREADS = 256;
-  static constexpr int NW = THREADS / WAVE;
-  static constexpr int NP = 4;                              // passes of 64 triplets a wave holds in registers
+  static_assert(NW_ == 4 || NW_ == 8, "four or eight waves per workgroup");
+  static constexpr int NW = NW_;
+  static constexpr int THREADS = NW * WAVE;
+  static constexpr int NP = 16 / NW;                        // passes of 64 triplets a wave holds in registers
   static constexpr int CAP = sizeof(real) == 8 ? 8 : 16;    // channels tabulated at a time
   static constexpr int CAPP = CAP + 1;                      // table row pitch in entries
   // der3b rows requested one sweep ahead and held in registers across the channel loop: measured, no gain in
   // fp32 (the kernel is bound by vector-ALU issue) and slower in fp64 (a third of the resident waves lost)
+  // measured and not faster either: the rows of a wave's first pass requested ahead of the channel loop, rolling
+  // requests in single precision, one element of every 128-byte line of the rows requested at the kernel's start
+  static constexpr bool EARLY1 = false;
   static constexpr bool PREFETCH = false;
+  // waves per SIMD the register allocation is held to (what the LDS footprint of the reference's sizes admits:
+  // six workgroups per CU in single precision, four in double)
+  static constexpr int MIN_WAVES = NW == 8 ? (sizeof(real) == 8 ? 6 : 8) : (sizeof(real) == 8 ? 4 : 6);
   __host__ __device__ static bool fits(int nr, int nt) { return nr <= 255 && nt <= NT_MAX; }   // slots packed in 8 bits
   __host__ __device__ static int pitch(int Aa) { return (Aa + 3) & ~3; }   // parameter row pitch (channels)
   __host__ __device__ static size_t n_reals(int nr, int Aa, int nt, bool fused = false) {
     const int nsig = 2 * nt - 1;
     return (size_t)nsig * pitch(Aa) * 6 /*prm, prE*/ + (((size_t)CAPP * nt * nr + 1) & ~(size_t)1) * 2 /*E*/ +
-           (size_t)NW * 8 * nr /*accJ, accK per wave*/ + nr /*D*/ + 3 * nr /*grad fc*/ +
-           (size_t)NW * 4 * WAVE /*scan exchange per wave*/ + (fused ? 4 * nr : 0) /*unit vectors, 1/r*/;
+           (size_t)NW * 4 * nr /*slot sums per wave*/ + nr /*D*/ + 3 * nr /*grad fc*/ +
+           (size_t)NW * 4 /*the waves' shares of the centre's own force*/ + (fused ? 4 * nr : 0) /*unit vectors, 1/r*/;
   }
   __host__ __device__ static size_t bytes(int nr, int Aa, int nt, bool fused = false) {
     return n_reals(nr, Aa, nt, fused) * sizeof(real) + (size_t)(16 + nr) * sizeof(int);
@@ -83,8 +93,8 @@ struct Force3Cfg {
 // STAF/src/descriptor_builder/reforce.cu.cc:195-228), with c = u_j . u_k, h = (c + 1)/2:
 //   T = h fc_j fc_k,   dT/dd_j = 1/2 fc_j fc_k / r_j (u_k - c u_j) + h fc_k grad fc_j,   j <-> k for dT/dd_k
 // `unit` is [nf, ld, 4, nr] = (u_x, u_y, u_z, 1/r) per sorted neighbour, written by the radial-only descriptor call.
-template <typename real, bool FUSED = false>
-__global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
+template <typename real, bool FUSED = false, int NWAVES = 4>
+__global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real, NWAVES>::MIN_WAVES)) void force3_kernel(
     const real* __restrict__ G, const real* __restrict__ Dsup, const real* __restrict__ Tang,
     const real* __restrict__ dDsup, const real* __restrict__ d3b, const real* __restrict__ unit,
     const int* __restrict__ im2,
@@ -94,7 +104,7 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
   using real2 = typename Vec2<real>::type;
   using real4 = typename Vec4<real>::type;
   using HE = HotExp<real>;
-  using L = Force3Cfg<real>;
+  using L = Force3Cfg<real, NWAVES>;
   constexpr int NP = L::NP, NW = L::NW, THREADS = L::THREADS, CAP = L::CAP, CAPP = L::CAPP;
   extern __shared__ __align__(16) unsigned char smem[];
   const int nsig = 2 * nt - 1;
@@ -103,11 +113,11 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
   real* prm = (real*)smem;                                 // [nsig*Ap][4] = a1+a2, a1-a2, scaled beta, 1/4 G c3 (active channels)
   real* prE = prm + (size_t)nsig * Ap * 4;                 // [nsig*Ap][2] = a1, a2 in the units of the hot exponential
   real2* E = (real2*)(prE + (size_t)nsig * Ap * 2);        // [RT][CAPP]
-  real* acc = (real*)(E + (((size_t)RT * CAPP + 1) & ~(size_t)1));   // [NW][2][nr][4]: per wave, slot sums as j and as k
-  real* sD = acc + (size_t)NW * 8 * nr;                    // [nr]
+  real* acc = (real*)(E + (((size_t)RT * CAPP + 1) & ~(size_t)1));   // [NW][nr][4]: per wave, slot sums (as j and as k)
+  real* sD = acc + (size_t)NW * 4 * nr;                    // [nr]
   real* sg = sD + nr;                                      // [3*nr] grad fc (der3bsupp)
-  real* xch = sg + 3 * nr;                                 // [NW][4][64] prefix sums of a pass
-  real* sU = xch + NW * 4 * WAVE;                          // FUSED: [4][nr] unit vector, 1/r
+  real* xch = sg + 3 * nr;                                 // [NW][4] the waves' shares of the centre's own force
+  real* sU = xch + NW * 4;                                 // FUSED: [4][nr] unit vector, 1/r
   int* nact = (int*)(sU + (FUSED ? 4 * nr : 0));           // [16] active channels per sigma (0 beyond nsig)
   int* stp = nact + 16;                                    // [nr] species of every slot
   PHASE_CLOCK_BEGIN();
@@ -124,9 +134,7 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
   if (ntri > na) ntri = na;
   const real* Trow = Tang + rowAtom * na;
   const real2* d3 = (const real2*)d3b + rowAtom * 3 * na;
-  real4* accJ = (real4*)(acc + (size_t)wave * 8 * nr);   // [nr] x (force x, y, z, radial factor)
-  real4* accK = accJ + nr;
-  real* myx = xch + wave * 4 * WAVE;
+  real4* accW = (real4*)(acc + (size_t)wave * 4 * nr);   // [nr] x (force x, y, z, radial factor)
 
   // ---- set-up.  Global reads are issued back to back in two levels: (1) everything addressed by the centre alone,
   // the neighbour index first (read up to nr: padded slots are never used); (2) the neighbour's species, which
@@ -160,7 +168,7 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
   int t_s = 0;
   if (slot) t_s = type_map[nj];
   if (tid >= nsig && tid < 16) nact[tid] = 0;
-  for (int q = tid; q < NW * 8 * nr; q += THREADS) acc[q] = 0;
+  for (int q = tid; q < NW * 4 * nr; q += THREADS) acc[q] = 0;
   for (int sgm = wave; sgm < nsig; sgm += NW) {
     int base = 0;
     for (int a0 = 0; a0 < Aa; a0 += WAVE) {
@@ -215,6 +223,11 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
   // The der3b rows of a sweep are requested one sweep ahead (those of the first here, after the last wait of the
   // set-up): all workgroups of a launch run in step, so reads issued only where they are needed arrive as one
   // burst with the vector units idle.
+  // LATE: the products of a pass are formed where the pass is reduced.  Always so in the fused form; in double
+  // precision too, where in addition the der3b rows of a pass are requested while the pass before it is reduced (all
+  // passes' rows or products at once do not fit the registers of four waves per SIMD).
+  constexpr bool LATE = FUSED || sizeof(real) == 8;
+  constexpr bool ROLL = !FUSED && LATE && !L::PREFETCH;
   real2 dn[NP][3];
   if constexpr (L::PREFETCH && !FUSED) {
 #pragma unroll
@@ -246,13 +259,18 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
           T[p] = Tn[p];
         }
         const int tj = stp[j], tk = stp[k];
-        rj[p] = (tk * nr + j) * CAPP;
-        rk[p] = (tj * nr + k) * CAPP;
-        rp[p] = (tj + tk) * Ap * 4;
+        rj[p] = mul24(mul24(tk, nr) + j, CAPP);
+        rk[p] = mul24(mul24(tj, nr) + k, CAPP);
+        rp[p] = mul24(tj + tk, Ap * 4);
         jk[p] = j | (k << 8);
       }
     }
     PHASE_MARK(1);
+    if constexpr (ROLL && L::EARLY1) {   // der3b rows of the wave's first pass: on their way during the channel loop
+      const int nn = w0 + wave * WAVE + lane;
+#pragma unroll
+      for (int c = 0; c < 3; c++) dn[0][c] = d3[c * na + (nn < nlast ? nn : nlast)];
+    }
 
     for (int c0 = 0; c0 < maxact; c0 += CAP) {
       const int nch = (maxact - c0) < CAP ? (maxact - c0) : CAP;
@@ -266,12 +284,12 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
         if (ia < nch2) {
           for (int tb = 0; tb < nt; tb++) {
             for (int s_ = r0; s_ < m; s_ += RPI) {
-              const real2 o = *(const real2*)(prE + ((size_t)(stp[s_] + tb) * Ap + c0 + ia) * 2);
+              const real2 o = *(const real2*)(prE + (mul24(stp[s_] + tb, Ap) + c0 + ia) * 2);
               const real d = sD[s_];
               real2 v;
               v.x = HE::eval(o.x * d);
               v.y = HE::eval(o.y * d);
-              E[(tb * nr + s_) * CAPP + ia] = v;
+              E[mul24(mul24(tb, nr) + s_, CAPP) + ia] = v;
             }
           }
         }
@@ -319,13 +337,21 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
           }
         }
       };
-      static_assert(NP == 4, "one case per pass count below");
-      switch (npass) {
-        case 1: channels(std::integral_constant<int, 1>{}); break;
-        case 2: channels(std::integral_constant<int, 2>{}); break;
-        case 3: channels(std::integral_constant<int, 3>{}); break;
-        case 4: channels(std::integral_constant<int, 4>{}); break;
-        default: break;
+      static_assert(NP == 4 || NP == 2, "one case per pass count below");
+      if constexpr (NP == 4) {
+        switch (npass) {
+          case 1: channels(std::integral_constant<int, 1>{}); break;
+          case 2: channels(std::integral_constant<int, 2>{}); break;
+          case 3: channels(std::integral_constant<int, 3>{}); break;
+          case 4: channels(std::integral_constant<int, 4>{}); break;
+          default: break;
+        }
+      } else {
+        switch (npass) {
+          case 1: channels(std::integral_constant<int, 1>{}); break;
+          case 2: channels(std::integral_constant<int, 2>{}); break;
+          default: break;
+        }
       }
       PHASE_MARK(3);
     }
@@ -334,9 +360,9 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
     // computed on row 0: their products are forced to 0.
     if constexpr (FUSED) {
       // nothing to load: a pass's Jacobian is rebuilt from the slot tile where it is used
-    } else if constexpr (!L::PREFETCH) {
+    } else if constexpr (!L::PREFETCH && !(ROLL && L::EARLY1)) {
 #pragma unroll
-      for (int p = 0; p < NP; p++) {
+      for (int p = 0; p < (ROLL ? 1 : NP); p++) {
         const int nn = w0 + (p * NW + wave) * WAVE + lane;
 #pragma unroll
         for (int c = 0; c < 3; c++) dn[p][c] = d3[c * na + (nn < nlast ? nn : nlast)];
@@ -375,7 +401,7 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
       vj[3] = (U[p] + V[p]) * hT;
       vk[3] = (U[p] - V[p]) * hT;
     };
-    if constexpr (!FUSED) {
+    if constexpr (!LATE) {
 #pragma unroll
       for (int p = 0; p < NP; p++) pass_products(p, vjs[p], vks[p]);
     }
@@ -402,34 +428,38 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
       const bool valid = nn < ntri;
       const int j = jk[p] & 0xff, k = jk[p] >> 8;
       real vj[4], vk[4];
-      if constexpr (FUSED) {
+      if constexpr (ROLL) {
+        if (p + 1 < NP) {   // rows of the next pass (a pass this wave has no triplets in re-reads the last triplet)
+          const int nx = w0 + ((p + 1) * NW + wave) * WAVE + lane;
+#pragma unroll
+          for (int c = 0; c < 3; c++) dn[(p + 1) % NP][c] = d3[c * na + (nx < nlast ? nx : nlast)];
+        }
+      }
+      if constexpr (LATE) {
         pass_products(p, vj, vk);
       } else {
 #pragma unroll
         for (int c = 0; c < 4; c++) { vj[c] = vjs[p][c]; vk[c] = vks[p][c]; }
       }
       // slot j: the lanes of a row are contiguous.  Row sum = prefix at the row's last lane minus prefix
-      // before its first lane of this pass.
-      __builtin_amdgcn_wave_barrier();
+      // before its first lane of this pass (taken with a lane read: no memory is involved).
       wave_scan4(vj);
+      const int first = lane - (k - j - 1);   // lane of the row's first triplet (not positive: starts earlier)
+      const int before = first > 0 ? first - 1 : 0;   // lanes past the last triplet hold j = k = 0: their own lane
+      real pre[4];
 #pragma unroll
-      for (int c = 0; c < 4; c++) myx[c * WAVE + lane] = vj[c];
-      __builtin_amdgcn_wave_barrier();
+      for (int c = 0; c < 4; c++) pre[c] = __shfl(vj[c], before, WAVE);
       const int jn = __shfl_down(valid ? j : -1, 1, WAVE);
       const bool row_end = valid && (lane == WAVE - 1 || jn != j);
       if (row_end) {
-        const int first = lane - (k - j - 1);   // lane of the row's first triplet (not positive: starts earlier)
-        const int before = first > 0 ? first - 1 : 0;
-        real sj[4];
-#pragma unroll
-        for (int c = 0; c < 4; c++) {
-          const real pre = myx[c * WAVE + before];
-          sj[c] = vj[c] - (first > 0 ? pre : real(0));
-        }
-        real4 t = accJ[j];
-        t.x += sj[0]; t.y += sj[1]; t.z += sj[2]; t.w += sj[3];
-        accJ[j] = t;
+        real4 t = accW[j];
+        t.x += vj[0] - (first > 0 ? pre[0] : real(0));
+        t.y += vj[1] - (first > 0 ? pre[1] : real(0));
+        t.z += vj[2] - (first > 0 ? pre[2] : real(0));
+        t.w += vj[3] - (first > 0 ? pre[3] : real(0));
+        accW[j] = t;
       }
+      __builtin_amdgcn_wave_barrier();   // the wave's memory operations stay in program order: slot k sums follow
       // slot k: row by row (the k of one row are distinct).  LDS floating-point adds instead of this loop were
       // measured: much slower in fp32 (1.6x the kernel), a few percent faster in fp64.
       const int jlo = __builtin_amdgcn_readfirstlane(j);
@@ -437,9 +467,9 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
       const int jhi = __builtin_amdgcn_readlane(j, llast);
       for (int g = jlo; g <= jhi; g++) {
         if (valid && j == g) {
-          real4 t = accK[k];
+          real4 t = accW[k];
           t.x += vk[0]; t.y += vk[1]; t.z += vk[2]; t.w += vk[3];
-          accK[k] = t;
+          accW[k] = t;
         }
         __builtin_amdgcn_wave_barrier();
       }
@@ -455,9 +485,8 @@ __global__ __launch_bounds__(Force3Cfg<real>::THREADS) void force3_kernel(
     real t4[4] = {0, 0, 0, 0};
 #pragma unroll
     for (int w = 0; w < NW; w++) {
-      const real4 a = ((const real4*)(acc + (size_t)w * 8 * nr))[tid];
-      const real4 c_ = ((const real4*)(acc + (size_t)w * 8 * nr))[nr + tid];
-      t4[0] += a.x + c_.x; t4[1] += a.y + c_.y; t4[2] += a.z + c_.z; t4[3] += a.w + c_.w;
+      const real4 a = ((const real4*)(acc + (size_t)w * 4 * nr))[tid];
+      t4[0] += a.x; t4[1] += a.y; t4[2] += a.z; t4[3] += a.w;
     }
 #pragma unroll
     for (int c = 0; c < 3; c++) f3[c] = t4[c] + t4[3] * sg[c * nr + tid];
