@@ -21,6 +21,10 @@ constexpr int NT_MAX = 8;  // species supported by the per-type bookkeeping
 template <typename real> struct Vec2;
 template <> struct Vec2<float> { using type = float2; };
 template <> struct Vec2<double> { using type = double2; };
+// 16 bytes of reals: the widest LDS and global access
+template <typename real> struct Vec16;
+template <> struct Vec16<float> { using type = float4; };
+template <> struct Vec16<double> { using type = double2; };
 template <typename real> struct Vec4;
 template <> struct Vec4<float> { using type = float4; };
 template <> struct Vec4<double> { using type = double4; };

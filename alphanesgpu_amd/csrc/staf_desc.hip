@@ -225,6 +225,19 @@ __global__ __launch_bounds__(CELL_THREADS) void cell_build_kernel(const real* __
   }
 }
 
+// Zeroes nbytes (a multiple of 4) from p (4-byte aligned), all threads of a 256-thread workgroup calling: single
+// words up to the first 16-byte boundary and after the last, 16-byte stores between.
+__device__ inline void zero_fill(char* p, unsigned nbytes, int tid) {
+  const unsigned head_max = (unsigned)((16 - ((size_t)p & 15)) & 15);
+  const unsigned head = head_max < nbytes ? head_max : nbytes;
+  const unsigned body = (nbytes - head) & ~15u;
+  const unsigned tail = nbytes - head - body;
+  if ((unsigned)tid * 4u < head) *(int*)(p + tid * 4u) = 0;
+  char* q = p + head;
+  for (unsigned o = (unsigned)tid * 16u; o < body; o += 256u * 16u) *(int4*)(q + o) = make_int4(0, 0, 0, 0);
+  if ((unsigned)tid * 4u < tail) *(int*)(q + body + tid * 4u) = 0;
+}
+
 template <typename real>
 __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
   using real2 = typename Vec2<real>::type;
@@ -233,12 +246,14 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
   // LDS carve-up
   real* c_d2 = (real*)smem;            // [nr] candidate dist2
   real* c_d = c_d2 + nr;               // [3*nr] candidate delta (neighbour - centre)
-  // [8][nr] per sorted neighbour: unit vector centre - neighbour (3), 1/r, grad of fc wrt d (3), fc.  Component-
-  // major: the lanes of a wave hold consecutive triplets, i.e. one j and consecutive k, so a component of the k
-  // records is read from consecutive words (no bank conflict) and of the j record as a broadcast (records of 8
-  // components side by side cost 2-4 conflict cycles per read)
-  real* s_rec = c_d + 3 * nr;
-  int* c_j = (int*)(s_rec + 8 * nr);   // [nr] candidate index
+  // Per sorted neighbour: unit vector centre - neighbour (3), 1/r, grad of fc wrt d (3), fc, kept as 16-byte pieces
+  // in REC_P arrays of nr pieces each (piece q of slot s at s_rec[q * nr + s]): the lanes of a wave hold consecutive
+  // triplets, i.e. one j and consecutive k, so a piece of the k records is read from consecutive 16-byte words (no
+  // bank conflict) and of the j record as a broadcast, with one address and REC_P wide reads per record.
+  using rec_t = typename Vec16<real>::type;
+  constexpr int REC_P = 8 * (int)sizeof(real) / 16, REC_N = 16 / (int)sizeof(real);
+  rec_t* s_rec = (rec_t*)(c_d + 3 * nr);
+  int* c_j = (int*)((real*)s_rec + 8 * nr);   // [nr] candidate index
   int* s_j = c_j + nr;                 // [nr] sorted neighbour index
   int* s_rank = s_j + nr;              // [nr] rank of every candidate
   __shared__ int cnt_all, cnt_ang;
@@ -445,18 +460,21 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
       A.des3bsupp[row + rank] = fc;
       im[1 + rank] = j;
       s_j[rank] = j;
-      s_rec[3 * nr + rank] = invr;
-      s_rec[7 * nr + rank] = fc;
       if (A.unit) A.unit[(atom * 4 + 3) * nr + rank] = invr;
+      alignas(16) real rec[8];
+      rec[3] = invr;
+      rec[7] = fc;
 #pragma unroll
       for (int c = 0; c < 3; c++) {
         const real u = d[c] * invr;
         A.der2b[row3 + c * nr + rank] = dD * u;
         A.der3bsupp[row3 + c * nr + rank] = dfc * u;
-        s_rec[c * nr + rank] = u;
-        s_rec[(4 + c) * nr + rank] = dfc * u;
+        rec[c] = u;
+        rec[4 + c] = dfc * u;
         if (A.unit) A.unit[(atom * 4 + c) * nr + rank] = u;
       }
+#pragma unroll
+      for (int q = 0; q < REC_P; q++) s_rec[q * nr + rank] = *(const rec_t*)(rec + q * REC_N);
     } else {
       if (A.unit) {
 #pragma unroll
@@ -490,48 +508,54 @@ __global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
   real2* d3 = (real2*)A.der3b + atom * 3 * na;
   // Consecutive lanes take consecutive triplets: the stores of a wave are whole cache lines.  (Four consecutive
   // triplets per thread with one index decode was measured: fewer instructions, but the strided stores made the
-  // kernel a third slower.)
+  // kernel a third slower.)  Row bases are workgroup-uniform and element offsets unsigned 32-bit byte counts, so a
+  // store's address is a scalar base plus a vector offset.
+  char* angp = (char*)ang;
+  char* im3p = (char*)im3;
+  char* d3p0 = (char*)d3;
+  char* d3p1 = (char*)(d3 + na);
+  char* d3p2 = (char*)(d3 + 2 * (size_t)na);
+  for (unsigned nn = tid; nn < (unsigned)ntr; nn += 256u) {
+    int j, k;
+    tri_decode((int)nn, m, j, k);
+    alignas(16) real rj[8];
+    alignas(16) real rk[8];
+#pragma unroll
+    for (int q = 0; q < REC_P; q++) {
+      *(rec_t*)(rj + q * REC_N) = s_rec[q * nr + j];
+      *(rec_t*)(rk + q * REC_N) = s_rec[q * nr + k];
+    }
+    const real uj0 = rj[0], uj1 = rj[1], uj2 = rj[2];
+    const real uk0 = rk[0], uk1 = rk[1], uk2 = rk[2];
+    const real cs = uj0 * uk0 + uj1 * uk1 + uj2 * uk2;
+    const real fj = rj[7], fk = rk[7];
+    const real half = real(0.5) * (cs + real(1));
+    const real ff = fj * fk;
+    const real aj = real(0.5) * rj[3] * ff, ak = real(0.5) * rk[3] * ff;
+    const real hk = half * fk, hj = half * fj;
+    const unsigned o1 = nn * (unsigned)sizeof(real), o2 = nn * (unsigned)sizeof(real2);
+    *(real*)(angp + o1) = half * ff;
+    *(int2*)(im3p + nn * 8u) = make_int2(s_j[j], s_j[k]);
+    real2 o;
+    o.x = aj * (uk0 - cs * uj0) + hk * rj[4];
+    o.y = ak * (uj0 - cs * uk0) + hj * rk[4];
+    *(real2*)(d3p0 + o2) = o;
+    o.x = aj * (uk1 - cs * uj1) + hk * rj[5];
+    o.y = ak * (uj1 - cs * uk1) + hj * rk[5];
+    *(real2*)(d3p1 + o2) = o;
+    o.x = aj * (uk2 - cs * uj2) + hk * rj[6];
+    o.y = ak * (uj2 - cs * uk2) + hj * rk[6];
+    *(real2*)(d3p2 + o2) = o;
+  }
   // angdescr and intmap3b are written over the whole row (the reference zeroes both tensors before its kernels
   // run, STAF/src/descriptor_builder/reforce.cc:357-358,385-386); der3b beyond the triplets only on request
-  for (int nn = tid; nn < na; nn += blockDim.x) {
-    if (nn < ntr) {
-      int j, k;
-      tri_decode(nn, m, j, k);
-      real rj[8], rk[8];
-#pragma unroll
-      for (int c = 0; c < 8; c++) { rj[c] = s_rec[c * nr + j]; rk[c] = s_rec[c * nr + k]; }
-      const real uj0 = rj[0], uj1 = rj[1], uj2 = rj[2];
-      const real uk0 = rk[0], uk1 = rk[1], uk2 = rk[2];
-      const real cs = uj0 * uk0 + uj1 * uk1 + uj2 * uk2;
-      const real fj = rj[7], fk = rk[7];
-      const real half = real(0.5) * (cs + real(1));
-      const real ff = fj * fk;
-      const real aj = real(0.5) * rj[3] * ff, ak = real(0.5) * rk[3] * ff;
-      const real hk = half * fk, hj = half * fj;
-      ang[nn] = half * ff;
-      im3[nn] = make_int2(s_j[j], s_j[k]);
-      real2 o;
-      o.x = aj * (uk0 - cs * uj0) + hk * rj[4];
-      o.y = ak * (uj0 - cs * uk0) + hj * rk[4];
-      d3[nn] = o;
-      o.x = aj * (uk1 - cs * uj1) + hk * rj[5];
-      o.y = ak * (uj1 - cs * uk1) + hj * rk[5];
-      d3[na + nn] = o;
-      o.x = aj * (uk2 - cs * uj2) + hk * rj[6];
-      o.y = ak * (uj2 - cs * uk2) + hj * rk[6];
-      d3[2 * na + nn] = o;
-    } else {
-      ang[nn] = 0;
-      im3[nn] = make_int2(0, 0);
-      if (A.zero_padding) {
-        real2 z;
-        z.x = 0;
-        z.y = 0;
-        d3[nn] = z;
-        d3[na + nn] = z;
-        d3[2 * na + nn] = z;
-      }
-    }
+  const unsigned npad = (unsigned)(na - ntr);
+  zero_fill(angp + (size_t)ntr * sizeof(real), npad * (unsigned)sizeof(real), tid);
+  zero_fill(im3p + (size_t)ntr * 8, npad * 8u, tid);
+  if (A.zero_padding) {
+    zero_fill(d3p0 + (size_t)ntr * sizeof(real2), npad * (unsigned)sizeof(real2), tid);
+    zero_fill(d3p1 + (size_t)ntr * sizeof(real2), npad * (unsigned)sizeof(real2), tid);
+    zero_fill(d3p2 + (size_t)ntr * sizeof(real2), npad * (unsigned)sizeof(real2), tid);
   }
   PHASE_MARK(4);
   PHASE_CLOCK_END();
