@@ -89,6 +89,21 @@ __device__ inline void group_slots_by_type(int m, int nt, const int* stp, int* l
   if (lane == 0) off[nt] = base;
 }
 
+// The same for m <= 64 with the species of slot `lane` in a register (t_mine; anything for lane >= m): no memory
+// is read, so the wave that loaded the species needs no barrier before it groups.
+__device__ inline void group_slots_by_type_reg(int m, int nt, int t_mine, int* lst, int* off) {
+  const int lane = lane_id();
+  int base = 0;
+  for (int t = 0; t < nt; t++) {
+    if (lane == 0) off[t] = base;
+    const bool on = lane < m && t_mine == t;
+    const unsigned long long mask = __ballot(on);
+    if (on) lst[base + __popcll(mask & ((1ull << lane) - 1ull))] = lane;
+    base += __popcll(mask);
+  }
+  if (lane == 0) off[nt] = base;
+}
+
 // Class (ta,tb) pair index q -> slots (j<k) and storage index nn.
 // na_ = population of ta, nb_ = population of tb; la/lb the two slot lists.
 __device__ inline void class_pair(int q, bool same, int nb_, const int* la, const int* lb, int m, int& j, int& k,

@@ -27,6 +27,8 @@
 //     MODE 2 the contraction U of der3b with dL/dF), so tensors laid out by
 //     the storage index nn are read exactly once.
 #pragma once
+#include <type_traits>
+
 #include "staf_tile.hpp"
 
 namespace staf {
@@ -39,9 +41,9 @@ constexpr int TRI_SUBS = TRI_BLOCK / TRI_CAP;
 template <typename real, int MODE>
 struct TriCfg {
   static constexpr int QB = 512;   // triplets staged per block
-  // waves per SIMD the register allocation is held to: the double-precision force gradient would otherwise come
-  // out two registers above the 128 that let four workgroups share a CU
-  static constexpr int MIN_WAVES = (MODE == 2 && sizeof(real) == 8) ? 4 : 1;
+  // waves per SIMD the register allocation is held to: without a bound the allocation comes out a few registers
+  // above the next occupancy step (the fused double-precision fingerprint kernel is held to four)
+  static constexpr int MIN_WAVES = sizeof(real) == 8 ? (MODE == 0 ? 5 : 4) : (MODE == 0 ? 8 : MODE == 1 ? 7 : 5);
 };
 constexpr int TRI_GRID_MAX = 2048;  // workgroups of the persistent gradient modes (one partial row each)
 
@@ -142,7 +144,8 @@ struct TriLds {
 // the slots' unit vectors and cutoff values, T = 1/2 (u_j . u_k + 1) fc_j fc_k
 // (DescriptorsAngular_kernel, STAF/src/descriptor_builder/reforce.cu.cc:195-212), so no na-wide tensor exists.
 template <typename real, int MODE, bool FUSED = false>
-__global__ __launch_bounds__(TRI_BLOCK, (TriCfg<real, MODE>::MIN_WAVES)) void tri_reduce_kernel(TriArgs<real> A) {
+__global__ __launch_bounds__(TRI_BLOCK, ((FUSED && sizeof(real) == 8) ? 4 : TriCfg<real, MODE>::MIN_WAVES)) void
+tri_reduce_kernel(TriArgs<real> A) {
   static_assert(!FUSED || MODE == 0, "only the fingerprint mode rebuilds T");
   using real2 = typename Vec2<real>::type;
   using HE = HotExp<real>;
@@ -176,6 +179,29 @@ __global__ __launch_bounds__(TRI_BLOCK, (TriCfg<real, MODE>::MIN_WAVES)) void tr
   const int tid = threadIdx.x;
   const int lane = tid & (WAVE - 1), wave = tid / WAVE;
   const int ia = tid & (TRI_CAP - 1), sub = tid / TRI_CAP;
+  // The reads of the workgroup's first centre that need no other read's result (triplet count, neighbour index and
+  // descriptor values of slot tid) are issued ahead of everything else, together with the parameter rows: a centre
+  // then waits for two rounds of global reads (these, and what the neighbour index addresses) instead of four.
+  // Slots are read up to nr whatever the count: rows are nr long.
+  int m0, nj0 = 0;
+  real d0 = 0, gr0[3] = {0, 0, 0}, un0[3] = {0, 0, 0};
+  {
+    const int b0 = blockIdx.x / A.Nl, p0 = blockIdx.x - b0 * A.Nl;
+    const size_t row0 = (size_t)b0 * A.ld + p0;
+    m0 = A.numtriplet[row0];
+    if (tid < nr) {
+      nj0 = A.im2[row0 * (nr + 1) + 1 + tid];
+      d0 = A.Dsup[row0 * nr + tid];
+      if (MODE == 2) {
+#pragma unroll
+        for (int c = 0; c < 3; c++) gr0[c] = A.dDsup[row0 * 3 * nr + c * nr + tid];
+      }
+      if (FUSED) {
+#pragma unroll
+        for (int c = 0; c < 3; c++) un0[c] = A.unit[(row0 * 4 + c) * nr + tid];
+      }
+    }
+  }
   tab.build(A.alpha3b, A.emb3b);
   if (MODE != 0)
     for (int q = tid; q < nacc; q += TRI_BLOCK) accw[q] = 0;
@@ -205,23 +231,33 @@ __global__ __launch_bounds__(TRI_BLOCK, (TriCfg<real, MODE>::MIN_WAVES)) void tr
   __syncthreads();
 
   const int total = A.nf * A.Nl;
-  for (int atom = blockIdx.x; atom < total; atom += gridDim.x) {
+  // Per-centre set-up: slot data into LDS.  The first centre takes what was read at the kernel's start (a separate
+  // copy of the code, so that those registers are free afterwards); later centres of a persistent workgroup read here.
+  int m = 0, t_mine = -1;   // neighbours inside the angular cutoff; species of slot tid
+  const real* Trow = nullptr;
+  const real2* d3 = nullptr;
+  auto centre_setup = [&](int atom, auto early_c) {
     const int b = atom / A.Nl, p = atom - b * A.Nl;
     const size_t rowAtom = (size_t)b * A.ld + p;
     const int* im = A.im2 + rowAtom * (nr + 1);
-    int m = A.numtriplet[rowAtom];
+    constexpr bool early = decltype(early_c)::value;   // the centre whose first reads were issued at the kernel's start
+    m = early ? m0 : A.numtriplet[rowAtom];
     if (m > nr) m = nr;
-    const real* Trow = A.Tang + rowAtom * na;
-    const real2* d3 = (const real2*)A.d3b + rowAtom * 3 * na;
+    Trow = A.Tang + rowAtom * na;
+    d3 = (const real2*)A.d3b + rowAtom * 3 * na;
     // ---- per-atom slot data
+    t_mine = -1;
     for (int s = tid; s < m; s += TRI_BLOCK) {
-      sD[s] = A.Dsup[rowAtom * nr + s];
+      const bool have = early && s == tid;
+      sD[s] = have ? d0 : A.Dsup[rowAtom * nr + s];
       if (FUSED) {
 #pragma unroll
-        for (int c = 0; c < 3; c++) sUn[c * nr + s] = A.unit[(rowAtom * 4 + c) * nr + s];
+        for (int c = 0; c < 3; c++) sUn[c * nr + s] = have ? un0[c] : A.unit[(rowAtom * 4 + c) * nr + s];
       }
-      const int nj = im[1 + s];
-      stp[s] = A.type_map[nj];
+      const int nj = have ? nj0 : im[1 + s];
+      const int t_s = A.type_map[nj];
+      stp[s] = t_s;
+      if (s == tid) t_mine = t_s;
       if (MODE == 2) {
         const real* Qj = A.Q + ((size_t)b * A.N + nj) * 3;
         const real* Qi = A.Q + ((size_t)b * A.N + p + shift) * 3;
@@ -237,16 +273,27 @@ __global__ __launch_bounds__(TRI_BLOCK, (TriCfg<real, MODE>::MIN_WAVES)) void tr
           q2 -= Wg[6] * r[0] + Wg[7] * r[1] + Wg[8] * r[2];
         }
         const real* gr = A.dDsup + rowAtom * 3 * nr + s;
+        const real g0 = have ? gr0[0] : gr[0], g1 = have ? gr0[1] : gr[nr], g2 = have ? gr0[2] : gr[2 * nr];
         sQ[3 * s] = q0; sQ[3 * s + 1] = q1; sQ[3 * s + 2] = q2;
-        sV[s] = q0 * gr[0] + q1 * gr[nr] + q2 * gr[2 * nr];
+        sV[s] = q0 * g0 + q1 * g1 + q2 * g2;
       }
     }
     for (int a = tid; a < Aa; a += TRI_BLOCK)
       if (MODE != 0) sP[a] = A.P[(size_t)atom * Aa + a];
     for (int q = tid; q < TRI_WAVES * Aa; q += TRI_BLOCK) outw[q] = 0;
-    __syncthreads();
-    if (tid < WAVE) group_slots_by_type(m, nt, stp, lst, off);
-    __syncthreads();
+  };
+  int atom = blockIdx.x;
+  centre_setup(atom, std::true_type{});
+  while (true) {
+    if (m <= WAVE) {
+      // all slots are in the first wave's registers: it groups them by species before the barrier
+      if (tid < WAVE) group_slots_by_type_reg(m, nt, t_mine, lst, off);
+      __syncthreads();
+    } else {
+      __syncthreads();
+      if (tid < WAVE) group_slots_by_type(m, nt, stp, lst, off);
+      __syncthreads();
+    }
 
     bool first = true;
     for (int ta = 0; ta < nt; ta++) {
@@ -438,6 +485,9 @@ __global__ __launch_bounds__(TRI_BLOCK, (TriCfg<real, MODE>::MIN_WAVES)) void tr
         A.out[(size_t)atom * Aa + a] = s;
       }
     __syncthreads();
+    atom += gridDim.x;
+    if (atom >= total) break;
+    centre_setup(atom, std::false_type{});
   }
   if (MODE != 0) {
     for (int q = tid; q < nacc; q += TRI_BLOCK) A.partial[(size_t)blockIdx.x * nacc + q] = accw[q];
