@@ -30,8 +30,8 @@ REPEATS = 5          # timed blocks of --steps steps each; the median block is r
 PROFILES = os.path.join(ROOT, "profiles")
 # bench.py's kernel names (the library's timing names) -> the names the profiler prints
 PROFILED_NAME = {
-    ("force3_kernel", "f32"): "staf::force3_kernel<float, false>",
-    ("force3_kernel", "f64"): "staf::force3_kernel<double, false>",
+    ("force3_kernel", "f32"): "staf::force3_kernel<float, false, 8>",
+    ("force3_kernel", "f64"): "staf::force3_kernel<double, false, 4>",
     ("gradforce3_kernel", "f32"): "staf::tri_reduce_kernel<float, 2, false>",
     ("gradforce3_kernel", "f64"): "staf::tri_reduce_kernel<double, 2, false>",
     ("af3_kernel", "f32"): "staf::tri_reduce_kernel<float, 0, false>",
