@@ -215,7 +215,7 @@ def main():
                     help="copy per-species tensors like tf.split instead of passing views")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build measures one GPU only (frames are independent; see DESIGN.md for sharding); "
+        print("bench.py: this build measures one GPU only (frames are independent: a data-parallel run gives each GPU its share of the frame batch); "
               "run with --gpus 1", file=sys.stderr)
         sys.exit(2)
     import torch

@@ -197,7 +197,7 @@ def test_compute_before_construct_other_precision():
 
 
 def test_full_size_properties(oracle):
-    """BASELINE config 2 at full size (768 atoms, 4 frames, fp32): size-independent checks.
+    """The benchmark's headline configuration at full size (768 atoms, 4 frames, fp32): size-independent checks.
     Newton's third law (sum of forces = 0 per frame), linearity of the force ops in G, and the exact
     adjoint relation between the force op and its gradient: sum(Q * F(G)) == sum(G * dG(Q))."""
     import torch
@@ -635,22 +635,22 @@ def test_default_options_write_the_reference_padding(oracle, dtype):
 
 
 def test_config2_full_size_fp32(oracle):
-    """BASELINE config 2 as benchmarked: 768 atoms, 4 frames, fp32, every op against the oracle."""
+    """The headline configuration as benchmarked: 768 atoms, 4 frames, fp32, every op against the oracle."""
     print(_run_case(oracle, _synth("water768_f32"), np.float32))
 
 
 def test_config3_full_size_fp64(oracle):
-    """BASELINE config 3: 768 atoms, 4 frames, fp64, full training step (all eight ops)."""
+    """The double-precision training configuration: 768 atoms, 4 frames, fp64, full training step (all eight ops)."""
     print(_run_case(oracle, _synth("water768_f64"), np.float64))
 
 
 def test_config4_train8_fp32(oracle):
-    """BASELINE config 4: eight 768-atom frames, fp32, all eight ops of a training step."""
+    """The eight-frame training configuration: eight 768-atom frames, fp32, all eight ops of a training step."""
     print(_run_case(oracle, _synth("water768_train8"), np.float32))
 
 
 def test_config5_water6144_fp64(oracle):
-    """BASELINE config 5: 6144 atoms, one frame, fp64; above the library's default threshold, so the neighbours are
+    """The large-box configuration: 6144 atoms, one frame, fp64; above the library's default threshold, so the neighbours are
     found through the cell list (8 x 8 x 8 cells) while the oracle tests all pairs."""
     from alphanesgpu_amd import ops
     ops.descriptor_cell_threshold(2048)
