@@ -68,12 +68,13 @@ struct Force3Cfg {
   static constexpr int CAPP = CAP + 1;                      // table row pitch in entries
   // der3b rows requested one sweep ahead and held in registers across the channel loop: measured, no gain in
   // fp32 (the kernel is bound by vector-ALU issue) and slower in fp64 (a third of the resident waves lost)
-  // measured and not faster either: the rows of a wave's first pass requested ahead of the channel loop, rolling
-  // requests in single precision, one element of every 128-byte line of the rows requested at the kernel's start
-  static constexpr bool EARLY1 = false;
+  // (measured and not faster either: the rows of a wave's first pass alone requested ahead of the channel loop,
+  // rolling requests in single precision, one element of every 128-byte line of the rows requested at the kernel's
+  // start to have the lines in the L2)
   static constexpr bool PREFETCH = false;
-  // waves per SIMD the register allocation is held to (what the LDS footprint of the reference's sizes admits:
-  // six workgroups per CU in single precision, four in double)
+  // waves per SIMD the register allocation is held to: with four waves per workgroup what the LDS footprint of the
+  // reference's sizes admits (six workgroups per CU in single precision, four in double), with eight waves the
+  // hardware's eight waves per SIMD in single precision
   static constexpr int MIN_WAVES = NW == 8 ? (sizeof(real) == 8 ? 6 : 8) : (sizeof(real) == 8 ? 4 : 6);
   __host__ __device__ static bool fits(int nr, int nt) { return nr <= 255 && nt <= NT_MAX; }   // slots packed in 8 bits
   __host__ __device__ static int pitch(int Aa) { return (Aa + 3) & ~3; }   // parameter row pitch (channels)
@@ -266,12 +267,6 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
       }
     }
     PHASE_MARK(1);
-    if constexpr (ROLL && L::EARLY1) {   // der3b rows of the wave's first pass: on their way during the channel loop
-      const int nn = w0 + wave * WAVE + lane;
-#pragma unroll
-      for (int c = 0; c < 3; c++) dn[0][c] = d3[c * na + (nn < nlast ? nn : nlast)];
-    }
-
     for (int c0 = 0; c0 < maxact; c0 += CAP) {
       const int nch = (maxact - c0) < CAP ? (maxact - c0) : CAP;
       const int nch2 = (nch + 1) & ~1;            // the channel loop runs in pairs (c0 + nch2 <= Ap)
@@ -360,7 +355,7 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
     // computed on row 0: their products are forced to 0.
     if constexpr (FUSED) {
       // nothing to load: a pass's Jacobian is rebuilt from the slot tile where it is used
-    } else if constexpr (!L::PREFETCH && !(ROLL && L::EARLY1)) {
+    } else if constexpr (!L::PREFETCH) {
 #pragma unroll
       for (int p = 0; p < (ROLL ? 1 : NP); p++) {
         const int nn = w0 + (p * NW + wave) * WAVE + lane;
