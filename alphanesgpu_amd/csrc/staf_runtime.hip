@@ -216,6 +216,9 @@ static int fetch_status(DeviceState* st, hipStream_t stream) {
 int finish_op(DeviceState* st, hipStream_t stream) {
   if (hipGetLastError() != hipSuccess) return STAF_E_HIP;
   if (!sync_errors_enabled()) return STAF_OK;
+  // A stream that is being captured cannot be waited for (and the copy and the clear would become nodes of the
+  // graph): the condition stays in the status word for staf_ops_poll_status after a replay.
+  if (stream_is_capturing(stream)) return STAF_OK;
   return fetch_status(st, stream);
 }
 

@@ -513,6 +513,43 @@ def test_hip_graph_replay_with_two_streams_matches_eager():
 
 
 @pytest.mark.gpu
+def test_capture_with_synchronising_error_returns_left_on():
+    """With the default error mode (every op waits for its stream to return a device-detected condition) an op that is
+    being captured must not wait: the capture succeeds, the replay gives the eager result, and the condition is read
+    with poll_status afterwards."""
+    import torch
+    from alphanesgpu_amd import ops, synth
+    dev = torch.device("cuda:0")
+    batch = synth.water_batch("water96")
+    nr, na = synth.NR, synth.NA
+    nf, N = batch["nf"], batch["N"]
+    T = lambda a: torch.as_tensor(np.ascontiguousarray(a)).to(dev)
+    pos, box, tm = T(batch["pos"]), T(batch["box"]), T(batch["type_map"])
+    p = {k: T(v) for k, v in synth.fingerprint_params(dtype=batch["dtype"])[0].items()}
+    ops.construct_descriptors_light(synth.RC, nr, na, N, box, synth.RS, synth.RA, nf, dtype=torch.float64)
+    ops.set_sync_errors(True)
+
+    def step(out=None):
+        d = ops.compute_descriptors_light(pos, box, out=out)
+        return d, ops.compute_sort_proj(d[0], d[3], p["alpha2b"], p["emb2b"], tm)
+
+    d_want, af_want = step()
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        d_held, _ = step()              # the stream's work areas exist before the capture
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s):
+        _, af_held = step(out=d_held)
+    for rep in range(2):
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(af_held, af_want), f"replay {rep}"
+        assert torch.equal(d_held[3], d_want[3])
+    ops.poll_status()
+
+
+@pytest.mark.gpu
 def test_random_configurations(oracle):
     """Twelve seeded random configurations through every op: 1-3 species with 1-13 atoms each (parameter rows and
     classes of every shape), 1-3 frames, orthorhombic and triclinic boxes with the cluster shifted far outside the
