@@ -78,8 +78,10 @@ const char* staf_ops_version(void);
 
 /* Error reporting of conditions only the GPU can detect (neighbour-buffer overflow,
  * scatter overflow).  mode 1 (default, reference behaviour): the call that can hit
- * the condition synchronises its stream and returns the code.  mode 0: nothing
- * synchronises; conditions accumulate in a device word read by staf_ops_poll_status. */
+ * the condition synchronises its stream and returns the code -- except on a stream
+ * that is being captured into a graph, which cannot be waited for: there the call
+ * behaves as in mode 0.  mode 0: nothing synchronises; conditions accumulate in a
+ * device word (one per device, shared by its streams) read by staf_ops_poll_status. */
 void staf_ops_set_sync_errors(int mode);
 
 /* Synchronises `stream`, returns the accumulated device-side status (0 or a
