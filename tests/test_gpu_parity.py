@@ -591,6 +591,50 @@ def test_random_configurations(oracle):
 
 
 @pytest.mark.gpu
+def test_random_dense_clusters(oracle):
+    """Eleven seeded dense clusters through every op: 1-3 species with 8-33 atoms each inside a cutoff of 5-6.5, so
+    that an atom has up to ~85 neighbours inside the angular cutoff -- several sweeps of the 3-body force kernel, more
+    than 64 slots to group by species, up to 19 channels per species pair (more than one table chunk), angular
+    buffers that cut the triplet list, either precision, block or dense embeddings."""
+    rng = np.random.default_rng(7)
+    seen_wide = seen_chunks = False
+    for case in range(11):
+        nt = int(rng.integers(1, 4))
+        tip = [int(x) for x in rng.integers(8, 34, nt)]
+        n = sum(tip)
+        nf = int(rng.integers(1, 3))
+        L = float(rng.uniform(14.0, 18.0))
+        spread = float(rng.uniform(2.6, 3.6))
+        pos, box = np.zeros((nf, 3 * n)), np.zeros((nf, 6))
+        for b in range(nf):
+            pts = []
+            while len(pts) < n:
+                c = rng.uniform(-spread, spread, 3)
+                if all(np.linalg.norm(c - q) > 0.75 for q in pts):
+                    pts.append(c)
+            pos[b] = (np.array(pts) + rng.uniform(-5, 5, 3)).reshape(-1)
+            box[b] = [L, 0.5, -0.3, L + 0.7, 0.4, L + 1.3]
+        rc = float(rng.uniform(5.0, 6.5))
+        ra = float(rng.uniform(0.8 * rc, rc))
+        rs = float(rng.uniform(0.9, 2.0))
+        nr = n + 2
+        na = int(rng.integers(nr * (nr - 1) // 4, nr * (nr - 1) // 2 + 1))
+        ar = tuple(int(x) for x in rng.integers(1, 7, nt))
+        aa = tuple(int(x) for x in rng.integers(1, 20, nt * (nt + 1) // 2))
+        dtype = np.float64 if rng.random() < 0.5 else np.float32
+        dense = bool(rng.random() < 0.5)
+        seen_wide |= nr > 64
+        seen_chunks |= max(aa) > 16
+        try:
+            _generic_case(oracle, pos, box, tip, dtype, nr=nr, na=na, rc=rc, ra=ra, rs=rs, nt=nt, seed=case + 1,
+                          dense=dense, maps=(ar, aa))
+        except AssertionError as e:
+            raise AssertionError(f"case {case}: nt={nt} tipos={tip} nf={nf} rc={rc:.2f} ra={ra:.2f} rs={rs:.2f} "
+                                 f"nr={nr} na={na} ar={ar} aa={aa} {np.dtype(dtype).name} dense={dense}: {e}") from e
+    assert seen_wide and seen_chunks   # the draws cover what the test is for
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 def test_add_n_is_the_sequential_sum(dtype):
     """ops.add_n (the callers' sum of per-op force arrays) against adding the arrays one after the other: same
