@@ -116,6 +116,54 @@ struct TriArgs {
   int nf, N, Nl, ld, nr, na, Aa, nt;
 };
 
+// A staged triplet: the offsets of its two table rows (16 bits each, in one word), T and -- force gradient -- the
+// contraction U, laid out so that the inner loop takes them with one LDS read (two in the double-precision force
+// gradient, whose LDS budget has no room for padding): every lane of a subset reads the same record.
+//   float,  fingerprint / its gradient: {ab, T}          8 bytes
+//   float,  force gradient:             {ab, T, U, -}   16 bytes
+//   double, fingerprint / its gradient: {ab, -, T}      16 bytes
+//   double, force gradient:             {T, U} 16 bytes in one array, ab in a second one
+template <typename real, int MODE>
+struct TriStage {
+  static constexpr bool SPLIT = MODE == 2 && sizeof(real) == 8;
+  static constexpr int BYTES = SPLIT ? 20 : ((sizeof(real) == 4 && MODE != 2) ? 8 : 16);
+  unsigned char* base;   // 16-byte aligned; SPLIT: QB records of 16 bytes, then QB words
+  int qb;
+  __device__ void put(int qq, unsigned ab, real T, real U) const {
+    if constexpr (SPLIT) {
+      double2 v;
+      v.x = T; v.y = U;
+      ((double2*)base)[qq] = v;
+      ((unsigned*)(base + (size_t)qb * 16))[qq] = ab;
+    } else if constexpr (sizeof(real) == 4 && MODE != 2) {
+      ((uint2*)base)[qq] = make_uint2(ab, __float_as_uint((float)T));
+    } else if constexpr (sizeof(real) == 4) {
+      ((uint4*)base)[qq] = make_uint4(ab, __float_as_uint((float)T), __float_as_uint((float)U), 0u);
+    } else {
+      const unsigned long long t = (unsigned long long)__double_as_longlong((double)T);
+      ((uint4*)base)[qq] = make_uint4(ab, 0u, (unsigned)(t & 0xffffffffull), (unsigned)(t >> 32));
+    }
+  }
+  __device__ void get(int qq, unsigned& ab, real& T, real& U) const {
+    if constexpr (SPLIT) {
+      const double2 v = ((const double2*)base)[qq];
+      T = (real)v.x; U = (real)v.y;
+      ab = ((const unsigned*)(base + (size_t)qb * 16))[qq];
+    } else if constexpr (sizeof(real) == 4 && MODE != 2) {
+      const uint2 v = ((const uint2*)base)[qq];
+      ab = v.x; T = (real)__uint_as_float(v.y); U = 0;
+    } else if constexpr (sizeof(real) == 4) {
+      const uint4 v = ((const uint4*)base)[qq];
+      ab = v.x; T = (real)__uint_as_float(v.y); U = (real)__uint_as_float(v.z);
+    } else {
+      const uint4 v = ((const uint4*)base)[qq];
+      ab = v.x;
+      T = (real)__longlong_as_double((long long)(((unsigned long long)v.w << 32) | v.z));
+      U = 0;
+    }
+  }
+};
+
 template <typename real, int MODE>
 struct TriLds {
   static constexpr int NV = (MODE == 0) ? 1 : (MODE == 1 ? 3 : 4);
@@ -130,12 +178,12 @@ struct TriLds {
     if (MODE != 0) r += (size_t)nsig * Aa * 3;              // parameter-gradient sums of the workgroup
     if (MODE != 0) r += (size_t)TRI_WAVES * TRI_CAP * 3;    // exchange buffer of a pass
     if (MODE == 2) r += (size_t)4 * nr;                     // sV, sQ
-    r += (size_t)QB * (MODE == 2 ? 2 : 1);                  // staged T (and U)
     return r;
   }
   __host__ __device__ static size_t bytes(int nr, int Aa, int nt, bool fused = false) {
     size_t b = chan_table_bytes<real>(2 * nt - 1, Aa) + n_reals(nr, Aa, nt, fused) * sizeof(real);
-    b += (size_t)2 * QB * sizeof(unsigned short) + (size_t)(2 * nr + NT_MAX + 1) * sizeof(int);
+    b += 16 + (size_t)QB * TriStage<real, MODE>::BYTES;     // staged triplets, 16-byte aligned
+    b += (size_t)(2 * nr + NT_MAX + 1) * sizeof(int);
     return (b + 15) & ~(size_t)15;
   }
 };
@@ -168,11 +216,10 @@ tri_reduce_kernel(TriArgs<real> A) {
   real* sV = rp;
   real* sQ = rp + nr;
   if (MODE == 2) rp += (size_t)4 * nr;
-  real* sT = rp; rp += TRI_QB;
-  real* sU = rp; if (MODE == 2) rp += TRI_QB;
-  unsigned short* offA = (unsigned short*)rp;   // [TRI_QB] first table row of the staged triplet, times TRI_CAPP
-  unsigned short* offB = offA + TRI_QB;         // [TRI_QB] second
-  int* lst = (int*)(offB + TRI_QB);
+  TriStage<real, MODE> stage;                   // [TRI_QB] staged triplets
+  stage.base = smem + ((((unsigned char*)rp - smem) + 15) & ~(ptrdiff_t)15);   // an offset into smem, not an integer cast
+  stage.qb = TRI_QB;
+  int* lst = (int*)(stage.base + (size_t)TRI_QB * TriStage<real, MODE>::BYTES);
   int* stp = lst + nr;
   int* off = stp + nr;
 
@@ -353,12 +400,7 @@ tri_reduce_kernel(TriArgs<real> A) {
             const int nq_pad = (nq + TRI_SUBS - 1) & ~(TRI_SUBS - 1);
             if (q0 > 0) __syncthreads();   // previous block consumed
             // ---- stage a block of triplets
-            for (int qq = nq + tid; qq < nq_pad; qq += TRI_BLOCK) {
-              offA[qq] = 0;
-              offB[qq] = 0;
-              sT[qq] = 0;
-              if (MODE == 2) sU[qq] = 0;
-            }
+            for (int qq = nq + tid; qq < nq_pad; qq += TRI_BLOCK) stage.put(qq, 0u, real(0), real(0));
             for (int qq = tid; qq < nq; qq += TRI_BLOCK) {
               const int q = q0 + qq;
               int x, y;
@@ -368,9 +410,8 @@ tri_reduce_kernel(TriArgs<real> A) {
               const int j = s1 < s2 ? s1 : s2, k = s1 < s2 ? s2 : s1;
               const int nn = tri_rowstart(j, m) + k - j - 1;
               const bool ok = nn < na;
-              offA[qq] = (unsigned short)(x * TRI_CAPP);
-              offB[qq] = (unsigned short)((rowB0 + y) * TRI_CAPP);
-              real T = 0;
+              const unsigned ab = (unsigned)(x * TRI_CAPP) | ((unsigned)((rowB0 + y) * TRI_CAPP) << 16);
+              real T = 0, U = 0;
               if (ok) {
                 if constexpr (FUSED) {
                   const real cs = sUn[j] * sUn[k] + sUn[nr + j] * sUn[nr + k] + sUn[2 * nr + j] * sUn[2 * nr + k];
@@ -379,9 +420,7 @@ tri_reduce_kernel(TriArgs<real> A) {
                   T = Trow[nn];
                 }
               }
-              sT[qq] = T;
               if (MODE == 2) {
-                real U = 0;
                 if (ok) {
 #pragma unroll
                   for (int c = 0; c < 3; c++) {
@@ -389,8 +428,8 @@ tri_reduce_kernel(TriArgs<real> A) {
                     U += sQ[3 * j + c] * dv.x + sQ[3 * k + c] * dv.y;
                   }
                 }
-                sU[qq] = U;
               }
+              stage.put(qq, ab, T, U);
             }
             __syncthreads();
             // ---- thread <-> (channel ia, subset sub)
@@ -399,9 +438,11 @@ tri_reduce_kernel(TriArgs<real> A) {
 #pragma unroll 2
               for (int it = 0; it < rounds; it++) {
                 const int qq = sub + it * TRI_SUBS;
-                const real2* r1 = tabE + (unsigned)offA[qq];
-                const real2* r2 = tabE + (unsigned)offB[qq];
-                const real T = sT[qq];
+                unsigned ab;
+                real T, U;
+                stage.get(qq, ab, T, U);
+                const real2* r1 = tabE + (ab & 0xffffu);
+                const real2* r2 = tabE + (ab >> 16);
                 const real2 e1 = r1[ia];
                 const real2 e2 = r2[ia];
                 const real ebt = HE::eval(bes * T);
@@ -418,7 +459,6 @@ tri_reduce_kernel(TriArgs<real> A) {
                 } else {
                   const real2 g1 = r1[TRI_CAP], g2 = r2[TRI_CAP];
                   const real D1 = g1.x, D2 = g2.x, V1 = g1.y, V2 = g2.y;
-                  const real U = sU[qq];
                   // With X1 = sim2 V1 + sim1 V2, X2 = sim1 V1 + sim2 V2, W = a1 X1 + a2 X2 (the factor 1/2 of both
                   // weights is applied once per channel at the end):
                   //   d/dG      : hU ss + hT W                         hT = e^{bT} T,  hU = e^{bT} (1 + bT) U
