@@ -274,13 +274,16 @@ struct Transpose {
   unsigned long long stamp = 0;        // last use, for replacement
 };
 constexpr int TRANSPOSE_SLOTS = 8;     // descriptor output tensors whose transposes are kept at a time
+constexpr int STATUS_WORDS = 64;       // error words of a device, one per stream
 
 struct DeviceState {
   int device = -1;
-  // One word per device, shared by every stream and model that uses the device: kernels OR their error bits into it,
-  // and a poll (or the synchronising return of an op) reports and clears whatever any of them raised.
-  int* status_d = nullptr;
-  int* status_h = nullptr;   // pinned host mirror
+  // Error words kernels OR their bits into: one per stream that has used the device (STATUS_WORDS of them, allocated
+  // with the state; later streams share the last one).  The synchronising return of an op reports and clears the word
+  // of the op's own stream, so a condition goes to the caller that raised it; a poll reports and clears all of them.
+  int* status_d = nullptr;   // [STATUS_WORDS]
+  int* status_h = nullptr;   // pinned host mirror, [STATUS_WORDS]
+  std::unordered_map<hipStream_t, int> status_slot;
   std::unordered_map<hipStream_t, StreamWork> work;
   Transpose transposes[TRANSPOSE_SLOTS];
   std::vector<void*> retired;   // outgrown blocks, freed by staf_ops_release
@@ -293,6 +296,8 @@ DeviceState* device_state(hipStream_t stream);
 // True while `stream` is being captured into a graph: memory may then neither be freed nor allocated, and a fill
 // launched to initialise a fresh block would become part of the graph.
 bool stream_is_capturing(hipStream_t stream);
+// The error word of `stream` on this device (see DeviceState::status_d).
+int* status_word(DeviceState* st, hipStream_t stream);
 // Both grow on demand and never shrink; under capture a request that does not fit what the stream already holds
 // returns null (the caller reports STAF_E_CAPTURE) instead of freeing and allocating.
 void* scratch_reserve(DeviceState* st, hipStream_t stream, size_t bytes);

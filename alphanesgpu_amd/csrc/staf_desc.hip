@@ -674,7 +674,7 @@ int desc_launch(const DescConfig<real>& c, const real* pos, const real* box, int
   A.raddescr = raddescr; A.angdescr = angdescr; A.des3bsupp = des3bsupp; A.intmap2b = intmap2b;
   A.intmap3b = intmap3b; A.der2b = der2b; A.der3b = der3b; A.der3bsupp = der3bsupp; A.numtriplet = numtriplet;
   A.unit = unit; A.angular = angular ? 1 : 0;
-  A.status = st->status_d;
+  A.status = status_word(st, stream);
   if (N >= (1 << (31 - KEY_SLOT_BITS))) return STAF_E_LIMIT;
   // The library's own search finds j from i exactly when it finds i from j (the squared distance is computed from
   // the negated difference vector: same bits), so the map it writes needs no transposing; a caller's list may name

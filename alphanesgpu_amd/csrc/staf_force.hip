@@ -443,7 +443,7 @@ static int force_transpose(DeviceState* st, const int* im2, int nf, int N, int N
   if (!bucket_reserve(st, (size_t)nf * N, cap, stream, tr)) return reserve_failure(stream);
   const int total = nf * Nl * nr;
   hipLaunchKernelGGL(transpose_push_kernel, dim3((total + TR_BLOCK - 1) / TR_BLOCK), dim3(TR_BLOCK), 0, stream, im2,
-                     tr->build_cnt, tr->keys, tr->cap, st->status_d, nf, N, Nl, ld, nr);
+                     tr->build_cnt, tr->keys, tr->cap, status_word(st, stream), nf, N, Nl, ld, nr);
   launch_transpose_sort(*tr, nf * N, stream);
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }
@@ -485,7 +485,7 @@ int force_doublets(const real* G, const real* D, const real* dD, const int* im2,
   if (rc) return rc;
   A.G = G; A.D = D; A.dD = dD; A.im2 = im2; A.alpha2b = alpha2b; A.emb2b = emb2b; A.type_map = type_map;
   A.tipos = tipos; A.actual_type = actual_type; A.force = force; A.vpart = nullptr; A.pos = pos; A.box = box;
-  A.status = st->status_d; A.skip_pbc = skip_pbc;
+  A.status = status_word(st, stream); A.skip_pbc = skip_pbc;
   A.host_shift = cached ? A.tr.key_shift : -1;
   A.nf = nf; A.N = N; A.Nl = Nl; A.ld = ld; A.nr = nr; A.Ar = Ar; A.nt = nt;
   if (virial) {
@@ -572,7 +572,7 @@ int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* d
     KernelTimer kt_("gather_kernel", stream);
     const int recv = nf * N;
     hipLaunchKernelGGL(gather_kernel<real>, dim3((recv + F_WAVES - 1) / F_WAVES), dim3(F_BLOCK), 0, stream,
-                       (const real*)gslot, (const real*)self, im2, tr, tipos, actual_type, force, st->status_d,
+                       (const real*)gslot, (const real*)self, im2, tr, tipos, actual_type, force, status_word(st, stream),
                        cached ? tr.key_shift : -1, nf, N, Nl, ld, nr);
   }
   return finish_op(st, stream);

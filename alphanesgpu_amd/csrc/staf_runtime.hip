@@ -41,14 +41,26 @@ DeviceState* device_state(hipStream_t stream) {
   if (stream_is_capturing(stream)) return nullptr;
   auto st = std::unique_ptr<DeviceState>(new DeviceState());
   st->device = dev;
-  if (hipMalloc((void**)&st->status_d, sizeof(int)) != hipSuccess) return nullptr;
+  if (hipMalloc((void**)&st->status_d, STATUS_WORDS * sizeof(int)) != hipSuccess) return nullptr;
   // the clear runs on the legacy default stream: wait for it, callers' streams need not be ordered after that one
-  if (hipMemset(st->status_d, 0, sizeof(int)) != hipSuccess || hipDeviceSynchronize() != hipSuccess) return nullptr;
-  if (hipHostMalloc((void**)&st->status_h, sizeof(int), hipHostMallocDefault) != hipSuccess) return nullptr;
-  *st->status_h = 0;
+  if (hipMemset(st->status_d, 0, STATUS_WORDS * sizeof(int)) != hipSuccess || hipDeviceSynchronize() != hipSuccess)
+    return nullptr;
+  if (hipHostMalloc((void**)&st->status_h, STATUS_WORDS * sizeof(int), hipHostMallocDefault) != hipSuccess)
+    return nullptr;
+  for (int w = 0; w < STATUS_WORDS; w++) st->status_h[w] = 0;
   DeviceState* raw = st.get();
   g_state.emplace(dev, std::move(st));
   return raw;
+}
+
+int* status_word(DeviceState* st, hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  auto it = st->status_slot.find(stream);
+  if (it == st->status_slot.end()) {
+    const int n = (int)st->status_slot.size();
+    it = st->status_slot.emplace(stream, n < STATUS_WORDS ? n : STATUS_WORDS - 1).first;
+  }
+  return st->status_d + it->second;
 }
 
 static StreamWork* stream_work(DeviceState* st, hipStream_t stream) {
@@ -201,13 +213,20 @@ static int decode_status(int bits) {
   return STAF_OK;
 }
 
-static int fetch_status(DeviceState* st, hipStream_t stream) {
-  if (hipMemcpyAsync(st->status_h, st->status_d, sizeof(int), hipMemcpyDeviceToHost, stream) != hipSuccess)
-    return STAF_E_HIP;
+// Reads and clears, after waiting for `stream`, the stream's own error word (all = false) or every word of the
+// device (all = true: the poll, whose caller has waited for the other streams itself).
+static int fetch_status(DeviceState* st, hipStream_t stream, bool all) {
+  static std::mutex mirror_mu;   // one pinned mirror per device
+  std::lock_guard<std::mutex> lock(mirror_mu);
+  int* word = all ? st->status_d : status_word(st, stream);
+  const int nw = all ? STATUS_WORDS : 1;
+  int* host = st->status_h + (word - st->status_d);
+  if (hipMemcpyAsync(host, word, nw * sizeof(int), hipMemcpyDeviceToHost, stream) != hipSuccess) return STAF_E_HIP;
   if (hipStreamSynchronize(stream) != hipSuccess) return STAF_E_HIP;
-  int bits = *st->status_h;
+  int bits = 0;
+  for (int w = 0; w < nw; w++) bits |= host[w];
   if (bits) {
-    if (hipMemsetAsync(st->status_d, 0, sizeof(int), stream) != hipSuccess) return STAF_E_HIP;
+    if (hipMemsetAsync(word, 0, nw * sizeof(int), stream) != hipSuccess) return STAF_E_HIP;
     if (hipStreamSynchronize(stream) != hipSuccess) return STAF_E_HIP;
   }
   return decode_status(bits);
@@ -219,7 +238,7 @@ int finish_op(DeviceState* st, hipStream_t stream) {
   // A stream that is being captured cannot be waited for (and the copy and the clear would become nodes of the
   // graph): the condition stays in the status word for staf_ops_poll_status after a replay.
   if (stream_is_capturing(stream)) return STAF_OK;
-  return fetch_status(st, stream);
+  return fetch_status(st, stream, false);
 }
 
 }  // namespace staf
@@ -233,7 +252,7 @@ void staf_ops_set_sync_errors(int mode) { staf::g_sync_errors = mode ? 1 : 0; }
 int staf_ops_poll_status(void* stream) {
   staf::DeviceState* st = staf::device_state((hipStream_t)stream);
   if (!st) return staf::reserve_failure((hipStream_t)stream);
-  return staf::fetch_status(st, (hipStream_t)stream);
+  return staf::fetch_status(st, (hipStream_t)stream, true);
 }
 
 void staf_ops_kernel_timing(int enable) { staf::g_kernel_timing = enable ? 1 : 0; }

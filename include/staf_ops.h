@@ -32,8 +32,10 @@
  *     zeros; the other pointers are not read.
  *   - state is per device.  Work areas are kept per stream, so calls issued on
  *     different streams of a device may overlap; calls on one stream are ordered.
- *     The error word of staf_ops_poll_status is one per device, shared by all
- *     streams: a poll reports what any of them raised.
+ *     Error words are per stream too (the first 63 streams that use a device
+ *     get their own, later ones share one): the synchronising return of an op
+ *     reports what its own stream raised; staf_ops_poll_status reports what
+ *     any stream of the device raised.
  *   - the force ops are owner-computes: every atom collects the pair forces of
  *     the slots that list it.  The descriptor op remembers, by address, the
  *     intmap2b tensors it has written (the 8 most recent per device); such a
@@ -80,12 +82,14 @@ const char* staf_ops_version(void);
  * scatter overflow).  mode 1 (default, reference behaviour): the call that can hit
  * the condition synchronises its stream and returns the code -- except on a stream
  * that is being captured into a graph, which cannot be waited for: there the call
- * behaves as in mode 0.  mode 0: nothing synchronises; conditions accumulate in a
- * device word (one per device, shared by its streams) read by staf_ops_poll_status. */
+ * behaves as in mode 0.  mode 0: nothing synchronises; conditions accumulate in
+ * the stream's device word, read by staf_ops_poll_status. */
 void staf_ops_set_sync_errors(int mode);
 
-/* Synchronises `stream`, returns the accumulated device-side status (0 or a
- * negative STAF_E_* code) and clears it. */
+/* Synchronises `stream`, returns the accumulated device-side status of every
+ * stream of the device (0 or a negative STAF_E_* code) and clears it.  Work on
+ * other streams that `stream` has not been made to wait for may still raise
+ * conditions afterwards; they stay for the next poll. */
 int staf_ops_poll_status(void* stream);
 
 /* Measurement aid with no counterpart in the reference: when enabled, the library brackets its kernels with HIP

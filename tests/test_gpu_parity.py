@@ -187,6 +187,33 @@ def test_radial_overflow_is_reported():
         ops.set_sync_errors(True)
 
 
+def test_condition_stays_with_the_stream_that_raised_it():
+    """Each stream has its own error word: an overflow raised (and left unfetched) on a side stream does not
+    make a later, valid op on another stream return it; the poll, which reads every word, still reports it."""
+    import torch
+    from alphanesgpu_amd import ops, _lib
+    b = _synth("water96")
+    dev = torch.device("cuda:0")
+    pos, box = torch.as_tensor(b["pos"]).to(dev), torch.as_tensor(b["box"]).to(dev)
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    ops.set_sync_errors(False)
+    try:
+        ops.construct_descriptors_light(4.5, 20, 190, b["N"], None, 2.25, 4.5, 1, dtype=torch.float64)
+        with torch.cuda.stream(side):
+            ops.compute_descriptors_light(pos, box)
+        side.synchronize()
+        ops.set_sync_errors(True)
+        ops.construct_descriptors_light(4.5, 60, 1770, b["N"], None, 2.25, 4.5, 1, dtype=torch.float64)
+        ops.compute_descriptors_light(pos, box)   # valid, on the default stream: returns STAF_OK
+        with pytest.raises(_lib.StafError) as e:
+            ops.poll_status()
+        assert e.value.code == -10
+        ops.poll_status()  # cleared
+    finally:
+        ops.set_sync_errors(True)
+
+
 def test_compute_before_construct_other_precision():
     import torch
     from alphanesgpu_amd import ops, _lib
