@@ -315,7 +315,8 @@ int angular_afs(const real* Dsup, const real* Tang, const real* unit, int nr, in
   if (nt > NT_MAX) return STAF_E_LIMIT;
   if (ld <= 0) ld = Nl;
   size_t lds = TriLds<real, 0>::bytes(nr, Aa, nt, unit != nullptr);
-  if (lds > 64 * 1024) return STAF_E_LIMIT;
+  if (!(unit ? lds_request(tri_reduce_kernel<real, 0, true>, lds) : lds_request(tri_reduce_kernel<real, 0>, lds)))
+    return STAF_E_LIMIT;
   TriArgs<real> A = {};
   A.Dsup = Dsup; A.Tang = Tang; A.unit = unit; A.im2 = im2; A.alpha3b = alpha3b; A.emb3b = emb3b;
   A.type_map = type_map; A.numtriplet = numtriplet; A.out = out;
@@ -361,7 +362,7 @@ static int alphagrad_ang(const real* Dsup, const real* Tang, int nr, int na, con
   real* red_tmp = partial ? partial + (size_t)nb * nout : nullptr;
   if (!partial) return reserve_failure(stream);
   size_t lds = TriLds<real, 1>::bytes(nr, Aa, nt);
-  if (lds > 64 * 1024) return STAF_E_LIMIT;
+  if (!lds_request(tri_reduce_kernel<real, 1>, lds)) return STAF_E_LIMIT;
   // rows sigma >= nsig of the outputs receive no contribution
   const int nall = ntc * Aa * 3;
   TriArgs<real> A = {};

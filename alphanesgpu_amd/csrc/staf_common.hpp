@@ -296,6 +296,14 @@ DeviceState* device_state(hipStream_t stream);
 // True while `stream` is being captured into a graph: memory may then neither be freed nor allocated, and a fill
 // launched to initialise a fresh block would become part of the graph.
 bool stream_is_capturing(hipStream_t stream);
+// Dynamic LDS of a launch of `kernel`: up to 64 KB needs nothing, up to the 160 KB of a CU is requested for the
+// kernel (host-side attribute, no stream work).  False: the launch cannot be made (STAF_E_LIMIT).
+template <typename K>
+inline bool lds_request(K kernel, size_t lds) {
+  if (lds <= 64 * 1024) return true;
+  return lds <= 160 * 1024 &&
+         hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) == hipSuccess;
+}
 // The error word of `stream` on this device (see DeviceState::status_d).
 int* status_word(DeviceState* st, hipStream_t stream);
 // Both grow on demand and never shrink; under capture a request that does not fit what the stream already holds

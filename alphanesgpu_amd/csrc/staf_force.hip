@@ -651,7 +651,7 @@ static int gradforce_tripl(const real* Q, const real* G, const real* Dsup, const
   real* red_tmp = partial ? partial + (size_t)nb * nout : nullptr;
   if (!partial) return reserve_failure(stream);
   size_t lds = TriLds<real, 2>::bytes(nr, Aa, nt);
-  if (lds > 64 * 1024) return STAF_E_LIMIT;
+  if (!lds_request(tri_reduce_kernel<real, 2>, lds)) return STAF_E_LIMIT;
   const int nall = ntc * Aa * 3;
   TriArgs<real> A = {};
   A.Dsup = Dsup; A.Tang = Tang; A.im2 = im2; A.alpha3b = alpha3b; A.emb3b = emb3b; A.type_map = type_map;

@@ -663,6 +663,26 @@ def test_random_dense_clusters(oracle):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_wide_channel_sets(oracle, dtype):
+    """Three species with 141 three-body and 57 two-body channels: the parameter tables and gradient accumulators of
+    the triplet kernels then take more than the 64 KB of LDS a launch gets without asking (the library requests up to
+    the CU's 160 KB per kernel), and a class has up to 42 active channels (three table chunks)."""
+    rng = np.random.default_rng(21)
+    tip = [18, 15, 13]
+    n = sum(tip)
+    pts = []
+    while len(pts) < n:
+        c = rng.uniform(-3.2, 3.2, 3)
+        if all(np.linalg.norm(c - q) > 0.75 for q in pts):
+            pts.append(c)
+    pos = (np.array(pts) + rng.uniform(-5, 5, 3)).reshape(1, -1)
+    box = np.array([[16.0, 0.5, -0.3, 16.7, 0.4, 17.3]])
+    _generic_case(oracle, pos, box, tip, dtype, nr=n + 2, na=938, rc=5.4, ra=4.9, rs=1.5, nt=3, seed=2,
+                  maps=((11, 16, 30), (12, 5, 40, 4, 42, 38)))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
 def test_add_n_is_the_sequential_sum(dtype):
     """ops.add_n (the callers' sum of per-op force arrays) against adding the arrays one after the other: same
     order, same bits, for 1 to 9 inputs, also in place."""
