@@ -182,6 +182,36 @@ def test_compute_6144_atom_box_matches_oracle_pipeline(oracle):
 
 
 @pytest.mark.gpu
+def test_compute_is_invariant_under_periodic_replication():
+    """A size-independent property at a size the oracle does not reach: the 6144-atom box replicated 2x2x2 (49152
+    atoms, species-sorted, box edges doubled) has the same local environments, so the energy and the virial are
+    eight times those of the single box and every replica carries the single box's forces (1e-12; the sums are
+    the same, only the neighbour search runs over other cells)."""
+    from alphanesgpu_amd import libstaf, synth
+    b = synth.water_batch("water6144")
+    x = b["pos"][0].reshape(-1, 3).astype(np.float64)
+    box = b["box"][0].astype(np.float64)
+    tm = b["type_map"]
+    L = box[0]
+    n_o = int((tm == 0).sum())
+    shifts = np.array([[i, j, k] for i in range(2) for j in range(2) for k in range(2)], float) * L
+    xo = np.concatenate([x[:n_o] + s for s in shifts])
+    xh = np.concatenate([x[n_o:] + s for s in shifts])
+    big_x = np.concatenate([xo, xh]) - L / 2
+    big_tm = np.array([0] * len(xo) + [1] * len(xh), np.int32)
+    big_box = box.copy()
+    big_box[[0, 3, 5]] *= 2
+    m = libstaf.StafModel(os.path.join(GOLDEN, "model_double"), precision=1)
+    e, f, v = m.compute(x, box, tm)
+    E, F, V = m.compute(big_x, big_box, big_tm)
+    m.close()
+    assert abs(E - 8 * e) <= 1e-12 * abs(8 * e)
+    want = np.concatenate([np.concatenate([f[:n_o]] * 8), np.concatenate([f[n_o:]] * 8)])
+    assert nerr(F.reshape(-1), want.reshape(-1)) <= 1e-12
+    assert nerr(V, 8 * v) <= 1e-12
+
+
+@pytest.mark.gpu
 def test_compute_reproduces_recorded_energies_fp32_model(oracle):
     """float32 MLP (the reference's default build): E and rms(F) recorded by the reference for its 768-atom frame
     (test/test-lammps-STAF-inference-STAF-comp/results/frames.csv:2) and PE of data.water_smoke
