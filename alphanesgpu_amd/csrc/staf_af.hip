@@ -184,7 +184,8 @@ static int radial_afs(const real* D, int nr, const real* alpha2b, int Ar, real* 
 }
 
 // Work area of the 2-body parameter gradient: one row of 2*nt*Ar partial sums per workgroup of grad2_kernel, then
-// RED_SLICES rows for the first pass of the reduction.
+// RED_SLICES spare rows (an earlier form of the reduction used them; the size is part of the documented limit of
+// the entry point that allocates nothing).
 static inline size_t grad2_work_reals(int nf, int Nl, int nt, int Ar) {
   return ((size_t)grad_blocks(nf * Nl) + RED_SLICES) * 2 * nt * Ar;
 }
