@@ -147,6 +147,7 @@ struct StafModel {
     // ranks every few steps) doubles `need`, one that lived long resets it.
     int seen = 0, replays = 0, need = 2;
     int nlocal = 0, nall = 0, ext = 0, want_w = 0;
+    unsigned epoch = 0;        // staf::release_epoch() when the shape was first seen
     std::vector<int> tipos;
     const void* in_d = nullptr;
     const void* out_d = nullptr;
@@ -554,7 +555,8 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
   if (m->dev_mlp) {
     StafModel::Replay& rp = m->replay;
     const bool same = rp.state > 0 && rp.nlocal == nlocal && rp.nall == nall && rp.ext == (int)ext &&
-                      rp.want_w == (int)want_w && rp.tipos == tipos && rp.in_d == m->in_d.p && rp.out_d == m->out_d.p;
+                      rp.want_w == (int)want_w && rp.tipos == tipos && rp.in_d == m->in_d.p && rp.out_d == m->out_d.p &&
+                      rp.epoch == staf::release_epoch();   // staf_ops_release frees what a recorded graph points into
     if (!m->use_graph || !same) {
       if (rp.state == 2) rp.need = rp.replays < 12 ? (rp.need < 64 ? 2 * rp.need : 64) : 2;
       rp.drop();
@@ -565,6 +567,7 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
         rp.replays = 0;
         rp.nlocal = nlocal; rp.nall = nall; rp.ext = ext; rp.want_w = want_w; rp.tipos = tipos;
         rp.in_d = m->in_d.p; rp.out_d = m->out_d.p;
+        rp.epoch = staf::release_epoch();
       }
     } else if (rp.state == 1 && ++rp.seen < rp.need) {
       if (device_sequence() != 0) return -20;

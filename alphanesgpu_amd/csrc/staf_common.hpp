@@ -296,6 +296,9 @@ DeviceState* device_state(hipStream_t stream);
 // True while `stream` is being captured into a graph: memory may then neither be freed nor allocated, and a fill
 // launched to initialise a fresh block would become part of the graph.
 bool stream_is_capturing(hipStream_t stream);
+// Counts the calls of staf_ops_release: work-area addresses recorded anywhere (a captured graph of the MD entry)
+// are valid only while it stands still.
+unsigned release_epoch();
 // Dynamic LDS of a launch of `kernel`: up to 64 KB needs nothing, up to the 160 KB of a CU is requested for the
 // kernel (host-side attribute, no stream work).  False: the launch cannot be made (STAF_E_LIMIT).
 template <typename K>

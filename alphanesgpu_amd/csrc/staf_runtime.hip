@@ -2,6 +2,7 @@
 #include "staf_common.hpp"
 #include "staf_reduce.hpp"
 
+#include <atomic>
 #include <mutex>
 #include <unordered_map>
 #include <memory>
@@ -13,6 +14,8 @@
 namespace staf {
 
 static std::mutex g_mu;
+static std::atomic<unsigned> g_release_epoch{0};
+unsigned release_epoch() { return g_release_epoch.load(); }
 static std::unordered_map<int, std::unique_ptr<DeviceState>> g_state;
 static int g_sync_errors = 1;
 // Calls made by this thread leave their device-detected conditions in the status word (no synchronisation per op)
@@ -279,6 +282,7 @@ void staf_ops_release(void) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return;
   std::lock_guard<std::mutex> lock(staf::g_mu);
+  staf::g_release_epoch++;
   auto it = staf::g_state.find(dev);
   if (it == staf::g_state.end()) return;
   staf::DeviceState* st = it->second.get();

@@ -104,6 +104,12 @@ def kernel_time(kernel):
     return ms.value, n.value
 
 
+def release():
+    """Frees every work area the library holds on the current device (after waiting for it); the next call sizes
+    them again.  Graphs captured before hold pointers into the freed areas and must not be replayed afterwards."""
+    _lib.lib().staf_ops_release()
+
+
 def version():
     return _lib.lib().staf_ops_version().decode()
 

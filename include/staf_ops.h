@@ -101,7 +101,10 @@ int staf_ops_poll_status(void* stream);
 void staf_ops_kernel_timing(int enable);
 int staf_ops_kernel_time(const char* kernel, double* total_ms, int* launches);
 
-/* Frees all device memory the library holds on the current device. */
+/* Waits for the current device and frees all device memory the library holds on it (work areas, remembered
+ * neighbour maps, error words); the next call builds them again.  Graphs the caller captured before point into the
+ * freed areas and must not be replayed afterwards; a handle of the MD entry (staf.h) notices the release and records
+ * its own graph again. */
 void staf_ops_release(void);
 
 /* ---- descriptor op ------------------------------------------------------ */

@@ -816,6 +816,40 @@ def test_stale_neighbour_map_is_reported():
                              T(params[0]["alpha2b"]), T(params[0]["emb2b"]), tm, tp, at)
 
 
+def test_release_frees_the_work_areas_and_the_next_calls_rebuild_them():
+    """staf_ops_release between two runs of every op: same bits before and after.  A force op handed descriptor
+    outputs from before the release no longer finds them among the maps the library remembers and transposes the
+    map itself: same forces to rounding (its sums run in another order)."""
+    import torch
+    from alphanesgpu_amd import ops
+    b = _synth("water96")
+    dtype = np.dtype(np.float64)
+    params = _params(dtype)
+    pos, box = b["pos"].astype(dtype), b["box"].astype(dtype)
+    up = pipeline.synthetic_upstream(1, b["tipos"], params, 3, dtype)
+    r1 = pipeline.run_hip(pos, box, b["tipos"], b["type_map"], params, up, NR, NA, dtype)
+    dev = torch.device("cuda:0")
+    T = lambda a: torch.as_tensor(np.ascontiguousarray(a)).to(dev)
+    rad, ang, sup, im2, im3, d2, d3, d3s, ntr = ops.compute_descriptors_light(T(pos), T(box))
+    n0 = int(b["tipos"][0])
+    tm, tp = T(b["type_map"]), T(b["tipos"])
+    at = torch.tensor([0], dtype=torch.int32, device=dev)
+    args = (T(up["G2"][0]), d2[:, :n0], im2[:, :n0], rad[:, :n0], T(params[0]["alpha2b"]), T(params[0]["emb2b"]),
+            tm, tp, at)
+    before = ops.compute_force_radial(*args).cpu().numpy()
+    ops.release()
+    after = ops.compute_force_radial(*args).cpu().numpy()
+    assert nerr(after, before) <= 1e-13
+    r2 = pipeline.run_hip(pos, box, b["tipos"], b["type_map"], params, up, NR, NA, dtype)
+    for key in ("af2", "af3", "f2", "f3"):
+        for x, y in zip(r1[key], r2[key]):
+            assert np.array_equal(x, y), key
+    for key in ("g2", "g3", "gf2", "gf3"):
+        for x, y in zip(r1[key], r2[key]):
+            for u, v in zip(x, y):
+                assert np.array_equal(u, v), key
+
+
 def test_growth_under_capture_is_refused():
     """An op that meets a shape it has no work area for while its stream is being captured returns STAF_E_CAPTURE
     and launches nothing; after one eager call of the same shape the capture goes through and replays correctly."""

@@ -379,6 +379,24 @@ def test_replayed_calls_give_the_bits_of_eager_calls_and_follow_shape_changes():
 
 
 @pytest.mark.gpu
+def test_release_of_the_ops_state_between_replayed_calls():
+    """staf_ops_release (the op interface's call that frees the library's work areas) while a handle of the MD entry
+    holds a recorded graph: the graph points into freed memory, so the handle drops it, evaluates eagerly and
+    records again -- same bits on every call."""
+    from alphanesgpu_amd import libstaf, ops
+    pos, box, _, type_map = load_frame_mbpol(np.float64)
+    m = libstaf.StafModel(os.path.join(GOLDEN, "model_double"), precision=1, full_virial=True)
+    x = pos.reshape(-1, 3)
+    ref = [m.compute(x, box[0], type_map) for _ in range(4)][-1]      # recorded and replayed by now
+    for _ in range(2):
+        ops.release()
+        for _ in range(4):
+            e, f, w = m.compute(x, box[0], type_map)
+            assert e == ref[0] and np.array_equal(f, ref[1]) and np.array_equal(w, ref[2])
+    m.close()
+
+
+@pytest.mark.gpu
 def test_compute_return_codes():
     """Validation order and codes of libstaf/src/staf_api.cpp:196-337."""
     from alphanesgpu_amd import libstaf
