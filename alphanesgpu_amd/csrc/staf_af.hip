@@ -358,12 +358,13 @@ static int alphagrad_ang(const real* Dsup, const real* Tang, int nr, int na, con
   hipStream_t stream = (hipStream_t)stream_;
   const int nsig = 2 * nt - 1;
   const int nout = nsig * Aa * 3;
-  const int nb = nf * Nl < TRI_GRID_MAX ? nf * Nl : TRI_GRID_MAX;
-  real* partial = (real*)scratch_reserve(st, stream, ((size_t)nb + RED_SLICES) * nout * sizeof(real));
-  real* red_tmp = partial ? partial + (size_t)nb * nout : nullptr;
+  const int nb_max = nf * Nl < TRI_GRID_MAX ? nf * Nl : TRI_GRID_MAX;   // the work area does not depend on occupancy
+  real* partial = (real*)scratch_reserve(st, stream, ((size_t)nb_max + RED_SLICES) * nout * sizeof(real));
+  real* red_tmp = partial ? partial + (size_t)nb_max * nout : nullptr;
   if (!partial) return reserve_failure(stream);
   size_t lds = TriLds<real, 1>::bytes(nr, Aa, nt);
   if (!lds_request(tri_reduce_kernel<real, 1>, lds)) return STAF_E_LIMIT;
+  const int nb = tri_grid((const void*)tri_reduce_kernel<real, 1>, lds, nf * Nl);
   // rows sigma >= nsig of the outputs receive no contribution
   const int nall = ntc * Aa * 3;
   TriArgs<real> A = {};

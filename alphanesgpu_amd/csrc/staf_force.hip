@@ -646,12 +646,13 @@ static int gradforce_tripl(const real* Q, const real* G, const real* Dsup, const
   const int ntc = nt * (nt + 1) / 2;
   const int nsig = 2 * nt - 1;
   const int nout = nsig * Aa * 3;
-  const int nb = nf * Nl < TRI_GRID_MAX ? nf * Nl : TRI_GRID_MAX;
-  real* partial = (real*)scratch_reserve(st, stream, ((size_t)nb + RED_SLICES) * nout * sizeof(real));
-  real* red_tmp = partial ? partial + (size_t)nb * nout : nullptr;
+  const int nb_max = nf * Nl < TRI_GRID_MAX ? nf * Nl : TRI_GRID_MAX;   // the work area does not depend on occupancy
+  real* partial = (real*)scratch_reserve(st, stream, ((size_t)nb_max + RED_SLICES) * nout * sizeof(real));
+  real* red_tmp = partial ? partial + (size_t)nb_max * nout : nullptr;
   if (!partial) return reserve_failure(stream);
   size_t lds = TriLds<real, 2>::bytes(nr, Aa, nt);
   if (!lds_request(tri_reduce_kernel<real, 2>, lds)) return STAF_E_LIMIT;
+  const int nb = tri_grid((const void*)tri_reduce_kernel<real, 2>, lds, nf * Nl);
   const int nall = ntc * Aa * 3;
   TriArgs<real> A = {};
   A.Dsup = Dsup; A.Tang = Tang; A.im2 = im2; A.alpha3b = alpha3b; A.emb3b = emb3b; A.type_map = type_map;

@@ -27,7 +27,10 @@
 //     MODE 2 the contraction U of der3b with dL/dF), so tensors laid out by
 //     the storage index nn are read exactly once.
 #pragma once
+#include <map>
+#include <mutex>
 #include <type_traits>
+#include <utility>
 
 #include "staf_tile.hpp"
 
@@ -46,6 +49,51 @@ struct TriCfg {
   static constexpr int MIN_WAVES = sizeof(real) == 8 ? (MODE == 0 ? 5 : 4) : (MODE == 0 ? 8 : MODE == 1 ? 7 : 5);
 };
 constexpr int TRI_GRID_MAX = 2048;  // workgroups of the persistent gradient modes (one partial row each)
+
+// Workgroups of a persistent gradient launch over `centres` centres.  Workgroup w takes centres w, w + W, ...: the
+// launch lasts about ceil(W / resident) rounds of workgroups times ceil(centres / W) centres each, `resident` being
+// the workgroups the device holds at once for this kernel and LDS size.  Within a number of rounds the largest W
+// is best, so one candidate per number of rounds; ties go to the larger W (more, shorter workgroups even out the
+// centres' unequal work).  E.g. 4096 centres, 1792 resident: 1792 workgroups (1 round x 3) rather than 2048 (2 x 2).
+inline int tri_grid(const void* kernel, size_t lds, int centres) {
+  const int wmax = centres < TRI_GRID_MAX ? centres : TRI_GRID_MAX;
+  static int cus = 0;   // one device kind per process
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      cus = n;
+    else
+      cus = -1;
+  }
+  // the occupancy query is made once per (kernel, LDS size)
+  static std::mutex mu;
+  static std::map<std::pair<const void*, size_t>, int> known;
+  int per_cu = 0;
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = known.find({kernel, lds});
+    if (it != known.end()) {
+      per_cu = it->second;
+    } else {
+      if (cus <= 0 || hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, TRI_BLOCK, lds) != hipSuccess) {
+        (void)hipGetLastError();
+        per_cu = 0;
+      }
+      known[{kernel, lds}] = per_cu;
+    }
+  }
+  if (per_cu <= 0) return wmax;
+  const long resident = (long)per_cu * cus;
+  int best = wmax;
+  long best_span = ((wmax + resident - 1) / resident) * (long)((centres + wmax - 1) / wmax);
+  for (long k = (wmax + resident - 1) / resident - 1; k >= 1; k--) {
+    const int w = (int)(k * resident);   // < wmax
+    const long span = k * (long)((centres + w - 1) / w);
+    if (span < best_span) { best = w; best_span = span; }
+  }
+  return best;
+}
 
 // Exponential of the hot loops.
 // float: the argument is pre-scaled by log2(e) and fed to the hardware exp2 (two instructions; the rounding of the
