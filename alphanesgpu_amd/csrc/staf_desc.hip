@@ -238,8 +238,11 @@ __device__ inline void zero_fill(char* p, unsigned nbytes, int tid) {
   if ((unsigned)tid * 4u < tail) *(int*)(q + body + tid * 4u) = 0;
 }
 
+// Waves per SIMD the allocation is held to: without a bound the single-precision kernel takes 112 scalar registers
+// (seven waves: 1792 resident workgroups for the 3072 centres of four 768-atom frames) and the double-precision
+// one 104 vector registers (four waves); at eight and five the launch needs fewer rounds of workgroups.
 template <typename real>
-__global__ __launch_bounds__(256) void desc_kernel(DescArgs<real> A) {
+__global__ __launch_bounds__(256, sizeof(real) == 4 ? 8 : 5) void desc_kernel(DescArgs<real> A) {
   using real2 = typename Vec2<real>::type;
   extern __shared__ __align__(16) unsigned char smem[];
   const int nr = A.nr, na = A.na, N = A.N;
