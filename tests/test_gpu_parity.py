@@ -850,6 +850,52 @@ def test_release_frees_the_work_areas_and_the_next_calls_rebuild_them():
                 assert np.array_equal(u, v), key
 
 
+def test_three_host_threads_on_their_own_streams(monkeypatch):
+    """The library's state is per device and per stream behind one lock: three host threads, each on a stream of its
+    own, run the whole op sequence at the same time (a framework's executor calls ops from several threads), and
+    every result has the bits of the single-threaded run."""
+    import threading
+    import torch
+    from alphanesgpu_amd import ops
+    b = _synth("water96")
+    dtype = np.dtype(np.float64)
+    params = _params(dtype)
+    pos, box = b["pos"].astype(dtype), b["box"].astype(dtype)
+    up = pipeline.synthetic_upstream(1, b["tipos"], params, 3, dtype)
+    want = pipeline.run_hip(pos, box, b["tipos"], b["type_map"], params, up, NR, NA, dtype)
+    # the geometry and the options stay as the call above set them: threads only compute
+    monkeypatch.setattr(ops, "construct_descriptors_light", lambda *a, **k: None)
+    monkeypatch.setattr(ops, "descriptor_options", lambda *a, **k: None)
+    bad = []
+
+    def same(x, y):
+        if isinstance(x, tuple):
+            return all(same(u, v) for u, v in zip(x, y))
+        return np.array_equal(x, y)
+
+    def worker(t):
+        try:
+            with torch.cuda.stream(torch.cuda.Stream()):
+                for it in range(3):
+                    got = pipeline.run_hip(pos, box, b["tipos"], b["type_map"], params, up, NR, NA, dtype)
+                    for key in ("af2", "af3", "f2", "f3", "g2", "g3", "gf2", "gf3"):
+                        for x, y in zip(got[key], want[key]):
+                            if not same(x, y):
+                                bad.append((t, it, key))
+                    for k in ("intmap2b", "intmap3b", "numtriplet", "raddescr", "angdescr", "der2b"):
+                        if not np.array_equal(got["desc"][k], want["desc"][k]):
+                            bad.append((t, it, k))
+        except Exception as e:   # a thread's exception would otherwise be lost
+            bad.append((t, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(3)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not bad, bad[:10]
+
+
 def test_growth_under_capture_is_refused():
     """An op that meets a shape it has no work area for while its stream is being captured returns STAF_E_CAPTURE
     and launches nothing; after one eager call of the same shape the capture goes through and replays correctly."""
