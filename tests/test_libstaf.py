@@ -397,6 +397,42 @@ def test_release_of_the_ops_state_between_replayed_calls():
 
 
 @pytest.mark.gpu
+def test_three_handles_on_three_host_threads():
+    """Three handles, each used by a host thread of its own at the same time (every handle records and replays its
+    own graph on its own streams): every call returns the bits a single handle returned for the same positions."""
+    import threading
+    from alphanesgpu_amd import libstaf
+    pos, box, _, type_map = load_frame_mbpol(np.float64)
+    x = pos.reshape(-1, 3)
+    d = os.path.join(GOLDEN, "model_double")
+    rng = np.random.default_rng(1)
+    xs = [x + 0.02 * rng.standard_normal(x.shape) for _ in range(8)]
+    ref = libstaf.StafModel(d, precision=1, full_virial=True)
+    want = [ref.compute(xx, box[0], type_map) for xx in xs]
+    ref.close()
+    bad = []
+
+    def worker(t):
+        try:
+            m = libstaf.StafModel(d, precision=1, full_virial=True)
+            for rep in range(2):
+                for i, xx in enumerate(xs):
+                    e, f, w = m.compute(xx, box[0], type_map)
+                    if e != want[i][0] or not np.array_equal(f, want[i][1]) or not np.array_equal(w, want[i][2]):
+                        bad.append((t, rep, i))
+            m.close()
+        except Exception as ex:   # a thread's exception would otherwise be lost
+            bad.append((t, repr(ex)))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(3)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not bad, bad[:10]
+
+
+@pytest.mark.gpu
 def test_compute_return_codes():
     """Validation order and codes of libstaf/src/staf_api.cpp:196-337."""
     from alphanesgpu_amd import libstaf
