@@ -663,6 +663,26 @@ def test_random_dense_clusters(oracle):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_tiny_systems(oracle, dtype):
+    """One atom (no neighbour at all), two atoms of one or two species, one water molecule, three atoms: every op,
+    one and three frames, buffers larger and smaller than the neighbour counts."""
+    cases = [([1], [[0.1, 0.2, 0.3]]),
+             ([2], [[0, 0, 0], [1.1, 0.2, 0.1]]),
+             ([1, 1], [[0, 0, 0], [1.0, 0.3, 0.2]]),
+             ([1, 2], [[0, 0, 0], [0.96, 0, 0], [-0.24, 0.93, 0]]),
+             ([3], [[0, 0, 0], [1.0, 0, 0], [0, 1.2, 0]])]
+    for tip, pts in cases:
+        n = sum(tip)
+        for nf in (1, 3):
+            pos = np.tile(np.array(pts, float).reshape(1, -1), (nf, 1)) + np.arange(nf)[:, None] * 0.01
+            box = np.tile(np.array([[12.0, 0.3, -0.2, 12.5, 0.1, 13.0]]), (nf, 1))
+            for nr, na in ((n + 2, 3), (4, 6)):
+                _generic_case(oracle, pos, box, tip, dtype, nr=nr, na=na, rc=4.5, ra=4.5, rs=2.25, nt=len(tip),
+                              seed=2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
 def test_wide_channel_sets(oracle, dtype):
     """Three species with 141 three-body and 57 two-body channels: the parameter tables and gradient accumulators of
     the triplet kernels then take more than the 64 KB of LDS a launch gets without asking (the library requests up to
