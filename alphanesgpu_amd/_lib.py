@@ -18,6 +18,10 @@ ERRORS = {
     -10: "STAF_E_RADIAL_OVERFLOW: an atom has more neighbours than radial_buffer",
     -11: "STAF_E_SCATTER_OVERFLOW: an atom is listed by more centres than the force scatter holds",
     -12: "STAF_E_LIMIT: dimension beyond the kernels' limits, or feature not built",
+    -13: "STAF_E_CAPTURE: the stream is being captured into a graph and the call would have to allocate; run the "
+         "same call once outside the capture first",
+    -14: "STAF_E_STALE_MAP: a force op was handed a view of a descriptor output whose intmap2b no longer holds what "
+         "the descriptor op wrote, or whose first row is not the first atom of the centre species",
 }
 
 

@@ -438,5 +438,3 @@ int staf_op_alphagrad_ang_f64(const double* Dsup, const double* Tang, int nr, in
 }
 
 }  // extern "C"
-
-PHASE_CLOCK_READER(staf_debug_phase_clock_af)

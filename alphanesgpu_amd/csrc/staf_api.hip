@@ -703,6 +703,7 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
   // the call's synchronisation: results are on the host, and so is what the kernels reported
   rc = staf_ops_poll_status(st);
   if (rc == STAF_E_RADIAL_OVERFLOW) return -10;
+  if (rc == STAF_E_SCATTER_OVERFLOW) return -11;
   if (rc != STAF_OK) return -20;
   if (m->dev_mlp) {
     const double* e_atom_h = m->out_h.p + (size_t)n3 + 9;

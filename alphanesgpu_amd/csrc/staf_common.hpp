@@ -186,53 +186,6 @@ __device__ inline void mic_cart_from_cart(const real* pi, const real* pj, const 
 // Pair index q inside an n-item triangle (x<y) -> (x,y); same numbering.
 __device__ inline void tri_decode_xy(int q, int n, int& x, int& y) { tri_decode(q, n, x, y); }
 
-// Phase clock (profiling builds only, -DSTAF_PHASE_CLOCK): thread 0 of every workgroup adds the shader-clock
-// cycles between consecutive marks to a per-phase total when it ends.  Every translation unit has its own totals, read back
-// and cleared with the staf_debug_phase_clock_<unit>() it defines through PHASE_CLOCK_READER.
-#ifdef STAF_PHASE_CLOCK
-static __device__ unsigned long long g_phase_clock[32];
-#define PHASE_CLOCK_READER(name)                                                                            \
-  extern "C" int name(unsigned long long* out) {                                                            \
-    if (hipDeviceSynchronize() != hipSuccess) return STAF_E_HIP;                                            \
-    if (hipMemcpyFromSymbol(out, HIP_SYMBOL(staf::g_phase_clock), 32 * sizeof(unsigned long long)) !=       \
-        hipSuccess)                                                                                         \
-      return STAF_E_HIP;                                                                                    \
-    unsigned long long zero[32] = {0};                                                                      \
-    if (hipMemcpyToSymbol(HIP_SYMBOL(staf::g_phase_clock), zero, sizeof(zero)) != hipSuccess)               \
-      return STAF_E_HIP;                                                                                    \
-    return STAF_OK;                                                                                         \
-  }
-#define PHASE_CLOCK_BEGIN()                           \
-  unsigned long long phase_acc_[16] = {0};            \
-  const unsigned long long phase_w0_ = wall_clock64(); \
-  unsigned long long phase_t_ = clock64()
-#define PHASE_MARK(i)                                   \
-  do {                                                  \
-    const unsigned long long now_ = clock64();          \
-    phase_acc_[i] += now_ - phase_t_;                   \
-    phase_t_ = now_;                                    \
-  } while (0)
-#define PHASE_CLOCK_END()                                                   \
-  do {                                                                      \
-    if (threadIdx.x == 0) {                                                 \
-      for (int i_ = 0; i_ < 16; i_++)                                       \
-        if (phase_acc_[i_]) atomicAdd(&g_phase_clock[i_], phase_acc_[i_]);  \
-      /* wall-clock (100 MHz) extremes of workgroup start and end; entry 16 holds ~min start */ \
-      const unsigned long long w1_ = wall_clock64();                        \
-      atomicMax(&g_phase_clock[16], ~phase_w0_);                            \
-      atomicMax(&g_phase_clock[17], phase_w0_);                             \
-      atomicMax(&g_phase_clock[18], ~w1_);                                  \
-      atomicMax(&g_phase_clock[19], w1_);                                   \
-      atomicAdd(&g_phase_clock[20], w1_ - phase_w0_);                       \
-    }                                                                       \
-  } while (0)
-#else
-#define PHASE_CLOCK_READER(name)
-#define PHASE_CLOCK_BEGIN() do {} while (0)
-#define PHASE_MARK(i) do {} while (0)
-#define PHASE_CLOCK_END() do {} while (0)
-#endif
-
 // ---- library-owned device state (per device) -------------------------------
 struct Workspace {
   void* buf = nullptr;

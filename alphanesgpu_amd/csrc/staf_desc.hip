@@ -265,7 +265,6 @@ __global__ __launch_bounds__(256, sizeof(real) == 4 ? 8 : 5) void desc_kernel(De
   const int tid = threadIdx.x;
   const int b = blockIdx.x / N;
   const int i = blockIdx.x - b * N;
-  PHASE_CLOCK_BEGIN();
   if (tid == 0) { cnt_all = 0; cnt_ang = 0; }
   for (int e = tid; e < nr; e += blockDim.x) s_rank[e] = 0;
   // Box and centre position are the same for the whole workgroup: every thread reads them itself (reads of
@@ -383,7 +382,6 @@ __global__ __launch_bounds__(256, sizeof(real) == 4 ? 8 : 5) void desc_kernel(De
     }
   }
   __syncthreads();
-  PHASE_MARK(0);
   const int hm = cnt_all;
   const int n = hm < nr ? hm : nr;
   if (hm > nr && tid == 0) atomicOr(A.status, 1);
@@ -413,7 +411,6 @@ __global__ __launch_bounds__(256, sizeof(real) == 4 ? 8 : 5) void desc_kernel(De
     }
     __syncthreads();
   }
-  PHASE_MARK(1);
   // A caller's list: every slot registers with the atom it points at (the transposed map the force ops gather
   // through; the library's own lists are symmetric and need none).  The second wave does it while the first one
   // fills the radial rows.
@@ -493,9 +490,7 @@ __global__ __launch_bounds__(256, sizeof(real) == 4 ? 8 : 5) void desc_kernel(De
       }
     }
   }
-  PHASE_MARK(2);
   __syncthreads();
-  PHASE_MARK(3);
   const int m = cnt_ang;
   if (tid == 0) {
     im[0] = hm;
@@ -560,8 +555,6 @@ __global__ __launch_bounds__(256, sizeof(real) == 4 ? 8 : 5) void desc_kernel(De
     zero_fill(d3p1 + (size_t)ntr * sizeof(real2), npad * (unsigned)sizeof(real2), tid);
     zero_fill(d3p2 + (size_t)ntr * sizeof(real2), npad * (unsigned)sizeof(real2), tid);
   }
-  PHASE_MARK(4);
-  PHASE_CLOCK_END();
 }
 
 template <typename real>
@@ -747,7 +740,6 @@ static int compute(const real* pos, const real* box, int nf, int N, real* raddes
 }
 
 }  // namespace staf
-PHASE_CLOCK_READER(staf_debug_phase_clock_desc)
 
 extern "C" {
 

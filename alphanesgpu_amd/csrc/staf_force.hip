@@ -726,5 +726,3 @@ STAF_FORCE_ENTRY(float, f32)
 STAF_FORCE_ENTRY(double, f64)
 
 }  // extern "C"
-
-PHASE_CLOCK_READER(staf_debug_phase_clock_force)

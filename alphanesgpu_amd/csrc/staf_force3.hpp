@@ -121,7 +121,6 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
   real* sU = xch + NW * 4;                                 // FUSED: [4][nr] unit vector, 1/r
   int* nact = (int*)(sU + (FUSED ? 4 * nr : 0));           // [16] active channels per sigma (0 beyond nsig)
   int* stp = nact + 16;                                    // [nr] species of every slot
-  PHASE_CLOCK_BEGIN();
 
   const int tid = threadIdx.x;
   const int lane = tid & (WAVE - 1), wave = uniform(tid / WAVE);
@@ -215,7 +214,6 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
   }
   if (slot) stp[tid] = t_s;
   __syncthreads();
-  PHASE_MARK(0);
   int maxact = 0;
   for (int sgm = 0; sgm < nsig; sgm++) {
     const int n_ = uniform(nact[sgm]);
@@ -266,7 +264,6 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
         jk[p] = j | (k << 8);
       }
     }
-    PHASE_MARK(1);
     for (int c0 = 0; c0 < maxact; c0 += CAP) {
       const int nch = (maxact - c0) < CAP ? (maxact - c0) : CAP;
       const int nch2 = (nch + 1) & ~1;            // the channel loop runs in pairs (c0 + nch2 <= Ap)
@@ -290,7 +287,6 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
         }
       }
       __syncthreads();
-      PHASE_MARK(2);
       // One copy of the loop per number of passes, so that no branch separates the (triplet, channel) items and
       // the LDS reads of the next items are in flight while the current ones are computed.
       auto channels = [&](auto npass_c) {
@@ -348,7 +344,6 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
           default: break;
         }
       }
-      PHASE_MARK(3);
     }
 
     // ---- contraction with der3b, slot sums of this wave.  Lanes past the last triplet hold T = 0 and finite sums
@@ -469,10 +464,8 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
         __builtin_amdgcn_wave_barrier();
       }
     }
-    PHASE_MARK(4);
   }
   __syncthreads();
-  PHASE_MARK(5);
 
   // ---- slot forces (waves added in a fixed order; one slot per thread: m <= nr < THREADS), centre's own force
   real f3[3] = {0, 0, 0};
@@ -505,8 +498,6 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
     for (int w = 0; w < NW; w++) a += xch[w * 4 + tid];
     self[(size_t)atom * 3 + tid] = -a;
   }
-  PHASE_MARK(6);
-  PHASE_CLOCK_END();
 }
 
 }  // namespace staf

@@ -115,7 +115,6 @@ __global__ __launch_bounds__(MLP_BLOCK) void mlp_kernel(MlpArgs<T> A) {
   const int tid = threadIdx.x;
   const int a0 = blockIdx.x * MLP_TA;
   const int n_af = A.n_af;
-  PHASE_CLOCK_BEGIN();
   for (int q = tid; q < MLP_TA * n_af; q += MLP_BLOCK) {
     const int t = q / n_af, i = q - t * n_af;
     const int atom = a0 + t;
@@ -127,7 +126,6 @@ __global__ __launch_bounds__(MLP_BLOCK) void mlp_kernel(MlpArgs<T> A) {
     buf[t * A.tot + i] = v;
   }
   __syncthreads();
-  PHASE_MARK(0);
   // ---- forward
   int off_in = 0;
   for (int l = 0; l < A.nl; l++) {
@@ -150,7 +148,6 @@ __global__ __launch_bounds__(MLP_BLOCK) void mlp_kernel(MlpArgs<T> A) {
     } else {
       const int KS = matvec_slices<T, MLP_TA>(A.W[l], in_f, out_f, buf + off_in, A.tot, part);
       __syncthreads();
-      PHASE_MARK(1);
       for (int q = tid; q < MLP_TA * out_f; q += MLP_BLOCK) {
         const int t = q / out_f, j = q - t * out_f;
         T y = A.b[l][j];
@@ -161,7 +158,6 @@ __global__ __launch_bounds__(MLP_BLOCK) void mlp_kernel(MlpArgs<T> A) {
       }
     }
     __syncthreads();
-    PHASE_MARK(2);
     off_in = off_out;
   }
   // off_in is now the offset of the last layer's output (one value per atom)
@@ -184,10 +180,8 @@ __global__ __launch_bounds__(MLP_BLOCK) void mlp_kernel(MlpArgs<T> A) {
     }
     __syncthreads();
     // delta of the layer's input: Wt [out, in] is the matrix, the delta the vector
-    PHASE_MARK(3);
     const int KS = matvec_slices<T, MLP_TA>(A.Wt[l], out_f, in_f, dl, A.maxw, part);
     __syncthreads();
-    PHASE_MARK(4);
     for (int q = tid; q < MLP_TA * in_f; q += MLP_BLOCK) {
       const int t = q / in_f, i = q - t * in_f;
       T g = 0;
@@ -195,7 +189,6 @@ __global__ __launch_bounds__(MLP_BLOCK) void mlp_kernel(MlpArgs<T> A) {
       dl[t * A.maxw + i] = g;
     }
     __syncthreads();
-    PHASE_MARK(5);
     off_out = off_i;
   }
   // ---- d sum(atomic) / d af = delta / (af + 1e-3)
@@ -209,8 +202,6 @@ __global__ __launch_bounds__(MLP_BLOCK) void mlp_kernel(MlpArgs<T> A) {
     if (two) A.g2[(size_t)atom * A.Ar + i] = g;
     else A.g3[(size_t)atom * A.Aa + (i - A.Ar)] = g;
   }
-  PHASE_MARK(6);
-  PHASE_CLOCK_END();
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -303,7 +294,6 @@ __global__ __launch_bounds__(MM_BLOCK) void mlp_matrix_kernel(MlpArgs<T> A) {
   const int tid = threadIdx.x;
   const int a0 = blockIdx.x * MM_TA;
   const int n_af = A.n_af;
-  PHASE_CLOCK_BEGIN();
   for (int q = tid; q < MM_TA * n_af; q += MM_BLOCK) {
     const int t = q / n_af, i = q - t * n_af;
     const int atom = a0 + t;
@@ -315,7 +305,6 @@ __global__ __launch_bounds__(MM_BLOCK) void mlp_matrix_kernel(MlpArgs<T> A) {
     X[i * MM_TA + t] = v;
   }
   __syncthreads();
-  PHASE_MARK(0);
   // ---- forward
   int off_in = 0;
   for (int l = 0; l < A.nl; l++) {
@@ -323,7 +312,6 @@ __global__ __launch_bounds__(MM_BLOCK) void mlp_matrix_kernel(MlpArgs<T> A) {
     const int off_out = off_in + in_f;
     const int nsl = mm_products<T>(A.W[l], in_f, out_f, X + (size_t)off_in * MM_TA, part);
     __syncthreads();
-    PHASE_MARK(1);
     for (int q = tid; q < out_f * MM_TA; q += MM_BLOCK) {
       const int j = q / MM_TA;
       T y = A.b[l][j];
@@ -333,7 +321,6 @@ __global__ __launch_bounds__(MM_BLOCK) void mlp_matrix_kernel(MlpArgs<T> A) {
       X[(size_t)off_out * MM_TA + q] = y;
     }
     __syncthreads();
-    PHASE_MARK(2);
     off_in = off_out;
   }
   // off_in is now the offset of the last layer's output (one value per atom)
@@ -355,17 +342,14 @@ __global__ __launch_bounds__(MM_BLOCK) void mlp_matrix_kernel(MlpArgs<T> A) {
     }
     __syncthreads();
     // delta of the layer's input: Wt [out, in] is the matrix, the deltas [out][atoms] the vectors
-    PHASE_MARK(3);
     const int nsl = mm_products<T>(A.Wt[l], out_f, in_f, dl, part);
     __syncthreads();
-    PHASE_MARK(4);
     for (int q = tid; q < in_f * MM_TA; q += MM_BLOCK) {
       T g = 0;
       for (int sl = 0; sl < nsl; sl++) g += part[(size_t)sl * in_f * MM_TA + q];
       dl[q] = g;
     }
     __syncthreads();
-    PHASE_MARK(5);
     off_out = off_i;
   }
   // ---- d sum(atomic) / d af = delta / (af + 1e-3)
@@ -379,8 +363,6 @@ __global__ __launch_bounds__(MM_BLOCK) void mlp_matrix_kernel(MlpArgs<T> A) {
     if (two) A.g2[(size_t)atom * A.Ar + i] = g;
     else A.g3[(size_t)atom * A.Aa + (i - A.Ar)] = g;
   }
-  PHASE_MARK(6);
-  PHASE_CLOCK_END();
 }
 
 // LDS of a workgroup of the matrix kernel: activations, deltas, slice sums of the widest product
@@ -519,5 +501,3 @@ int dev_mlp_eval(const DevMlpNet& net, const double* af2, int Ar, const double* 
 }
 
 }  // namespace staf
-
-PHASE_CLOCK_READER(staf_debug_phase_clock_mlp)

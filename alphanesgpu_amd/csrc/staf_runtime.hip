@@ -216,6 +216,14 @@ static int decode_status(int bits) {
   return STAF_OK;
 }
 
+// Clears in every error word exactly the bits the host has just read: a bit a kernel of another stream sets between
+// the read and this clear stays for the next poll (a plain fill of the words would lose it).
+struct StatusSeen { int bits[STATUS_WORDS]; };
+__global__ void status_clear_kernel(int* word, StatusSeen seen, int nw) {
+  const int w = threadIdx.x;
+  if (w < nw && seen.bits[w]) atomicAnd(&word[w], ~seen.bits[w]);
+}
+
 // Reads and clears, after waiting for `stream`, the stream's own error word (all = false) or every word of the
 // device (all = true: the poll, whose caller has waited for the other streams itself).
 static int fetch_status(DeviceState* st, hipStream_t stream, bool all) {
@@ -227,10 +235,18 @@ static int fetch_status(DeviceState* st, hipStream_t stream, bool all) {
   if (hipMemcpyAsync(host, word, nw * sizeof(int), hipMemcpyDeviceToHost, stream) != hipSuccess) return STAF_E_HIP;
   if (hipStreamSynchronize(stream) != hipSuccess) return STAF_E_HIP;
   int bits = 0;
+  StatusSeen seen;
+  for (int w = 0; w < STATUS_WORDS; w++) seen.bits[w] = w < nw ? host[w] : 0;
   for (int w = 0; w < nw; w++) bits |= host[w];
   if (bits) {
-    if (hipMemsetAsync(word, 0, nw * sizeof(int), stream) != hipSuccess) return STAF_E_HIP;
-    if (hipStreamSynchronize(stream) != hipSuccess) return STAF_E_HIP;
+    hipLaunchKernelGGL(status_clear_kernel, dim3(1), dim3(STATUS_WORDS), 0, stream, word, seen, nw);
+    if (hipGetLastError() != hipSuccess || hipStreamSynchronize(stream) != hipSuccess) return STAF_E_HIP;
+    if (bits & 4) {
+      // A remembered neighbour map no longer holds what the descriptor op wrote: nothing remembered is trusted any
+      // more.  Force ops then transpose the map they are handed themselves until the descriptor op writes again.
+      std::lock_guard<std::mutex> lock2(g_mu);
+      for (auto& e : st->transposes) e.im2 = nullptr;
+    }
   }
   return decode_status(bits);
 }

@@ -22,6 +22,7 @@ RETURN_CODES = {
     -8: "unsupported atom type",
     -9: "neighbour index out of range",
     -10: "an atom has more neighbours than Buffer_radial_descriptors",
+    -11: "an atom of the caller's list is named by more than 4 x the radial buffer centres",
     -20: "GPU runtime error",
 }
 

@@ -130,3 +130,19 @@ def fingerprint_params(nt=2, ar_map=AR_MAP, aa_map=AA_MAP, seed=7, dtype=np.floa
             emb2b=e2.astype(dtype), emb3b=e3.astype(dtype),
             mu=rng.uniform(-1.0, 1.0, Ar + Aa).astype(dtype)))
     return out
+
+
+def synthetic_upstream(nf, tipos, params, seed, dtype):
+    """Stand-ins for what the MLP and the loss feed into the ops: G = d(sum e)/dAF ~ N(0,1), P = dL/dAF ~ N(0,1),
+    Q = dL/dF ~ N(0,1)."""
+    rng = np.random.Generator(np.random.Philox(seed))
+    N = int(np.sum(tipos))
+    up = dict(Q=rng.standard_normal((nf, 3 * N)).astype(dtype), G2=[], G3=[], P2=[], P3=[])
+    for k, n in enumerate(tipos):
+        Ar = params[k]["alpha2b"].shape[1]
+        Aa = params[k]["alpha3b"].shape[1] // 3
+        up["G2"].append(rng.standard_normal((nf, int(n), Ar)).astype(dtype))
+        up["G3"].append(rng.standard_normal((nf, int(n), Aa)).astype(dtype))
+        up["P2"].append(rng.standard_normal((nf, int(n), Ar)).astype(dtype))
+        up["P3"].append(rng.standard_normal((nf, int(n), Aa)).astype(dtype))
+    return up

@@ -235,8 +235,6 @@ def main():
 def run_workload(args, workload, mode):
     import torch
     from alphanesgpu_amd import ops, synth
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
-    import pipeline
 
     dev = torch.device("cuda:0")
     batch = synth.water_batch(workload)
@@ -249,7 +247,7 @@ def run_workload(args, workload, mode):
     nt = len(tipos)
     params = synth.fingerprint_params(dtype=dtype)
     Ar, Aa = params[0]["alpha2b"].shape[1], params[0]["alpha3b"].shape[1] // 3
-    up = pipeline.synthetic_upstream(nf, batch["tipos"], params, 11, dtype)
+    up = synth.synthetic_upstream(nf, batch["tipos"], params, 11, dtype)
 
     T = lambda a: torch.as_tensor(np.ascontiguousarray(a)).to(dev)
     pos, box = T(batch["pos"]), T(batch["box"])

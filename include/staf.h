@@ -54,7 +54,9 @@ StafModel* staf_load(const char* model_dir, const StafOptions* opt);
  *   reverse-communicated); virial [6] = xx yy zz xy xz yz.
  * Returns 0, or: -1 null model / allocation, -3 nlocal <= 0, -4 model files unreadable, -7 zero box diagonal,
  * -8 species out of range, -9 neighbour index out of range, -10 more neighbours than the radial buffer,
- * -20 GPU runtime failure.  (-2 and -5 of the reference, "built without engine" and "cwd", cannot occur.) */
+ * -11 (this library only) an atom of a caller's list is named by more than 4 x the radial buffer centres, which
+ * no list cut at the model's cutoff can hold while -10 does not occur, -20 GPU runtime failure.  (-2 and -5 of the
+ * reference, "built without engine" and "cwd", cannot occur.) */
 int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const double* box, const int* type,
                  const int* howmany, const int* with, int maxneigh, double* e_rank, double* f, double* virial);
 

@@ -52,6 +52,14 @@
  *     allocate under capture returns STAF_E_CAPTURE and allocates nothing.
  *     Outgrown work areas stay allocated until staf_ops_release, so graphs
  *     recorded earlier keep valid addresses.
+ *     Tested bound: a capture that forks the op chains onto at most THREE
+ *     streams beside the capture stream (captured, instantiated, replayed and
+ *     compared bit for bit with the eager step).  A capture that forked onto
+ *     four side streams has ended the process inside the end of the capture /
+ *     the instantiation of the graph, twice, with the cause unknown; under
+ *     capture the library itself only looks up per-stream state it already
+ *     holds and launches kernels, exactly as with three streams.  Keep a
+ *     captured step to three forked streams.
  */
 #ifndef STAF_OPS_H
 #define STAF_OPS_H

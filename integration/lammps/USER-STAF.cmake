@@ -5,9 +5,12 @@
 # staf_compute and staf_free (lammps/USER-STAF/pair_staf.cpp:152-256); include/staf.h of this repository declares
 # those with the reference's argument lists and return codes.
 #
-#   cmake -C <this file> -D STAF_HIP_DIR=<checkout of this repository> -D PKG_USER-STAF=on ../cmake
+# Use: place the block below in cmake/Modules/Packages/USER-STAF.cmake in place of the find of the reference's
+# libstaf (that file is included after the `lammps` target exists, which the target_* commands below need; this file
+# cannot serve as an initial-cache script for `cmake -C`), then configure with
 #
-# or append the block below to cmake/Modules/Packages/USER-STAF.cmake in place of the find of the reference's libstaf.
+#   cmake -D STAF_HIP_DIR=<checkout of this repository> -D PKG_USER-STAF=on ../cmake
+#
 if(NOT DEFINED STAF_HIP_DIR)
   message(FATAL_ERROR "set STAF_HIP_DIR to a checkout in which `python -m alphanesgpu_amd.build` has been run")
 endif()

@@ -3,25 +3,10 @@ gradients -- once through the CPU oracle and once through the HIP library, with 
 argument mapping (STAF/source_routine/*.py, STAF/gradient_utility/*.py), and returns every tensor of both."""
 import numpy as np
 
+from alphanesgpu_amd.synth import synthetic_upstream  # noqa: F401  (the tests call it through this module)
 from util import species_slices
 
 RC, RA, RS = 4.5, 4.5, 2.25
-
-
-def synthetic_upstream(nf, tipos, params, seed, dtype):
-    """Stand-ins for what the MLP and the loss feed into the ops: G = d(sum e)/dAF ~ N(0,1), P = dL/dAF ~ N(0,1),
-    Q = dL/dF ~ N(0,1)."""
-    rng = np.random.Generator(np.random.Philox(seed))
-    N = int(np.sum(tipos))
-    up = dict(Q=rng.standard_normal((nf, 3 * N)).astype(dtype), G2=[], G3=[], P2=[], P3=[])
-    for k, n in enumerate(tipos):
-        Ar = params[k]["alpha2b"].shape[1]
-        Aa = params[k]["alpha3b"].shape[1] // 3
-        up["G2"].append(rng.standard_normal((nf, int(n), Ar)).astype(dtype))
-        up["G3"].append(rng.standard_normal((nf, int(n), Aa)).astype(dtype))
-        up["P2"].append(rng.standard_normal((nf, int(n), Ar)).astype(dtype))
-        up["P3"].append(rng.standard_normal((nf, int(n), Aa)).astype(dtype))
-    return up
 
 
 def promote(ref, params, up):

@@ -506,8 +506,12 @@ def test_hip_graph_replay_with_two_streams_matches_eager():
             with torch.cuda.stream(streams[k]):
                 streams[k].wait_event(ready)
                 r = chain(k, d)
-                for t in r:
-                    t.record_stream(main)
+                # eager steps tell the allocator that the step's stream reads these; under capture the graph's
+                # private pool keeps them and the returned list holds the references: no allocator event is
+                # queued inside the captured region
+                if not torch.cuda.is_current_stream_capturing():
+                    for t in r:
+                        t.record_stream(main)
                 outs.append(r)
                 done.append(streams[k].record_event())
         for ev in done:
@@ -830,10 +834,47 @@ def test_stale_neighbour_map_is_reported():
     with pytest.raises(_lib.StafError) as e:
         ops.compute_force_radial(*args())
     assert e.value.code == -14
+    # once a remembered map has failed its check the library forgets what it remembered: the same view is now
+    # transposed by the op itself, like the private copy below, and gives that copy's forces
+    f_view = ops.compute_force_radial(*args())
+    f_copy = ops.compute_force_radial(G2, d2[:, :n0].clone(), im2[:, :n0].clone(), rad[:, :n0].clone(),
+                                      T(params[0]["alpha2b"]), T(params[0]["emb2b"]), tm, tp, at)
+    assert torch.equal(f_view, f_copy)
     # a private copy of the modified map is transposed by the op itself: no complaint
     # (clone: a leading slice of a one-frame tensor already is contiguous, .contiguous() would hand back the view)
     ops.compute_force_radial(G2, d2[:, :n0].clone(), im2[:, :n0].clone(), rad[:, :n0].clone(),
                              T(params[0]["alpha2b"]), T(params[0]["emb2b"]), tm, tp, at)
+
+
+def test_scatter_overflow_is_reported():
+    """A neighbour map of unknown origin in which one atom is listed by more centres than the force op's transposed
+    map holds keys for (4 x nr): the op returns STAF_E_SCATTER_OVERFLOW (detected on the device, returned by the
+    host after the op's synchronisation; every kernel runs to its end) and the next valid call is not affected."""
+    import torch
+    from alphanesgpu_amd import ops, _lib
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(5)
+    nf, Nl, N, nr, nt, Ar = 1, 40, 64, 8, 2, 6
+    assert Nl > 4 * nr
+    T = lambda a: torch.as_tensor(np.ascontiguousarray(a)).to(dev)
+    im = np.zeros((nf, Nl, nr + 1), np.int32)
+    im[..., 0] = 2
+    im[..., 1] = 63                                    # every centre names atom 63 in its first slot
+    im[..., 2] = np.arange(Nl)[None, :] % 20 + 40      # and one of atoms 40..59 in its second
+    D = T(rng.uniform(0.1, 1.0, (nf, Nl, nr)))
+    dD = T(rng.standard_normal((nf, Nl, 3, nr)))
+    G = T(rng.standard_normal((nf, Nl, Ar)))
+    al, em = T(rng.uniform(0.5, 2.0, (nt, Ar))), T(rng.uniform(0.2, 1.0, (nt, Ar)))
+    tm = T((np.arange(N) >= Nl).astype(np.int32))
+    tp = T(np.array([Nl, N - Nl], np.int32))
+    at = torch.tensor([0], dtype=torch.int32, device=dev)
+    with pytest.raises(_lib.StafError) as e:
+        ops.compute_force_radial(G, dD, T(im), D, al, em, tm, tp, at)
+    assert e.value.code == -11
+    assert ops.poll_status() == 0                      # reported once, then cleared
+    im[:, 4 * nr:, 1] = 62                             # 32 centres name atom 63: exactly what the map holds
+    f = ops.compute_force_radial(G, dD, T(im), D, al, em, tm, tp, at)
+    assert torch.isfinite(f).all()
 
 
 def test_release_frees_the_work_areas_and_the_next_calls_rebuild_them():

@@ -451,6 +451,12 @@ def test_compute_return_codes():
     w = np.zeros((len(pos), 4), np.int32)
     w[3, 0] = len(pos)
     assert code(x=pos, box=box[0], types=types, howmany=hm, neigh=w) == -9
+    # one atom named by more centres than the force gather holds keys for (4 x the radial buffer): every other atom
+    # of the frame lists atom 0.  Detected on the device, returned by the host; every kernel runs to its end.
+    w[:] = 0
+    w[0, 0] = 1
+    assert len(pos) - 1 > 4 * 60
+    assert code(x=pos, box=box[0], types=types, howmany=hm, neigh=w) == -11
     # a valid call still works afterwards
     e, f, v = m.compute(pos, box[0], types)
     assert abs(e - KNOWN["water_smoke_model_float"]["PE"]) < 2e-4
