@@ -348,6 +348,6 @@ int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* d
                 const real* emb3b, int nt,
                 const int* tipos, const int* actual_type, real* force, const int* numtriplet, const real* alpha3b,
                 const int* type_map, int Nl, real* virial, const real* pos, const real* box, int ld, int skip_pbc,
-                void* stream);
+                void* stream, real* slots_out = nullptr, real* self_out = nullptr);
 
 }  // namespace staf

@@ -310,6 +310,84 @@ __global__ __launch_bounds__(F_BLOCK) void gather_kernel(const real* __restrict_
 }
 
 // ---------------------------------------------------------------------------
+// Total force in one launch: for every atom the 3-body forces of all centre species (what gather_kernel does per
+// species, from the slot forces force3_kernel left) and the per-op force arrays the caller adds to them (the 2-body
+// forces), summed in the order 2-body of species 0, 3-body of species 0, 2-body of species 1, ...  One wave per
+// atom; the lane sums of a species run over the same lanes in the same tree as in gather_kernel, so the result has
+// the bits of the per-op outputs added in that order.  The map must be one the library's own neighbour search
+// wrote (symmetric); atoms are species-sorted, first[k] is the first atom of species k.
+// ---------------------------------------------------------------------------
+template <typename real>
+struct TotalArgs {
+  const real* gslot[NT_MAX];   // [nf, Nl_k, nr, 3] slot forces of centre species k (null: no 3-body term of k)
+  const real* self[NT_MAX];    // [nf, Nl_k, 3]
+  const real* f2[NT_MAX];      // [nf, 3N] a per-op force array added ahead of the 3-body term of species k (or null)
+  int first[NT_MAX + 1];
+  const int* full;             // intmap2b [nf, N, nr+1]
+  real* total;                 // [nf, 3N]
+  int* status;
+  int nf, N, nr, nt;
+};
+
+template <typename real, int NT>   // NT: species the unrolled selections below cover (nt <= NT)
+__global__ __launch_bounds__(F_BLOCK) void force_total_kernel(TotalArgs<real> A) {
+  const int wave = threadIdx.x / WAVE, lane = lane_id();
+  const int recv = blockIdx.x * F_WAVES + wave;
+  if (recv >= A.nf * A.N) return;
+  const int nr = A.nr, N = A.N, nt = A.nt;
+  const int b = recv / N, a = recv - b * N;
+  real acc[NT][3];
+#pragma unroll
+  for (int k = 0; k < NT; k++) acc[k][0] = acc[k][1] = acc[k][2] = 0;
+  const int* mine = A.full + ((size_t)b * N + a) * (nr + 1);
+  int cnt = mine[0];
+  if (cnt > nr) cnt = nr;
+  for (int t = lane; t < nr; t += WAVE) {
+    const int i = mine[1 + t];
+    if (t >= cnt) break;
+    int k = 0;
+#pragma unroll
+    for (int q = 1; q < NT; q++) k += (q < nt && i >= A.first[q]) ? 1 : 0;
+    const real* gs = nullptr;
+#pragma unroll
+    for (int q = 0; q < NT; q++) gs = (q == k) ? A.gslot[q] : gs;
+    if (!gs) continue;
+    const int s = slot_of(A.full, b, N, nr, i, a);
+    if (s < 0) { atomicOr(A.status, 4); continue; }   // a lists i but i does not list a
+    int f0 = 0, f1 = 0;
+#pragma unroll
+    for (int q = 0; q < NT; q++) { f0 = (q == k) ? A.first[q] : f0; f1 = (q == k) ? A.first[q + 1] : f1; }
+    const real* g = gs + (((size_t)b * (f1 - f0) + (i - f0)) * nr + s) * 3;
+    const real g0 = g[0], g1 = g[1], g2 = g[2];
+#pragma unroll
+    for (int q = 0; q < NT; q++) {
+      if (q == k) { acc[q][0] += g0; acc[q][1] += g1; acc[q][2] += g2; }
+    }
+  }
+  real tot = 0;
+  bool have = false;
+#pragma unroll
+  for (int k = 0; k < NT; k++) {
+    if (k >= nt) break;
+    if (A.f2[k]) {
+      real v = 0;
+      if (lane < 3) v = A.f2[k][((size_t)b * N + a) * 3 + lane];
+      tot = have ? tot + v : v;
+      have = true;
+    }
+    if (A.gslot[k]) {
+      const real s0 = wave_sum(acc[k][0]), s1 = wave_sum(acc[k][1]), s2 = wave_sum(acc[k][2]);
+      real o = lane == 0 ? s0 : (lane == 1 ? s1 : s2);
+      const int pl = a - A.first[k];
+      if (lane < 3 && pl >= 0 && a < A.first[k + 1]) o += A.self[k][((size_t)b * (A.first[k + 1] - A.first[k]) + pl) * 3 + lane];
+      tot = have ? tot + o : o;
+      have = true;
+    }
+  }
+  if (lane < 3) A.total[((size_t)b * N + a) * 3 + lane] = tot;
+}
+
+// ---------------------------------------------------------------------------
 // gradient of the 2-body force op.  Q = dL/dF.
 //   w_s   = sum_c (Q[j_s,c] - Q[i,c]) * 1/2 dD_s,c
 //   dG[a]      = sum_s w_s c2 e(1+alpha D)
@@ -516,11 +594,17 @@ int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* d
                 const real* emb3b, int nt,
                 const int* tipos, const int* actual_type, real* force, const int* numtriplet, const real* alpha3b,
                 const int* type_map, int Nl, real* virial, const real* pos, const real* box, int ld, int skip_pbc,
-                void* stream_) {
+                void* stream_, real* slots_out, real* self_out) {
   (void)im3;
   if ((virial || pos || box) && !(virial && pos && box)) return STAF_E_BAD_ARG;
+  // slots_out / self_out: the slot forces [nf, Nl, nr, 3] and the centres' own forces [nf, Nl, 3] go to the caller
+  // instead of the library's work area and no atom gathers them here (force is not written and may be null)
+  const bool deferred = slots_out != nullptr;
+  if (deferred && (!self_out || virial)) return STAF_E_BAD_ARG;
+  if (deferred && Nl == 0) return STAF_OK;
   if (Nl == 0 && nf > 0 && N > 0 && force) return empty_species_force<real>(force, virial, nf, N, stream_);
-  if (!G || !Dsup || (!unit && (!Tang || !d3b)) || !dDsup || !im2 || !emb3b || !tipos || !actual_type || !force ||
+  if (!G || !Dsup || (!unit && (!Tang || !d3b)) || !dDsup || !im2 || !emb3b || !tipos || !actual_type ||
+      (!force && !deferred) ||
       !numtriplet || !alpha3b || !type_map || nr <= 0 || na <= 0 || N <= 0 || nf <= 0 || Aa <= 0 || nt <= 0 ||
       Nl <= 0 || Nl > N)
     return STAF_E_BAD_ARG;
@@ -532,12 +616,12 @@ int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* d
   if (!Force3Cfg<real, 4>::fits(nr, nt) || N >= (1 << (31 - KEY_SLOT_BITS))) return STAF_E_LIMIT;
   TransposeRef tr;
   bool cached = false;
-  int rc = force_transpose(st, im2, nf, N, Nl, ld, nr, stream, &tr, &cached);
+  int rc = deferred ? STAF_OK : force_transpose(st, im2, nf, N, Nl, ld, nr, stream, &tr, &cached);
   if (rc) return rc;
   const size_t ng = (size_t)nf * Nl * nr * 3, ns = (size_t)nf * Nl * 3, nv = virial ? (size_t)nf * Nl * 9 : 0;
-  real* gslot = (real*)scratch_reserve(st, stream, (ng + ns + nv) * sizeof(real));
+  real* gslot = deferred ? slots_out : (real*)scratch_reserve(st, stream, (ng + ns + nv) * sizeof(real));
   if (!gslot) return reserve_failure(stream);
-  real* self = gslot + ng;
+  real* self = deferred ? self_out : gslot + ng;
   real* vpart = self + ns;
   const bool fused = unit != nullptr;   // the MD entry: T and its Jacobian rebuilt from the unit vectors
   // Single precision: eight waves per workgroup (a wave's registers then admit eight waves per SIMD, and a centre's
@@ -561,6 +645,7 @@ int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* d
   };
   rc = fused ? launch(std::integral_constant<bool, true>{}) : launch(std::integral_constant<bool, false>{});
   if (rc) return rc;
+  if (deferred) return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
   if (virial) {
     const int atoms = nf * Nl;
     hipLaunchKernelGGL(virial_centre_kernel<real>, dim3((atoms + F_WAVES - 1) / F_WAVES), dim3(F_BLOCK), 0, stream,
@@ -585,7 +670,7 @@ template int force_tripl<double>(const double*, const double*, const double*, co
                                  const double*, const int*, const int*, int, int, int, int, int, const double*, int,
                                  const int*,
                                  const int*, double*, const int*, const double*, const int*, int, double*,
-                                 const double*, const double*, int, int, void*);
+                                 const double*, const double*, int, int, void*, double*, double*);
 
 template <typename real>
 static int gradforce_2b(const real* Q, const real* D, int nr, const real* alpha2b, int Ar, const real* dD,
@@ -669,6 +754,110 @@ static int gradforce_tripl(const real* Q, const real* G, const real* Dsup, const
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }
 
+template <typename real>
+static int force_total(const int* im2_full, int nr, int N, int nf, int nt, const int* n_local,
+                       const real* const* slot_forces, const real* const* self_forces, const real* const* force_2b,
+                       real* total, void* stream_) {
+  if (!im2_full || !n_local || !slot_forces || !self_forces || !total || nr <= 0 || N <= 0 || nf <= 0 || nt <= 0)
+    return STAF_E_BAD_ARG;
+  if (nt > NT_MAX) return STAF_E_LIMIT;
+  hipStream_t stream = (hipStream_t)stream_;
+  DeviceState* st = device_state(stream);
+  if (!st) return reserve_failure(stream);
+  TotalArgs<real> A;
+  int sum = 0;
+  bool any = false;
+  for (int k = 0; k < NT_MAX; k++) {
+    A.first[k] = sum;
+    A.gslot[k] = A.self[k] = A.f2[k] = nullptr;
+    if (k >= nt) continue;
+    if (n_local[k] < 0) return STAF_E_BAD_ARG;
+    if (n_local[k] > 0 && slot_forces[k]) {
+      if (!self_forces[k]) return STAF_E_BAD_ARG;
+      A.gslot[k] = slot_forces[k];
+      A.self[k] = self_forces[k];
+      any = true;
+    }
+    if (force_2b && force_2b[k]) { A.f2[k] = force_2b[k]; any = true; }
+    sum += n_local[k];
+  }
+  A.first[NT_MAX] = sum;
+  for (int k = nt; k < NT_MAX; k++) A.first[k] = sum;
+  if (sum != N) return STAF_E_BAD_ARG;
+  if (!any) {
+    launch_fill_zero<real>(total, nf * 3 * N, stream);
+    return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
+  }
+  // the slots that list an atom are found through the atom's own row: only a map the library's own neighbour search
+  // wrote, and remembers, is known to be symmetric
+  TransposeRef tr;
+  if (!transpose_find(st, im2_full, nf, N, N, N, nr, &tr) || !tr.symmetric || tr.key_shift != 0) return STAF_E_BAD_ARG;
+  A.full = im2_full; A.total = total; A.status = status_word(st, stream);
+  A.nf = nf; A.N = N; A.nr = nr; A.nt = nt;
+  {
+    KernelTimer kt_("force_total_kernel", stream);
+    const int recv = nf * N;
+    const dim3 grid((recv + F_WAVES - 1) / F_WAVES);
+    if (nt <= 2) hipLaunchKernelGGL((force_total_kernel<real, 2>), grid, dim3(F_BLOCK), 0, stream, A);
+    else if (nt <= 4) hipLaunchKernelGGL((force_total_kernel<real, 4>), grid, dim3(F_BLOCK), 0, stream, A);
+    else hipLaunchKernelGGL((force_total_kernel<real, NT_MAX>), grid, dim3(F_BLOCK), 0, stream, A);
+  }
+  return finish_op(st, stream);
+}
+
+// Both 3-body parameter gradients of a training step in one pass (tri_reduce_kernel<3>): the gradient of the force
+// op (gradnet, dL/dalpha3b from dL/dF) and the gradient of the fingerprint op (dL/dalpha3b from dL/dAF3).  Outputs
+// as the two separate ops give them; the embedding gradient (identically zero in both, as in the reference) once.
+template <typename real>
+static int grads_tripl_fused(const real* Q, const real* G, const real* PE, const real* Dsup, const real* Tang,
+                             const real* dDsup, const real* d3b, const int* im2, const int* im3, int nr, int na, int N,
+                             int nf, int Aa, const real* emb3b, int nt, const int* tipos, const int* actual_type,
+                             const int* numtriplet, const real* alpha3b, const int* type_map, int Nl, real* gnet,
+                             real* g_alpha_force, real* g_alpha_energy, real* g_emb, const real* Qvir, const real* pos,
+                             const real* box, int ld, int skip_pbc, void* stream_) {
+  (void)im3;
+  if ((Qvir || pos || box) && !(Qvir && pos && box)) return STAF_E_BAD_ARG;
+  const int ntc = nt * (nt + 1) / 2;
+  if (Nl == 0 && nf > 0 && Aa > 0 && nt > 0 && g_alpha_force && g_alpha_energy && g_emb) {
+    launch_fill_zero<real>(g_alpha_force, ntc * Aa * 3, (hipStream_t)stream_);
+    launch_fill_zero<real>(g_alpha_energy, ntc * Aa * 3, (hipStream_t)stream_);
+    launch_fill_zero<real>(g_emb, ntc * Aa, (hipStream_t)stream_);
+    return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
+  }
+  if (!Q || !G || !PE || !Dsup || !Tang || !dDsup || !d3b || !im2 || !emb3b || !tipos || !actual_type || !numtriplet ||
+      !alpha3b || !type_map || !gnet || !g_alpha_force || !g_alpha_energy || !g_emb || nr <= 0 || na <= 0 || N <= 0 ||
+      nf <= 0 || Aa <= 0 || nt <= 0 || Nl <= 0 || Nl > N)
+    return STAF_E_BAD_ARG;
+  if (nt > NT_MAX) return STAF_E_LIMIT;
+  if (ld <= 0) ld = Nl;
+  DeviceState* st = device_state((hipStream_t)stream_);
+  if (!st) return reserve_failure((hipStream_t)stream_);
+  hipStream_t stream = (hipStream_t)stream_;
+  const int nsig = 2 * nt - 1;
+  const int nacc = nsig * Aa * 3, nout = 2 * nacc;
+  const int nb_max = nf * Nl < TRI_GRID_MAX ? nf * Nl : TRI_GRID_MAX;   // the work area does not depend on occupancy
+  real* partial = (real*)scratch_reserve(st, stream, (size_t)nb_max * nout * sizeof(real));
+  if (!partial) return reserve_failure(stream);
+  size_t lds = TriLds<real, 3>::bytes(nr, Aa, nt);
+  if (!lds_request(tri_reduce_kernel<real, 3>, lds)) return STAF_E_LIMIT;
+  const int nb = tri_grid((const void*)tri_reduce_kernel<real, 3>, lds, nf * Nl);
+  const int nall = ntc * Aa * 3;
+  TriArgs<real> A = {};
+  A.Dsup = Dsup; A.Tang = Tang; A.im2 = im2; A.alpha3b = alpha3b; A.emb3b = emb3b; A.type_map = type_map;
+  A.numtriplet = numtriplet; A.P = G; A.PE = PE; A.Q = Q; A.dDsup = dDsup; A.d3b = d3b; A.tipos = tipos;
+  A.actual_type = actual_type; A.out = gnet; A.partial = partial; A.Qvir = Qvir; A.pos = pos; A.box = box;
+  A.skip_pbc = skip_pbc;
+  A.nf = nf; A.N = N; A.Nl = Nl; A.ld = ld; A.nr = nr; A.na = na; A.Aa = Aa; A.nt = nt;
+  {
+    KernelTimer kt_("grads3_kernel", stream);
+    hipLaunchKernelGGL((tri_reduce_kernel<real, 3>), dim3(nb), dim3(TRI_BLOCK), lds, stream, A);
+  }
+  // rows sigma >= nsig of both parameter gradients and the embedding gradient are zero-filled by the same launch
+  launch_reduce_partials<real>(partial, nb, nout, g_alpha_force, nacc, nall, g_alpha_energy, nacc, nall, nullptr, stream,
+                               g_emb, 0, ntc * Aa);
+  return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
+}
+
 }  // namespace staf
 
 extern "C" {
@@ -695,7 +884,27 @@ void staf_op_force_set_skip_pbc(int skip) { staf::g_force_skip_pbc = skip ? 1 : 
                                    intmap_a, nr, na, N,                                                                \
                                    dimbat, num_finger, type_emb3b, nt, tipos, actual_type, forces3b, num_triplets,     \
                                    smooth_a, type_map, N_local, virial, pos, box, ld_atoms, staf::g_force_skip_pbc,    \
-                                   stream);                                                                            \
+                                   stream, (real*)nullptr, (real*)nullptr);                                            \
+  }                                                                                                                    \
+  int staf_op_force_tripl_slots_##SFX(const real* netderiv, const real* desr, const real* desa,                        \
+                                      const real* intderiv_r, const real* intderiv_a, const int* intmap_r,             \
+                                      const int* intmap_a, int nr, int na, int N, int dimbat, int num_finger,          \
+                                      const real* type_emb3b, int nt, const int* tipos, const int* actual_type,        \
+                                      real* slot_forces, real* self_forces, const int* num_triplets,                   \
+                                      const real* smooth_a, const int* type_map, int N_local, int ld_atoms,            \
+                                      void* stream) {                                                                  \
+    if (!slot_forces || !self_forces) return STAF_E_BAD_ARG;                                                           \
+    return staf::force_tripl<real>(netderiv, desr, desa, intderiv_r, intderiv_a, (const real*)nullptr, intmap_r,      \
+                                   intmap_a, nr, na, N, dimbat, num_finger, type_emb3b, nt, tipos, actual_type,        \
+                                   (real*)nullptr, num_triplets, smooth_a, type_map, N_local, (real*)nullptr,          \
+                                   (const real*)nullptr, (const real*)nullptr, ld_atoms, staf::g_force_skip_pbc,       \
+                                   stream, slot_forces, self_forces);                                                  \
+  }                                                                                                                    \
+  int staf_op_force_total_##SFX(const int* intmap_r_full, int nr, int N, int dimbat, int nt, const int* n_local,       \
+                                const real* const* slot_forces, const real* const* self_forces,                        \
+                                const real* const* forces2b, real* total, void* stream) {                              \
+    return staf::force_total<real>(intmap_r_full, nr, N, dimbat, nt, n_local, slot_forces, self_forces, forces2b,      \
+                                   total, stream);                                                                     \
   }                                                                                                                    \
   int staf_op_gradforce_2b_##SFX(const real* prevgrad, const real* radiale, int nr, const real* alpha_radiale,         \
                                  int num_finger, const real* desder, const int* intmap_r, int dimbat, int N,           \
@@ -724,5 +933,22 @@ void staf_op_force_set_skip_pbc(int skip) { staf::g_force_skip_pbc = skip ? 1 : 
 
 STAF_FORCE_ENTRY(float, f32)
 STAF_FORCE_ENTRY(double, f64)
+
+#define STAF_FUSED_GRAD_ENTRY(real, SFX)                                                                               \
+  int staf_op_grads_tripl_fused_##SFX(                                                                                 \
+      const real* prevgrad_force, const real* netderiv, const real* prevgrad_energy, const real* desr,                 \
+      const real* desa, const real* intderiv_r, const real* intderiv_a, const int* intmap_r, const int* intmap_a,      \
+      int nr, int na, int N, int dimbat, int num_finger, const real* type_emb3b, int nt, const int* tipos,             \
+      const int* actual_type, const int* num_triplets, const real* smooth_a, const int* type_map, int N_local,         \
+      real* gradnet_3b, real* grad_alpha3b_force, real* grad_alpha3b_energy, real* grad_emb3b,                         \
+      const real* prevgrad_virial, const real* pos, const real* box, int ld_atoms, void* stream) {                     \
+    return staf::grads_tripl_fused<real>(prevgrad_force, netderiv, prevgrad_energy, desr, desa, intderiv_r,            \
+                                         intderiv_a, intmap_r, intmap_a, nr, na, N, dimbat, num_finger, type_emb3b,    \
+                                         nt, tipos, actual_type, num_triplets, smooth_a, type_map, N_local,            \
+                                         gradnet_3b, grad_alpha3b_force, grad_alpha3b_energy, grad_emb3b,              \
+                                         prevgrad_virial, pos, box, ld_atoms, staf::g_force_skip_pbc, stream);         \
+  }
+STAF_FUSED_GRAD_ENTRY(float, f32)
+STAF_FUSED_GRAD_ENTRY(double, f64)
 
 }  // extern "C"

@@ -14,7 +14,7 @@
 //       Sd += h (1 + beta T) P                          h = 1/4 G c3 e^{beta T}   (1/2 of E, 1/2 of T)
 //       U  += h (a1 + a2) P     V += h (a1 - a2) M
 //       SBj = (U + V)/2 = sum h (a1 sim2 + a2 sim1)     SBk = (U - V)/2          (times T at the end)
-//     The table is stored row-major ([row][channel], rows padded by one entry against bank conflicts) and the
+//     The table is stored row-major ([row][channel], rows padded against bank conflicts, see ROWP) and the
 //     channel loop is unrolled, so that every LDS read of the loop is a per-triplet base address plus an
 //     immediate offset.
 //   * der3b contraction in the same lanes: the contributions to slot j of a pass form contiguous lane groups
@@ -65,7 +65,15 @@ struct Force3Cfg {
   static constexpr int THREADS = NW * WAVE;
   static constexpr int NP = 16 / NW;                        // passes of 64 triplets a wave holds in registers
   static constexpr int CAP = sizeof(real) == 8 ? 8 : 16;    // channels tabulated at a time
-  static constexpr int CAPP = CAP + 1;                      // table row pitch in entries
+  // Exponential table: one row per (partner species, slot), ROWP reals long.
+  //   float:  (x, y) pairs of the CAP channels, then one pair of padding: 8-byte reads, rows 136 bytes apart
+  //   double: the CAP x values, the CAP y values, one real of padding: two 8-byte reads per entry (one instruction
+  //           with two offsets), rows 136 bytes apart as well
+  // With 136 = 8 x 17 bytes between the rows of consecutive slots, the 8-byte reads of the lanes of a wave -- a few
+  // runs of consecutive slots, since a wave's triplets span two or three rows of the triplet triangle -- fall on the
+  // same banks only for slots 32 apart.  (16-byte entries in double precision, 144 bytes apart, collide for slots
+  // 16 apart: measured 1.9 conflict cycles per LDS instruction of the whole kernel.)
+  static constexpr int ROWP = sizeof(real) == 8 ? 2 * CAP + 1 : 2 * (CAP + 1);
   // der3b rows requested one sweep ahead and held in registers across the channel loop: measured, no gain in
   // fp32 (the kernel is bound by vector-ALU issue) and slower in fp64 (a third of the resident waves lost)
   // (measured and not faster either: the rows of a wave's first pass alone requested ahead of the channel loop,
@@ -78,9 +86,15 @@ struct Force3Cfg {
   static constexpr int MIN_WAVES = NW == 8 ? (sizeof(real) == 8 ? 6 : 8) : (sizeof(real) == 8 ? 4 : 6);
   __host__ __device__ static bool fits(int nr, int nt) { return nr <= 255 && nt <= NT_MAX; }   // slots packed in 8 bits
   __host__ __device__ static int pitch(int Aa) { return (Aa + 3) & ~3; }   // parameter row pitch (channels)
+  // Distance, in channels, between the weight rows of consecutive sigma.  The lanes of a wave read the 16- or 32-byte
+  // entry of one channel from the rows of two or three different sigma at once: with a row of pitch(Aa) entries
+  // (a multiple of 128 bytes for the usual channel counts) those entries would share their banks; one entry more
+  // puts consecutive rows one entry apart.
+  __host__ __device__ static int rowp(int Aa) { return pitch(Aa) + 1; }
   __host__ __device__ static size_t n_reals(int nr, int Aa, int nt, bool fused = false) {
     const int nsig = 2 * nt - 1;
-    return (size_t)nsig * pitch(Aa) * 6 /*prm, prE*/ + (((size_t)CAPP * nt * nr + 1) & ~(size_t)1) * 2 /*E*/ +
+    return (size_t)nsig * rowp(Aa) * 4 /*prm*/ + (size_t)nsig * pitch(Aa) * 2 /*prE*/ +
+           (((size_t)ROWP * nt * nr + 1) & ~(size_t)1) /*E*/ +
            (size_t)NW * 4 * nr /*slot sums per wave*/ + nr /*D*/ + 3 * nr /*grad fc*/ +
            (size_t)NW * 4 /*the waves' shares of the centre's own force*/ + (fused ? 4 * nr : 0) /*unit vectors, 1/r*/;
   }
@@ -106,15 +120,15 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
   using real4 = typename Vec4<real>::type;
   using HE = HotExp<real>;
   using L = Force3Cfg<real, NWAVES>;
-  constexpr int NP = L::NP, NW = L::NW, THREADS = L::THREADS, CAP = L::CAP, CAPP = L::CAPP;
+  constexpr int NP = L::NP, NW = L::NW, THREADS = L::THREADS, CAP = L::CAP, ROWP = L::ROWP;
   extern __shared__ __align__(16) unsigned char smem[];
   const int nsig = 2 * nt - 1;
   const int RT = nt * nr;                                  // table rows (tb, s)
-  const int Ap = L::pitch(Aa);
-  real* prm = (real*)smem;                                 // [nsig*Ap][4] = a1+a2, a1-a2, scaled beta, 1/4 G c3 (active channels)
-  real* prE = prm + (size_t)nsig * Ap * 4;                 // [nsig*Ap][2] = a1, a2 in the units of the hot exponential
-  real2* E = (real2*)(prE + (size_t)nsig * Ap * 2);        // [RT][CAPP]
-  real* acc = (real*)(E + (((size_t)RT * CAPP + 1) & ~(size_t)1));   // [NW][nr][4]: per wave, slot sums (as j and as k)
+  const int Ap = L::pitch(Aa), Apr = L::rowp(Aa);
+  real* prm = (real*)smem;                                 // [nsig][Apr][4] = a1+a2, a1-a2, scaled beta, 1/4 G c3 (active channels)
+  real* prE = prm + (size_t)nsig * Apr * 4;                // [nsig*Ap][2] = a1, a2 in the units of the hot exponential
+  real* E = prE + (size_t)nsig * Ap * 2;                   // [RT][ROWP], see Force3Cfg::ROWP
+  real* acc = E + (((size_t)RT * ROWP + 1) & ~(size_t)1);  // [NW][4 nr]: per wave, slot sums (as j and as k), see accW
   real* sD = acc + (size_t)NW * 4 * nr;                    // [nr]
   real* sg = sD + nr;                                      // [3*nr] grad fc (der3bsupp)
   real* xch = sg + 3 * nr;                                 // [NW][4] the waves' shares of the centre's own force
@@ -134,7 +148,30 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
   if (ntri > na) ntri = na;
   const real* Trow = Tang + rowAtom * na;
   const real2* d3 = (const real2*)d3b + rowAtom * 3 * na;
-  real4* accW = (real4*)(acc + (size_t)wave * 4 * nr);   // [nr] x (force x, y, z, radial factor)
+  // A wave's slot sums (force x, y, z, radial factor).  Single precision: one 16-byte entry per slot.  Double
+  // precision: two arrays of 16-byte halves, (x, y) and (z, w), so that the lanes of a row, which hold consecutive
+  // slots, read consecutive 16-byte words (32-byte entries would put every other lane on the same banks).
+  real* accW = acc + (size_t)wave * 4 * nr;
+  auto acc_get = [&](const real* base, int s_) -> real4 {
+    if constexpr (sizeof(real) == 8) {
+      const real2 a = ((const real2*)base)[s_], b2 = ((const real2*)base)[nr + s_];
+      real4 t;
+      t.x = a.x; t.y = a.y; t.z = b2.x; t.w = b2.y;
+      return t;
+    } else {
+      return ((const real4*)base)[s_];
+    }
+  };
+  auto acc_put = [&](real* base, int s_, const real4& t) {
+    if constexpr (sizeof(real) == 8) {
+      real2 a, b2;
+      a.x = t.x; a.y = t.y; b2.x = t.z; b2.y = t.w;
+      ((real2*)base)[s_] = a;
+      ((real2*)base)[nr + s_] = b2;
+    } else {
+      ((real4*)base)[s_] = t;
+    }
+  };
 
   // ---- set-up.  Global reads are issued back to back in two levels: (1) everything addressed by the centre alone,
   // the neighbour index first (read up to nr: padded slots are never used); (2) the neighbour's species, which
@@ -183,23 +220,23 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
       const bool on = (a < Aa) && (c != real(0));
       const unsigned long long mask = __ballot(on);
       if (on) {
-        const int ch = sgm * Ap + base + __popcll(mask & ((1ull << lane) - 1ull));
+        const int cpos = base + __popcll(mask & ((1ull << lane) - 1ull));
         real4 o;
         o.x = al0 + al1;
         o.y = al0 - al1;
         o.z = HE::scale(al2);   // beta in the units of the hot exponential
         o.w = real(0.25) * gv * c;
-        *(real4*)(prm + (size_t)ch * 4) = o;
+        *(real4*)(prm + (size_t)(sgm * Apr + cpos) * 4) = o;
         real2 e;
         e.x = HE::scale(al0);
         e.y = HE::scale(al1);
-        *(real2*)(prE + (size_t)ch * 2) = e;
+        *(real2*)(prE + (size_t)(sgm * Ap + cpos) * 2) = e;
       }
       base += __popcll(mask);
     }
     // Rows are Ap long and zero beyond the active channels: a triplet whose sigma has fewer channels than the
     // workgroup's maximum reads weight 0 (and exponent 0: table entries 1) there.
-    for (int q = base * 4 + lane; q < Ap * 4; q += WAVE) prm[(size_t)sgm * Ap * 4 + q] = 0;
+    for (int q = base * 4 + lane; q < Ap * 4; q += WAVE) prm[(size_t)sgm * Apr * 4 + q] = 0;
     for (int q = base * 2 + lane; q < Ap * 2; q += WAVE) prE[(size_t)sgm * Ap * 2 + q] = 0;
     if (lane == 0) nact[sgm] = base;
   }
@@ -258,9 +295,9 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
           T[p] = Tn[p];
         }
         const int tj = stp[j], tk = stp[k];
-        rj[p] = mul24(mul24(tk, nr) + j, CAPP);
-        rk[p] = mul24(mul24(tj, nr) + k, CAPP);
-        rp[p] = mul24(tj + tk, Ap * 4);
+        rj[p] = mul24(mul24(tk, nr) + j, ROWP);
+        rk[p] = mul24(mul24(tj, nr) + k, ROWP);
+        rp[p] = mul24(tj + tk, Apr * 4);
         jk[p] = j | (k << 8);
       }
     }
@@ -281,7 +318,13 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
               real2 v;
               v.x = HE::eval(o.x * d);
               v.y = HE::eval(o.y * d);
-              E[mul24(mul24(tb, nr) + s_, CAPP) + ia] = v;
+              real* row = E + mul24(mul24(tb, nr) + s_, ROWP);
+              if constexpr (sizeof(real) == 8) {
+                row[ia] = v.x;
+                row[CAP + ia] = v.y;
+              } else {
+                ((real2*)row)[ia] = v;
+              }
             }
           }
         }
@@ -291,9 +334,19 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
       // the LDS reads of the next items are in flight while the current ones are computed.
       auto channels = [&](auto npass_c) {
         constexpr int NPASS = decltype(npass_c)::value;
-        const real2* pj[NPASS];
-        const real2* pk[NPASS];
+        const real* pj[NPASS];
+        const real* pk[NPASS];
         const real* po[NPASS];
+        auto entry = [](const real* row, int c) -> real2 {   // (exp(a1 D), exp(a2 D)) of channel c of a table row
+          if constexpr (sizeof(real) == 8) {
+            real2 v;
+            v.x = row[c];
+            v.y = row[CAP + c];
+            return v;
+          } else {
+            return ((const real2*)row)[c];
+          }
+        };
 #pragma unroll
         for (int p = 0; p < NPASS; p++) {
           pj[p] = E + rj[p];
@@ -313,8 +366,8 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
 #pragma unroll
             for (int p = 0; p < NPASS; p++) {
               const real4 o = *(const real4*)(po[p] + (ia + u) * 4);   // a1+a2, a1-a2, scaled beta, weight
-              const real2 e1 = pj[p][ia + u];
-              const real2 e2 = pk[p][ia + u];
+              const real2 e1 = entry(pj[p], ia + u);
+              const real2 e2 = entry(pk[p], ia + u);
               const real bts = o.z * T[p];
               const real h = HE::eval(bts) * o.w;
               const real sim1 = e1.y * e2.x;                      // exp(a2 Dj + a1 Dk)
@@ -442,12 +495,12 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
       const int jn = __shfl_down(valid ? j : -1, 1, WAVE);
       const bool row_end = valid && (lane == WAVE - 1 || jn != j);
       if (row_end) {
-        real4 t = accW[j];
+        real4 t = acc_get(accW, j);
         t.x += vj[0] - (first > 0 ? pre[0] : real(0));
         t.y += vj[1] - (first > 0 ? pre[1] : real(0));
         t.z += vj[2] - (first > 0 ? pre[2] : real(0));
         t.w += vj[3] - (first > 0 ? pre[3] : real(0));
-        accW[j] = t;
+        acc_put(accW, j, t);
       }
       __builtin_amdgcn_wave_barrier();   // the wave's memory operations stay in program order: slot k sums follow
       // slot k: row by row (the k of one row are distinct).  LDS floating-point adds instead of this loop were
@@ -457,9 +510,9 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
       const int jhi = __builtin_amdgcn_readlane(j, llast);
       for (int g = jlo; g <= jhi; g++) {
         if (valid && j == g) {
-          real4 t = accW[k];
+          real4 t = acc_get(accW, k);
           t.x += vk[0]; t.y += vk[1]; t.z += vk[2]; t.w += vk[3];
-          accW[k] = t;
+          acc_put(accW, k, t);
         }
         __builtin_amdgcn_wave_barrier();
       }
@@ -473,7 +526,7 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
     real t4[4] = {0, 0, 0, 0};
 #pragma unroll
     for (int w = 0; w < NW; w++) {
-      const real4 a = ((const real4*)(acc + (size_t)w * 4 * nr))[tid];
+      const real4 a = acc_get(acc + (size_t)w * 4 * nr, tid);
       t4[0] += a.x; t4[1] += a.y; t4[2] += a.z; t4[3] += a.w;
     }
 #pragma unroll

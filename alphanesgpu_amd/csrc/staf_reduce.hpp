@@ -13,12 +13,15 @@ constexpr int RED_SLICES = 32;  // rows callers still reserve behind their parti
 // of a wavefront are combined by a butterfly over the lane bits above the element index, the four wavefronts'
 // sums in ascending order by the first lanes.  One launch instead of a sliced first pass and a final one: the
 // partial rows are a few MB and a segment's column a few hundred KB, which one CU reads in the time a launch costs.
-// Element e of the padded output space [0, z0) -> out0, [z0, z0+z1) -> out1: e < n0 takes column e, z0 <= e < z0+n1
-// column n0 + (e - z0), the rest is written as zero (z0 >= n0, z1 >= n1; out1 may be null when z1 == 0).
+// The padded output space is a sequence of up to three pieces: piece i takes the next n[i] columns of the partial
+// rows and is z[i] >= n[i] elements long, the rest written as zero (a piece with n = 0 is a zero fill).
+struct ReduceOut {
+  void* out[3];
+  int n[3], z[3];
+};
 template <typename real>
 __global__ __launch_bounds__(RED_THREADS) void reduce_partials_kernel(const real* __restrict__ partial, int nblocks,
-                                                                      int nout, real* out0, int n0, int z0, real* out1,
-                                                                      int n1, int z1) {
+                                                                      int nout, ReduceOut O) {
   constexpr int EL = 64 / (int)sizeof(real);
   constexpr int PARTS = RED_THREADS / EL;
   constexpr int NWV = RED_THREADS / WAVE;
@@ -26,7 +29,10 @@ __global__ __launch_bounds__(RED_THREADS) void reduce_partials_kernel(const real
   const int tid = threadIdx.x;
   const int el = tid % EL, part = tid / EL;
   const int e = blockIdx.x * EL + el;
-  const int src = e < z0 ? (e < n0 ? e : -1) : ((e - z0) < n1 ? n0 + (e - z0) : -1);
+  // piece and position of element e, column of the partial rows it sums (-1: padding)
+  int piece = 0, at = e, col0 = 0;
+  while (piece < 2 && at >= O.z[piece]) { at -= O.z[piece]; col0 += O.n[piece]; piece++; }
+  const int src = at < O.n[piece] ? col0 + at : -1;
   real s = 0;
   if (src >= 0 && src < nout) {
     int g = part;
@@ -47,20 +53,24 @@ __global__ __launch_bounds__(RED_THREADS) void reduce_partials_kernel(const real
     real t = 0;
 #pragma unroll
     for (int w = 0; w < NWV; w++) t += sh[w][tid];
-    if (e < z0) out0[e] = t;
-    else if (e - z0 < z1) out1[e - z0] = t;
+    if (at < O.z[piece]) ((real*)O.out[piece])[at] = t;
   }
 }
 
 // tmp is not used (callers reserve it with their partial rows).
 template <typename real>
 inline void launch_reduce_partials(const real* partial, int nblocks, int nout, real* out0, int n0, int z0, real* out1,
-                                   int n1, int z1, real* tmp, hipStream_t stream) {
+                                   int n1, int z1, real* tmp, hipStream_t stream, real* out2 = nullptr, int n2 = 0,
+                                   int z2 = 0) {
   (void)tmp;
   constexpr int EL = 64 / (int)sizeof(real);
-  const int etot = z0 + z1;
+  const int etot = z0 + z1 + z2;
+  ReduceOut O;
+  O.out[0] = out0; O.n[0] = n0; O.z[0] = z0;
+  O.out[1] = out1; O.n[1] = n1; O.z[1] = z1;
+  O.out[2] = out2; O.n[2] = n2; O.z[2] = z2;
   hipLaunchKernelGGL(reduce_partials_kernel<real>, dim3((etot + EL - 1) / EL), dim3(RED_THREADS), 0, stream, partial,
-                     nblocks, nout, out0, n0, z0, out1, n1, z1);
+                     nblocks, nout, O);
 }
 
 template <typename real>

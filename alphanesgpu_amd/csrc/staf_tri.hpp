@@ -1,7 +1,10 @@
 // Triplet kernels that reduce over an atom's triplets: 3-body fingerprints
-// (MODE 0), their parameter gradient (MODE 1) and the gradient of the 3-body
-// force op (MODE 2).  One 256-thread workgroup per centre atom (persistent
-// over atoms for the gradient modes).  These kernels are bound by vector-ALU
+// (MODE 0), their parameter gradient (MODE 1), the gradient of the 3-body
+// force op (MODE 2), and both gradients in one pass (MODE 3: a training step
+// needs both, and everything but the last few accumulations per item -- set-up,
+// tables, staging, the exponential, the pair factors -- is shared).  One
+// 256-thread workgroup per centre atom (persistent over atoms for the gradient
+// modes).  These kernels are bound by vector-ALU
 // issue, so the layout below is chosen to keep the instruction count per
 // (triplet, channel) item low.
 //
@@ -43,10 +46,15 @@ constexpr int TRI_CAPP = TRI_CAP + 1;   // table row pitch: the entry after a ro
 constexpr int TRI_SUBS = TRI_BLOCK / TRI_CAP;
 template <typename real, int MODE>
 struct TriCfg {
-  static constexpr int QB = 512;   // triplets staged per block
+  // triplets staged per block.  The double-precision pass that gives both gradients stages half as many: with 512
+  // its LDS footprint would admit three workgroups per CU instead of four.
+  static constexpr int QB = (MODE == 3 && sizeof(real) == 8) ? 256 : 512;
   // waves per SIMD the register allocation is held to: without a bound the allocation comes out a few registers
   // above the next occupancy step (the fused double-precision fingerprint kernel is held to four)
-  static constexpr int MIN_WAVES = sizeof(real) == 8 ? (MODE == 0 ? 5 : 4) : (MODE == 0 ? 8 : MODE == 1 ? 7 : 5);
+  static constexpr int MIN_WAVES = sizeof(real) == 8 ? (MODE == 0 ? 5 : 4)
+                                                     : (MODE == 0 ? 8 : MODE == 1 ? 7 : MODE == 3 ? 4 : 5);
+  static constexpr bool FORCE_BRANCH = MODE == 2 || MODE == 3;    // dL/dF comes in: der3b, der3bsupp are read
+  static constexpr bool ENERGY_BRANCH = MODE == 1 || MODE == 3;   // dL/dAF3 comes in
 };
 constexpr int TRI_GRID_MAX = 2048;  // workgroups of the persistent gradient modes (one partial row each)
 
@@ -149,8 +157,9 @@ struct TriArgs {
   const real* emb3b;      // [ntc, Aa]
   const int* type_map;    // [N]
   const int* numtriplet;  // [nf, ld]
-  const real* P;          // MODE 1: dL/dAF3, MODE 2: netderiv  [nf, Nl, Aa] contiguous
-  const real* Q;          // MODE 2: dL/dF [nf, 3N]
+  const real* P;          // MODE 1: dL/dAF3, MODE 2 and 3: netderiv  [nf, Nl, Aa] contiguous
+  const real* PE;         // MODE 3: dL/dAF3 [nf, Nl, Aa] contiguous
+  const real* Q;          // MODE 2, 3: dL/dF [nf, 3N]
   const real* dDsup;      // MODE 2: der3bsupp [nf, ld, 3, nr]
   const real* d3b;        // MODE 2: der3b [nf, ld, 3, na, 2]
   const int* tipos;       // MODE 2
@@ -159,8 +168,8 @@ struct TriArgs {
   const real* pos;        // MODE 2, virial form: positions [nf, 3N]
   const real* box;        // MODE 2, virial form: [nf, 6]
   int skip_pbc;           // MODE 2, virial form: no minimum-image wrap
-  real* out;              // MODE 0: AF3, MODE 2: gradnet  [nf, Nl, Aa] contiguous
-  real* partial;          // MODE 1/2: [gridDim.x, nsig*Aa*3]
+  real* out;              // MODE 0: AF3, MODE 2, 3: gradnet  [nf, Nl, Aa] contiguous
+  real* partial;          // MODE 1, 2: [gridDim.x, nsig*Aa*3]; MODE 3: [gridDim.x, 2, nsig*Aa*3] force branch, energy branch
   int nf, N, Nl, ld, nr, na, Aa, nt;
 };
 
@@ -173,8 +182,9 @@ struct TriArgs {
 //   double, force gradient:             {T, U} 16 bytes in one array, ab in a second one
 template <typename real, int MODE>
 struct TriStage {
-  static constexpr bool SPLIT = MODE == 2 && sizeof(real) == 8;
-  static constexpr int BYTES = SPLIT ? 20 : ((sizeof(real) == 4 && MODE != 2) ? 8 : 16);
+  static constexpr bool WITH_U = MODE == 2 || MODE == 3;
+  static constexpr bool SPLIT = WITH_U && sizeof(real) == 8;
+  static constexpr int BYTES = SPLIT ? 20 : ((sizeof(real) == 4 && !WITH_U) ? 8 : 16);
   unsigned char* base;   // 16-byte aligned; SPLIT: QB records of 16 bytes, then QB words
   int qb;
   __device__ void put(int qq, unsigned ab, real T, real U) const {
@@ -183,7 +193,7 @@ struct TriStage {
       v.x = T; v.y = U;
       ((double2*)base)[qq] = v;
       ((unsigned*)(base + (size_t)qb * 16))[qq] = ab;
-    } else if constexpr (sizeof(real) == 4 && MODE != 2) {
+    } else if constexpr (sizeof(real) == 4 && !WITH_U) {
       ((uint2*)base)[qq] = make_uint2(ab, __float_as_uint((float)T));
     } else if constexpr (sizeof(real) == 4) {
       ((uint4*)base)[qq] = make_uint4(ab, __float_as_uint((float)T), __float_as_uint((float)U), 0u);
@@ -197,7 +207,7 @@ struct TriStage {
       const double2 v = ((const double2*)base)[qq];
       T = (real)v.x; U = (real)v.y;
       ab = ((const unsigned*)(base + (size_t)qb * 16))[qq];
-    } else if constexpr (sizeof(real) == 4 && MODE != 2) {
+    } else if constexpr (sizeof(real) == 4 && !WITH_U) {
       const uint2 v = ((const uint2*)base)[qq];
       ab = v.x; T = (real)__uint_as_float(v.y); U = 0;
     } else if constexpr (sizeof(real) == 4) {
@@ -214,18 +224,19 @@ struct TriStage {
 
 template <typename real, int MODE>
 struct TriLds {
-  static constexpr int NV = (MODE == 0) ? 1 : (MODE == 1 ? 3 : 4);
+  static constexpr int NV = (MODE == 0) ? 1 : (MODE == 1 ? 3 : (MODE == 2 ? 4 : 7));
+  static constexpr int NG = MODE == 3 ? 2 : 1;   // parameter-gradient sets (force branch, energy branch)
   static constexpr int QB = TriCfg<real, MODE>::QB;
   __host__ __device__ static size_t n_reals(int nr, int Aa, int nt, bool fused = false) {
     const int nsig = 2 * nt - 1;
     size_t r = (size_t)nr * TRI_CAPP * 2;                   // pair tables (real2 per (row, channel)), + (D, V) per row
     if (fused) r += (size_t)3 * nr;                         // unit vectors of the slots
     r += nr;                                                // sD
-    r += Aa;                                                // sP
+    r += (size_t)NG * Aa;                                   // sP (and sPE)
     r += (size_t)TRI_WAVES * Aa;                            // per-wave channel sums
-    if (MODE != 0) r += (size_t)nsig * Aa * 3;              // parameter-gradient sums of the workgroup
-    if (MODE != 0) r += (size_t)TRI_WAVES * TRI_CAP * 3;    // exchange buffer of a pass
-    if (MODE == 2) r += (size_t)4 * nr;                     // sV, sQ
+    if (MODE != 0) r += (size_t)NG * nsig * Aa * 3;         // parameter-gradient sums of the workgroup
+    if (MODE != 0) r += (size_t)NG * TRI_WAVES * TRI_CAP * 3;   // exchange buffer of a pass
+    if (MODE == 2 || MODE == 3) r += (size_t)4 * nr;        // sV, sQ
     return r;
   }
   __host__ __device__ static size_t bytes(int nr, int Aa, int nt, bool fused = false) {
@@ -245,8 +256,9 @@ tri_reduce_kernel(TriArgs<real> A) {
   static_assert(!FUSED || MODE == 0, "only the fingerprint mode rebuilds T");
   using real2 = typename Vec2<real>::type;
   using HE = HotExp<real>;
-  constexpr int NV = TriLds<real, MODE>::NV;
+  constexpr int NV = TriLds<real, MODE>::NV, NG = TriLds<real, MODE>::NG;
   constexpr int TRI_QB = TriCfg<real, MODE>::QB;
+  constexpr bool FB = TriCfg<real, MODE>::FORCE_BRANCH;
   extern __shared__ __align__(16) unsigned char smem[];
   const int nr = A.nr, na = A.na, Aa = A.Aa, nt = A.nt;
   const int nsig = 2 * nt - 1;
@@ -258,12 +270,13 @@ tri_reduce_kernel(TriArgs<real> A) {
   real* sUn = rp; if (FUSED) rp += (size_t)3 * nr;             // [3][nr] unit vectors
   real* sD = rp; rp += nr;
   real* sP = rp; rp += Aa;
+  real* sPE = rp; if (MODE == 3) rp += Aa;                     // MODE 3: dL/dAF3 of the centre beside its netderiv
   real* outw = rp; rp += (size_t)TRI_WAVES * Aa;
-  real* accw = rp; if (MODE != 0) rp += (size_t)nacc;
-  real* xch = rp; if (MODE != 0) rp += (size_t)TRI_WAVES * TRI_CAP * 3;
+  real* accw = rp; if (MODE != 0) rp += (size_t)NG * nacc;     // [NG][nacc]
+  real* xch = rp; if (MODE != 0) rp += (size_t)TRI_WAVES * TRI_CAP * 3 * NG;   // [wave][channel][3 NG]
   real* sV = rp;
   real* sQ = rp + nr;
-  if (MODE == 2) rp += (size_t)4 * nr;
+  if (FB) rp += (size_t)4 * nr;
   TriStage<real, MODE> stage;                   // [TRI_QB] staged triplets
   stage.base = smem + ((((unsigned char*)rp - smem) + 15) & ~(ptrdiff_t)15);   // an offset into smem, not an integer cast
   stage.qb = TRI_QB;
@@ -287,7 +300,7 @@ tri_reduce_kernel(TriArgs<real> A) {
     if (tid < nr) {
       nj0 = A.im2[row0 * (nr + 1) + 1 + tid];
       d0 = A.Dsup[row0 * nr + tid];
-      if (MODE == 2) {
+      if (FB) {
 #pragma unroll
         for (int c = 0; c < 3; c++) gr0[c] = A.dDsup[row0 * 3 * nr + c * nr + tid];
       }
@@ -299,14 +312,14 @@ tri_reduce_kernel(TriArgs<real> A) {
   }
   tab.build(A.alpha3b, A.emb3b);
   if (MODE != 0)
-    for (int q = tid; q < nacc; q += TRI_BLOCK) accw[q] = 0;
+    for (int q = tid; q < NG * nacc; q += TRI_BLOCK) accw[q] = 0;
   int shift = 0;
-  if (MODE == 2) {
+  if (FB) {
     const int at = A.actual_type[0];
     for (int y = 0; y < at; y++) shift += A.tipos[y];
   }
   real* my_out = outw + wave * Aa;
-  real* my_xch = xch + (size_t)wave * TRI_CAP * 3;
+  real* my_xch = xch + (size_t)wave * TRI_CAP * 3 * NG;
   // Parameter-gradient sums of the last pass: thread ia < 16 of the workgroup adds the four waves' values of its
   // channel to accumulator row `pending` (-1: nothing to add).  Called right after a barrier that follows the pass
   // and before the next one, so that the exchange buffer is complete and not yet rewritten.
@@ -314,11 +327,14 @@ tri_reduce_kernel(TriArgs<real> A) {
   auto flush_pass = [&]() {
     if (MODE != 0 && tid < TRI_CAP && pending >= 0) {
 #pragma unroll
-      for (int v = 0; v < 3; v++) {
-        real s = xch[ia * 3 + v];
+      for (int g = 0; g < NG; g++) {
 #pragma unroll
-        for (int w = 1; w < TRI_WAVES; w++) s += xch[(w * TRI_CAP + ia) * 3 + v];
-        accw[pending + v] += s;
+        for (int v = 0; v < 3; v++) {
+          real s = xch[ia * 3 * NG + g * 3 + v];
+#pragma unroll
+          for (int w = 1; w < TRI_WAVES; w++) s += xch[(w * TRI_CAP + ia) * 3 * NG + g * 3 + v];
+          accw[g * nacc + pending + v] += s;
+        }
       }
     }
     pending = -1;
@@ -353,7 +369,7 @@ tri_reduce_kernel(TriArgs<real> A) {
       const int t_s = A.type_map[nj];
       stp[s] = t_s;
       if (s == tid) t_mine = t_s;
-      if (MODE == 2) {
+      if (FB) {
         const real* Qj = A.Q + ((size_t)b * A.N + nj) * 3;
         const real* Qi = A.Q + ((size_t)b * A.N + p + shift) * 3;
         real q0 = Qj[0] - Qi[0], q1 = Qj[1] - Qi[1], q2 = Qj[2] - Qi[2];
@@ -373,8 +389,10 @@ tri_reduce_kernel(TriArgs<real> A) {
         sV[s] = q0 * g0 + q1 * g1 + q2 * g2;
       }
     }
-    for (int a = tid; a < Aa; a += TRI_BLOCK)
+    for (int a = tid; a < Aa; a += TRI_BLOCK) {
       if (MODE != 0) sP[a] = A.P[(size_t)atom * Aa + a];
+      if (MODE == 3) sPE[a] = A.PE[(size_t)atom * Aa + a];
+    }
     for (int q = tid; q < TRI_WAVES * Aa; q += TRI_BLOCK) outw[q] = 0;
   };
   int atom = blockIdx.x;
@@ -433,7 +451,7 @@ tri_reduce_kernel(TriArgs<real> A) {
             if (ia == 0) {
               real2 v;
               v.x = d;
-              v.y = MODE == 2 ? sV[s] : real(0);
+              v.y = FB ? sV[s] : real(0);
               tabE[row * TRI_CAPP + TRI_CAP] = v;
             }
           }
@@ -468,7 +486,7 @@ tri_reduce_kernel(TriArgs<real> A) {
                   T = Trow[nn];
                 }
               }
-              if (MODE == 2) {
+              if (FB) {
                 if (ok) {
 #pragma unroll
                   for (int c = 0; c < 3; c++) {
@@ -530,7 +548,14 @@ tri_reduce_kernel(TriArgs<real> A) {
                   const real Z1 = r_fma(r_, V1, t_ * V2), Z2 = r_fma(t_, V1, r_ * V2);
                   acc[2] = r_fma(hU, r_ + t_, acc[2]);
                   acc[2] = r_fma(hT, r_fma(a1, Z2, r_fma(a2, Z1, X2)), acc[2]);
-                  acc[NV - 1] = r_fma(hT, r_fma((real(2) + bT) * ss, U, T * W), acc[NV - 1]);
+                  acc[3] = r_fma(hT, r_fma((real(2) + bT) * ss, U, T * W), acc[3]);
+                  if constexpr (MODE == 3) {
+                    // the energy branch's sums of the same item (MODE 1 above with w = hT):
+                    // d/da1: (sim2 D1 + sim1 D2) w,  d/da2: (sim2 D2 + sim1 D1) w,  d/dbeta: (sim1 + sim2) w T
+                    acc[4] = r_fma(p_ + q_, hT, acc[4]);
+                    acc[5] = r_fma(r_ + t_, hT, acc[5]);
+                    acc[6] = r_fma(ss * hT, T, acc[6]);
+                  }
                 }
               }
             }
@@ -545,7 +570,7 @@ tri_reduce_kernel(TriArgs<real> A) {
           }
           if (lane < TRI_CAP && chan) {
             const int a = tab.ch[pb + c0 + ia];
-            const real c3h = tab.c3[pb + c0 + ia] * real(MODE == 2 ? 0.25 : 0.5);
+            const real c3h = tab.c3[pb + c0 + ia] * real(FB ? 0.25 : 0.5);
             if constexpr (MODE == 0) {
               my_out[a] += acc[0] * c3h;
             } else if constexpr (MODE == 1) {
@@ -556,7 +581,12 @@ tri_reduce_kernel(TriArgs<real> A) {
               my_out[a] += acc[0] * c3h;
               const real f = c3h * sP[a];
 #pragma unroll
-              for (int v = 0; v < 3; v++) my_xch[ia * 3 + v] = acc[v + 1] * f;
+              for (int v = 0; v < 3; v++) my_xch[ia * 3 * NG + v] = acc[v + 1] * f;
+              if constexpr (MODE == 3) {
+                const real fe = (c3h + c3h) * sPE[a];   // 1/2 c3 dL/dAF3: the energy branch's weight
+#pragma unroll
+                for (int v = 0; v < 3; v++) my_xch[ia * 6 + 3 + v] = acc[v + 4] * fe;
+              }
             }
             if (MODE != 0) pending = (sg * Aa + a) * 3;
           }
@@ -578,7 +608,7 @@ tri_reduce_kernel(TriArgs<real> A) {
     centre_setup(atom, std::false_type{});
   }
   if (MODE != 0) {
-    for (int q = tid; q < nacc; q += TRI_BLOCK) A.partial[(size_t)blockIdx.x * nacc + q] = accw[q];
+    for (int q = tid; q < NG * nacc; q += TRI_BLOCK) A.partial[(size_t)blockIdx.x * NG * nacc + q] = accw[q];
   }
 }
 

@@ -333,6 +333,61 @@ def compute_force_tripl(netderiv, radial_descriptor, angular_descriptor, descrip
     return force if pos is None else (force, virial)
 
 
+def compute_force_tripl_slots(netderiv, radial_descriptor, angular_descriptor, descriptor_derivative_rad,
+                              descriptor_derivative_ang, interaction_map_rad, interaction_map_ang, alpha3b_parameters,
+                              type_emb3b_parameters, type_map, tipos, actual_type, num_triplets):
+    """First half of ComputeForceTripl: the 3-body forces of one centre species as they act on each centre's
+    neighbour slots, (slot_forces [nf,Nl,nr,3], self_forces [nf,Nl,3]), not yet collected by the atoms that receive
+    them.  force_total() collects them for all species, and adds the 2-body forces, in one launch."""
+    dtype = angular_descriptor.dtype
+    s, _ = sfx(dtype)
+    dev = angular_descriptor.device
+    nf, Nl, na = angular_descriptor.shape
+    nr = radial_descriptor.shape[2]
+    N = type_map.shape[0]
+    nt = tipos.shape[0]
+    Aa = alpha3b_parameters.shape[1] // 3
+    v = _Views()
+    pD = v(radial_descriptor)
+    pT = v(angular_descriptor)
+    pdD = v(descriptor_derivative_rad)
+    pd3 = v(descriptor_derivative_ang)
+    pI2 = v(_i32(interaction_map_rad))
+    pI3 = v(_i32(interaction_map_ang))
+    pN = v(_i32(num_triplets))
+    slots = torch.empty((nf, Nl, nr, 3), dtype=dtype, device=dev)
+    own = torch.empty((nf, Nl, 3), dtype=dtype, device=dev)
+    at = _scalar_dev(actual_type, dev)
+    call(f"staf_op_force_tripl_slots_{s}", ptr(_dense(netderiv)), pD, pT, pdD, pd3, pI2, pI3, _I(nr), _I(na), _I(N),
+         _I(nf), _I(Aa), ptr(_dense(type_emb3b_parameters)), _I(nt), ptr(_i32(tipos)), ptr(at), ptr(slots), ptr(own),
+         pN, ptr(_dense(alpha3b_parameters)), ptr(_i32(type_map)), _I(Nl), _I(v.ld), _stream())
+    return slots, own
+
+
+def force_total(interaction_map_rad_full, n_local, slot_forces, self_forces, forces2b=None, out=None):
+    """Total force [nf,3N] in one launch: for every species k, in this order, forces2b[k] (a per-op force array,
+    e.g. what compute_force_radial returned for centre species k; None to skip) plus the 3-body forces of species k
+    collected from slot_forces[k] / self_forces[k] (compute_force_tripl_slots; None to skip).  Same bits as adding
+    the per-op force arrays in that order.  interaction_map_rad_full is the whole intmap2b tensor [nf,N,nr+1] the
+    descriptor op wrote; n_local the atoms per species (host integers)."""
+    im = _i32(interaction_map_rad_full)
+    if not im.is_contiguous():
+        raise ValueError("force_total needs the descriptor op's whole intmap2b tensor")
+    nf, N, nr1 = im.shape
+    nt = len(n_local)
+    some = next(t for t in list(slot_forces) + list(forces2b or []) if t is not None)
+    dtype, dev = some.dtype, some.device
+    s, _ = sfx(dtype)
+    arr = lambda ts: (C.c_void_p * nt)(*[None if t is None else _dense(t).data_ptr() for t in ts])
+    keep = [None if t is None else _dense(t) for t in list(slot_forces) + list(self_forces) + list(forces2b or [])]
+    total = torch.empty((nf, 3 * N), dtype=dtype, device=dev) if out is None else out
+    call(f"staf_op_force_total_{s}", ptr(im), _I(nr1 - 1), _I(N), _I(nf), _I(nt), (C.c_int * nt)(*[int(n) for n in n_local]),
+         arr(slot_forces), arr(self_forces), arr(forces2b if forces2b is not None else [None] * nt), ptr(total),
+         _stream())
+    del keep
+    return total
+
+
 def compute_force_tripl_virial(netderiv, radial_descriptor, angular_descriptor, descriptor_derivative_rad,
                                descriptor_derivative_ang, interaction_map_rad, interaction_map_ang,
                                alpha3b_parameters, type_emb3b_parameters, type_map, tipos, actual_type, num_triplets,
@@ -454,6 +509,46 @@ def compute_force_tripl_grad(prevgrad, netderiv, radial_descriptor, angular_desc
          ptr(None if prevgrad_virial is None else _dense(prevgrad_virial)),
          ptr(None if pos is None else _dense(pos)), ptr(None if box is None else _dense(box)), _I(v.ld), _stream())
     return gn, ga, ge
+
+
+def compute_tripl_grads_fused(prevgrad_force, netderiv, prevgrad_energy, radial_descriptor, angular_descriptor,
+                              descriptor_derivative_rad, descriptor_derivative_ang, interaction_map_rad,
+                              interaction_map_ang, alpha3b_parameters, type_emb3b_parameters, type_map, tipos,
+                              actual_type, num_triplets, prevgrad_virial=None, pos=None, box=None):
+    """Both 3-body parameter gradients of a training step in one launch (no counterpart as one op in the reference):
+    what compute_force_tripl_grad(prevgrad_force, netderiv, ...) and compute_sort_proj3body_grad(prevgrad_energy,
+    ...) return, as (gradnet [nf,Nl,Aa], gradalpha_force [ntc,3Aa], gradalpha_energy [ntc,3Aa], gradck [ntc,Aa] == 0).
+    The two ops share everything but a few accumulations per (triplet, channel), so this costs about what the
+    force-branch op costs alone."""
+    dtype = angular_descriptor.dtype
+    s, _ = sfx(dtype)
+    dev = angular_descriptor.device
+    nf, Nl, na = angular_descriptor.shape
+    nr = radial_descriptor.shape[2]
+    N = type_map.shape[0]
+    nt = tipos.shape[0]
+    ntc = nt * (nt + 1) // 2
+    Aa = alpha3b_parameters.shape[1] // 3
+    v = _Views()
+    pD = v(radial_descriptor)
+    pT = v(angular_descriptor)
+    pdD = v(descriptor_derivative_rad)
+    pd3 = v(descriptor_derivative_ang)
+    pI2 = v(_i32(interaction_map_rad))
+    pI3 = v(_i32(interaction_map_ang))
+    pN = v(_i32(num_triplets))
+    gn = torch.empty((nf, Nl, Aa), dtype=dtype, device=dev)
+    gaf = torch.empty((ntc, 3 * Aa), dtype=dtype, device=dev)
+    gae = torch.empty((ntc, 3 * Aa), dtype=dtype, device=dev)
+    ge = torch.empty((ntc, Aa), dtype=dtype, device=dev)
+    at = _scalar_dev(actual_type, dev)
+    call(f"staf_op_grads_tripl_fused_{s}", ptr(_dense(prevgrad_force)), ptr(_dense(netderiv)),
+         ptr(_dense(prevgrad_energy)), pD, pT, pdD, pd3, pI2, pI3, _I(nr), _I(na), _I(N), _I(nf), _I(Aa),
+         ptr(_dense(type_emb3b_parameters)), _I(nt), ptr(_i32(tipos)), ptr(at), pN, ptr(_dense(alpha3b_parameters)),
+         ptr(_i32(type_map)), _I(Nl), ptr(gn), ptr(gaf), ptr(gae), ptr(ge),
+         ptr(None if prevgrad_virial is None else _dense(prevgrad_virial)),
+         ptr(None if pos is None else _dense(pos)), ptr(None if box is None else _dense(box)), _I(v.ld), _stream())
+    return gn, gaf, gae, ge
 
 
 def compute_force_radial_virial_grad(prevgrad, prevgrad_virial, netderiv, descriptor_derivative_rad,

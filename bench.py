@@ -38,6 +38,8 @@ PROFILED_NAME = {
     ("af3_kernel", "f64"): "staf::tri_reduce_kernel<double, 0, false>",
     ("grad3_kernel", "f32"): "staf::tri_reduce_kernel<float, 1, false>",
     ("grad3_kernel", "f64"): "staf::tri_reduce_kernel<double, 1, false>",
+    ("grads3_kernel", "f32"): "staf::tri_reduce_kernel<float, 3, false>",
+    ("grads3_kernel", "f64"): "staf::tri_reduce_kernel<double, 3, false>",
     ("desc_kernel", "f32"): "staf::desc_kernel<float>",
     ("desc_kernel", "f64"): "staf::desc_kernel<double>",
 }
@@ -104,7 +106,7 @@ def algorithmic_bytes(N, tipos, nr, na, Ar, Aa, nt, s):
     per-species calls summed.  Keys are the kernels that do the op's work."""
     ntc = nt * (nt + 1) // 2
     out = dict(desc_kernel=(N * (8 * nr + 7 * na)) * s + N * (nr + 1 + 2 * na + 1) * 4 + (3 * N + 6) * s)
-    for k in ("af2", "af3", "force2", "force3", "grad2", "grad3", "gradforce2", "gradforce3"):
+    for k in ("af2", "af3", "force2", "force3", "grad2", "grad3", "gradforce2", "gradforce3", "grads3"):
         out[k + "_kernel"] = 0
     for Nl in tipos:
         par2 = 2 * nt * Ar * s
@@ -126,6 +128,11 @@ def algorithmic_bytes(N, tipos, nr, na, Ar, Aa, nt, s):
         out["gradforce3_kernel"] += (3 * N * s + Nl * (Aa + nr + na + 3 * nr + 6 * na) * s
                                      + Nl * (nr + 1 + 2 * na + 1) * 4 + par3 + tm + Nl * Aa * s
                                      + (3 * ntc * Aa + ntc * Aa) * s)                             # ComputeForceTriplGrad
+        # both 3-body parameter gradients in one pass: the inputs of ComputeForceTriplGrad, dL/dAF3 beside them, and
+        # one more parameter-gradient array out
+        out["grads3_kernel"] += (3 * N * s + Nl * (2 * Aa + nr + na + 3 * nr + 6 * na) * s
+                                 + Nl * (nr + 1 + 2 * na + 1) * 4 + par3 + tm + Nl * Aa * s
+                                 + (2 * 3 * ntc * Aa + ntc * Aa) * s)
     return out
 
 
@@ -211,6 +218,14 @@ def main():
                          "on one stream")
     ap.add_argument("--no-graph", action="store_true",
                     help="launch every op of every step from Python instead of replaying one captured HIP graph")
+    ap.add_argument("--reference-op-sequence", action="store_true",
+                    help="call the ops one by one as the reference's layers and gradient registry do: a force array per "
+                         "force op (ComputeForceRadial, ComputeForceTripl) summed by one more launch, and the 3-body "
+                         "parameter gradients as two ops (ComputeSortProj3bodyGrad, ComputeForceTriplGrad).  Default: "
+                         "the library's step-level entry points -- the 3-body slot forces of all species collected "
+                         "and added to the 2-body forces in one launch (staf_op_force_tripl_slots + "
+                         "staf_op_force_total), both 3-body parameter gradients in one pass "
+                         "(staf_op_grads_tripl_fused); same results")
     ap.add_argument("--contiguous-splits", action="store_true",
                     help="copy per-species tensors like tf.split instead of passing views")
     args = ap.parse_args()
@@ -316,10 +331,22 @@ def run_workload(args, workload, mode):
         if phase == 0:
             return timed("af3", lambda: ops.compute_sort_proj3body(angk, supk, im3k, im2k, p["alpha3b"], p["emb3b"],
                                                                    tm, ntrk, nt=nt), record)
+        if phase == 1 and not args.reference_op_sequence:
+            # slot forces only: the atoms collect them, for all species at once, in the step's last launch
+            return timed("force3", lambda: ops.compute_force_tripl_slots(G3[k], supk, angk, d3sk, d3k, im2k, im3k,
+                                                                         p["alpha3b"], p["emb3b"], tm, tp, at[k],
+                                                                         ntrk), record)
         if phase == 1:
             return timed("force3", lambda: ops.compute_force_tripl(G3[k], supk, angk, d3sk, d3k, im2k, im3k,
                                                                    p["alpha3b"], p["emb3b"], tm, tp, at[k], ntrk),
                          record)
+        if phase == 2 and not args.reference_op_sequence:
+            # both 3-body parameter gradients (energy branch and force branch) in one pass
+            return timed("grads3", lambda: ops.compute_tripl_grads_fused(Q, G3[k], P3[k], supk, angk, d3sk, d3k, im2k,
+                                                                         im3k, p["alpha3b"], p["emb3b"], tm, tp,
+                                                                         at[k], ntrk), record)
+        if phase == 3 and not args.reference_op_sequence:
+            return None
         if phase == 2:
             return timed("grad3", lambda: ops.compute_sort_proj3body_grad(P3[k], angk, supk, im3k, im2k,
                                                                           p["alpha3b"], p["emb3b"], tm, ntrk, nt=nt),
@@ -349,6 +376,7 @@ def run_workload(args, workload, mode):
             main_stream = torch.cuda.current_stream()   # the capture stream while a graph is recorded
             ready = main_stream.record_event()
             done = []
+            forces_done = []   # events behind the force op of a side chain: all the total force waits for
 
             def small_species():
                 for k in sorted(range(nt), key=lambda k: -tipos[k]):
@@ -366,9 +394,11 @@ def run_workload(args, workload, mode):
                             body_op(k, vk, 3, 0, record)
                             fingerprints = streams[k].record_event()
                             forces[(k, 3)] = body_op(k, vk, 3, 1, record)
+                            forces_done.append(streams[k].record_event())
                             for phase in range(2, n_phase):
                                 body_op(k, vk, 3, phase, record)
-                            done.append(streams[k].record_event())
+                            if n_phase > 2:
+                                done.append(streams[k].record_event())
                         main_stream.wait_event(fingerprints)
                         forces[(k, 2)] = body_op(k, vk, 2, 1, record)
                         for phase in range(2, n_phase):
@@ -377,7 +407,7 @@ def run_workload(args, workload, mode):
                     with torch.cuda.stream(streams[k]):
                         streams[k].wait_event(ready)
                         species_chain(k, d, record, forces)
-                        done.append(streams[k].record_event())
+                        forces_done.append(streams[k].record_event())
 
             if args.streams == 3:
                 # The largest species in two chains: its 3-body ops on its own stream, its 2-body ops on the
@@ -404,23 +434,37 @@ def run_workload(args, workload, mode):
                     else:
                         forces[(big, 2)], forces[(big, 3)] = out2, out3
                 with torch.cuda.stream(sb):
+                    forces_done.append(e3)
                     for phase in range(2, n_phase):
                         body_op(big, v, 3, phase, record)
-                    done.append(sb.record_event())
+                    if n_phase > 2:
+                        done.append(sb.record_event())
                 for phase in range(2, n_phase):
                     body_op(big, v, 2, phase, record)
             small_species()
-            for ev in done:
+            for ev in forces_done:
                 main_stream.wait_event(ev)
             # eager steps: the force arrays were allocated on the side streams and are consumed on this one.  Under
             # capture the graph's private pool keeps them (and `forces` holds them until the sum is recorded): no
             # allocator event is queued inside the captured region.
             if not torch.cuda.is_current_stream_capturing():
                 for f in forces.values():
-                    f.record_stream(main_stream)
-        # total force = sum of the per-op force arrays (the reference's force_radial + force_angular and add_n over
-        # the species), one launch, always in the same order
-        return ops.add_n([forces[(k, body)] for k in range(nt) for body in (2, 3)])
+                    for t in (f if isinstance(f, tuple) else (f,)):
+                        t.record_stream(main_stream)
+        # Total force, one launch, always in the same order (2-body of species 0, 3-body of species 0, 2-body of
+        # species 1, ...): the sum of the per-op force arrays (the reference's force_radial + force_angular and add_n
+        # over the species) or, with the library's step-level entry points, the same sum with the 3-body slot forces
+        # of all species collected by the receiving atoms inside that launch.
+        if args.reference_op_sequence:
+            total = timed("total", lambda: ops.add_n([forces[(k, body)] for k in range(nt) for body in (2, 3)]), record)
+        else:
+            total = timed("total", lambda: ops.force_total(d[3], tipos, [forces[(k, 3)][0] for k in range(nt)],
+                                                           [forces[(k, 3)][1] for k in range(nt)],
+                                                           [forces[(k, 2)] for k in range(nt)]), record)
+        if streams is not None:
+            for ev in done:
+                main_stream.wait_event(ev)   # the side chains' gradient ops end the step
+        return total
 
     # One step = one replay of a HIP graph that holds the whole op sequence (the ops run on the stream they are
     # called on, so stream capture records their kernels; scratch is grown by the eager warm-up steps first).
@@ -477,6 +521,11 @@ def run_workload(args, workload, mode):
     el1 = el
     if side is not None:
         torch.cuda.synchronize()
+        # (three untimed steps first: the eager tensors of this arrangement are new to the allocator, whose first
+        # device allocations after a capture have taken tens of milliseconds)
+        for _ in range(3):
+            step(streams=None)
+        torch.cuda.synchronize()
         t1 = time.perf_counter()
         for _ in range(nprof):
             step(streams=None)
@@ -513,7 +562,7 @@ def run_workload(args, workload, mode):
     s = np.dtype(dtype).itemsize
     ab = algorithmic_bytes(N, tipos, nr, na, Ar, Aa, nt, s)
     kern = {}
-    for name in list(ab) + ["gather_kernel", "transpose_sort_kernel", "cell_build_kernel"]:
+    for name in list(ab) + ["gather_kernel", "force_total_kernel", "transpose_sort_kernel", "cell_build_kernel"]:
         ms, n = ops.kernel_time(name)
         if n:
             kern[name] = dict(ms_per_step=ms / nprof, launches_per_step=n // nprof, avg_launch_ms=ms / n)
@@ -570,6 +619,13 @@ def run_workload(args, workload, mode):
                    "schedule": {1: "one stream", 2: "one stream per species",
                                 3: "one stream per species; on the step's stream the 2-body ops of the largest "
                                    "species and the 2-body force ops of the others"}[args.streams],
+                   "op_sequence": ("the reference's: one force array per force op and one launch that adds them; "
+                                   "one op per parameter gradient" if args.reference_op_sequence else
+                                   "the library's step-level entry points: 3-body slot forces of all species collected "
+                                   "and added to the 2-body forces in one launch (staf_op_force_tripl_slots, "
+                                   "staf_op_force_total)" + ("; both 3-body parameter gradients in one pass "
+                                                             "(staf_op_grads_tripl_fused)" if mode == "full_step"
+                                                             else "")),
                    "launch": "python per op" if graph is None else "hip graph replay",
                    "timing": f"median of {REPEATS} blocks of {args.steps} steps"},
         "block_ms_per_step": [b / args.steps * 1e3 for b in block_s],

@@ -104,7 +104,7 @@ int staf_ops_poll_status(void* stream);
  * events on the stream they are launched on.  staf_ops_kernel_time waits for the device, returns the summed duration
  * and the number of launches of the named kernel ("desc_kernel", "af2_kernel", "af3_kernel", "force2_kernel",
  * "force3_kernel", "gather_kernel", "grad2_kernel", "grad3_kernel", "gradforce2_kernel", "gradforce3_kernel",
- * "transpose_sort_kernel", "cell_build_kernel")
+ * "grads3_kernel", "force_total_kernel", "transpose_sort_kernel", "cell_build_kernel")
  * since the last call for that name, and forgets them. */
 void staf_ops_kernel_timing(int enable);
 int staf_ops_kernel_time(const char* kernel, double* total_ms, int* launches);
@@ -320,6 +320,73 @@ int staf_op_gradforce_tripl_f64(const double* prevgrad, const double* netderiv, 
                                 const int* type_map, int N_local, double* gradnet_3b, double* grad_alpha3b,
                                 double* grad_emb3b, const double* prevgrad_virial, const double* pos,
                                 const double* box, int ld_atoms, void* stream);
+
+/* Both 3-body parameter gradients of a training step in one launch.  No counterpart as one op in the reference: it
+ * stands for the pair ComputeForceTriplGrad (STAF/src/grad_force/ang/reforce.cc:39-66, reforce.cu.cc:47-254; with
+ * prevgrad_virial/pos/box the virial form, :172-206) and ComputeSortProj3bodyGrad (STAF/src/grad_finger/ang/
+ * reforce.cc:24-31, reforce.cu.cc:13-111), which the modules of STAF/gradient_utility register as the gradients of the 3-body
+ * force op and of the 3-body fingerprint op and which every energy+force training step runs on the same descriptor
+ * tensors.  They share the species grouping, the exponential tables, the staged triplets and exp(beta T) of every
+ * (triplet, channel), so one pass costs about what the force-branch op costs alone.
+ *   prevgrad_force [nf,3N] = dL/dF, netderiv [nf,Nl,num_finger] = dE/dAF3, prevgrad_energy [nf,Nl,num_finger] = dL/dAF3
+ *   -> gradnet_3b [nf,Nl,num_finger] and grad_alpha3b_force [ntc,3*num_finger] as staf_op_gradforce_tripl,
+ *      grad_alpha3b_energy [ntc,3*num_finger] as staf_op_alphagrad_ang, grad_emb3b [ntc,num_finger] (zero, once).
+ * Results agree with the separate ops to rounding (same sums, other order of a few operations). */
+int staf_op_grads_tripl_fused_f32(const float* prevgrad_force, const float* netderiv, const float* prevgrad_energy,
+                                  const float* desr, const float* desa, const float* intderiv_r,
+                                  const float* intderiv_a, const int* intmap_r, const int* intmap_a, int nr, int na,
+                                  int N, int dimbat, int num_finger, const float* type_emb3b, int nt,
+                                  const int* tipos, const int* actual_type, const int* num_triplets,
+                                  const float* smooth_a, const int* type_map, int N_local, float* gradnet_3b,
+                                  float* grad_alpha3b_force, float* grad_alpha3b_energy, float* grad_emb3b,
+                                  const float* prevgrad_virial, const float* pos, const float* box, int ld_atoms,
+                                  void* stream);
+int staf_op_grads_tripl_fused_f64(const double* prevgrad_force, const double* netderiv, const double* prevgrad_energy,
+                                  const double* desr, const double* desa, const double* intderiv_r,
+                                  const double* intderiv_a, const int* intmap_r, const int* intmap_a, int nr, int na,
+                                  int N, int dimbat, int num_finger, const double* type_emb3b, int nt,
+                                  const int* tipos, const int* actual_type, const int* num_triplets,
+                                  const double* smooth_a, const int* type_map, int N_local, double* gradnet_3b,
+                                  double* grad_alpha3b_force, double* grad_alpha3b_energy, double* grad_emb3b,
+                                  const double* prevgrad_virial, const double* pos, const double* box, int ld_atoms,
+                                  void* stream);
+
+/* The 3-body force op in two halves, for a caller that owns the whole step.  No counterpart in the reference, whose
+ * ComputeForceTripl (STAF/src/force/ang/reforce.cc:44-66) scatters with atomicAdd inside the op and whose callers
+ * then add the per-op force arrays (force_radial + force_angular, STAF/source_routine/force_layer_mod.py:24-43;
+ * tf.math.add_n over the species, STAF/staf_models/staf_model.py:210).
+ *
+ * staf_op_force_tripl_slots: arguments of staf_op_force_tripl (no virial form); instead of forces3b it returns the
+ *   force of every centre on each of its neighbour slots, slot_forces [nf,N_local,nr,3], and on the centre itself,
+ *   self_forces [nf,N_local,3] (caller-owned, fully written).  No atom collects anything yet.
+ * staf_op_force_total: one launch that, for every atom, collects the slot forces of all centre species and adds
+ *   the per-op force arrays to them: total [nf,3N] = sum over species k = 0..nt-1, in this order, of forces2b[k]
+ *   (any [nf,3N] array, e.g. the output of staf_op_force_doublets for centre species k; null to skip) and of the
+ *   3-body forces of centre species k (slot_forces[k], self_forces[k]; null to skip).  The result has the bits of
+ *   the per-op outputs added in that order.  slot_forces, self_forces, forces2b are HOST arrays of nt device
+ *   pointers; n_local is a HOST array of the atoms per species (atoms are stored species-sorted, summing to N);
+ *   intmap_r_full is the whole [nf,N,nr+1] tensor the descriptor op wrote and still remembers (its own neighbour
+ *   search: the map is symmetric), else STAF_E_BAD_ARG -- callers with other maps use staf_op_force_tripl. */
+int staf_op_force_tripl_slots_f32(const float* netderiv, const float* desr, const float* desa,
+                                  const float* intderiv_r, const float* intderiv_a, const int* intmap_r,
+                                  const int* intmap_a, int nr, int na, int N, int dimbat, int num_finger,
+                                  const float* type_emb3b, int nt, const int* tipos, const int* actual_type,
+                                  float* slot_forces, float* self_forces, const int* num_triplets,
+                                  const float* smooth_a, const int* type_map, int N_local, int ld_atoms,
+                                  void* stream);
+int staf_op_force_tripl_slots_f64(const double* netderiv, const double* desr, const double* desa,
+                                  const double* intderiv_r, const double* intderiv_a, const int* intmap_r,
+                                  const int* intmap_a, int nr, int na, int N, int dimbat, int num_finger,
+                                  const double* type_emb3b, int nt, const int* tipos, const int* actual_type,
+                                  double* slot_forces, double* self_forces, const int* num_triplets,
+                                  const double* smooth_a, const int* type_map, int N_local, int ld_atoms,
+                                  void* stream);
+int staf_op_force_total_f32(const int* intmap_r_full, int nr, int N, int dimbat, int nt, const int* n_local,
+                            const float* const* slot_forces, const float* const* self_forces,
+                            const float* const* forces2b, float* total, void* stream);
+int staf_op_force_total_f64(const int* intmap_r_full, int nr, int N, int dimbat, int nt, const int* n_local,
+                            const double* const* slot_forces, const double* const* self_forces,
+                            const double* const* forces2b, double* total, void* stream);
 
 /* Sum of up to four arrays of n elements, dst[e] = ((a[e] + b[e]) + c[e]) + d[e] (c, d may be null), in one launch:
  * what the callers do with the per-op force arrays (force_radial + force_angular in

