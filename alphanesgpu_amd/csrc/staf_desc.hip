@@ -44,7 +44,7 @@ struct DescArgs {
   // cell list of the frame (null: every atom is a candidate): atoms grouped by cell, see cell_build_kernel
   const int* cell_dims;    // [nf, 4] cells along a, b, c (1: the axis is not divided), number of cells
   const int* cell_start;   // [nf, CELL_MAX + 1]
-  const int* cell_atoms;   // [nf, N]
+  const void* cell_recs;   // [nf, N] CellRec<real>: position and index of every atom, in cell order
   const int* cell_of;      // [nf, N] cell of every atom
   real* raddescr;
   real* angdescr;
@@ -120,19 +120,52 @@ __device__ inline real norm_plain(const real* d) {
 // ---------------------------------------------------------------------------
 constexpr int CELL_MAX = 4096;
 constexpr int CELL_THREADS = 1024;   // one workgroup bins a whole frame: as wide as a workgroup gets
+constexpr int CELL_APT = 8;          // atoms a thread holds in registers from the counting pass to the fill pass
+
+// An atom as the neighbour search reads it: Cartesian position and index in one 16-byte (float) or 32-byte (double)
+// record, stored in cell order, so that the atoms of a cell -- and of the cells next to it along the last axis --
+// are one contiguous run of records.
+template <typename real> struct CellRec;
+template <> struct __align__(16) CellRec<float> { float x, y, z; int j; };
+template <> struct __align__(16) CellRec<double> { double x, y, z; int j, pad; };
+
+// inclusive prefix sum over the 1024 threads of the workgroup (two barriers); sc: 16 ints of LDS
+__device__ inline int block_scan_1024(int v, int* sc) {
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+#pragma unroll
+  for (int o = 1; o < WAVE; o <<= 1) {
+    const int t = __shfl_up(v, o, WAVE);
+    if (lane >= o) v += t;
+  }
+  if (lane == WAVE - 1) sc[wave] = v;
+  __syncthreads();
+  int before = 0;
+  for (int w = 0; w < wave; w++) before += sc[w];
+  __syncthreads();
+  return v + before;
+}
 
 template <typename real>
 __global__ __launch_bounds__(CELL_THREADS) void cell_build_kernel(const real* __restrict__ pos, const real* __restrict__ boxes,
                                                          int N, real Rc, int* __restrict__ cell_dims,
-                                                         int* __restrict__ cell_start, int* __restrict__ cell_atoms,
+                                                         int* __restrict__ cell_start, CellRec<real>* __restrict__ cell_recs,
                                                          int* __restrict__ cell_of) {
   __shared__ int cnt[CELL_MAX];
   __shared__ int dims[4];
-  __shared__ int carry;
+  __shared__ int sc[CELL_THREADS / WAVE];
   const int tid = threadIdx.x, b = blockIdx.x;
   real box[6], inv[6];
 #pragma unroll
   for (int c = 0; c < 6; c++) box[c] = boxes[b * 6 + c];
+  const real* pf = pos + (size_t)b * N * 3;
+  // the positions of the first CELL_APT x 1024 atoms are requested before anything is computed, and kept
+  real px[CELL_APT], py[CELL_APT], pz[CELL_APT];
+  int cl[CELL_APT];
+#pragma unroll
+  for (int u = 0; u < CELL_APT; u++) {
+    const int a = tid + u * CELL_THREADS < N ? tid + u * CELL_THREADS : N - 1;
+    px[u] = pf[3 * a]; py[u] = pf[3 * a + 1]; pz[u] = pf[3 * a + 2];
+  }
   inverse_box(box, inv);
   if (tid == 0) {
     // lattice vectors a = (b0,0,0), b = (b1,b3,0), c = (b2,b4,b5); heights = volume / area of the opposite face
@@ -151,77 +184,78 @@ __global__ __launch_bounds__(CELL_THREADS) void cell_build_kernel(const real* __
     }
     dims[0] = n[0]; dims[1] = n[1]; dims[2] = n[2]; dims[3] = n[0] * n[1] * n[2];
     for (int c = 0; c < 4; c++) cell_dims[b * 4 + c] = dims[c];
-    carry = 0;
   }
+  for (int c = tid; c < CELL_MAX; c += CELL_THREADS) cnt[c] = 0;
   __syncthreads();
   const int nx = dims[0], ny = dims[1], nz = dims[2], ncell = dims[3];
-  for (int c = tid; c < ncell; c += CELL_THREADS) cnt[c] = 0;
-  __syncthreads();
-  const real* pf = pos + (size_t)b * N * 3;
   int* of = cell_of + (size_t)b * N;
-  // eight atoms per thread at a time: their position reads are in flight together
-  for (int a0 = tid; a0 < N; a0 += 8 * CELL_THREADS) {
-    real px[8], py[8], pz[8];
+  auto cell_index = [&](real x, real y, real z) -> int {
+    real s[3];
+    to_frac(inv, x, y, z, s);
+    int c3[3];
+    const int nn[3] = {nx, ny, nz};
 #pragma unroll
-    for (int u = 0; u < 8; u++) {
-      const int a = a0 + u * CELL_THREADS < N ? a0 + u * CELL_THREADS : N - 1;
-      px[u] = pf[3 * a]; py[u] = pf[3 * a + 1]; pz[u] = pf[3 * a + 2];
+    for (int c = 0; c < 3; c++) {
+      const real f = s[c] - r_floor(s[c]);   // [0, 1]
+      int q = (int)(f * (real)nn[c]);
+      c3[c] = q < 0 ? 0 : (q >= nn[c] ? nn[c] - 1 : q);
     }
+    return (c3[0] * ny + c3[1]) * nz + c3[2];
+  };
+  // ---- counting pass
 #pragma unroll
-    for (int u = 0; u < 8; u++) {
-      const int a = a0 + u * CELL_THREADS;
-      if (a >= N) break;
-      real s[3];
-      to_frac(inv, px[u], py[u], pz[u], s);
-      int c3[3];
-      const int nn[3] = {nx, ny, nz};
-#pragma unroll
-      for (int c = 0; c < 3; c++) {
-        const real f = s[c] - r_floor(s[c]);   // [0, 1]
-        int q = (int)(f * (real)nn[c]);
-        c3[c] = q < 0 ? 0 : (q >= nn[c] ? nn[c] - 1 : q);
-      }
-      const int cell = (c3[0] * ny + c3[1]) * nz + c3[2];
-      of[a] = cell;
-      atomicAdd(&cnt[cell], 1);
+  for (int u = 0; u < CELL_APT; u++) {
+    const int a = tid + u * CELL_THREADS;
+    cl[u] = 0;
+    if (a < N) {
+      cl[u] = cell_index(px[u], py[u], pz[u]);
+      of[a] = cl[u];
+      atomicAdd(&cnt[cl[u]], 1);
     }
+  }
+  for (int a = tid + CELL_APT * CELL_THREADS; a < N; a += CELL_THREADS) {   // frames beyond 8192 atoms
+    const int c = cell_index(pf[3 * a], pf[3 * a + 1], pf[3 * a + 2]);
+    of[a] = c;
+    atomicAdd(&cnt[c], 1);
   }
   __syncthreads();
-  // exclusive prefix over the cells, one block of threads at a time
+  // ---- exclusive prefix over the cells: a thread takes CPT consecutive cells
   int* start = cell_start + (size_t)b * (CELL_MAX + 1);
-  for (int c0 = 0; c0 < ncell; c0 += CELL_THREADS) {
-    const int c = c0 + tid;
-    const int v = c < ncell ? cnt[c] : 0;
-    // inclusive scan of v over the threads through LDS
-    __shared__ int sc[CELL_THREADS];
-    sc[tid] = v;
-    __syncthreads();
-    for (int o = 1; o < CELL_THREADS; o <<= 1) {
-      const int t = tid >= o ? sc[tid - o] : 0;
-      __syncthreads();
-      sc[tid] += t;
-      __syncthreads();
-    }
-    const int base = carry;
-    if (c < ncell) {
-      start[c] = base + sc[tid] - v;
-      cnt[c] = base + sc[tid] - v;   // becomes the fill cursor
-    }
-    __syncthreads();
-    if (tid == CELL_THREADS - 1) carry = base + sc[CELL_THREADS - 1];
-    __syncthreads();
+  constexpr int CPT = CELL_MAX / CELL_THREADS;
+  int mine[CPT], tot = 0;
+#pragma unroll
+  for (int u = 0; u < CPT; u++) {
+    const int c = tid * CPT + u;
+    mine[u] = c < ncell ? cnt[c] : 0;
+    tot += mine[u];
   }
-  if (tid == 0) start[ncell] = carry;
-  int* atoms = cell_atoms + (size_t)b * N;
-  for (int a0 = tid; a0 < N; a0 += 8 * CELL_THREADS) {
-    int cl[8];
+  int run = block_scan_1024(tot, sc) - tot;   // atoms in the cells before this thread's
 #pragma unroll
-    for (int u = 0; u < 8; u++) cl[u] = of[a0 + u * CELL_THREADS < N ? a0 + u * CELL_THREADS : N - 1];
-#pragma unroll
-    for (int u = 0; u < 8; u++) {
-      const int a = a0 + u * CELL_THREADS;
-      if (a < N) atoms[atomicAdd(&cnt[cl[u]], 1)] = a;
+  for (int u = 0; u < CPT; u++) {
+    const int c = tid * CPT + u;
+    if (c < ncell) {
+      start[c] = run;
+      cnt[c] = run;   // becomes the fill cursor
     }
+    run += mine[u];
+  }
+  if (tid == CELL_THREADS - 1) start[ncell] = run;
+  __syncthreads();
+  // ---- fill pass: records in cell order (the order inside a cell is arbitrary: the search sorts what it finds)
+  CellRec<real>* recs = cell_recs + (size_t)b * N;
+#pragma unroll
+  for (int u = 0; u < CELL_APT; u++) {
+    const int a = tid + u * CELL_THREADS;
+    if (a < N) {
+      CellRec<real> r;
+      r.x = px[u]; r.y = py[u]; r.z = pz[u]; r.j = a;
+      recs[atomicAdd(&cnt[cl[u]], 1)] = r;
+    }
+  }
+  for (int a = tid + CELL_APT * CELL_THREADS; a < N; a += CELL_THREADS) {
+    CellRec<real> r;
+    r.x = pf[3 * a]; r.y = pf[3 * a + 1]; r.z = pf[3 * a + 2]; r.j = a;
+    recs[atomicAdd(&cnt[of[a]], 1)] = r;
   }
 }
 
@@ -290,41 +324,53 @@ __global__ __launch_bounds__(256, sizeof(real) == 4 ? 8 : 5) void desc_kernel(De
   // 1. candidate scan -- or the caller's list (already cut off and sorted by distance)
   const bool injected = A.inj_howmany != nullptr;
   if (!injected && A.cell_start) {
-    // candidates = the atoms of the centre's cell and its neighbours (every atom appears once: an axis has one
-    // cell or at least three)
-    __shared__ int nb_start[27], nb_off[28];
+    // Candidates = the atoms of the centre's cell and its neighbours (every atom appears once: an axis has one cell or
+    // at least three).  Cells that follow each other along the last axis are contiguous in the record array, so the
+    // 27 cells are at most 18 runs of records: one per (dx, dy), two where the last axis wraps.  Each wave takes
+    // every fourth run, lane <-> record: one coalesced read per run, all of a wave's runs requested before the first
+    // is used.
+    constexpr int RUNS = 18, RPW = (RUNS + 3) / 4;
+    __shared__ int run_start[RUNS], run_len[RUNS];
     const int* dm = A.cell_dims + b * 4;
     const int nx = dm[0], ny = dm[1], nz = dm[2];
     const int* cstart = A.cell_start + (size_t)b * (CELL_MAX + 1);
-    const int* catoms = A.cell_atoms + (size_t)b * N;
-    if (tid < 27) {
+    const CellRec<real>* recs = (const CellRec<real>*)A.cell_recs + (size_t)b * N;
+    if (tid < 9) {
       const int ci = A.cell_of[(size_t)b * N + i];
       const int cz = ci % nz, cy = (ci / nz) % ny, cx = ci / (nz * ny);
-      const int dx = tid / 9 - 1, dy = (tid / 3) % 3 - 1, dz = tid % 3 - 1;
-      int cnt = 0, st0 = 0;
-      if ((nx > 1 || dx == 0) && (ny > 1 || dy == 0) && (nz > 1 || dz == 0)) {
-        const int x = (cx + dx + nx) % nx, y = (cy + dy + ny) % ny, z = (cz + dz + nz) % nz;
-        const int c = (x * ny + y) * nz + z;
-        st0 = cstart[c];
-        cnt = cstart[c + 1] - st0;
+      const int dx = tid / 3 - 1, dy = tid % 3 - 1;
+      int s0 = 0, l0 = 0, s1 = 0, l1 = 0;
+      if ((nx > 1 || dx == 0) && (ny > 1 || dy == 0)) {
+        const int x = (cx + dx + nx) % nx, y = (cy + dy + ny) % ny;
+        const int base = (x * ny + y) * nz;
+        // cells z0 .. z1 of this column without wrapping; a wrapped end is a second run
+        int z0 = nz > 1 ? cz - 1 : cz, z1 = nz > 1 ? cz + 1 : cz;
+        int w = -1;                      // the wrapped cell, if any
+        if (z0 < 0) { z0 = 0; w = nz - 1; }
+        if (z1 >= nz) { z1 = nz - 1; w = 0; }
+        s0 = cstart[base + z0];
+        l0 = cstart[base + z1 + 1] - s0;
+        if (w >= 0) { s1 = cstart[base + w]; l1 = cstart[base + w + 1] - s1; }
       }
-      nb_start[tid] = st0;
-      nb_off[tid + 1] = cnt;
+      run_start[2 * tid] = s0; run_len[2 * tid] = l0;
+      run_start[2 * tid + 1] = s1; run_len[2 * tid + 1] = l1;
     }
     __syncthreads();
-    if (tid == 0) {
-      nb_off[0] = 0;
-      for (int c = 0; c < 27; c++) nb_off[c + 1] += nb_off[c];
+    const int lane = tid & (WAVE - 1), wave = tid / WAVE;
+    CellRec<real> rc_[RPW];
+    int rl[RPW], rs[RPW];
+#pragma unroll
+    for (int u = 0; u < RPW; u++) {
+      const int r = wave + 4 * u;
+      rl[u] = r < RUNS ? run_len[r] : 0;
+      rs[u] = r < RUNS ? run_start[r] : 0;
+      if (lane < rl[u]) rc_[u] = recs[rs[u] + lane];
     }
-    __syncthreads();
-    const int total = nb_off[27];
-    for (int q = tid; q < total; q += 256) {
-      int c = 0;
-      while (q >= nb_off[c + 1]) c++;
-      const int j = catoms[nb_start[c] + q - nb_off[c]];
-      if (j == i) continue;
+    auto candidate = [&](const CellRec<real>& c) {
+      const int j = c.j;
+      if (j == i) return;
       real sj[3], d[3];
-      to_frac(inv, pf[3 * j], pf[3 * j + 1], pf[3 * j + 2], sj);
+      to_frac(inv, c.x, c.y, c.z, sj);
       const real d2 = mic_delta(box, sj, si, A.dist2_fma, A.skip_pbc, d);
       if (d2 < rc2) {
         const int slot = atomicAdd(&cnt_all, 1);
@@ -336,6 +382,11 @@ __global__ __launch_bounds__(256, sizeof(real) == 4 ? 8 : 5) void desc_kernel(De
           c_d[3 * slot + 2] = d[2];
         }
       }
+    };
+#pragma unroll
+    for (int u = 0; u < RPW; u++) {
+      if (lane < rl[u]) candidate(rc_[u]);
+      for (int q = lane + WAVE; q < rl[u]; q += WAVE) candidate(recs[rs[u] + q]);   // runs of more than 64 atoms
     }
   } else if (!injected) {
     // the position reads of four candidates per thread are issued together
@@ -678,22 +729,25 @@ int desc_launch(const DescConfig<real>& c, const real* pos, const real* box, int
   const bool symmetric = inj_howmany == nullptr;
   if (!transpose_for_descriptor(st, intmap2b, nf, N, Npos, c.nr, 4 * c.nr, symmetric, stream, &A.tr))
     return reserve_failure(stream);
-  A.cell_dims = A.cell_start = A.cell_atoms = A.cell_of = nullptr;
+  A.cell_dims = A.cell_start = A.cell_of = nullptr;
+  A.cell_recs = nullptr;
   const int cell_from = g_cell_threshold;
   if (!inj_howmany && cell_from > 0 && N >= cell_from) {
-    const size_t ints = (size_t)nf * (4 + (CELL_MAX + 1) + 2 * (size_t)N);
-    int* w = (int*)scratch_reserve(st, stream, ints * sizeof(int));
+    // records first (16-byte aligned), then the integer tables
+    const size_t rec_bytes = (size_t)nf * N * sizeof(CellRec<real>);
+    const size_t ints = (size_t)nf * (4 + (CELL_MAX + 1) + (size_t)N);
+    char* w = (char*)scratch_reserve(st, stream, rec_bytes + ints * sizeof(int));
     if (!w) return reserve_failure(stream);
-    int* dims = w;
+    CellRec<real>* recs = (CellRec<real>*)w;
+    int* dims = (int*)(w + rec_bytes);
     int* start = dims + (size_t)nf * 4;
-    int* atoms = start + (size_t)nf * (CELL_MAX + 1);
-    int* of = atoms + (size_t)nf * N;
+    int* of = start + (size_t)nf * (CELL_MAX + 1);
     {
       KernelTimer kt_("cell_build_kernel", stream);
       hipLaunchKernelGGL(cell_build_kernel<real>, dim3(nf), dim3(CELL_THREADS), 0, stream, pos, box, N, c.Rc, dims, start,
-                         atoms, of);
+                         recs, of);
     }
-    A.cell_dims = dims; A.cell_start = start; A.cell_atoms = atoms; A.cell_of = of;
+    A.cell_dims = dims; A.cell_start = start; A.cell_recs = recs; A.cell_of = of;
   }
   size_t lds = desc_lds_bytes<real>(c.nr);
   if (lds > 60 * 1024) return STAF_E_LIMIT;

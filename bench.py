@@ -23,6 +23,15 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+# Vector-ALU roof: 256 CUs x 4 SIMDs, each issuing one 64-lane instruction per 4 cycles at the published 2.4 GHz
+# (= the published 78.6 TFLOP/s of fp64, and of non-packed fp32, when every instruction is an FMA)
+VALU_PEAK_WAVE_INST = 256 * 4 * 2.4e9 / 4
+# Vector instructions the formulas of a 3-body op need per (triplet, active channel) item, fp32 / fp64, counted on
+# the inner loops of csrc/staf_tri.hpp and csrc/staf_force3.hpp (pair factors from the exponential tables, exp(beta T),
+# the op's accumulations; fp64 carries the written-out exponential, 18 instructions instead of the hardware exp2).
+# Set-up, triplet decoding, table building, staging and reductions are overhead and not counted.
+ALGORITHMIC_INST = {"af3_kernel": (7, 24), "force3_kernel": (13, 30), "grad3_kernel": (14, 31),
+                    "gradforce3_kernel": (44, 61), "grads3_kernel": (48, 65)}
 
 SETTLE_STEPS = 300   # untimed graph replays of the set-up, see run_workload()
 REPEATS = 5          # timed blocks of --steps steps each; the median block is reported
@@ -42,6 +51,8 @@ PROFILED_NAME = {
     ("grads3_kernel", "f64"): "staf::tri_reduce_kernel<double, 3, false>",
     ("desc_kernel", "f32"): "staf::desc_kernel<float>",
     ("desc_kernel", "f64"): "staf::desc_kernel<double>",
+    ("af3_fused", "f64"): "staf::tri_reduce_kernel<double, 0, true>",
+    ("force3_fused", "f64"): "staf::force3_kernel<double, true, 4>",
 }
 
 
@@ -66,6 +77,11 @@ def profile_traffic(kernel, workload, prec):
         if not m:
             continue
         name, grid, ctr, v, n = m.group(1), int(m.group(2)), m.group(3), float(m.group(4)), int(m.group(5))
+        inst = re.search(r"staf::(force3_kernel|tri_reduce_kernel|desc_kernel)<[^>]*>", name)
+        if inst and inst.group(0) not in PROFILED_NAME.values():
+            # a row of an instantiation this library no longer builds: the file mixes runs of several builds
+            raise ProfileMissing(f"{path} holds rows of {inst.group(0)}, which the current library does not build: "
+                                 "regenerate it from one run")
         if name.startswith("__amd_rocclr_copyBuffer") and v > 1e5:
             copy[ctr] = v
         elif want in name:
@@ -136,9 +152,21 @@ def algorithmic_bytes(N, tipos, nr, na, Ar, Aa, nt, s):
     return out
 
 
-def cpu_baseline(batch, params, up, mode, nr, na, max_frames=2, threads=16):
+def host_threads():
+    """(threads the CPU legs use, cores the host shows).  The job's CPU share is what OMP_NUM_THREADS says where it
+    is set (a GPU box hands a one-GPU job 16 of its cores), else every core."""
+    cores = os.cpu_count() or 1
+    try:
+        share = int(os.environ.get("OMP_NUM_THREADS", cores))
+    except ValueError:
+        share = cores
+    return max(1, min(share, cores)), cores
+
+
+def cpu_baseline(batch, params, up, mode, nr, na, max_frames=2):
     """Times the CPU oracle on the first frames of the same batch: one thread (the reported value), and one frame per
-    thread on `threads` threads (frames are independent; ctypes releases the GIL inside the oracle's C++ calls)."""
+    thread on all threads of the job's CPU share (frames are independent; ctypes releases the GIL inside the
+    oracle's C++ calls)."""
     from concurrent.futures import ThreadPoolExecutor
 
     from oracle import staf_oracle as O
@@ -186,15 +214,268 @@ def cpu_baseline(batch, params, up, mode, nr, na, max_frames=2, threads=16):
         return float(np.median(ts))
 
     el = median_time(lambda: frames(0, nfs))
-    threads = max(1, min(threads, os.cpu_count() or 1))
+    threads, cores_visible = host_threads()
     nfr = batch["nf"]
     with ThreadPoolExecutor(threads) as ex:
         elm = median_time(lambda: list(ex.map(lambda i: frames(i % nfr, i % nfr + 1), range(threads))))
-    return dict(value=nfs / el, unit="frames/s", cores=1, kind="port",
+    return dict(value=nfs / el, unit="frames/s", cores=1, kind="port", host_cores=cores_visible,
                 sample=f"{nfs} frame(s) of the same batch, same ops, scalar C++ oracle (-O2 -ffp-contract=off), 1 thread, "
-                       f"median of {reps} after a warm-up",
-                multicore=dict(value=threads / elm, unit="frames/s", cores=threads,
-                               sample=f"{threads} frames, one per thread, same oracle, median of {reps}"))
+                       f"median of {reps} after a warm-up; the host shows {cores_visible} cores",
+                multicore=dict(value=threads / elm, unit="frames/s", cores=threads, host_cores=cores_visible,
+                               sample=f"{threads} frames, one per thread on the {threads} threads of the job's CPU "
+                                      f"share ({cores_visible} cores visible), same oracle, median of {reps}"))
+
+
+def triplet_channel_items(desc_out, type_map_dev, tipos, params, nr, na):
+    """Per centre species: sum over its centres and over the species pairs (ta <= tb) of the centre's triplets of
+    (triplets of that pair) x (channels with non-zero squared embedding in parameter row ta + tb).  From the
+    descriptor op's own outputs (numtriplet = neighbours inside the angular cutoff, the first of the sorted row)."""
+    import torch
+    im2, ntr = desc_out[3], desc_out[8]
+    nt = len(tipos)
+    nbr = im2[..., 1:].long()
+    inside = torch.arange(nr, device=im2.device)[None, None, :] < ntr[..., None]
+    sp = type_map_dev.long()[nbr]
+    counts = [((sp == t) & inside).sum(-1).double() for t in range(nt)]   # [nf, N] each
+    out = []
+    o = 0
+    for k, n in enumerate(tipos):
+        nact = [(np.asarray(params[k]["emb3b"])[sg] != 0).sum() for sg in range(2 * nt - 1)]
+        tot = 0.0
+        for ta in range(nt):
+            ca = counts[ta][:, o:o + n]
+            for tb in range(ta, nt):
+                cb = counts[tb][:, o:o + n]
+                size = ca * (ca - 1) / 2 if ta == tb else ca * cb
+                tot += float(size.sum()) * float(nact[ta + tb])
+        out.append(tot)
+        o += n
+    return out
+
+
+def numpy_mlp(af, mu, layers):
+    """The per-species network of the MD entry on the host (Dense stack on log(af + 1e-3) - mu, as
+    libstaf/src/mlp/staf_mlp_ort.cc:186-233): (sum of atomic energies, d sum / d af)."""
+    x = np.log(af + 1e-3) - mu
+    acts = [x]
+    for W, b, act in layers:
+        z = acts[-1] @ W + b
+        acts.append(np.tanh(z) if act == "tanh" else (np.maximum(z, 0) if act == "relu" else z))
+    g = np.ones_like(acts[-1])
+    for (W, b, act), a_out in zip(reversed(layers), reversed(acts[1:])):
+        if act == "tanh":
+            g = g * (1 - a_out * a_out)
+        elif act == "relu":
+            g = g * (a_out > 0)
+        g = g @ W.T
+    return float(acts[-1].sum()), g / (af + 1e-3)
+
+
+def run_md(args, workload):
+    """The MD entry end to end: staf_compute on the workload's first frame, host arrays in and out, the library's
+    own neighbour list rebuilt on every call, fingerprints -> device MLP -> forces without leaving the GPU.  The
+    model is a random-initialised one of the reference's architecture (60 fingerprints -> 140 -> 140 -> 1, tanh),
+    written as a model directory and loaded with staf_load."""
+    import tempfile
+
+    import torch
+    from alphanesgpu_amd import libstaf, model_dir, ops, synth
+    batch = synth.water_batch(workload)
+    N, tipos, type_map = batch["N"], [int(x) for x in batch["tipos"]], batch["type_map"]
+    nt = len(tipos)
+    nr, na = synth.NR, synth.NA
+    x = np.ascontiguousarray(batch["pos"][0].astype(np.float64).reshape(-1, 3))
+    box = np.ascontiguousarray(batch["box"][0].astype(np.float64))
+    params = synth.fingerprint_params(dtype=np.float64, dense_embedding=args.dense_embedding)
+    rng = np.random.Generator(np.random.Philox(23))
+    species = []
+    for p in params:
+        n_af = p["alpha2b"].shape[1] + p["alpha3b"].shape[1] // 3
+        dims = [n_af, 140, 140, 1]
+        layers = [(rng.standard_normal((a, b)) / np.sqrt(a), 0.1 * rng.standard_normal(b), "tanh" if b > 1 else "linear")
+                  for a, b in zip(dims[:-1], dims[1:])]
+        species.append(dict(p, layers=layers))
+    Ar, Aa = params[0]["alpha2b"].shape[1], params[0]["alpha3b"].shape[1] // 3
+    tmp = tempfile.mkdtemp(prefix="staf_bench_model_")
+    model_dir.write_model_dir(tmp, species, rc=synth.RC, rc_ang=synth.RA, rs=synth.RS, radial_buffer=nr,
+                              angular_buffer=na, tipos=tipos, precision="double")
+    m = libstaf.StafModel(tmp, precision=1)
+    for _ in range(8):     # sizes every buffer; the shape repeats, so the call's kernel sequence is recorded and replayed
+        e, f, vir = m.compute(x, box, type_map)
+    for _ in range(args.warmup):
+        m.compute(x, box, type_map)
+    block_s = []
+    for _ in range(REPEATS):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            m.compute(x, box, type_map)
+        torch.cuda.synchronize()     # every call ends with its own synchronisation; this one finds nothing to wait for
+        block_s.append(time.perf_counter() - t0)
+    el = float(np.median(block_s))
+    # per-kernel times from the library's events: a handle that launches every call eagerly (replayed graphs hold no events)
+    me = libstaf.StafModel(tmp, precision=1, eager=True)
+    for _ in range(3):
+        e2, f2, _ = me.compute(x, box, type_map)
+    if not (e2 == e and np.array_equal(f2, f)):
+        print("bench.py: replayed and eager calls of staf_compute differ", file=sys.stderr)
+        sys.exit(1)
+    nprof = max(3, min(args.steps, 20))
+    t1 = time.perf_counter()
+    ops.kernel_timing(True)
+    for _ in range(nprof):
+        me.compute(x, box, type_map)
+    ops.kernel_timing(False)
+    el_eager = (time.perf_counter() - t1) / nprof
+    kern = {}
+    for name in ("cell_build_kernel", "desc_kernel", "af2_kernel", "af3_kernel", "force2_kernel", "force3_kernel",
+                 "gather_kernel"):
+        ms, n = ops.kernel_time(name)
+        if n:
+            kern[name] = dict(ms_per_step=ms / nprof, launches_per_step=n // nprof, avg_launch_ms=ms / n)
+    me.close()
+    # items of the 3-body kernels, from an operator-level descriptor call on the same frame
+    dev = torch.device("cuda:0")
+    T = lambda a: torch.as_tensor(np.ascontiguousarray(a)).to(dev)
+    ops.construct_descriptors_light(synth.RC, nr, na, N, None, synth.RS, synth.RA, 1, dtype=torch.float64)
+    d_ = ops.compute_descriptors_light(T(batch["pos"][:1].astype(np.float64)), T(batch["box"][:1].astype(np.float64)))
+    items = float(sum(triplet_channel_items(d_, T(type_map), tipos, params, nr, na)))
+    pairs = float(d_[3][..., 0].clamp(max=nr).double().sum())
+    del d_
+    torch.cuda.empty_cache()
+    # Bytes the call's kernels move once through HBM by their signatures (no tensor of the angular buffer's width
+    # exists on this path).  In rows of N x nr doubles: the radial-only descriptor kernel writes 12 (raddescr,
+    # des3bsupp, der2b x3, der3bsupp x3, unit x4) and the neighbour map; the 2-body fingerprints read 1 and the map,
+    # the fused 3-body fingerprints 5 (des3bsupp, unit), the 2-body force 4 (raddescr, der2b), the fused 3-body force 8
+    # (des3bsupp, der3bsupp, unit); the slot forces are written and read once (3 rows); fingerprints and their
+    # gradients are written and read once each; positions in, four per-op force arrays and their sum out.
+    s = 8
+    row = N * nr * s
+    imap = N * (nr + 1) * 4
+    md_bytes = (12 * row + imap) + (row + imap) + (5 * row + imap) + (4 * row + imap) + (8 * row + imap) \
+        + 2 * 3 * row + 4 * N * (Ar + Aa) * s + 10 * N * 3 * s
+    dom = max(kern, key=lambda k: kern[k]["ms_per_step"])
+    alg = {"af3_kernel": ALGORITHMIC_INST["af3_kernel"][1], "force3_kernel": ALGORITHMIC_INST["force3_kernel"][1]}
+    valu_frac = {k: items * alg[k] / 64.0 / (kern[k]["ms_per_step"] * 1e-3) / VALU_PEAK_WAVE_INST for k in alg if k in kern}
+    try:
+        valu_share, valu_src = profile_valu_share_md(dom, workload)
+    except ProfileMissing as ex:
+        valu_share, valu_src = None, str(ex)
+    t_dom = kern[dom]["ms_per_step"] * 1e-3
+    out = {
+        "metric": "frames/s descriptor fwd+force/alpha bwd, 768-atom water fp32/fp64; % HBM roofline",
+        "value": args.steps / el,
+        "unit": "frames/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": el / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f64",
+        "data": "synthetic",
+        "config": {"workload": workload, "entry": "staf_compute (MD entry, include/staf.h)", "mode": "energy + forces + virial",
+                   "atoms": N, "frames_per_step": 1, "Rc": synth.RC, "radial_buffer": nr, "angular_buffer": na,
+                   "Ar": Ar, "Aa": Aa, "mlp": "60-140-140-1 tanh per species, float64, random init, on the GPU",
+                   "neighbour_list": "the library's own, rebuilt on every call (cell list from 2048 atoms on)",
+                   "boundary": "host arrays in (positions, box, species) and out (energy, forces, virial): the PCIe "
+                               "copies and the call's one synchronisation are inside the timed region",
+                   "launch": "the call's kernel sequence recorded once as a HIP graph and replayed",
+                   "timing": f"median of {REPEATS} blocks of {args.steps} calls"},
+        "block_ms_per_step": [b / args.steps * 1e3 for b in block_s],
+        "eager_ms_per_step": el_eager * 1e3,
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": md_bytes / (el / args.steps) / 1e9,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": md_bytes / (el / args.steps) / 1e9 / HBM_PEAK_GBS,
+                     "frac_is": "bytes of the whole call (nr-wide tensors only: this path holds no tensor of the angular "
+                                "buffer's width) over the call's time over peak: low by construction, the call is bound "
+                                "by vector-ALU issue and by the latency of its ~25 dependent launches",
+                     "traffic": None, "algorithmic_bytes_per_call": md_bytes,
+                     "valu": {"bound": "valu", "unit": "wave instructions/s", "kernel": dom,
+                              "algorithmic_inst_per_item": alg.get(dom), "items_per_call": items,
+                              "achieved": (items * alg[dom] / 64.0 / t_dom) if dom in alg else None,
+                              "peak": VALU_PEAK_WAVE_INST,
+                              "frac": valu_frac.get(dom), "exp_per_s": (items / t_dom) if dom in alg else None,
+                              "executed_issue_share": valu_share, "executed_issue_share_source": valu_src,
+                              "note": "per (triplet, active channel) item as in the operator chain; the fused kernels "
+                                      "also rebuild the angular descriptor and its Jacobian per triplet, which "
+                                      "executed_issue_share includes"}},
+        "kernel_valu_frac_algorithmic": valu_frac,
+        "kernel_ms_per_step": {k: v["ms_per_step"] for k, v in kern.items()},
+        "kernels_sum_ms": sum(v["ms_per_step"] for v in kern.values()),
+        "active_slots": {"pairs_per_atom": pairs / N, "triplet_channel_items": items},
+        "ms_per_frame": el / args.steps * 1e3,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = md_cpu_baseline(x, box, tipos, type_map, species, nr, na)
+    m.close()
+    return out
+
+
+def profile_valu_share_md(kernel, workload):
+    """Issue share of the MD call's dominant kernel from profiles/md_step_<workload>_sq_counters.txt."""
+    path = os.path.join(PROFILES, f"md_step_{workload}_sq_counters.txt")
+    if not os.path.exists(path):
+        raise ProfileMissing(f"{path} not found")
+    want = PROFILED_NAME[({"af3_kernel": "af3_fused", "force3_kernel": "force3_fused"}.get(kernel, kernel), "f64")]
+    want = want.replace("staf::", "")
+    num = den = 0.0
+    for line in open(path):
+        if not line.startswith(want):
+            continue
+        rest = line[len(want):].split()
+        us, issue = float(rest[2]), float(rest[5])
+        num += us * issue
+        den += us
+    if den == 0.0:
+        raise ProfileMissing(f"{path}: no row for {want}")
+    return num / den, os.path.relpath(path, ROOT)
+
+
+def md_cpu_baseline(x, box, tipos, type_map, species, nr, na):
+    """The same call on the host: the CPU oracle's ops wired in the order of the reference's inference
+    (STAF/staf_models/staf_model_inference_full.py:89-144) with the network as numpy matrix products, one thread
+    for the oracle; one call, median of 3 after a warm-up."""
+    from oracle import staf_oracle as O
+    pos = x.reshape(1, -1)
+    bx = box.reshape(1, 6)
+
+    def call():
+        d = O.compute_descriptors_light(pos, bx, 4.5, 4.5, 2.25, nr, na, dtype=np.float64)
+        o = 0
+        E = 0.0
+        F = np.zeros_like(pos)
+        for k, n in enumerate(tipos):
+            sl = slice(o, o + n)
+            o += n
+            m = species[k]
+            c = lambda a: np.ascontiguousarray(a[:, sl])
+            af2 = O.radial_afs(c(d["raddescr"]), c(d["intmap2b"]), m["alpha2b"], m["emb2b"], type_map)
+            af3 = O.angular_afs(c(d["angdescr"]), c(d["des3bsupp"]), c(d["intmap3b"]), m["alpha3b"], m["emb3b"],
+                                type_map, c(d["numtriplet"]))
+            af = np.concatenate([af2, af3], axis=2)
+            e, g = numpy_mlp(af[0], m["mu"], m["layers"])
+            E += 0.5 * e
+            A2 = af2.shape[2]
+            G = g[None]
+            F += O.force_radial(np.ascontiguousarray(G[:, :, :A2]), c(d["der2b"]), c(d["intmap2b"]), c(d["raddescr"]),
+                                m["alpha2b"], m["emb2b"], type_map, np.asarray(tipos, np.int32), k)
+            F += O.force_tripl(np.ascontiguousarray(G[:, :, A2:]), c(d["des3bsupp"]), c(d["angdescr"]),
+                               c(d["der3bsupp"]), c(d["der3b"]), c(d["intmap2b"]), c(d["intmap3b"]), m["alpha3b"],
+                               m["emb3b"], type_map, np.asarray(tipos, np.int32), k, c(d["numtriplet"]))
+        return E, F
+
+    call()
+    ts = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        call()
+        ts.append(time.perf_counter() - t0)
+    _, cores_visible = host_threads()
+    return dict(value=1.0 / float(np.median(ts)), unit="frames/s", cores=1, kind="port", host_cores=cores_visible,
+                sample="one call on the same frame: scalar C++ oracle ops (-O2 -ffp-contract=off, 1 thread; all-pairs "
+                       "neighbour search) and the network as numpy matrix products, median of 3 after a warm-up; "
+                       f"the host shows {cores_visible} cores")
 
 
 def main():
@@ -226,6 +507,12 @@ def main():
                          "and added to the 2-body forces in one launch (staf_op_force_tripl_slots + "
                          "staf_op_force_total), both 3-body parameter gradients in one pass "
                          "(staf_op_grads_tripl_fused); same results")
+    ap.add_argument("--dense-embedding", action="store_true",
+                    help="type embeddings without zeros: every 3-body channel is active for every species pair "
+                         "(default: the 0/1 block embeddings the reference trains with, a third of them active)")
+    ap.add_argument("--entry", default="ops", choices=["ops", "md"],
+                    help="ops: the operator chain (default).  md: the MD entry staf_compute end to end on the workload's "
+                         "first frame (host arrays in and out, own neighbour list rebuilt each call, device MLP)")
     ap.add_argument("--contiguous-splits", action="store_true",
                     help="copy per-species tensors like tf.split instead of passing views")
     args = ap.parse_args()
@@ -237,13 +524,15 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
-    if args.workload is not None:
+    if args.entry == "md":
+        out = run_md(args, args.workload or "water6144")
+    elif args.workload is not None:
         out = run_workload(args, args.workload, args.mode)
     else:
         # The metric names both halves: fp32 descriptor fwd + force (the headline line) and the fp64 full step with
         # the parameter-gradient ops, measured in the same process right behind it.
         out = run_workload(args, "water768_f32", "fwd_force")
-        out["also"] = [run_workload(args, "water768_f64", "full_step")]
+        out["also"] = [run_workload(args, "water768_f64", "full_step"), run_md(args, "water6144")]
     print(json.dumps(out))
 
 
@@ -260,7 +549,7 @@ def run_workload(args, workload, mode):
     nf, N = batch["nf"], batch["N"]
     tipos = [int(x) for x in batch["tipos"]]
     nt = len(tipos)
-    params = synth.fingerprint_params(dtype=dtype)
+    params = synth.fingerprint_params(dtype=dtype, dense_embedding=args.dense_embedding)
     Ar, Aa = params[0]["alpha2b"].shape[1], params[0]["alpha3b"].shape[1] // 3
     up = synth.synthetic_upstream(nf, batch["tipos"], params, 11, dtype)
 
@@ -577,6 +866,14 @@ def run_workload(args, workload, mode):
     na_act = float(torch.clamp(mtr * (mtr - 1) / 2, max=na).mean())
     ab_act = algorithmic_bytes(N, tipos, nr_act, na_act, Ar, Aa, nt, s)
     step_bytes_act = sum(ab_act[k] for k in kern if k in ab_act)
+    # (triplet, active channel) items of the 3-body ops per centre species: the triplets of a centre by the species
+    # pair of their two neighbours, times the channels whose squared embedding is not zero for that pair
+    items = triplet_channel_items(d_, tm, tipos, params, nr, na)
+    total_items = float(sum(items))
+    col = 0 if dtype == np.float32 else 1
+    valu_frac = {k: total_items * ALGORITHMIC_INST[k][col] / 64.0 / (kern[k]["ms_per_step"] * 1e-3) / VALU_PEAK_WAVE_INST
+                 for k in kern if k in ALGORITHMIC_INST}
+    step_alg_inst = sum(total_items * ALGORITHMIC_INST[k][col] / 64.0 for k in kern if k in ALGORITHMIC_INST)
     # the kernel the step spends most of its time in, priced against HBM with the bytes its op signature moves
     dom = max((k for k in kern if k in ab), key=lambda k: kern[k]["ms_per_step"])
     dom_bytes_per_launch = ab[dom] * nf / kern[dom]["launches_per_step"]
@@ -594,6 +891,22 @@ def run_workload(args, workload, mode):
         if workload in ("water768_f32", "water768_f64") and not args.profiling_run:
             raise SystemExit(f"bench.py: {e}")
         valu_share, valu_src = None, str(e)
+    valu = None
+    if dom in ALGORITHMIC_INST:
+        per_launch = total_items / kern[dom]["launches_per_step"]
+        t_launch = kern[dom]["avg_launch_ms"] * 1e-3
+        valu = {"bound": "valu", "unit": "wave instructions/s",
+                "algorithmic_inst_per_item": ALGORITHMIC_INST[dom][col],
+                "items_per_launch": per_launch,
+                "achieved": per_launch * ALGORITHMIC_INST[dom][col] / 64.0 / t_launch,
+                "peak": VALU_PEAK_WAVE_INST,
+                "frac": per_launch * ALGORITHMIC_INST[dom][col] / 64.0 / t_launch / VALU_PEAK_WAVE_INST,
+                "exp_per_s": per_launch / t_launch,
+                "executed_issue_share": valu_share, "executed_issue_share_source": valu_src,
+                "note": "algorithmic = the instructions the op's formulas need per (triplet, active channel) item; "
+                        "executed_issue_share = all vector instructions the kernel issues (SQ_INSTS_VALU x 4 cycles "
+                        "over the launch's SIMD-cycles, rocprofv3): the difference is set-up, decoding, tables, "
+                        "staging and reductions"}
     # bytes desc_kernel really writes: the nr-wide tensors, angdescr and intmap3b over their whole rows (padding is
     # written as 0 like the reference's memsets), der3b over the triplets that exist only
     desc_written = N * (8 * nr + na) * s + N * (nr + 1 + 2 * na + 1) * 4 + N * 6 * na_act * s + (3 * N + 6) * s
@@ -612,6 +925,9 @@ def run_workload(args, workload, mode):
         "data": "synthetic",
         "config": {"workload": workload, "mode": mode, "atoms": N, "frames_per_step": nf, "Rc": synth.RC,
                    "radial_buffer": nr, "angular_buffer": na, "Ar": Ar, "Aa": Aa,
+                   "type_embeddings": ("dense: every channel active for every species pair" if args.dense_embedding
+                                       else "0/1 blocks as the reference trains with: 14/13/13 of the 40 3-body "
+                                            "channels active per species pair"),
                    "descriptor_padding": "library default = the reference op's: angdescr, intmap2b, intmap3b, "
                                          "numtriplet zero beyond the active slots; der3b padding left untouched",
                    "species_tensors": "contiguous copies" if args.contiguous_splits else "views",
@@ -630,8 +946,13 @@ def run_workload(args, workload, mode):
                    "timing": f"median of {REPEATS} blocks of {args.steps} steps"},
         "block_ms_per_step": [b / args.steps * 1e3 for b in block_s],
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                     "traffic_source": traffic_src,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                     "frac_is": "algorithmic bytes of the op's signature (padded slots included) over launch time "
+                                "over peak; hbm_frac_measured prices the bytes the counters saw",
+                     "traffic": traffic, "traffic_source": traffic_src,
+                     "hbm_frac_measured": (None if traffic is None else
+                                           traffic / (kern[dom]["avg_launch_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS),
+                     "valu": valu,
                      "valu_issue_share": valu_share, "valu_issue_share_source": valu_src,
                      "measured_copy_GBs": copy_gbs, "frac_of_measured_copy": achieved / copy_gbs,
                      "algorithmic_bytes_per_launch": dom_bytes_per_launch,
@@ -642,6 +963,9 @@ def run_workload(args, workload, mode):
         # desc_kernel against the bytes it writes (its signature's bytes include der3b padding it leaves alone)
         "desc_kernel_hbm_frac_of_written_bytes": desc_written * nf / (kern["desc_kernel"]["ms_per_step"] * 1e-3) / 1e9
                                                  / HBM_PEAK_GBS,
+        "kernel_valu_frac_algorithmic": valu_frac,
+        "whole_step_valu_frac_algorithmic": step_alg_inst / (el / args.steps) / VALU_PEAK_WAVE_INST,
+        "triplet_channel_items_per_step": total_items,
         "kernel_ms_per_step": {k: v["ms_per_step"] for k, v in kern.items()},
         "whole_step_hbm_frac": step_bytes * nf / (el / args.steps) / 1e9 / HBM_PEAK_GBS,
         "whole_step_frac_of_measured_copy": step_bytes * nf / (el / args.steps) / 1e9 / copy_gbs,
