@@ -342,12 +342,14 @@ template <typename real>
 int angular_afs(const real* Dsup, const real* Tang, const real* unit, int nr, int na, real* out, int nf, int Nl,
                 const int* im3, const int* im2, const real* alpha3b, int Aa, const real* emb3b, const int* type_map,
                 const int* numtriplet, int nt, int ld, void* stream);
+template <typename real> struct Force2In;   // staf_force3.hpp: the 2-body inputs of the fused slot forces
 template <typename real>
 int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* dDsup, const real* d3b,
                 const real* unit, const int* im2, const int* im3, int nr, int na, int N, int nf, int Aa,
                 const real* emb3b, int nt,
                 const int* tipos, const int* actual_type, real* force, const int* numtriplet, const real* alpha3b,
                 const int* type_map, int Nl, real* virial, const real* pos, const real* box, int ld, int skip_pbc,
-                void* stream, real* slots_out = nullptr, real* self_out = nullptr);
+                void* stream, real* slots_out = nullptr, real* self_out = nullptr,
+                const struct Force2In<real>* two_body = nullptr);
 
 }  // namespace staf

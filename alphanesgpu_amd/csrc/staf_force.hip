@@ -594,13 +594,17 @@ int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* d
                 const real* emb3b, int nt,
                 const int* tipos, const int* actual_type, real* force, const int* numtriplet, const real* alpha3b,
                 const int* type_map, int Nl, real* virial, const real* pos, const real* box, int ld, int skip_pbc,
-                void* stream_, real* slots_out, real* self_out) {
+                void* stream_, real* slots_out, real* self_out, const Force2In<real>* two_body) {
   (void)im3;
   if ((virial || pos || box) && !(virial && pos && box)) return STAF_E_BAD_ARG;
   // slots_out / self_out: the slot forces [nf, Nl, nr, 3] and the centres' own forces [nf, Nl, 3] go to the caller
   // instead of the library's work area and no atom gathers them here (force is not written and may be null)
   const bool deferred = slots_out != nullptr;
   if (deferred && (!self_out || virial)) return STAF_E_BAD_ARG;
+  // two_body: the 2-body pair forces of the same centres are added to the slot forces (slot outputs only)
+  if (two_body && (!deferred || unit || !two_body->G2 || !two_body->D || !two_body->dD || !two_body->alpha2b ||
+                   !two_body->emb2b || two_body->Ar <= 0))
+    return STAF_E_BAD_ARG;
   if (deferred && Nl == 0) return STAF_OK;
   if (Nl == 0 && nf > 0 && N > 0 && force) return empty_species_force<real>(force, virial, nf, N, stream_);
   if (!G || !Dsup || (!unit && (!Tang || !d3b)) || !dDsup || !im2 || !emb3b || !tipos || !actual_type ||
@@ -628,22 +632,24 @@ int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* d
   // critical path is half as long: measured 20.5 against 22.4 us for 1024 centres, 32.0 against 34.0 for 2048);
   // double precision: four (eight measured no faster, its registers admit no more resident waves).
   constexpr int NWV = sizeof(real) == 4 ? 8 : 4;
-  auto launch = [&](auto fused_c) -> int {
-    constexpr bool FUSED = decltype(fused_c)::value;
+  auto launch = [&](auto fused_c, auto w2b_c) -> int {
+    constexpr bool FUSED = decltype(fused_c)::value, W2B = decltype(w2b_c)::value;
     using L = Force3Cfg<real, NWV>;
-    const size_t lds = L::bytes(nr, Aa, nt, FUSED);
+    const size_t lds = L::bytes(nr, Aa, nt, FUSED, W2B ? two_body->Ar : 0);
     if (lds > 64 * 1024) {
-      if (lds > 160 * 1024 || hipFuncSetAttribute((const void*)force3_kernel<real, FUSED, NWV>,
+      if (lds > 160 * 1024 || hipFuncSetAttribute((const void*)force3_kernel<real, FUSED, NWV, W2B>,
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
         return STAF_E_LIMIT;
     }
     KernelTimer kt_("force3_kernel", stream);
-    hipLaunchKernelGGL((force3_kernel<real, FUSED, NWV>), dim3(nf * Nl), dim3(L::THREADS), lds, stream, G, Dsup, Tang,
-                       dDsup, d3b, unit, im2, alpha3b, emb3b, type_map, numtriplet, gslot, self, nf, N, Nl, ld, nr, na,
-                       Aa, nt);
+    hipLaunchKernelGGL((force3_kernel<real, FUSED, NWV, W2B>), dim3(nf * Nl), dim3(L::THREADS), lds, stream, G, Dsup,
+                       Tang, dDsup, d3b, unit, im2, alpha3b, emb3b, type_map, numtriplet, gslot, self, nf, N, Nl, ld, nr,
+                       na, Aa, nt, two_body ? *two_body : Force2In<real>{});
     return STAF_OK;
   };
-  rc = fused ? launch(std::integral_constant<bool, true>{}) : launch(std::integral_constant<bool, false>{});
+  using T_ = std::integral_constant<bool, true>;
+  using F_ = std::integral_constant<bool, false>;
+  rc = fused ? launch(T_{}, F_{}) : (two_body ? launch(F_{}, T_{}) : launch(F_{}, F_{}));
   if (rc) return rc;
   if (deferred) return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
   if (virial) {
@@ -670,7 +676,8 @@ template int force_tripl<double>(const double*, const double*, const double*, co
                                  const double*, const int*, const int*, int, int, int, int, int, const double*, int,
                                  const int*,
                                  const int*, double*, const int*, const double*, const int*, int, double*,
-                                 const double*, const double*, int, int, void*, double*, double*);
+                                 const double*, const double*, int, int, void*, double*, double*,
+                                 const Force2In<double>*);
 
 template <typename real>
 static int gradforce_2b(const real* Q, const real* D, int nr, const real* alpha2b, int Ar, const real* dD,
@@ -884,7 +891,7 @@ void staf_op_force_set_skip_pbc(int skip) { staf::g_force_skip_pbc = skip ? 1 : 
                                    intmap_a, nr, na, N,                                                                \
                                    dimbat, num_finger, type_emb3b, nt, tipos, actual_type, forces3b, num_triplets,     \
                                    smooth_a, type_map, N_local, virial, pos, box, ld_atoms, staf::g_force_skip_pbc,    \
-                                   stream, (real*)nullptr, (real*)nullptr);                                            \
+                                   stream, (real*)nullptr, (real*)nullptr, (const staf::Force2In<real>*)nullptr);      \
   }                                                                                                                    \
   int staf_op_force_tripl_slots_##SFX(const real* netderiv, const real* desr, const real* desa,                        \
                                       const real* intderiv_r, const real* intderiv_a, const int* intmap_r,             \
@@ -898,7 +905,25 @@ void staf_op_force_set_skip_pbc(int skip) { staf::g_force_skip_pbc = skip ? 1 : 
                                    intmap_a, nr, na, N, dimbat, num_finger, type_emb3b, nt, tipos, actual_type,        \
                                    (real*)nullptr, num_triplets, smooth_a, type_map, N_local, (real*)nullptr,          \
                                    (const real*)nullptr, (const real*)nullptr, ld_atoms, staf::g_force_skip_pbc,       \
-                                   stream, slot_forces, self_forces);                                                  \
+                                   stream, slot_forces, self_forces, (const staf::Force2In<real>*)nullptr);           \
+  }                                                                                                                    \
+  int staf_op_forces_slots_##SFX(const real* netderiv3b, const real* netderiv2b, const real* desr, const real* desa,   \
+                                 const real* intderiv_r, const real* intderiv_a, const real* des_r2b,                  \
+                                 const real* intderiv_r2b, const int* intmap_r, const int* intmap_a, int nr, int na,   \
+                                 int N, int dimbat, int num_finger, int num_alpha_radiale, const real* type_emb3b,     \
+                                 const real* smooth_a, const real* alpha_radiale, const real* type_emb2b, int nt,      \
+                                 const int* tipos, const int* actual_type, real* slot_forces, real* self_forces,       \
+                                 const int* num_triplets, const int* type_map, int N_local, int ld_atoms,              \
+                                 void* stream) {                                                                       \
+    if (!slot_forces || !self_forces) return STAF_E_BAD_ARG;                                                           \
+    staf::Force2In<real> two;                                                                                          \
+    two.G2 = netderiv2b; two.D = des_r2b; two.dD = intderiv_r2b; two.alpha2b = alpha_radiale; two.emb2b = type_emb2b;  \
+    two.Ar = num_alpha_radiale;                                                                                        \
+    return staf::force_tripl<real>(netderiv3b, desr, desa, intderiv_r, intderiv_a, (const real*)nullptr, intmap_r,    \
+                                   intmap_a, nr, na, N, dimbat, num_finger, type_emb3b, nt, tipos, actual_type,        \
+                                   (real*)nullptr, num_triplets, smooth_a, type_map, N_local, (real*)nullptr,          \
+                                   (const real*)nullptr, (const real*)nullptr, ld_atoms, staf::g_force_skip_pbc,       \
+                                   stream, slot_forces, self_forces, &two);                                            \
   }                                                                                                                    \
   int staf_op_force_total_##SFX(const int* intmap_r_full, int nr, int N, int dimbat, int nt, const int* n_local,       \
                                 const real* const* slot_forces, const real* const* self_forces,                        \

@@ -91,15 +91,18 @@ struct Force3Cfg {
   // (a multiple of 128 bytes for the usual channel counts) those entries would share their banks; one entry more
   // puts consecutive rows one entry apart.
   __host__ __device__ static int rowp(int Aa) { return pitch(Aa) + 1; }
-  __host__ __device__ static size_t n_reals(int nr, int Aa, int nt, bool fused = false) {
+  // Ar2 > 0: the 2-body pair forces are added (Ar2 radial channels)
+  __host__ __device__ static size_t n_reals(int nr, int Aa, int nt, bool fused = false, int Ar2 = 0) {
     const int nsig = 2 * nt - 1;
     return (size_t)nsig * rowp(Aa) * 4 /*prm*/ + (size_t)nsig * pitch(Aa) * 2 /*prE*/ +
            (((size_t)ROWP * nt * nr + 1) & ~(size_t)1) /*E*/ +
            (size_t)NW * 4 * nr /*slot sums per wave*/ + nr /*D*/ + 3 * nr /*grad fc*/ +
-           (size_t)NW * 4 /*the waves' shares of the centre's own force*/ + (fused ? 4 * nr : 0) /*unit vectors, 1/r*/;
+           (size_t)NW * 4 /*the waves' shares of the centre's own force*/ + (fused ? 4 * nr : 0) /*unit vectors, 1/r*/ +
+           (Ar2 > 0 ? (size_t)NW * nr + nr + (size_t)(2 * nt + 1) * Ar2 : 0) /*2-body: the waves' shares of the pair
+           weights, D, parameter rows, the centre's dE/dAF2*/;
   }
-  __host__ __device__ static size_t bytes(int nr, int Aa, int nt, bool fused = false) {
-    return n_reals(nr, Aa, nt, fused) * sizeof(real) + (size_t)(16 + nr) * sizeof(int);
+  __host__ __device__ static size_t bytes(int nr, int Aa, int nt, bool fused = false, int Ar2 = 0) {
+    return n_reals(nr, Aa, nt, fused, Ar2) * sizeof(real) + (size_t)(16 + nr) * sizeof(int);
   }
 };
 
@@ -108,14 +111,27 @@ struct Force3Cfg {
 // STAF/src/descriptor_builder/reforce.cu.cc:195-228), with c = u_j . u_k, h = (c + 1)/2:
 //   T = h fc_j fc_k,   dT/dd_j = 1/2 fc_j fc_k / r_j (u_k - c u_j) + h fc_k grad fc_j,   j <-> k for dT/dd_k
 // `unit` is [nf, ld, 4, nr] = (u_x, u_y, u_z, 1/r) per sorted neighbour, written by the radial-only descriptor call.
-template <typename real, bool FUSED = false, int NWAVES = 4>
+// The 2-body pair forces of the same centre, added to its slot forces (W2B): with g(i,s) = 1/2 sum_ch G2[i,ch]
+// c2[t_s,ch] e^{alpha[t_s,ch] D(i,s)} (1 + alpha[t_s,ch] D(i,s)) grad D(i,s) (computeforce_doublets_kernel,
+// STAF/src/force/rad/reforce.cu.cc:70-131) the slot force becomes 3-body + g, over all im2[0] radial neighbours.
+template <typename real>
+struct Force2In {
+  const real* G2;       // [nf, Nl, Ar] dE/dAF2
+  const real* D;        // raddescr [nf, ld, nr]
+  const real* dD;       // der2b [nf, ld, 3, nr]
+  const real* alpha2b;  // [nt, Ar]
+  const real* emb2b;    // [nt, Ar]
+  int Ar;
+};
+
+template <typename real, bool FUSED = false, int NWAVES = 4, bool W2B = false>
 __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real, NWAVES>::MIN_WAVES)) void force3_kernel(
     const real* __restrict__ G, const real* __restrict__ Dsup, const real* __restrict__ Tang,
     const real* __restrict__ dDsup, const real* __restrict__ d3b, const real* __restrict__ unit,
     const int* __restrict__ im2,
     const real* __restrict__ alpha3b, const real* __restrict__ emb3b, const int* __restrict__ type_map,
     const int* __restrict__ numtriplet, real* __restrict__ gslot, real* __restrict__ self, int nf, int N, int Nl,
-    int ld, int nr, int na, int Aa, int nt) {
+    int ld, int nr, int na, int Aa, int nt, Force2In<real> B2) {
   using real2 = typename Vec2<real>::type;
   using real4 = typename Vec4<real>::type;
   using HE = HotExp<real>;
@@ -133,7 +149,10 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
   real* sg = sD + nr;                                      // [3*nr] grad fc (der3bsupp)
   real* xch = sg + 3 * nr;                                 // [NW][4] the waves' shares of the centre's own force
   real* sU = xch + NW * 4;                                 // FUSED: [4][nr] unit vector, 1/r
-  int* nact = (int*)(sU + (FUSED ? 4 * nr : 0));           // [16] active channels per sigma (0 beyond nsig)
+  real* w2p = sU + (FUSED ? 4 * nr : 0);                   // W2B: [NW][nr] the waves' shares of the 2-body pair weights
+  real* sD2 = w2p + (W2B ? NW * nr : 0);                   // W2B: [nr] raddescr of the slots
+  real* p2 = sD2 + (W2B ? nr : 0);                         // W2B: alpha2b [nt*Ar], emb2b [nt*Ar], dE/dAF2 of the centre [Ar]
+  int* nact = (int*)(p2 + (W2B ? (2 * nt + 1) * B2.Ar : 0));   // [16] active channels per sigma (0 beyond nsig)
   int* stp = nact + 16;                                    // [nr] species of every slot
 
   const int tid = threadIdx.x;
@@ -179,6 +198,15 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
   // Holding the der3b rows of the first sweep in registers from here on was measured and is slower.
   unsigned nj = 0;   // unsigned: no sign extension (and so no wait for the read) ahead of the reads that follow
   real d_s = 0, g_s[3] = {0, 0, 0}, u_s[4] = {0, 0, 0, 0};
+  int cnt2 = 0;      // W2B: radial neighbours of the centre
+  real d2_s = 0;
+  if constexpr (W2B) {
+    cnt2 = im[0];
+    if (tid < nr) d2_s = B2.D[rowAtom * nr + tid];
+    const int npar = nt * B2.Ar;
+    for (int q = tid; q < 2 * npar + B2.Ar; q += THREADS)
+      p2[q] = q < npar ? B2.alpha2b[q] : (q < 2 * npar ? B2.emb2b[q - npar] : B2.G2[(size_t)atom * B2.Ar + (q - 2 * npar)]);
+  }
   if (tid < nr) {
     nj = (unsigned)im[1 + tid];
     d_s = Dsup[rowAtom * nr + tid];
@@ -201,9 +229,11 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
       Tn[p] = Trow[nn < nlast ? nn : nlast];
     }
   }
+  if constexpr (W2B) cnt2 = cnt2 > nr ? nr : cnt2;
   const bool slot = tid < m;
+  const bool slot_t = W2B ? tid < cnt2 : slot;   // slots whose species is needed: with the pair forces, all radial ones
   int t_s = 0;
-  if (slot) t_s = type_map[nj];
+  if (slot_t) t_s = type_map[nj];
   if (tid >= nsig && tid < 16) nact[tid] = 0;
   for (int q = tid; q < NW * 4 * nr; q += THREADS) acc[q] = 0;
   for (int sgm = wave; sgm < nsig; sgm += NW) {
@@ -249,8 +279,30 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
       for (int c = 0; c < 4; c++) sU[c * nr + tid] = u_s[c];
     }
   }
-  if (slot) stp[tid] = t_s;
+  if (slot_t) stp[tid] = t_s;
+  if constexpr (W2B) {
+    if (tid < nr) sD2[tid] = d2_s;
+  }
   __syncthreads();
+  if constexpr (W2B) {
+    // 2-body pair weights: lane <-> slot, wave w takes every NW-th channel; the waves' shares are added in a fixed
+    // order where the slot forces are formed (several barriers from here)
+    const int Ar = B2.Ar;
+    for (int s_ = lane; s_ < nr; s_ += WAVE) {
+      real w = 0;
+      if (s_ < cnt2) {
+        const real d2 = sD2[s_];
+        const real* al = p2 + mul24(stp[s_], Ar);
+        const real* c2 = al + mul24(nt, Ar);
+        const real* g2 = p2 + 2 * mul24(nt, Ar);
+        for (int ch = wave; ch < Ar; ch += NW) {
+          const real ad = al[ch] * d2;
+          w += g2[ch] * (c2[ch] * HE::eval(HE::scale(ad)) * (real(1) + ad));
+        }
+      }
+      w2p[wave * nr + s_] = w;
+    }
+  }
   int maxact = 0;
   for (int sgm = 0; sgm < nsig; sgm++) {
     const int n_ = uniform(nact[sgm]);
@@ -531,6 +583,17 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
     }
 #pragma unroll
     for (int c = 0; c < 3; c++) f3[c] = t4[c] + t4[3] * sg[c * nr + tid];
+  }
+  if constexpr (W2B) {
+    // the pair force of slot tid (zero weight beyond the radial neighbours); slots beyond the angular cutoff carry it alone
+    if (tid < nr) {
+      real w = 0;
+#pragma unroll
+      for (int w_ = 0; w_ < NW; w_++) w += w2p[w_ * nr + tid];
+      w *= real(0.5);
+#pragma unroll
+      for (int c = 0; c < 3; c++) f3[c] += w * B2.dD[rowAtom * 3 * nr + c * nr + tid];
+    }
   }
 #pragma unroll
   for (int c = 0; c < 3; c++) {

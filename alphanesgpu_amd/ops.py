@@ -364,6 +364,43 @@ def compute_force_tripl_slots(netderiv, radial_descriptor, angular_descriptor, d
     return slots, own
 
 
+def compute_forces_slots(netderiv3b, netderiv2b, radial_descriptor, angular_descriptor, descriptor_derivative_rad,
+                         descriptor_derivative_ang, radial_descriptor_2b, descriptor_derivative_rad_2b,
+                         interaction_map_rad, interaction_map_ang, alpha3b_parameters, type_emb3b_parameters,
+                         alpha2b_parameters, type_emb2b_parameters, type_map, tipos, actual_type, num_triplets):
+    """compute_force_tripl_slots with the 2-body pair forces of the same centres (what ComputeForceRadial computes
+    from netderiv2b, raddescr = radial_descriptor_2b and der2b = descriptor_derivative_rad_2b) added to the slot
+    forces in the same launch: (slot_forces [nf,Nl,nr,3], self_forces [nf,Nl,3]) of 2-body + 3-body.  force_total()
+    then gives the total force without any per-op force array."""
+    dtype = angular_descriptor.dtype
+    s, _ = sfx(dtype)
+    dev = angular_descriptor.device
+    nf, Nl, na = angular_descriptor.shape
+    nr = radial_descriptor.shape[2]
+    N = type_map.shape[0]
+    nt = tipos.shape[0]
+    Aa = alpha3b_parameters.shape[1] // 3
+    Ar = alpha2b_parameters.shape[1]
+    v = _Views()
+    pD = v(radial_descriptor)
+    pT = v(angular_descriptor)
+    pdD = v(descriptor_derivative_rad)
+    pd3 = v(descriptor_derivative_ang)
+    pD2 = v(radial_descriptor_2b)
+    pdD2 = v(descriptor_derivative_rad_2b)
+    pI2 = v(_i32(interaction_map_rad))
+    pI3 = v(_i32(interaction_map_ang))
+    pN = v(_i32(num_triplets))
+    slots = torch.empty((nf, Nl, nr, 3), dtype=dtype, device=dev)
+    own = torch.empty((nf, Nl, 3), dtype=dtype, device=dev)
+    at = _scalar_dev(actual_type, dev)
+    call(f"staf_op_forces_slots_{s}", ptr(_dense(netderiv3b)), ptr(_dense(netderiv2b)), pD, pT, pdD, pd3, pD2, pdD2,
+         pI2, pI3, _I(nr), _I(na), _I(N), _I(nf), _I(Aa), _I(Ar), ptr(_dense(type_emb3b_parameters)),
+         ptr(_dense(alpha3b_parameters)), ptr(_dense(alpha2b_parameters)), ptr(_dense(type_emb2b_parameters)), _I(nt),
+         ptr(_i32(tipos)), ptr(at), ptr(slots), ptr(own), pN, ptr(_i32(type_map)), _I(Nl), _I(v.ld), _stream())
+    return slots, own
+
+
 def force_total(interaction_map_rad_full, n_local, slot_forces, self_forces, forces2b=None, out=None):
     """Total force [nf,3N] in one launch: for every species k, in this order, forces2b[k] (a per-op force array,
     e.g. what compute_force_radial returned for centre species k; None to skip) plus the 3-body forces of species k

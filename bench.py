@@ -39,8 +39,10 @@ REPEATS = 5          # timed blocks of --steps steps each; the median block is r
 PROFILES = os.path.join(ROOT, "profiles")
 # bench.py's kernel names (the library's timing names) -> the names the profiler prints
 PROFILED_NAME = {
-    ("force3_kernel", "f32"): "staf::force3_kernel<float, false, 8>",
-    ("force3_kernel", "f64"): "staf::force3_kernel<double, false, 4>",
+    ("force3_kernel", "f32"): "staf::force3_kernel<float, false, 8, true>",      # 2-body + 3-body slot forces
+    ("force3_kernel", "f64"): "staf::force3_kernel<double, false, 4, true>",
+    ("force3_kernel_3b_only", "f32"): "staf::force3_kernel<float, false, 8, false>",   # the reference's op sequence
+    ("force3_kernel_3b_only", "f64"): "staf::force3_kernel<double, false, 4, false>",
     ("gradforce3_kernel", "f32"): "staf::tri_reduce_kernel<float, 2, false>",
     ("gradforce3_kernel", "f64"): "staf::tri_reduce_kernel<double, 2, false>",
     ("af3_kernel", "f32"): "staf::tri_reduce_kernel<float, 0, false>",
@@ -52,7 +54,7 @@ PROFILED_NAME = {
     ("desc_kernel", "f32"): "staf::desc_kernel<float>",
     ("desc_kernel", "f64"): "staf::desc_kernel<double>",
     ("af3_fused", "f64"): "staf::tri_reduce_kernel<double, 0, true>",
-    ("force3_fused", "f64"): "staf::force3_kernel<double, true, 4>",
+    ("force3_fused", "f64"): "staf::force3_kernel<double, true, 4, false>",
 }
 
 
@@ -533,6 +535,19 @@ def main():
         # the parameter-gradient ops, measured in the same process right behind it.
         out = run_workload(args, "water768_f32", "fwd_force")
         out["also"] = [run_workload(args, "water768_f64", "full_step"), run_md(args, "water6144")]
+        if not args.reference_op_sequence:
+            # the same two steps launched op by op as the reference's layers call them (drop-in sequence), for comparison
+            import copy
+            ref_args = copy.copy(args)
+            ref_args.reference_op_sequence = True
+            ref_args.no_cpu_baseline = True
+            ref_args.profiling_run = True
+            for rec, (wl, md) in zip([out, out["also"][0]], [("water768_f32", "fwd_force"), ("water768_f64", "full_step")]):
+                r = run_workload(ref_args, wl, md)
+                rec["reference_op_sequence"] = {"value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"],
+                                                "block_ms_per_step": r["block_ms_per_step"],
+                                                "op_sequence": r["config"]["op_sequence"],
+                                                "kernel_ms_per_step": r["kernel_ms_per_step"]}
     print(json.dumps(out))
 
 
@@ -609,6 +624,8 @@ def run_workload(args, workload, mode):
         if body == 2:
             if phase == 0:
                 return timed("af2", lambda: ops.compute_sort_proj(radk, im2k, p["alpha2b"], p["emb2b"], tm), record)
+            if phase == 1 and not args.reference_op_sequence:
+                return None    # the pair forces are added to the slot forces by the 3-body force launch
             if phase == 1:
                 return timed("force2", lambda: ops.compute_force_radial(G2[k], d2k, im2k, radk, p["alpha2b"],
                                                                         p["emb2b"], tm, tp, at[k]), record)
@@ -621,10 +638,12 @@ def run_workload(args, workload, mode):
             return timed("af3", lambda: ops.compute_sort_proj3body(angk, supk, im3k, im2k, p["alpha3b"], p["emb3b"],
                                                                    tm, ntrk, nt=nt), record)
         if phase == 1 and not args.reference_op_sequence:
-            # slot forces only: the atoms collect them, for all species at once, in the step's last launch
-            return timed("force3", lambda: ops.compute_force_tripl_slots(G3[k], supk, angk, d3sk, d3k, im2k, im3k,
-                                                                         p["alpha3b"], p["emb3b"], tm, tp, at[k],
-                                                                         ntrk), record)
+            # slot forces of 2-body + 3-body only: the atoms collect them, for all species at once, in the step's
+            # last launch
+            return timed("force3", lambda: ops.compute_forces_slots(G3[k], G2[k], supk, angk, d3sk, d3k, radk, d2k,
+                                                                    im2k, im3k, p["alpha3b"], p["emb3b"],
+                                                                    p["alpha2b"], p["emb2b"], tm, tp, at[k], ntrk),
+                         record)
         if phase == 1:
             return timed("force3", lambda: ops.compute_force_tripl(G3[k], supk, angk, d3sk, d3k, im2k, im3k,
                                                                    p["alpha3b"], p["emb3b"], tm, tp, at[k], ntrk),
@@ -739,7 +758,8 @@ def run_workload(args, workload, mode):
             if not torch.cuda.is_current_stream_capturing():
                 for f in forces.values():
                     for t in (f if isinstance(f, tuple) else (f,)):
-                        t.record_stream(main_stream)
+                        if t is not None:
+                            t.record_stream(main_stream)
         # Total force, one launch, always in the same order (2-body of species 0, 3-body of species 0, 2-body of
         # species 1, ...): the sum of the per-op force arrays (the reference's force_radial + force_angular and add_n
         # over the species) or, with the library's step-level entry points, the same sum with the 3-body slot forces
@@ -748,8 +768,7 @@ def run_workload(args, workload, mode):
             total = timed("total", lambda: ops.add_n([forces[(k, body)] for k in range(nt) for body in (2, 3)]), record)
         else:
             total = timed("total", lambda: ops.force_total(d[3], tipos, [forces[(k, 3)][0] for k in range(nt)],
-                                                           [forces[(k, 3)][1] for k in range(nt)],
-                                                           [forces[(k, 2)] for k in range(nt)]), record)
+                                                           [forces[(k, 3)][1] for k in range(nt)]), record)
         if streams is not None:
             for ev in done:
                 main_stream.wait_event(ev)   # the side chains' gradient ops end the step
@@ -850,6 +869,10 @@ def run_workload(args, workload, mode):
     ops.kernel_timing(False)
     s = np.dtype(dtype).itemsize
     ab = algorithmic_bytes(N, tipos, nr, na, Ar, Aa, nt, s)
+    if not args.reference_op_sequence:
+        # the 3-body force launch also does the 2-body force op's work: it is priced on the bytes of both signatures
+        # less the force arrays neither op writes here, plus the slot forces it writes instead
+        ab["force3_kernel"] += ab["force2_kernel"] - 2 * nt * 3 * N * s + N * (nr + 1) * 3 * s
     kern = {}
     for name in list(ab) + ["gather_kernel", "force_total_kernel", "transpose_sort_kernel", "cell_build_kernel"]:
         ms, n = ops.kernel_time(name)
@@ -865,6 +888,8 @@ def run_workload(args, workload, mode):
     nr_act = float(cnt2.mean())
     na_act = float(torch.clamp(mtr * (mtr - 1) / 2, max=na).mean())
     ab_act = algorithmic_bytes(N, tipos, nr_act, na_act, Ar, Aa, nt, s)
+    if not args.reference_op_sequence:
+        ab_act["force3_kernel"] += ab_act["force2_kernel"] - 2 * nt * 3 * N * s + N * (nr_act + 1) * 3 * s
     step_bytes_act = sum(ab_act[k] for k in kern if k in ab_act)
     # (triplet, active channel) items of the 3-body ops per centre species: the triplets of a centre by the species
     # pair of their two neighbours, times the channels whose squared embedding is not zero for that pair
@@ -937,9 +962,9 @@ def run_workload(args, workload, mode):
                                    "species and the 2-body force ops of the others"}[args.streams],
                    "op_sequence": ("the reference's: one force array per force op and one launch that adds them; "
                                    "one op per parameter gradient" if args.reference_op_sequence else
-                                   "the library's step-level entry points: 3-body slot forces of all species collected "
-                                   "and added to the 2-body forces in one launch (staf_op_force_tripl_slots, "
-                                   "staf_op_force_total)" + ("; both 3-body parameter gradients in one pass "
+                                   "the library's step-level entry points: per species one launch for the 2-body and "
+                                   "3-body slot forces (staf_op_forces_slots), collected by the receiving atoms of all "
+                                   "species in one launch (staf_op_force_total)" + ("; both 3-body parameter gradients in one pass "
                                                              "(staf_op_grads_tripl_fused)" if mode == "full_step"
                                                              else "")),
                    "launch": "python per op" if graph is None else "hip graph replay",

@@ -381,6 +381,26 @@ int staf_op_force_tripl_slots_f64(const double* netderiv, const double* desr, co
                                   double* slot_forces, double* self_forces, const int* num_triplets,
                                   const double* smooth_a, const int* type_map, int N_local, int ld_atoms,
                                   void* stream);
+/* staf_op_force_tripl_slots with the 2-body pair forces of the same centre species added to the slot forces in the
+ * same launch (the arguments of staf_op_force_doublets beside those of staf_op_force_tripl: netderiv2b
+ * [nf,N_local,num_alpha_radiale], des_r2b = raddescr, intderiv_r2b = der2b, alpha_radiale, type_emb2b): slot_forces and
+ * self_forces then hold 2-body + 3-body, and staf_op_force_total gives the total force of a step without any per-op
+ * force array.  Agrees with the sum of the two ops' outputs to rounding (other order of the additions). */
+int staf_op_forces_slots_f32(const float* netderiv3b, const float* netderiv2b, const float* desr, const float* desa,
+                             const float* intderiv_r, const float* intderiv_a, const float* des_r2b,
+                             const float* intderiv_r2b, const int* intmap_r, const int* intmap_a, int nr, int na,
+                             int N, int dimbat, int num_finger, int num_alpha_radiale, const float* type_emb3b,
+                             const float* smooth_a, const float* alpha_radiale, const float* type_emb2b, int nt,
+                             const int* tipos, const int* actual_type, float* slot_forces, float* self_forces,
+                             const int* num_triplets, const int* type_map, int N_local, int ld_atoms, void* stream);
+int staf_op_forces_slots_f64(const double* netderiv3b, const double* netderiv2b, const double* desr,
+                             const double* desa, const double* intderiv_r, const double* intderiv_a,
+                             const double* des_r2b, const double* intderiv_r2b, const int* intmap_r,
+                             const int* intmap_a, int nr, int na, int N, int dimbat, int num_finger,
+                             int num_alpha_radiale, const double* type_emb3b, const double* smooth_a,
+                             const double* alpha_radiale, const double* type_emb2b, int nt, const int* tipos,
+                             const int* actual_type, double* slot_forces, double* self_forces,
+                             const int* num_triplets, const int* type_map, int N_local, int ld_atoms, void* stream);
 int staf_op_force_total_f32(const int* intmap_r_full, int nr, int N, int dimbat, int nt, const int* n_local,
                             const float* const* slot_forces, const float* const* self_forces,
                             const float* const* forces2b, float* total, void* stream);

@@ -955,6 +955,24 @@ def test_force_total_has_the_bits_of_the_per_op_forces_added(dtype, case):
     got = ops.force_total(im2, n_local, slots, own, f2)
     torch.cuda.synchronize()
     assert torch.equal(got, want)
+    # 2-body pair forces folded into the slot forces by the same launch: the total without any per-op force array,
+    # equal to the sum of the per-op arrays to rounding
+    slots23, own23 = [], []
+    for k, s in enumerate(species_slices(tipos)):
+        if int(tipos[k]) == 0:
+            slots23.append(None)
+            own23.append(None)
+            continue
+        p = {kk: T(vv) for kk, vv in params[k].items()}
+        at = torch.tensor([k], dtype=torch.int32, device=dev)
+        sl, ow = ops.compute_forces_slots(T(up["G3"][k]), T(up["G2"][k]), sup[:, s], ang[:, s], d3s[:, s], d3[:, s],
+                                          rad[:, s], d2[:, s], im2[:, s], im3[:, s], p["alpha3b"], p["emb3b"],
+                                          p["alpha2b"], p["emb2b"], tm, tp, at, ntr[:, s])
+        slots23.append(sl)
+        own23.append(ow)
+    got23 = ops.force_total(im2, n_local, slots23, own23).cpu().numpy()
+    tol = TOL[dtype]
+    assert max(nerr(got23, want.cpu().numpy()), eerr(got23, want.cpu().numpy())) <= tol
     # 3-body terms alone, and with the first species' terms left out
     assert torch.equal(ops.force_total(im2, n_local, slots, own), ops.add_n(f3))
     some2 = [None] + f2[1:]
