@@ -75,6 +75,14 @@ __global__ void add_into_kernel(double* dst, const double* src, int n) {
   if (e < n) dst[e] += src[e];
 }
 
+// Host-to-device copy that is complete when it returns, on a stream of the model: a blocking hipMemcpy runs on the
+// legacy default stream, and work on that stream while another host thread records a graph (every handle records
+// its own) is refused by the runtime and spoils that thread's recording.
+static bool upload_sync(void* dst, const void* src, size_t bytes, hipStream_t stream) {
+  return hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, stream) == hipSuccess &&
+         hipStreamSynchronize(stream) == hipSuccess;
+}
+
 // dst[e] = sum over the nb op outputs src[b*n + e], b ascending (fixed order); the same for the 3x3 virials
 __global__ void combine_kernel(double* dst, const double* src, int n, int nb, double* vdst, const double* vsrc) {
   const int e = blockIdx.x * blockDim.x + threadIdx.x;
@@ -166,6 +174,7 @@ struct StafModel {
   bool dev_mlp = false;
   std::vector<staf::DevMlpNet> dnets;
   DevBuf<double> raddescr, des3bsupp, der2b, der3bsupp, unit;   // nr-wide rows per owned atom; unit = (u, 1/r)
+  DevBuf<double> slotf, selff;   // slot forces [nlocal, nr, 3] and centres' own forces [nlocal, 3] (own-list calls)
   DevBuf<int> intmap2b, numtriplet, type_map, tipos, actual_type;
   // host staging
   std::vector<double> af_h, gr_h, tmp2, tmp3;
@@ -203,8 +212,7 @@ static bool load_species_params(StafModel* m) {
         {&m->alpha2b[k], &a2}, {&m->alpha3b[k], &a3}, {&m->emb2b[k], &e2}, {&m->emb3b[k], &e3}};
     for (auto& u : up) {
       if (!u.d->reserve(u.h->size())) return false;
-      if (hipMemcpy(u.d->p, u.h->data(), u.h->size() * sizeof(double), hipMemcpyHostToDevice) != hipSuccess)
-        return false;
+      if (!upload_sync(u.d->p, u.h->data(), u.h->size() * sizeof(double), m->stream)) return false;
     }
   }
   return true;
@@ -299,6 +307,19 @@ StafModel* staf_load(const char* model_dir, const StafOptions* opt) {
     return NULL;
   }
   m->ntc = m->nt * (m->nt + 1) / 2;
+  // Streams of the model (default priority; non-blocking: no implicit ordering with the legacy default stream).
+  bool ok = hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking) == hipSuccess &&
+            hipEventCreateWithFlags(&m->ev_fork, hipEventDisableTiming) == hipSuccess;
+  m->sstream.assign(m->nt, nullptr);
+  m->ev_join.assign(m->nt, nullptr);
+  for (int k = 0; k < m->nt && ok; k++)
+    ok = hipStreamCreateWithFlags(&m->sstream[k], hipStreamNonBlocking) == hipSuccess &&
+         hipEventCreateWithFlags(&m->ev_join[k], hipEventDisableTiming) == hipSuccess;
+  if (!ok) {
+    fprintf(stderr, "staf_load: cannot create the model's streams\n");
+    staf_free(m);
+    return NULL;
+  }
   if (!load_species_params(m)) {
     fprintf(stderr, "staf_load: cannot read the type*_alpha_*.dat / type*_type_emb_*.dat files of %s\n", model_dir);
     staf_free(m);
@@ -319,7 +340,7 @@ StafModel* staf_load(const char* model_dir, const StafOptions* opt) {
   if (!(m->opt.reserved & 2) && !getenv("STAF_MLP_HOST")) {
     m->dnets.resize(m->nt);
     m->dev_mlp = true;
-    for (int k = 0; k < m->nt && m->dev_mlp; k++) m->dev_mlp = staf::dev_mlp_upload(m->mlp, k, &m->dnets[k]);
+    for (int k = 0; k < m->nt && m->dev_mlp; k++) m->dev_mlp = staf::dev_mlp_upload(m->mlp, k, &m->dnets[k], m->stream);
     if (!m->dev_mlp) {
       for (auto& n : m->dnets) staf::dev_mlp_free(&n);
       m->dnets.clear();
@@ -330,23 +351,16 @@ StafModel* staf_load(const char* model_dir, const StafOptions* opt) {
     staf_free(m);
     return NULL;
   }
-  // Streams of the model (default priority; non-blocking: no implicit ordering with the legacy default stream).
-  bool ok = hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking) == hipSuccess &&
-            hipEventCreateWithFlags(&m->ev_fork, hipEventDisableTiming) == hipSuccess;
-  m->sstream.assign(m->nt, nullptr);
-  m->ev_join.assign(m->nt, nullptr);
-  for (int k = 0; k < m->nt && ok; k++)
-    ok = hipStreamCreateWithFlags(&m->sstream[k], hipStreamNonBlocking) == hipSuccess &&
-         hipEventCreateWithFlags(&m->ev_join[k], hipEventDisableTiming) == hipSuccess;
-  if (!ok) {
-    fprintf(stderr, "staf_load: cannot create the model's streams\n");
-    staf_free(m);
-    return NULL;
-  }
   return m;
 }
 
-#define STAF_HIP_OK(x) do { if ((x) != hipSuccess) return -20; } while (0)
+// A GPU runtime failure: -20 to the caller; with STAF_DEBUG set in the environment, where it came from on stderr.
+static int gpu_failure(int line, int code) {
+  static const bool verbose = getenv("STAF_DEBUG") != nullptr;
+  if (verbose) fprintf(stderr, "staf_compute: GPU runtime failure at staf_api.hip:%d (code %d)\n", line, code);
+  return -20;
+}
+#define STAF_HIP_OK(x) do { const hipError_t e_ = (x); if (e_ != hipSuccess) return gpu_failure(__LINE__, (int)e_); } while (0)
 
 int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const double* box, const int* type,
                  const int* howmany, const int* with, int maxneigh, double* e_rank, double* f, double* virial) {
@@ -356,7 +370,7 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
   if (nlocal <= 0) return -3;
   if (!x || !box || (ext && !with)) return -1;
   if (box[0] == 0.0 || box[3] == 0.0 || box[5] == 0.0) return -7;
-  if (hipSetDevice(m->opt.device_id) != hipSuccess) return -20;
+  if (hipSetDevice(m->opt.device_id) != hipSuccess) return gpu_failure(__LINE__, 0);
   const int nt = m->nt, nr = m->nr, na = m->na;
 
   // ---- owned atoms species-sorted into slots [0, nlocal), ghosts keep their order behind them
@@ -433,7 +447,7 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
             m->af3.reserve(L * amax3) && m->g2.reserve(L * amax2) && m->g3.reserve(L * amax3) &&
             m->raddescr.reserve(L * nr) && m->des3bsupp.reserve(L * nr) && m->der2b.reserve(L * 3 * nr) &&
             m->der3bsupp.reserve(L * 3 * nr) && m->unit.reserve(L * 4 * nr) && m->intmap2b.reserve(L * (nr + 1)) &&
-            m->numtriplet.reserve(L) &&
+            m->numtriplet.reserve(L) && m->slotf.reserve(L * nr * 3) && m->selff.reserve(L * 3) &&
             m->type_map.reserve(nall) && m->tipos.reserve(nt) && m->actual_type.reserve(nt);
   if (!ok) return -1;
   if (m->type_map.p != type_map_before) m->type_map_up.clear();   // a new block holds nothing yet
@@ -449,17 +463,17 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
   // species of the slots and atoms per species: sent when they differ from what the device holds (in MD they change
   // when atoms migrate, not every step); the blocking copies read host vectors that the next lines may replace
   if (m->type_map_up != m->type_map_h) {
-    STAF_HIP_OK(hipMemcpy(m->type_map.p, m->type_map_h.data(), (size_t)nall * sizeof(int), hipMemcpyHostToDevice));
+    if (!upload_sync(m->type_map.p, m->type_map_h.data(), (size_t)nall * sizeof(int), st)) return gpu_failure(__LINE__, 0);
     m->type_map_up = m->type_map_h;
   }
   if (m->tipos_up != tipos) {
-    STAF_HIP_OK(hipMemcpy(m->tipos.p, tipos.data(), nt * sizeof(int), hipMemcpyHostToDevice));
+    if (!upload_sync(m->tipos.p, tipos.data(), nt * sizeof(int), st)) return gpu_failure(__LINE__, 0);
     m->tipos_up = tipos;
   }
   if (!m->actual_type_up) {
     std::vector<int> ats(nt);
     for (int k = 0; k < nt; k++) ats[k] = k;
-    STAF_HIP_OK(hipMemcpy(m->actual_type.p, ats.data(), nt * sizeof(int), hipMemcpyHostToDevice));
+    if (!upload_sync(m->actual_type.p, ats.data(), nt * sizeof(int), st)) return gpu_failure(__LINE__, 0);
     m->actual_type_up = true;
   }
   // No synchronisation here: the pinned input block outlives the call's final synchronisation.
@@ -481,7 +495,7 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
   // ---- everything stays on the device: per species fingerprints -> MLP -> forces, one stream per species (the
   // chains meet only in the sum of the forces); one synchronisation at the end of the call
   auto device_sequence = [&]() -> int {
-    if (descriptors() != 0) return -20;
+    if (descriptors() != 0) return gpu_failure(__LINE__, 0);
     // every species stream branches off right behind the descriptors, and the call's stream waits for all of
     // them only after the last chain has been issued: a recorded graph then holds independent branches
     STAF_HIP_OK(hipEventRecord(m->ev_fork, st));
@@ -499,7 +513,13 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
       if (tipos[k] > 0) { op_slot[k] = sl++; by_size.push_back(k); }
     }
     std::stable_sort(by_size.begin(), by_size.end(), [&](int a, int b) { return tipos[a] > tipos[b]; });
+    // With the library's own neighbour list (a symmetric map) the forces take the step-level route: per species one
+    // launch leaves the 2-body + 3-body forces on the centres' neighbour slots (and their virial), and after the
+    // join one launch lets every atom collect them.  A caller's list (ghosts, not symmetric) keeps one force op per
+    // body and species, each with its own gather.
+    const bool slots_route = !ext;
     for (int step = 0; step < 5; step++) {
+      if (slots_route && step == 3) continue;
       for (int k : by_size) {
         const int Nl = tipos[k], Ar = m->Ar[k], Aa = m->Aa[k];
         const int shift = first_atom[k], slot = op_slot[k];
@@ -534,6 +554,25 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
                                               Nl, wo, px, bx, nlocal, skip_pbc, sk);
             break;
           default:
+            if (slots_route) {
+              staf::Force2In<double> two;
+              two.G2 = g2; two.D = m->raddescr.p + o * nr; two.dD = m->der2b.p + o * 3 * nr;
+              two.alpha2b = m->alpha2b[k].p; two.emb2b = m->emb2b[k].p; two.Ar = Ar;
+              double* sf = m->slotf.p + o * nr * 3;
+              rc = staf::force_tripl<double>(g3, m->des3bsupp.p + o * nr, nullptr, m->der3bsupp.p + o * 3 * nr, nullptr,
+                                             m->unit.p + o * 4 * nr, m->intmap2b.p + o * (nr + 1), nullptr, nr, na,
+                                             nall, 1, Aa, m->emb3b[k].p, nt, m->tipos.p, m->actual_type.p + k, nullptr,
+                                             m->numtriplet.p + o, m->alpha3b[k].p, m->type_map.p, Nl, nullptr, nullptr,
+                                             nullptr, nlocal, skip_pbc, sk, sf, m->selff.p + o * 3, &two);
+              if (rc == STAF_OK && want_w)
+                rc = staf::slots_virial<double>(sf, m->intmap2b.p + o * (nr + 1), d_pos, d_box, m->tipos.p,
+                                                m->actual_type.p + k, m->virial_op.p + slot * 9, 1, nall, Nl, nlocal, nr,
+                                                skip_pbc, sk);
+              STAF_HIP_OK(hipEventRecord(m->ev_join[k], sk));
+              if (rc != STAF_OK) return gpu_failure(__LINE__, rc);
+              nops = slot + 1 > nops ? slot + 1 : nops;
+              continue;
+            }
             rc = staf::force_tripl<double>(g3, m->des3bsupp.p + o * nr, nullptr, m->der3bsupp.p + o * 3 * nr, nullptr,
                                            m->unit.p + o * 4 * nr, m->intmap2b.p + o * (nr + 1), nullptr, nr, na, nall,
                                            1, Aa, m->emb3b[k].p, nt, m->tipos.p, m->actual_type.p + k, fo,
@@ -542,12 +581,24 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
             STAF_HIP_OK(hipEventRecord(m->ev_join[k], sk));
             break;
         }
-        if (rc != STAF_OK) return -20;
+        if (rc != STAF_OK) return gpu_failure(__LINE__, rc);
         if (step >= 3) nops = op + 1 > nops ? op + 1 : nops;
       }
     }
     for (int k = 0; k < nt; k++)
       if (tipos[k] > 0) STAF_HIP_OK(hipStreamWaitEvent(st, m->ev_join[k], 0));
+    if (slots_route) {
+      std::vector<const double*> sl(nt, nullptr), se(nt, nullptr);
+      for (int k = 0; k < nt; k++)
+        if (tipos[k] > 0) { sl[k] = m->slotf.p + (size_t)first_atom[k] * nr * 3; se[k] = m->selff.p + (size_t)first_atom[k] * 3; }
+      if (staf::force_total<double>(m->intmap2b.p, nr, nlocal, 1, nt, tipos.data(), sl.data(), se.data(), nullptr,
+                                    d_force, st) != STAF_OK)
+        return gpu_failure(__LINE__, 0);
+      // the species' virials (nothing to add to the forces: n = 0)
+      hipLaunchKernelGGL(combine_kernel, dim3(1), dim3(256), 0, st, d_force, m->force_op.p, 0, nops, d_W,
+                         want_w ? m->virial_op.p : nullptr);
+      return hipGetLastError() == hipSuccess ? 0 : -20;
+    }
     hipLaunchKernelGGL(combine_kernel, dim3((n3 + 255) / 256), dim3(256), 0, st, d_force, m->force_op.p, n3, nops,
                        d_W, want_w ? m->virial_op.p : nullptr);
     return hipGetLastError() == hipSuccess ? 0 : -20;
@@ -560,7 +611,7 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
     if (!m->use_graph || !same) {
       if (rp.state == 2) rp.need = rp.replays < 12 ? (rp.need < 64 ? 2 * rp.need : 64) : 2;
       rp.drop();
-      if (device_sequence() != 0) return -20;
+      if (device_sequence() != 0) return gpu_failure(__LINE__, 0);
       if (m->use_graph) {
         rp.state = 1;
         rp.seen = 1;
@@ -570,7 +621,7 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
         rp.epoch = staf::release_epoch();
       }
     } else if (rp.state == 1 && ++rp.seen < rp.need) {
-      if (device_sequence() != 0) return -20;
+      if (device_sequence() != 0) return gpu_failure(__LINE__, 0);
     } else {
       if (rp.state == 1) {
         // the shape keeps coming and every buffer and scratch block has its final size: record the sequence
@@ -582,12 +633,12 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
           if (g) (void)hipGraphDestroy(g);
           (void)hipGetLastError();
           rp.drop();
-          return -20;
+          return gpu_failure(__LINE__, 0);
         }
         rp.graph = g;
         if (hipGraphInstantiate(&rp.exec, rp.graph, nullptr, nullptr, 0) != hipSuccess) {
           rp.drop();
-          return -20;
+          return gpu_failure(__LINE__, 0);
         }
         rp.state = 2;
       }
@@ -595,7 +646,7 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
       rp.replays++;
     }
   } else {
-    if (descriptors() != 0) return -20;
+    if (descriptors() != 0) return gpu_failure(__LINE__, 0);
     // ---- fingerprints of every species, packed rows [Ar+Aa] for the MLP
     size_t total = 0;
     for (int k = 0; k < nt; k++) total += (size_t)tipos[k] * (m->Ar[k] + m->Aa[k]);
@@ -613,7 +664,7 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
         rc = staf::angular_afs<double>(m->des3bsupp.p + o * nr, nullptr, m->unit.p + o * 4 * nr, nr, na, m->af3.p, 1, Nl,
                                        nullptr, m->intmap2b.p + o * (nr + 1), m->alpha3b[k].p, Aa, m->emb3b[k].p,
                                        m->type_map.p, m->numtriplet.p + o, nt, nlocal, st);
-      if (rc != STAF_OK) return -20;
+      if (rc != STAF_OK) return gpu_failure(__LINE__, rc);
       m->tmp2.resize((size_t)Nl * Ar);
       m->tmp3.resize((size_t)Nl * Aa);
       STAF_HIP_OK(hipMemcpyAsync(m->tmp2.data(), m->af2.p, m->tmp2.size() * sizeof(double), hipMemcpyDeviceToHost, st));
@@ -644,14 +695,14 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
       ev.af_f32 = m->af_f.data();
       ev.energy_f32 = &e_f;
       ev.dE_daf_f32 = m->gr_f.data();
-      if (staf_mlp_eval(m->mlp, &ev) != 0) return -20;
+      if (staf_mlp_eval(m->mlp, &ev) != 0) return gpu_failure(__LINE__, 0);
       energy = (double)e_f;
       for (size_t i = 0; i < total; i++) m->gr_h[i] = (double)m->gr_f[i];
     } else {
       ev.af_f64 = m->af_h.data();
       ev.energy_f64 = &energy;
       ev.dE_daf_f64 = m->gr_h.data();
-      if (staf_mlp_eval(m->mlp, &ev) != 0) return -20;
+      if (staf_mlp_eval(m->mlp, &ev) != 0) return gpu_failure(__LINE__, 0);
     }
     if (!isfinite(energy))
       fprintf(stderr, "staf_compute: non-finite energy=%g nlocal=%d nghost=%d\n", energy, nlocal, nghost);
@@ -688,7 +739,7 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
                                          Aa, m->emb3b[k].p, nt, m->tipos.p, m->actual_type.p + k, m->force_op.p,
                                          m->numtriplet.p + o, m->alpha3b[k].p, m->type_map.p, Nl, m->virial_op.p,
                                          d_pos, d_box, nlocal, skip_pbc, st);
-        if (rc != STAF_OK) return -20;
+        if (rc != STAF_OK) return gpu_failure(__LINE__, rc);
         hipLaunchKernelGGL(add_into_kernel, dim3((n3 + 255) / 256), dim3(256), 0, st, d_force, m->force_op.p, n3);
         STAF_HIP_OK(hipMemcpyAsync(Wk, m->virial_op.p, 9 * sizeof(double), hipMemcpyDeviceToHost, st));
         STAF_HIP_OK(hipStreamSynchronize(st));
@@ -704,7 +755,7 @@ int staf_compute(StafModel* m, int nlocal, int nghost, const double* x, const do
   rc = staf_ops_poll_status(st);
   if (rc == STAF_E_RADIAL_OVERFLOW) return -10;
   if (rc == STAF_E_SCATTER_OVERFLOW) return -11;
-  if (rc != STAF_OK) return -20;
+  if (rc != STAF_OK) return gpu_failure(__LINE__, rc);
   if (m->dev_mlp) {
     const double* e_atom_h = m->out_h.p + (size_t)n3 + 9;
     for (int c = 0; c < 9; c++) W[c] = m->out_h.p[(size_t)n3 + c];

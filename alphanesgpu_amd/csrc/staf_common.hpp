@@ -342,7 +342,17 @@ template <typename real>
 int angular_afs(const real* Dsup, const real* Tang, const real* unit, int nr, int na, real* out, int nf, int Nl,
                 const int* im3, const int* im2, const real* alpha3b, int Aa, const real* emb3b, const int* type_map,
                 const int* numtriplet, int nt, int ld, void* stream);
-template <typename real> struct Force2In;   // staf_force3.hpp: the 2-body inputs of the fused slot forces
+// The 2-body inputs of the force launch that adds the pair forces to the 3-body slot forces (staf_force3.hpp).
+template <typename real>
+struct Force2In {
+  const real* G2;       // [nf, Nl, Ar] dE/dAF2
+  const real* D;        // raddescr [nf, ld, nr]
+  const real* dD;       // der2b [nf, ld, 3, nr]
+  const real* alpha2b;  // [nt, Ar]
+  const real* emb2b;    // [nt, Ar]
+  int Ar;
+};
+
 template <typename real>
 int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* dDsup, const real* d3b,
                 const real* unit, const int* im2, const int* im3, int nr, int na, int N, int nf, int Aa,
@@ -350,6 +360,14 @@ int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* d
                 const int* tipos, const int* actual_type, real* force, const int* numtriplet, const real* alpha3b,
                 const int* type_map, int Nl, real* virial, const real* pos, const real* box, int ld, int skip_pbc,
                 void* stream, real* slots_out = nullptr, real* self_out = nullptr,
-                const struct Force2In<real>* two_body = nullptr);
+                const Force2In<real>* two_body = nullptr);
+// Virial of slot forces (of 2-body, 3-body or both bodies in one array) and the total force collected from the slot
+// forces of all species: the internal forms of staf_op_force_total and of the virial kernels of the force ops.
+template <typename real>
+int slots_virial(const real* gslot, const int* im2, const real* pos, const real* box, const int* tipos,
+                 const int* actual_type, real* virial, int nf, int N, int Nl, int ld, int nr, int skip_pbc, void* stream);
+template <typename real>
+int force_total(const int* im2_full, int nr, int N, int nf, int nt, const int* n_local, const real* const* slot_forces,
+                const real* const* self_forces, const real* const* force_2b, real* total, void* stream);
 
 }  // namespace staf

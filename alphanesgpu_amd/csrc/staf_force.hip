@@ -602,7 +602,7 @@ int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* d
   const bool deferred = slots_out != nullptr;
   if (deferred && (!self_out || virial)) return STAF_E_BAD_ARG;
   // two_body: the 2-body pair forces of the same centres are added to the slot forces (slot outputs only)
-  if (two_body && (!deferred || unit || !two_body->G2 || !two_body->D || !two_body->dD || !two_body->alpha2b ||
+  if (two_body && (!deferred || !two_body->G2 || !two_body->D || !two_body->dD || !two_body->alpha2b ||
                    !two_body->emb2b || two_body->Ar <= 0))
     return STAF_E_BAD_ARG;
   if (deferred && Nl == 0) return STAF_OK;
@@ -649,7 +649,7 @@ int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* d
   };
   using T_ = std::integral_constant<bool, true>;
   using F_ = std::integral_constant<bool, false>;
-  rc = fused ? launch(T_{}, F_{}) : (two_body ? launch(F_{}, T_{}) : launch(F_{}, F_{}));
+  rc = fused ? (two_body ? launch(T_{}, T_{}) : launch(T_{}, F_{})) : (two_body ? launch(F_{}, T_{}) : launch(F_{}, F_{}));
   if (rc) return rc;
   if (deferred) return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
   if (virial) {
@@ -761,8 +761,31 @@ static int gradforce_tripl(const real* Q, const real* G, const real* Dsup, const
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }
 
+// Virial of slot forces (2-body, 3-body or both in one array): W = - sum over centres and radial slots of
+// gslot (x) r, r = minimum-image r_centre - r_neighbour (virial_centre_kernel, virial_frame_kernel above).
 template <typename real>
-static int force_total(const int* im2_full, int nr, int N, int nf, int nt, const int* n_local,
+int slots_virial(const real* gslot, const int* im2, const real* pos, const real* box, const int* tipos,
+                 const int* actual_type, real* virial, int nf, int N, int Nl, int ld, int nr, int skip_pbc,
+                 void* stream_) {
+  if (!gslot || !im2 || !pos || !box || !tipos || !actual_type || !virial || nf <= 0 || N <= 0 || Nl <= 0 || nr <= 0)
+    return STAF_E_BAD_ARG;
+  hipStream_t stream = (hipStream_t)stream_;
+  DeviceState* st = device_state(stream);
+  if (!st) return reserve_failure(stream);
+  if (ld <= 0) ld = Nl;
+  real* vpart = (real*)scratch_reserve(st, stream, (size_t)nf * Nl * 9 * sizeof(real));
+  if (!vpart) return reserve_failure(stream);
+  const int atoms = nf * Nl;
+  hipLaunchKernelGGL(virial_centre_kernel<real>, dim3((atoms + F_WAVES - 1) / F_WAVES), dim3(F_BLOCK), 0, stream, gslot,
+                     im2, (const int*)nullptr, pos, box, tipos, actual_type, vpart, nf, N, Nl, ld, nr, skip_pbc);
+  hipLaunchKernelGGL(virial_frame_kernel<real>, dim3(nf), dim3(F_BLOCK), 0, stream, (const real*)vpart, virial, Nl);
+  return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
+}
+template int slots_virial<double>(const double*, const int*, const double*, const double*, const int*, const int*,
+                                  double*, int, int, int, int, int, int, void*);
+
+template <typename real>
+int force_total(const int* im2_full, int nr, int N, int nf, int nt, const int* n_local,
                        const real* const* slot_forces, const real* const* self_forces, const real* const* force_2b,
                        real* total, void* stream_) {
   if (!im2_full || !n_local || !slot_forces || !self_forces || !total || nr <= 0 || N <= 0 || nf <= 0 || nt <= 0)
@@ -811,6 +834,11 @@ static int force_total(const int* im2_full, int nr, int N, int nf, int nt, const
   }
   return finish_op(st, stream);
 }
+
+template int force_total<double>(const int*, int, int, int, int, const int*, const double* const*, const double* const*,
+                                 const double* const*, double*, void*);
+template int force_total<float>(const int*, int, int, int, int, const int*, const float* const*, const float* const*,
+                                const float* const*, float*, void*);
 
 // Both 3-body parameter gradients of a training step in one pass (tri_reduce_kernel<3>): the gradient of the force
 // op (gradnet, dL/dalpha3b from dL/dF) and the gradient of the fingerprint op (dL/dalpha3b from dL/dAF3).  Outputs

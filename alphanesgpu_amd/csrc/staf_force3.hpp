@@ -114,16 +114,6 @@ struct Force3Cfg {
 // The 2-body pair forces of the same centre, added to its slot forces (W2B): with g(i,s) = 1/2 sum_ch G2[i,ch]
 // c2[t_s,ch] e^{alpha[t_s,ch] D(i,s)} (1 + alpha[t_s,ch] D(i,s)) grad D(i,s) (computeforce_doublets_kernel,
 // STAF/src/force/rad/reforce.cu.cc:70-131) the slot force becomes 3-body + g, over all im2[0] radial neighbours.
-template <typename real>
-struct Force2In {
-  const real* G2;       // [nf, Nl, Ar] dE/dAF2
-  const real* D;        // raddescr [nf, ld, nr]
-  const real* dD;       // der2b [nf, ld, 3, nr]
-  const real* alpha2b;  // [nt, Ar]
-  const real* emb2b;    // [nt, Ar]
-  int Ar;
-};
-
 template <typename real, bool FUSED = false, int NWAVES = 4, bool W2B = false>
 __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real, NWAVES>::MIN_WAVES)) void force3_kernel(
     const real* __restrict__ G, const real* __restrict__ Dsup, const real* __restrict__ Tang,

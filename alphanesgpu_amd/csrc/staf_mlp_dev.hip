@@ -388,7 +388,7 @@ static size_t mlp_lds_bytes(const DevMlpNet& net, int ta) {
 }
 
 template <typename T>
-static bool upload_net(const StafMlp* mlp, int type, DevMlpNet* net) {
+static bool upload_net(const StafMlp* mlp, int type, DevMlpNet* net, hipStream_t stream) {
   const int nl = staf_mlp_internal_nlayers(mlp, type);
   if (nl <= 0 || nl > DEV_MLP_MAX_LAYERS) return false;
   net->nl = nl;
@@ -423,7 +423,10 @@ static bool upload_net(const StafMlp* mlp, int type, DevMlpNet* net) {
   T* block = nullptr;
   if (hipMalloc((void**)&block, host.size() * sizeof(T)) != hipSuccess) return false;
   net->mu = block;   // the block's address: freed through it
-  if (hipMemcpy(block, host.data(), host.size() * sizeof(T), hipMemcpyHostToDevice) != hipSuccess) return false;
+  // on the model's stream, not the legacy default stream (another host thread may be recording a graph)
+  if (hipMemcpyAsync(block, host.data(), host.size() * sizeof(T), hipMemcpyHostToDevice, stream) != hipSuccess ||
+      hipStreamSynchronize(stream) != hipSuccess)
+    return false;
   (void)at_mu;       // 0: mu leads the block
   for (int l = 0; l < nl; l++) {
     net->W[l] = block + at_W[l];
@@ -450,10 +453,10 @@ static bool upload_net(const StafMlp* mlp, int type, DevMlpNet* net) {
   return net->matrix_path || mlp_lds_bytes<T>(*net, MLP_TA_MAX) <= 64 * 1024;
 }
 
-bool dev_mlp_upload(const StafMlp* mlp, int type, DevMlpNet* net) {
+bool dev_mlp_upload(const StafMlp* mlp, int type, DevMlpNet* net, hipStream_t stream) {
   *net = DevMlpNet();
   net->precision = staf_mlp_precision(mlp);
-  return net->precision ? upload_net<double>(mlp, type, net) : upload_net<float>(mlp, type, net);
+  return net->precision ? upload_net<double>(mlp, type, net, stream) : upload_net<float>(mlp, type, net, stream);
 }
 
 void dev_mlp_free(DevMlpNet* net) {

@@ -18,7 +18,7 @@ struct DevMlpNet {
   bool matrix_path = false;   // the matrix-core kernel can hold this stack (LDS), else the vector kernel runs
 };
 
-bool dev_mlp_upload(const StafMlp* mlp, int type, DevMlpNet* net);   // false: not representable (fall back to host)
+bool dev_mlp_upload(const StafMlp* mlp, int type, DevMlpNet* net, hipStream_t stream);   // false: not representable (fall back to host)
 void dev_mlp_free(DevMlpNet* net);
 // af2 [Nl, Ar], af3 [Nl, Aa] (float64 fingerprints) -> atomic energies e_atom [Nl] and d sum(e) / d af split into
 // g2 [Nl, Ar], g3 [Nl, Aa] (float64; computed in the network's precision like the host evaluation).

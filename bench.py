@@ -54,7 +54,7 @@ PROFILED_NAME = {
     ("desc_kernel", "f32"): "staf::desc_kernel<float>",
     ("desc_kernel", "f64"): "staf::desc_kernel<double>",
     ("af3_fused", "f64"): "staf::tri_reduce_kernel<double, 0, true>",
-    ("force3_fused", "f64"): "staf::force3_kernel<double, true, 4, false>",
+    ("force3_fused", "f64"): "staf::force3_kernel<double, true, 4, true>",
 }
 
 
@@ -331,7 +331,7 @@ def run_md(args, workload):
     el_eager = (time.perf_counter() - t1) / nprof
     kern = {}
     for name in ("cell_build_kernel", "desc_kernel", "af2_kernel", "af3_kernel", "force2_kernel", "force3_kernel",
-                 "gather_kernel"):
+                 "gather_kernel", "force_total_kernel"):
         ms, n = ops.kernel_time(name)
         if n:
             kern[name] = dict(ms_per_step=ms / nprof, launches_per_step=n // nprof, avg_launch_ms=ms / n)
@@ -348,9 +348,9 @@ def run_md(args, workload):
     # Bytes the call's kernels move once through HBM by their signatures (no tensor of the angular buffer's width
     # exists on this path).  In rows of N x nr doubles: the radial-only descriptor kernel writes 12 (raddescr,
     # des3bsupp, der2b x3, der3bsupp x3, unit x4) and the neighbour map; the 2-body fingerprints read 1 and the map,
-    # the fused 3-body fingerprints 5 (des3bsupp, unit), the 2-body force 4 (raddescr, der2b), the fused 3-body force 8
-    # (des3bsupp, der3bsupp, unit); the slot forces are written and read once (3 rows); fingerprints and their
-    # gradients are written and read once each; positions in, four per-op force arrays and their sum out.
+    # the fused 3-body fingerprints 5 (des3bsupp, unit), the force launch 12 (raddescr, der2b, des3bsupp, der3bsupp,
+    # unit) -- counted as 4 + 8 below; the slot forces are written and read once (3 rows); fingerprints and their
+    # gradients are written and read once each; positions in, forces out (and the virial pass over the slot forces).
     s = 8
     row = N * nr * s
     imap = N * (nr + 1) * 4
