@@ -212,6 +212,9 @@ __global__ __launch_bounds__(MLP_BLOCK) void mlp_kernel(MlpArgs<T> A) {
 // 16 output columns, slice of the inner dimension) with up to MM_STEPS weight reads in flight per lane; units are
 // dealt round-robin to the 16 waves; slice sums meet in LDS and are added in ascending slice order (fixed order).
 constexpr int MM_TA = 16;
+// Pitch of a column of slice sums in LDS: the lanes of a tile write the same atom row of 16 consecutive columns at
+// once, and 16 atoms (128 bytes in double precision) between them would put all of them on the same banks.
+constexpr int MM_TP = MM_TA + 1;
 constexpr int MM_BLOCK = 1024;
 constexpr int MM_WAVES = MM_BLOCK / WAVE;
 constexpr int MM_STEPS = 12;      // MFMA steps (4 rows of the inner dimension each) per batch of weight reads
@@ -279,7 +282,7 @@ __device__ inline int mm_products(const T* __restrict__ M, int K, int J, const T
     }
     if (col < J) {
 #pragma unroll
-      for (int v = 0; v < 4; v++) part[((size_t)sl * J + col) * MM_TA + MfmaOp<T>::acc_row(lane, v)] = acc[v];
+      for (int v = 0; v < 4; v++) part[((size_t)sl * J + col) * MM_TP + MfmaOp<T>::acc_row(lane, v)] = acc[v];
     }
   }
   return nsl;
@@ -290,7 +293,7 @@ __global__ __launch_bounds__(MM_BLOCK) void mlp_matrix_kernel(MlpArgs<T> A) {
   extern __shared__ __align__(16) unsigned char smem[];
   T* X = (T*)smem;                            // [tot][MM_TA]: input and every layer's output
   T* dl = X + (size_t)A.tot * MM_TA;          // [maxw][MM_TA]: back-propagated deltas
-  T* part = dl + (size_t)A.maxw * MM_TA;      // [slices][width][MM_TA]
+  T* part = dl + (size_t)A.maxw * MM_TA;      // [slices][width][MM_TP]
   const int tid = threadIdx.x;
   const int a0 = blockIdx.x * MM_TA;
   const int n_af = A.n_af;
@@ -313,9 +316,9 @@ __global__ __launch_bounds__(MM_BLOCK) void mlp_matrix_kernel(MlpArgs<T> A) {
     const int nsl = mm_products<T>(A.W[l], in_f, out_f, X + (size_t)off_in * MM_TA, part);
     __syncthreads();
     for (int q = tid; q < out_f * MM_TA; q += MM_BLOCK) {
-      const int j = q / MM_TA;
+      const int j = q / MM_TA, t = q - j * MM_TA;
       T y = A.b[l][j];
-      for (int sl = 0; sl < nsl; sl++) y += part[(size_t)sl * out_f * MM_TA + q];
+      for (int sl = 0; sl < nsl; sl++) y += part[((size_t)sl * out_f + j) * MM_TP + t];
       if (A.act[l] == 1) y = m_tanh(y);
       else if (A.act[l] == 2) y = y > T(0) ? y : T(0);
       X[(size_t)off_out * MM_TA + q] = y;
@@ -346,7 +349,8 @@ __global__ __launch_bounds__(MM_BLOCK) void mlp_matrix_kernel(MlpArgs<T> A) {
     __syncthreads();
     for (int q = tid; q < in_f * MM_TA; q += MM_BLOCK) {
       T g = 0;
-      for (int sl = 0; sl < nsl; sl++) g += part[(size_t)sl * in_f * MM_TA + q];
+      const int j = q / MM_TA, t = q - j * MM_TA;
+      for (int sl = 0; sl < nsl; sl++) g += part[((size_t)sl * in_f + j) * MM_TP + t];
       dl[q] = g;
     }
     __syncthreads();
@@ -375,7 +379,7 @@ static size_t mm_lds_bytes(const DevMlpNet& net) {
     npart = f > npart ? f : npart;
     npart = b > npart ? b : npart;
   }
-  return ((size_t)net.tot + net.maxw + npart) * MM_TA * sizeof(T);
+  return (((size_t)net.tot + net.maxw) * MM_TA + npart * MM_TP) * sizeof(T);
 }
 
 // LDS of one workgroup of ta atoms: activations, deltas, and slice sums (slices * ta * width <= ta * max(MLP_BLOCK,
