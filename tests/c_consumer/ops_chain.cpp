@@ -158,6 +158,8 @@ int main(int argc, char** argv) {
   check_i("numtriplet", ntr, A);
 
   const double* Q = up_d("Q");
+  // per species: the force ops' outputs and the slot forces, kept for the collecting launch after the loop
+  std::vector<const double*> f2_of(nt), f3_of(nt), slots_of(nt), selfs_of(nt), both_slots_of(nt), both_selfs_of(nt);
   int first = 0;   // first atom of the centre species: its rows are views into the descriptor outputs (ld_atoms = N)
   for (int k = 0; k < nt; first += tipos_h[k], k++) {
     const int Nl = tipos_h[k];
@@ -217,7 +219,31 @@ int main(int argc, char** argv) {
     STAF_CALL(staf_op_gradforce_tripl_f64(Q, G3, supk, angk, d3sk, d3k, im2k, im3k, nr, na, N, nf, Aa, e3, nt, tipos,
                                           actual, ntrk, a3, type_map, Nl, gf3n, gf3a, gf3e, nullptr, nullptr, nullptr,
                                           N, stream));
+    // step-level entry points: both 3-body gradients in one pass; the 3-body force (alone, and with the 2-body pair
+    // forces) left on the neighbour slots for staf_op_force_total
+    double* fgn = dev_alloc<double>(L * Aa);
+    double* fgaf = dev_alloc<double>(ntc * 3 * Aa);
+    double* fgae = dev_alloc<double>(ntc * 3 * Aa);
+    double* fge = dev_alloc<double>(ntc * Aa);
+    double* slots = dev_alloc<double>(L * nr * 3);
+    double* selfs = dev_alloc<double>(L * 3);
+    double* both_slots = dev_alloc<double>(L * nr * 3);
+    double* both_selfs = dev_alloc<double>(L * 3);
+    STAF_CALL(staf_op_grads_tripl_fused_f64(Q, G3, P3, supk, angk, d3sk, d3k, im2k, im3k, nr, na, N, nf, Aa, e3, nt,
+                                            tipos, actual, ntrk, a3, type_map, Nl, fgn, fgaf, fgae, fge, nullptr,
+                                            nullptr, nullptr, N, stream));
+    STAF_CALL(staf_op_force_tripl_slots_f64(G3, supk, angk, d3sk, d3k, im2k, im3k, nr, na, N, nf, Aa, e3, nt, tipos,
+                                            actual, slots, selfs, ntrk, a3, type_map, Nl, N, stream));
+    STAF_CALL(staf_op_forces_slots_f64(G3, G2, supk, angk, d3sk, d3k, radk, d2k, im2k, im3k, nr, na, N, nf, Aa, Ar, e3,
+                                       a3, a2, e2, nt, tipos, actual, both_slots, both_selfs, ntrk, type_map, Nl, N,
+                                       stream));
+    f2_of[k] = f2, f3_of[k] = f3, slots_of[k] = slots, selfs_of[k] = selfs;
+    both_slots_of[k] = both_slots, both_selfs_of[k] = both_selfs;
     HIP_OK(hipStreamSynchronize(stream));
+    check_d("gf3n_" + s, fgn, L * Aa);
+    check_d("gf3a_" + s, fgaf, ntc * 3 * Aa);
+    check_d("g3a_" + s, fgae, ntc * 3 * Aa);
+    check_d("g3e_" + s, fge, ntc * Aa);
     check_d("af2_" + s, af2, L * Ar);
     check_d("af3_" + s, af3, L * Aa);
     check_d("f2_" + s, f2, (size_t)nf * 3 * N);
@@ -232,6 +258,33 @@ int main(int argc, char** argv) {
     check_d("gf3n_" + s, gf3n, L * Aa);
     check_d("gf3a_" + s, gf3a, ntc * 3 * Aa);
     check_d("gf3e_" + s, gf3e, ntc * Aa);
+  }
+  // ---- the collecting launch: total force of the step from the slot forces of every centre species
+  const size_t F = (size_t)nf * 3 * N;
+  double* total = dev_alloc<double>(F);
+  double* total_both = dev_alloc<double>(F);
+  STAF_CALL(staf_op_force_total_f64(im2, nr, N, nf, nt, tipos_h.data(), slots_of.data(), selfs_of.data(),
+                                    f2_of.data(), total, stream));
+  STAF_CALL(staf_op_force_total_f64(im2, nr, N, nf, nt, tipos_h.data(), both_slots_of.data(), both_selfs_of.data(),
+                                    nullptr, total_both, stream));
+  HIP_OK(hipStreamSynchronize(stream));
+  check_d("ftot", total, F);
+  check_d("ftot", total_both, F);
+  {
+    // the same bits as the per-op force arrays added in the order f2[0], f3[0], f2[1], f3[1], ...
+    std::vector<double> want(F), part(F), got(F);
+    for (int k = 0; k < nt; k++)
+      for (const double* src : {f2_of[k], f3_of[k]}) {
+        HIP_OK(hipMemcpy(part.data(), src, F * 8, hipMemcpyDeviceToHost));
+        const bool start = k == 0 && src == f2_of[0];
+        for (size_t e = 0; e < F; e++) want[e] = start ? part[e] : want[e] + part[e];
+      }
+    HIP_OK(hipMemcpy(got.data(), total, F * 8, hipMemcpyDeviceToHost));
+    size_t bad = 0;
+    for (size_t e = 0; e < F; e++) bad += memcmp(&got[e], &want[e], 8) != 0;
+    printf("%-12s %9zu doubles  %zu differ in bits from the per-op arrays added  %s\n", "ftot", F, bad,
+           bad ? "FAIL" : "ok");
+    if (bad) failures++;
   }
   staf_ops_release();
   printf("ops_chain: %s\n", failures ? "FAILED" : "OK");

@@ -46,6 +46,11 @@ def write_fixture(path, oracle, nf=2, nr=60, na=1770):
             _record(f, k, d[k])     # the oracle leaves zeros in every padded slot
         for k in ("intmap2b", "intmap3b", "numtriplet"):
             _record(f, k, d[k].astype(np.int32))
+        ftot = None     # the callers' sum of the per-op force arrays, in the order of staf_op_force_total
+        for k in range(len(tipos)):
+            for part in (ref["f2"][k], ref["f3"][k]):
+                ftot = part.copy() if ftot is None else ftot + part
+        _record(f, "ftot", ftot)
         for k in range(len(tipos)):
             m = params[k]
             for name in ("alpha2b", "emb2b", "alpha3b", "emb3b"):
@@ -90,7 +95,7 @@ def test_fixture_writer_round_trip(oracle, tmp_path):
             kind, count = struct.unpack("<iq", f.read(12))
             names[h.rstrip(b"\0").decode()] = (kind, count)
             f.seek(count * (4 if kind == 0 else 8), 1)
-    assert names["dims"] == (0, 5) and names["der3b"] == (1, 96 * 3 * 2 * 1770)
+    assert names["ftot"] == (1, 3 * 96) and names["dims"] == (0, 5) and names["der3b"] == (1, 96 * 3 * 2 * 1770)
     for k in range(2):
         for nm in ("af2", "af3", "f2", "f3", "g2a", "g2e", "g3a", "g3e", "gf2n", "gf2a", "gf2e", "gf3n", "gf3a", "gf3e"):
             assert f"{nm}_{k}" in names
