@@ -324,11 +324,15 @@ int angular_afs(const real* Dsup, const real* Tang, const real* unit, int nr, in
   A.nf = nf; A.Nl = Nl; A.ld = ld; A.nr = nr; A.na = na; A.Aa = Aa; A.nt = nt;
   {
     KernelTimer kt_("af3_kernel", (hipStream_t)stream_);
+    // as many workgroups as the device holds at once (or a whole number of such rounds), each taking several centres
     if (unit)
-      hipLaunchKernelGGL((tri_reduce_kernel<real, 0, true>), dim3(nf * Nl), dim3(TRI_BLOCK), lds,
+      hipLaunchKernelGGL((tri_reduce_kernel<real, 0, true>),
+                         dim3(tri_grid((const void*)tri_reduce_kernel<real, 0, true>, lds, nf * Nl)), dim3(TRI_BLOCK), lds,
                          (hipStream_t)stream_, A);
     else
-      hipLaunchKernelGGL((tri_reduce_kernel<real, 0>), dim3(nf * Nl), dim3(TRI_BLOCK), lds, (hipStream_t)stream_, A);
+      hipLaunchKernelGGL((tri_reduce_kernel<real, 0>),
+                         dim3(tri_grid((const void*)tri_reduce_kernel<real, 0>, lds, nf * Nl)), dim3(TRI_BLOCK), lds,
+                         (hipStream_t)stream_, A);
   }
   return hipGetLastError() == hipSuccess ? STAF_OK : STAF_E_HIP;
 }

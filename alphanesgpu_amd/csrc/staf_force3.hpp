@@ -225,7 +225,11 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
   int t_s = 0;
   if (slot_t) t_s = type_map[nj];
   if (tid >= nsig && tid < 16) nact[tid] = 0;
-  for (int q = tid; q < NW * 4 * nr; q += THREADS) acc[q] = 0;
+  {
+    real4 z;
+    z.x = z.y = z.z = z.w = 0;
+    for (int q = tid; q < NW * nr; q += THREADS) ((real4*)acc)[q] = z;
+  }
   for (int sgm = wave; sgm < nsig; sgm += NW) {
     int base = 0;
     for (int a0 = 0; a0 < Aa; a0 += WAVE) {
@@ -562,33 +566,38 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
   }
   __syncthreads();
 
-  // ---- slot forces (waves added in a fixed order; one slot per thread: m <= nr < THREADS), centre's own force
+  // ---- slot forces (waves added in a fixed order; one slot per thread: m <= nr < THREADS), centre's own force.
+  // Only the waves that hold slots (the first one for up to 64 slots) form sums; the others' share is zero.
   real f3[3] = {0, 0, 0};
-  if (slot) {
-    real t4[4] = {0, 0, 0, 0};
+  if (wave * WAVE < nr) {
+    if (slot) {
+      real t4[4] = {0, 0, 0, 0};
 #pragma unroll
-    for (int w = 0; w < NW; w++) {
-      const real4 a = acc_get(acc + (size_t)w * 4 * nr, tid);
-      t4[0] += a.x; t4[1] += a.y; t4[2] += a.z; t4[3] += a.w;
+      for (int w = 0; w < NW; w++) {
+        const real4 a = acc_get(acc + (size_t)w * 4 * nr, tid);
+        t4[0] += a.x; t4[1] += a.y; t4[2] += a.z; t4[3] += a.w;
+      }
+#pragma unroll
+      for (int c = 0; c < 3; c++) f3[c] = t4[c] + t4[3] * sg[c * nr + tid];
+    }
+    if constexpr (W2B) {
+      // the pair force of slot tid (zero weight beyond the radial neighbours); slots beyond the angular cutoff carry it alone
+      if (tid < nr) {
+        real w = 0;
+#pragma unroll
+        for (int w_ = 0; w_ < NW; w_++) w += w2p[w_ * nr + tid];
+        w *= real(0.5);
+#pragma unroll
+        for (int c = 0; c < 3; c++) f3[c] += w * B2.dD[rowAtom * 3 * nr + c * nr + tid];
+      }
     }
 #pragma unroll
-    for (int c = 0; c < 3; c++) f3[c] = t4[c] + t4[3] * sg[c * nr + tid];
-  }
-  if constexpr (W2B) {
-    // the pair force of slot tid (zero weight beyond the radial neighbours); slots beyond the angular cutoff carry it alone
-    if (tid < nr) {
-      real w = 0;
-#pragma unroll
-      for (int w_ = 0; w_ < NW; w_++) w += w2p[w_ * nr + tid];
-      w *= real(0.5);
-#pragma unroll
-      for (int c = 0; c < 3; c++) f3[c] += w * B2.dD[rowAtom * 3 * nr + c * nr + tid];
+    for (int c = 0; c < 3; c++) {
+      const real t = wave_sum_to_last(f3[c]);
+      if (lane == WAVE - 1) xch[wave * 4 + c] = t;
     }
-  }
-#pragma unroll
-  for (int c = 0; c < 3; c++) {
-    const real t = wave_sum_to_last(f3[c]);
-    if (lane == WAVE - 1) xch[wave * 4 + c] = t;
+  } else if (lane < 3) {
+    xch[wave * 4 + lane] = 0;
   }
   __syncthreads();
   // global stores after the last barrier: nothing waits for them
