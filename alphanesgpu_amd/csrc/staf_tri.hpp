@@ -525,35 +525,36 @@ tri_reduce_kernel(TriArgs<real> A) {
                 } else {
                   const real2 g1 = r1[TRI_CAP], g2 = r2[TRI_CAP];
                   const real D1 = g1.x, D2 = g2.x, V1 = g1.y, V2 = g2.y;
-                  // With X1 = sim2 V1 + sim1 V2, X2 = sim1 V1 + sim2 V2, W = a1 X1 + a2 X2 (the factor 1/2 of both
-                  // weights is applied once per channel at the end):
+                  // With A = a1 V1 + a2 V2, B = a1 V2 + a2 V1 (the factor 1/2 of both weights is applied once per
+                  // channel at the end) and W = sim2 A + sim1 B:
                   //   d/dG      : hU ss + hT W                         hT = e^{bT} T,  hU = e^{bT} (1 + bT) U
-                  //   d/da1     : hU (p + q) + hT (X1 + a1 (p V1 + q V2) + a2 (q V1 + p V2)),  p = sim2 D1, q = sim1 D2
-                  //   d/da2     : hU (r + t) + hT (X2 + a2 (r V1 + t V2) + a1 (t V1 + r V2)),  r = sim1 D1, t = sim2 D2
-                  //   d/dbeta   : hT ((2 + bT) ss U + T W)
+                  //   d/da1     : hU (sim2 D1 + sim1 D2) + hT (sim2 (V1 + D1 A) + sim1 (V2 + D2 B))
+                  //   d/da2     : hU (sim1 D1 + sim2 D2) + hT (sim1 (V1 + D1 B) + sim2 (V2 + D2 A))
+                  //   d/dbeta   : hT ((2 + bT) ss U + T W) = T (hU ss + hT W + e^{bT} U ss): T times (the d/dG term + eU ss)
+                  // (the sums of the reference's per-term products, STAF/src/grad_force/ang/reforce.cu.cc:120-200,
+                  // with the common factors taken out: 38 operations per item beside the exponential)
                   const real bT = be * T;
                   const real hT = ebt * T;
                   const real eU = ebt * U;
                   const real hU = r_fma(eU, bT, eU);
                   const real ss = sim1 + sim2;
-                  const real X1 = r_fma(sim2, V1, sim1 * V2);
-                  const real X2 = r_fma(sim1, V1, sim2 * V2);
-                  const real W = r_fma(a1, X1, a2 * X2);
-                  acc[0] = r_fma(hU, ss, acc[0]);
-                  acc[0] = r_fma(hT, W, acc[0]);
-                  const real p_ = sim2 * D1, q_ = sim1 * D2, r_ = sim1 * D1, t_ = sim2 * D2;
-                  const real Y1 = r_fma(p_, V1, q_ * V2), Y2 = r_fma(q_, V1, p_ * V2);
-                  acc[1] = r_fma(hU, p_ + q_, acc[1]);
-                  acc[1] = r_fma(hT, r_fma(a2, Y2, r_fma(a1, Y1, X1)), acc[1]);
-                  const real Z1 = r_fma(r_, V1, t_ * V2), Z2 = r_fma(t_, V1, r_ * V2);
-                  acc[2] = r_fma(hU, r_ + t_, acc[2]);
-                  acc[2] = r_fma(hT, r_fma(a1, Z2, r_fma(a2, Z1, X2)), acc[2]);
-                  acc[3] = r_fma(hT, r_fma((real(2) + bT) * ss, U, T * W), acc[3]);
+                  const real Aw = r_fma(a1, V1, a2 * V2);
+                  const real Bw = r_fma(a1, V2, a2 * V1);
+                  const real W = r_fma(sim2, Aw, sim1 * Bw);
+                  const real dG = r_fma(hT, W, hU * ss);
+                  acc[0] += dG;
+                  const real pq = r_fma(sim2, D1, sim1 * D2);
+                  const real rt = r_fma(sim1, D1, sim2 * D2);
+                  acc[1] = r_fma(hU, pq, acc[1]);
+                  acc[1] = r_fma(hT, r_fma(sim2, r_fma(D1, Aw, V1), sim1 * r_fma(D2, Bw, V2)), acc[1]);
+                  acc[2] = r_fma(hU, rt, acc[2]);
+                  acc[2] = r_fma(hT, r_fma(sim1, r_fma(D1, Bw, V1), sim2 * r_fma(D2, Aw, V2)), acc[2]);
+                  acc[3] = r_fma(T, r_fma(eU, ss, dG), acc[3]);
                   if constexpr (MODE == 3) {
                     // the energy branch's sums of the same item (MODE 1 above with w = hT):
                     // d/da1: (sim2 D1 + sim1 D2) w,  d/da2: (sim2 D2 + sim1 D1) w,  d/dbeta: (sim1 + sim2) w T
-                    acc[4] = r_fma(p_ + q_, hT, acc[4]);
-                    acc[5] = r_fma(r_ + t_, hT, acc[5]);
+                    acc[4] = r_fma(pq, hT, acc[4]);
+                    acc[5] = r_fma(rt, hT, acc[5]);
                     acc[6] = r_fma(ss * hT, T, acc[6]);
                   }
                 }

@@ -31,7 +31,7 @@ VALU_PEAK_WAVE_INST = 256 * 4 * 2.4e9 / 4
 # the op's accumulations; fp64 carries the written-out exponential, 18 instructions instead of the hardware exp2).
 # Set-up, triplet decoding, table building, staging and reductions are overhead and not counted.
 ALGORITHMIC_INST = {"af3_kernel": (7, 24), "force3_kernel": (13, 30), "grad3_kernel": (14, 31),
-                    "gradforce3_kernel": (44, 61), "grads3_kernel": (48, 65)}
+                    "gradforce3_kernel": (36, 53), "grads3_kernel": (40, 57)}
 
 SETTLE_STEPS = 300   # untimed graph replays of the set-up, see run_workload()
 REPEATS = 5          # timed blocks of --steps steps each; the median block is reported
