@@ -133,11 +133,24 @@ __device__ inline int mul24(int a, int b) { return __mul24(a, b); }
 // STAF/src/descriptor_builder/reforce.cu.cc:137-146.  j m - j (j + 1) / 2 = j (2 m - 1 - j) / 2, m <= 2048.
 __device__ inline int tri_rowstart(int j, int m) { return mul24(j, 2 * m - 1 - j) >> 1; }
 
-// Inverse of the numbering: nn -> (j,k), 0 <= nn < m(m-1)/2, m <= 2048.  The hardware square root (1 ulp) puts
-// the row estimate within one of the exact row (two steps each way are taken); the row start follows the row in
-// steps of the row length m - 1 - j, so that the comparisons with the exact integer row starts cost no multiply.
+// Inverse of the numbering: nn -> (j,k), 0 <= nn < m(m-1)/2, m <= 2048.
+// With t = 2m - 1 the row is j = floor((t - sqrt(t^2 - 8 nn)) / 2); the root is an integer exactly at a row's first
+// pair, where a rounding error would decide the row.
+// m <= 255: the root is taken of t^2 - 8 nn - 4 instead, which moves the quotient 1/(t - 2j) >= 0.002 away from the
+// integers on either side (up at a row's first pair, down at the last pair of the row before) -- sixty times the
+// error of the single-precision root and subtraction, so the truncation is the row and no correction step follows
+// (checked for every m <= 255 and every nn, with the root off by up to two units in the last place).
+// m > 255: the hardware square root (1 ulp) puts the row estimate within one of the exact row (two steps each way
+// are taken); the row start follows the row in steps of the row length m - 1 - j, so that the comparisons with the
+// exact integer row starts cost no multiply.
 __device__ inline void tri_decode(int nn, int m, int& j, int& k) {
   const int t = 2 * m - 1;
+  if (m <= 255) {
+    const int jj = (int)(((float)t - __builtin_amdgcn_sqrtf((float)(mul24(t, t) - 4 - 8 * nn))) * 0.5f);
+    j = jj;
+    k = nn - (mul24(jj, t - jj) >> 1) + jj + 1;
+    return;
+  }
   int jj = (int)(((float)t - __builtin_amdgcn_sqrtf((float)(mul24(t, t) - 8 * nn))) * 0.5f);
   jj = jj < 0 ? 0 : (jj > m - 2 ? m - 2 : jj);
   int rs = mul24(jj, t - jj) >> 1;

@@ -152,7 +152,7 @@ __global__ __launch_bounds__((Force3Cfg<real, NWAVES>::THREADS), (Force3Cfg<real
   const size_t rowAtom = (size_t)b * ld + p_;
   const int* im = im2 + rowAtom * (nr + 1);
   int m = numtriplet[rowAtom];
-  if (m > nr) m = nr;
+  m = m > nr ? nr : (m < 0 ? 0 : m);
   int ntri = (m * (m - 1)) / 2;
   if (ntri > na) ntri = na;
   const real* Trow = Tang + rowAtom * na;

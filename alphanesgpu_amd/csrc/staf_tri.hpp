@@ -353,7 +353,7 @@ tri_reduce_kernel(TriArgs<real> A) {
     const int* im = A.im2 + rowAtom * (nr + 1);
     constexpr bool early = decltype(early_c)::value;   // the centre whose first reads were issued at the kernel's start
     m = early ? m0 : A.numtriplet[rowAtom];
-    if (m > nr) m = nr;
+    m = m > nr ? nr : (m < 0 ? 0 : m);
     Trow = A.Tang + rowAtom * na;
     d3 = (const real2*)A.d3b + rowAtom * 3 * na;
     // ---- per-atom slot data
