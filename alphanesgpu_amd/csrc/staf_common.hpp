@@ -101,6 +101,42 @@ __device__ inline double dpp_get(double v) {
   const int hi = __builtin_amdgcn_update_dpp(0, (int)(b >> 32), CTRL, ROW_MASK, 0xf, false);
   return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
 }
+// The two steps that carry a prefix across the rows of 16 lanes: s += (lane 15 of the row before) in rows 1 and 3,
+// then s += (lane 31) in rows 2 and 3.  Written as `s += dpp_get<..>(s)` each costs a zero, a move and an add,
+// because the rows that receive nothing need a 0 to add; as one add whose result is written in the selected rows
+// only (the others keep s) it is a single instruction.  Single precision only: the lane moves are 32 bits wide.
+// A lane move reads a register two cycles after the instruction that wrote it at the earliest: the idle cycles
+// stand in front of the moves, and behind them for whatever lane operation follows.
+__device__ inline void dpp_rows_carry(float& a) {
+  asm("s_nop 1\n\t"
+      "v_add_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa\n\t"
+      "s_nop 1\n\t"
+      "v_add_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc\n\t"
+      "s_nop 1"
+      : "+v"(a));
+}
+__device__ inline void dpp_rows_carry(float& a, float& b, float& c, float& d) {
+  asm("s_nop 1\n\t"
+      "v_add_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa\n\t"
+      "v_add_f32_dpp %1, %1, %1 row_bcast:15 row_mask:0xa\n\t"
+      "v_add_f32_dpp %2, %2, %2 row_bcast:15 row_mask:0xa\n\t"
+      "v_add_f32_dpp %3, %3, %3 row_bcast:15 row_mask:0xa\n\t"
+      "v_add_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc\n\t"
+      "v_add_f32_dpp %1, %1, %1 row_bcast:31 row_mask:0xc\n\t"
+      "v_add_f32_dpp %2, %2, %2 row_bcast:31 row_mask:0xc\n\t"
+      "v_add_f32_dpp %3, %3, %3 row_bcast:31 row_mask:0xc\n\t"
+      "s_nop 1"
+      : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+}
+__device__ inline void dpp_rows_carry(double& s) {
+  s += dpp_get<0x142, 0xa>(s);   // lane 15 of a row -> every lane of the next row (rows 1 and 3 take it)
+  s += dpp_get<0x143, 0xc>(s);   // lane 31 -> rows 2 and 3
+}
+__device__ inline void dpp_rows_carry(double& a, double& b, double& c, double& d) {
+  a += dpp_get<0x142, 0xa>(a); b += dpp_get<0x142, 0xa>(b); c += dpp_get<0x142, 0xa>(c); d += dpp_get<0x142, 0xa>(d);
+  a += dpp_get<0x143, 0xc>(a); b += dpp_get<0x143, 0xc>(b); c += dpp_get<0x143, 0xc>(c); d += dpp_get<0x143, 0xc>(d);
+}
+
 // Sum over the 64 lanes with register-to-register lane moves only; the total is valid in lane 63 alone.
 // Fixed tree: prefix steps 1,2,3,4,8 inside each row of 16, then row 0->1, 2->3, and rows 0-1 -> 2-3.
 template <typename T>
@@ -110,8 +146,7 @@ __device__ inline T wave_sum_to_last(T v) {
   s += dpp_get<0x113, 0xf>(v);
   s += dpp_get<0x114, 0xf>(s);
   s += dpp_get<0x118, 0xf>(s);
-  s += dpp_get<0x142, 0xa>(s);   // lane 15 of a row -> every lane of the next row (rows 1 and 3 take it)
-  s += dpp_get<0x143, 0xc>(s);   // lane 31 -> rows 2 and 3
+  dpp_rows_carry(s);
   return s;
 }
 // Wave-uniform value loaded through a vector path (e.g. from LDS) moved to a scalar register, so that loop

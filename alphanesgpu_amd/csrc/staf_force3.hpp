@@ -48,10 +48,7 @@ __device__ inline void wave_scan4(T (&v)[4]) {
   for (int c = 0; c < 4; c++) s[c] += dpp_get<0x114, 0xf>(s[c]);
 #pragma unroll
   for (int c = 0; c < 4; c++) s[c] += dpp_get<0x118, 0xf>(s[c]);
-#pragma unroll
-  for (int c = 0; c < 4; c++) s[c] += dpp_get<0x142, 0xa>(s[c]);   // lane 15 of a row -> every lane of the next row
-#pragma unroll
-  for (int c = 0; c < 4; c++) s[c] += dpp_get<0x143, 0xc>(s[c]);   // lane 31 -> rows 2 and 3
+  dpp_rows_carry(s[0], s[1], s[2], s[3]);
 #pragma unroll
   for (int c = 0; c < 4; c++) v[c] = s[c];
 }
