@@ -28,10 +28,11 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 VALU_PEAK_WAVE_INST = 256 * 4 * 2.4e9 / 4
 # Vector instructions the formulas of a 3-body op need per (triplet, active channel) item, fp32 / fp64, counted on
 # the inner loops of csrc/staf_tri.hpp and csrc/staf_force3.hpp (pair factors from the exponential tables, exp(beta T),
-# the op's accumulations; fp64 carries the written-out exponential, 18 instructions instead of the hardware exp2).
+# the op's accumulations; fp64 carries the written-out exponential instead of the hardware exp2: 15 instructions and a
+# table read in the reduce kernels, 18 in the force kernel).
 # Set-up, triplet decoding, table building, staging and reductions are overhead and not counted.
-ALGORITHMIC_INST = {"af3_kernel": (7, 24), "force3_kernel": (13, 30), "grad3_kernel": (14, 31),
-                    "gradforce3_kernel": (36, 53), "grads3_kernel": (40, 57)}
+ALGORITHMIC_INST = {"af3_kernel": (7, 21), "force3_kernel": (13, 30), "grad3_kernel": (14, 28),
+                    "gradforce3_kernel": (36, 50), "grads3_kernel": (40, 54)}
 
 SETTLE_STEPS = 300   # untimed graph replays of the set-up, see run_workload()
 REPEATS = 5          # timed blocks of --steps steps each; the median block is reported
