@@ -331,7 +331,10 @@ int staf_op_gradforce_tripl_f64(const double* prevgrad, const double* netderiv, 
  *   prevgrad_force [nf,3N] = dL/dF, netderiv [nf,Nl,num_finger] = dE/dAF3, prevgrad_energy [nf,Nl,num_finger] = dL/dAF3
  *   -> gradnet_3b [nf,Nl,num_finger] and grad_alpha3b_force [ntc,3*num_finger] as staf_op_gradforce_tripl,
  *      grad_alpha3b_energy [ntc,3*num_finger] as staf_op_alphagrad_ang, grad_emb3b [ntc,num_finger] (zero, once).
- * Results agree with the separate ops to rounding (same sums, other order of a few operations). */
+ * Results agree with the separate ops to rounding (same sums, other order of a few operations).
+ * grad_alpha3b_energy is linear in prevgrad_energy, which must be complete when the pass runs: where dL/dAF3 has a
+ * part that is itself derived from gradnet_3b (a force loss back-propagated through the network's second
+ * derivative), that part is added afterwards with staf_op_alphagrad_ang. */
 int staf_op_grads_tripl_fused_f32(const float* prevgrad_force, const float* netderiv, const float* prevgrad_energy,
                                   const float* desr, const float* desa, const float* intderiv_r,
                                   const float* intderiv_a, const int* intmap_r, const int* intmap_a, int nr, int na,
