@@ -50,9 +50,12 @@ struct TriCfg {
   // 256 beside the table of the exponential) its LDS footprint would admit three workgroups per CU instead of four.
   static constexpr int QB = sizeof(real) == 8 ? (MODE == 3 ? 192 : MODE == 2 ? 448 : 512) : 512;
   // waves per SIMD the register allocation is held to: without a bound the allocation comes out a few registers
-  // above the next occupancy step (the fused double-precision fingerprint kernel is held to four)
+  // above the next occupancy step (the fused double-precision fingerprint kernel is held to four).  The
+  // single-precision pass for both gradients is held to six (80 registers, 56 bytes of spill per lane outside the
+  // item loop) where it would take 95 and run four: 146 against 168 us per 8-frame step; seven (with a staging block
+  // of 256 so that seven workgroups fit a CU's LDS) is slower again (156 us).
   static constexpr int MIN_WAVES = sizeof(real) == 8 ? (MODE == 0 ? 5 : 4)
-                                                     : (MODE == 0 ? 8 : MODE == 1 ? 7 : MODE == 3 ? 4 : 5);
+                                                     : (MODE == 0 ? 8 : MODE == 1 ? 7 : MODE == 3 ? 6 : 5);
   static constexpr bool FORCE_BRANCH = MODE == 2 || MODE == 3;    // dL/dF comes in: der3b, der3bsupp are read
   static constexpr bool ENERGY_BRANCH = MODE == 1 || MODE == 3;   // dL/dAF3 comes in
 };
