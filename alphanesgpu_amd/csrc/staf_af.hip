@@ -315,7 +315,7 @@ int angular_afs(const real* Dsup, const real* Tang, const real* unit, int nr, in
     return STAF_E_BAD_ARG;
   if (nt > NT_MAX) return STAF_E_LIMIT;
   if (ld <= 0) ld = Nl;
-  size_t lds = TriLds<real, 0>::bytes(nr, Aa, nt, unit != nullptr);
+  size_t lds = unit ? TriLds<real, 0, true>::bytes(nr, Aa, nt, true) : TriLds<real, 0>::bytes(nr, Aa, nt, false);
   if (!(unit ? lds_request(tri_reduce_kernel<real, 0, true>, lds) : lds_request(tri_reduce_kernel<real, 0>, lds)))
     return STAF_E_LIMIT;
   TriArgs<real> A = {};

@@ -44,17 +44,19 @@ constexpr int TRI_WAVES = TRI_BLOCK / WAVE;
 constexpr int TRI_CAP = 16;    // channels tabulated per pass = lanes of a subset
 constexpr int TRI_CAPP = TRI_CAP + 1;   // table row pitch: the entry after a row's channels holds (D, V) of its slot
 constexpr int TRI_SUBS = TRI_BLOCK / TRI_CAP;
-template <typename real, int MODE>
+template <typename real, int MODE, bool FUSED = false>
 struct TriCfg {
   // triplets staged per block.  The double-precision pass that gives both gradients stages fewer: with 512 (or with
   // 256 beside the table of the exponential) its LDS footprint would admit three workgroups per CU instead of four.
-  static constexpr int QB = sizeof(real) == 8 ? (MODE == 3 ? 192 : MODE == 2 ? 448 : 512) : 512;
+  // The fused double-precision fingerprint kernel (the MD entry: thousands of centres per launch, several per
+  // workgroup) stages 160: five workgroups per CU instead of four.
+  static constexpr int QB = sizeof(real) == 8 ? (MODE == 3 ? 192 : MODE == 2 ? 448 : FUSED ? 160 : 512) : 512;
   // waves per SIMD the register allocation is held to: without a bound the allocation comes out a few registers
-  // above the next occupancy step (the fused double-precision fingerprint kernel is held to four).  The
+  // above the next occupancy step.  The
   // single-precision pass for both gradients is held to six (80 registers, 56 bytes of spill per lane outside the
   // item loop) where it would take 95 and run four: 146 against 168 us per 8-frame step; seven (with a staging block
   // of 256 so that seven workgroups fit a CU's LDS) is slower again (156 us).
-  static constexpr int MIN_WAVES = sizeof(real) == 8 ? (MODE == 0 ? 5 : 4)
+  static constexpr int MIN_WAVES = sizeof(real) == 8 ? (MODE == 0 ? 5 : 4)   // also the fused fingerprint kernel's
                                                      : (MODE == 0 ? 8 : MODE == 1 ? 7 : MODE == 3 ? 6 : 5);
   static constexpr bool FORCE_BRANCH = MODE == 2 || MODE == 3;    // dL/dF comes in: der3b, der3bsupp are read
   static constexpr bool ENERGY_BRANCH = MODE == 1 || MODE == 3;   // dL/dAF3 comes in
@@ -284,11 +286,11 @@ struct TriStage {
   }
 };
 
-template <typename real, int MODE>
+template <typename real, int MODE, bool FUSED = false>
 struct TriLds {
   static constexpr int NV = (MODE == 0) ? 1 : (MODE == 1 ? 3 : (MODE == 2 ? 4 : 7));
   static constexpr int NG = MODE == 3 ? 2 : 1;   // parameter-gradient sets (force branch, energy branch)
-  static constexpr int QB = TriCfg<real, MODE>::QB;
+  static constexpr int QB = TriCfg<real, MODE, FUSED>::QB;
   __host__ __device__ static size_t n_reals(int nr, int Aa, int nt, bool fused = false) {
     const int nsig = 2 * nt - 1;
     size_t r = (size_t)nr * TRI_CAPP * 2;                   // pair tables (real2 per (row, channel)), + (D, V) per row
@@ -314,13 +316,13 @@ struct TriLds {
 // the slots' unit vectors and cutoff values, T = 1/2 (u_j . u_k + 1) fc_j fc_k
 // (DescriptorsAngular_kernel, STAF/src/descriptor_builder/reforce.cu.cc:195-212), so no na-wide tensor exists.
 template <typename real, int MODE, bool FUSED = false>
-__global__ __launch_bounds__(TRI_BLOCK, ((FUSED && sizeof(real) == 8) ? 4 : TriCfg<real, MODE>::MIN_WAVES)) void
+__global__ __launch_bounds__(TRI_BLOCK, (TriCfg<real, MODE, FUSED>::MIN_WAVES)) void
 tri_reduce_kernel(TriArgs<real> A) {
   static_assert(!FUSED || MODE == 0, "only the fingerprint mode rebuilds T");
   using real2 = typename Vec2<real>::type;
   using HE = HotExp<real>;
   constexpr int NV = TriLds<real, MODE>::NV, NG = TriLds<real, MODE>::NG;
-  constexpr int TRI_QB = TriCfg<real, MODE>::QB;
+  constexpr int TRI_QB = TriCfg<real, MODE, FUSED>::QB;
   constexpr bool FB = TriCfg<real, MODE>::FORCE_BRANCH;
   extern __shared__ __align__(16) unsigned char smem[];
   const int nr = A.nr, na = A.na, Aa = A.Aa, nt = A.nt;
