@@ -177,7 +177,9 @@ int staf_op_radial_afs_f64(const double* radial_descriptor, int nr, const double
  *   radial_descriptor = des3bsupp [nf,Nl,nr]; angular_descriptor [nf,Nl,na]; alpha3b [ntc,3*nsmooth_a]
  *   (alpha1,alpha2,beta per channel), type_emb3b [ntc,nsmooth_a]; row = t_j + t_k.
  *   interaction_map_rad [nf,Nl,nr+1] supplies the neighbour species; interaction_map_angular must be the
- *   one the descriptor op produced with it (it is not re-read). */
+ *   one the descriptor op produced with it (it is not re-read).
+ *   num_triplets [nf,Nl] = neighbours inside the angular cutoff; every 3-body op of this library takes an entry
+ *   below 0 as 0 and an entry above nr as nr, so no kernel leaves its rows whatever the tensor holds. */
 int staf_op_angular_afs_f32(const float* radial_descriptor, const float* angular_descriptor, int nr, int na,
                             float* three_body_AFs, int dimbat, int N_local, const int* interaction_map_angular,
                             const int* interaction_map_rad, const float* alpha3b, int nsmooth_a,

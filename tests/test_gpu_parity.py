@@ -1133,3 +1133,54 @@ def test_growth_under_capture_is_refused():
         torch.cuda.synchronize()
         for x, y in zip(held, want):
             assert torch.equal(x, y)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_triplet_counts_out_of_range_are_clamped(dtype):
+    """A caller's numtriplet tensor with entries below zero or above the radial buffer: the 3-body ops clamp them to
+    0 .. nr (a negative count means no triplet, a count above nr the whole row), so the outputs are those of the
+    clamped tensor, bit for bit, and no kernel reads outside its rows."""
+    import torch
+    from alphanesgpu_amd import ops
+    from util import species_slices
+    dtype = np.dtype(dtype)
+    b = _synth("water96")
+    params = _params(dtype)
+    pos, box = b["pos"].astype(dtype), b["box"].astype(dtype)
+    nf = box.shape[0]
+    up = pipeline.synthetic_upstream(nf, b["tipos"], params, 23, dtype)
+    dev = torch.device("cuda:0")
+    T = lambda a: torch.as_tensor(np.ascontiguousarray(a)).to(dev)
+    tdt = torch.float32 if dtype == np.float32 else torch.float64
+    ops.construct_descriptors_light(4.5, NR, NA, b["N"], None, 2.25, 4.5, nf, dtype=tdt)
+    ops.descriptor_options(False, True)   # every padded slot zero: a count above the row's own is well defined
+    names = ["raddescr", "angdescr", "des3bsupp", "intmap2b", "intmap3b", "der2b", "der3b", "der3bsupp", "numtriplet"]
+    g = dict(zip(names, ops.compute_descriptors_light(T(pos), T(box))))
+    tm, tp, Q = T(b["type_map"]), T(b["tipos"]), T(up["Q"])
+    bad = g["numtriplet"].clone()
+    bad[:, 0::3] = -7
+    bad[:, 1::3] = NR + 1000
+    good = bad.clamp(0, NR)
+    for k, s in enumerate(species_slices(b["tipos"])):
+        m = params[k]
+        v = lambda key: g[key][:, s]
+        al, em = T(m["alpha3b"]), T(m["emb3b"])
+        at = torch.tensor([k], dtype=torch.int32, device=dev)
+        G3, P3 = T(up["G3"][k]), T(up["P3"][k])
+
+        def run(ntr):
+            common = (v("des3bsupp"), v("angdescr"), v("der3bsupp"), v("der3b"), v("intmap2b"), v("intmap3b"), al,
+                      em, tm, tp, at, ntr[:, s])
+            out = [ops.compute_sort_proj3body(v("angdescr"), v("des3bsupp"), v("intmap3b"), v("intmap2b"), al, em, tm,
+                                              ntr[:, s], nt=len(b["tipos"])),
+                   ops.compute_force_tripl(G3, *common)]
+            out += list(ops.compute_tripl_grads_fused(Q, G3, P3, *common))
+            torch.cuda.synchronize()
+            return [o.clone() for o in out]
+
+        for x, y in zip(run(bad), run(good)):
+            assert torch.isfinite(x).all()
+            assert torch.equal(x, y), k
+    ops.descriptor_options(False, False)
+    ops.poll_status()
