@@ -95,6 +95,10 @@ __device__ inline float dpp_get(float v) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
 }
 template <int CTRL, int ROW_MASK>
+__device__ inline unsigned dpp_get(unsigned v) {
+  return (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROW_MASK, 0xf, false);
+}
+template <int CTRL, int ROW_MASK>
 __device__ inline double dpp_get(double v) {
   const long long b = __double_as_longlong(v);
   const int lo = __builtin_amdgcn_update_dpp(0, (int)(b & 0xffffffffll), CTRL, ROW_MASK, 0xf, false);
@@ -127,6 +131,14 @@ __device__ inline void dpp_rows_carry(float& a, float& b, float& c, float& d) {
       "v_add_f32_dpp %3, %3, %3 row_bcast:31 row_mask:0xc\n\t"
       "s_nop 1"
       : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+}
+__device__ inline void dpp_rows_carry(unsigned& a) {
+  asm("s_nop 1\n\t"
+      "v_add_u32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa\n\t"
+      "s_nop 1\n\t"
+      "v_add_u32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc\n\t"
+      "s_nop 1"
+      : "+v"(a));
 }
 __device__ inline void dpp_rows_carry(double& s) {
   s += dpp_get<0x142, 0xa>(s);   // lane 15 of a row -> every lane of the next row (rows 1 and 3 take it)
@@ -258,6 +270,9 @@ struct StreamWork {
 struct TransposeRef {
   int symmetric = 0;
   const int* full = nullptr; // symmetric: the intmap2b tensor the view points into
+  const unsigned* rowsum = nullptr;   // symmetric: [nf * N] checksum of every row as the descriptor op wrote it (row_hash
+                                      // in staf_transpose.hpp), or null where no block could be had: an atom that
+                                      // collects through its own row compares, and reports a stale map on a difference
   int* build_cnt = nullptr;  // [nf * Nrecv] fill cursors of a build, all zero between builds
   int* cnt = nullptr;        // [nf * Nrecv] keys per receiving atom
   int* keys = nullptr;       // [nf * Nrecv, cap]

@@ -294,12 +294,13 @@ __global__ __launch_bounds__(256, sizeof(real) == 4 ? 8 : 5) void desc_kernel(De
   int* s_j = c_j + nr;                 // [nr] sorted neighbour index
   int* s_rank = s_j + nr;              // [nr] rank of every candidate
   __shared__ int cnt_all, cnt_ang;
+  __shared__ unsigned row_sum;   // checksum of the row being written (row_hash over its slots)
   __shared__ real sinv[6];
 
   const int tid = threadIdx.x;
   const int b = blockIdx.x / N;
   const int i = blockIdx.x - b * N;
-  if (tid == 0) { cnt_all = 0; cnt_ang = 0; }
+  if (tid == 0) { cnt_all = 0; cnt_ang = 0; row_sum = 0; }
   for (int e = tid; e < nr; e += blockDim.x) s_rank[e] = 0;
   // Box and centre position are the same for the whole workgroup: every thread reads them itself (reads of
   // workgroup-uniform addresses).  The inverse box costs six divisions -- in double precision more instructions
@@ -473,6 +474,7 @@ __global__ __launch_bounds__(256, sizeof(real) == 4 ? 8 : 5) void desc_kernel(De
   // 3. radial fill
   const bool same_cut = A.Ra == A.Rc;
   const bool std_pow = A.pa == real(1) && A.pb == real(-30);   // the exponents fill_repulsion uses
+  unsigned hloc = 0;   // this thread's share of the row's checksum
   for (int e = tid; e < nr; e += blockDim.x) {
     if (e < n) {
       const int j = c_j[e];
@@ -510,6 +512,7 @@ __global__ __launch_bounds__(256, sizeof(real) == 4 ? 8 : 5) void desc_kernel(De
       A.raddescr[row + rank] = D;
       A.des3bsupp[row + rank] = fc;
       im[1 + rank] = j;
+      hloc += row_hash(j, rank);
       s_j[rank] = j;
       if (A.unit) A.unit[(atom * 4 + 3) * nr + rank] = invr;
       alignas(16) real rec[8];
@@ -541,11 +544,16 @@ __global__ __launch_bounds__(256, sizeof(real) == 4 ? 8 : 5) void desc_kernel(De
       }
     }
   }
+  if (A.tr.rowsum && tid < ((nr + WAVE - 1) & ~(WAVE - 1))) {   // the waves that hold slots: a lane sum each, one LDS add per wave
+    const unsigned hw = wave_sum_to_last(hloc);
+    if ((tid & (WAVE - 1)) == WAVE - 1) atomicAdd(&row_sum, hw);
+  }
   __syncthreads();
   const int m = cnt_ang;
   if (tid == 0) {
     im[0] = hm;
     A.numtriplet[atom] = m;
+    if (A.tr.rowsum) const_cast<unsigned*>(A.tr.rowsum)[atom] = row_sum + (unsigned)n;
   }
 
   if (!A.angular) return;

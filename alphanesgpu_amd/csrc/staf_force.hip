@@ -139,9 +139,11 @@ __global__ __launch_bounds__(F_BLOCK) void force2_kernel(Force2Args<real> A) {
     const int* mine = A.tr.full + ((size_t)b * A.N + a) * (nr + 1);
     int cnt = mine[0];
     if (cnt > nr) cnt = nr;
+    unsigned hsum = 0;
     for (int t = lane; t < nr; t += WAVE) {
       const int i = mine[1 + t];
       if (t >= cnt) break;
+      hsum += row_hash(i, t);
       const int p = i - A.tr.key_shift;
       if (p < 0 || p >= Nl) continue;
       const int s = slot_of(A.tr.full, b, A.N, nr, i, a);
@@ -151,6 +153,7 @@ __global__ __launch_bounds__(F_BLOCK) void force2_kernel(Force2Args<real> A) {
 #pragma unroll
       for (int c = 0; c < 3; c++) f[c] += w * A.dD[row * 3 * nr + c * nr + s];
     }
+    row_check(A.tr, (size_t)b * A.N + a, cnt, hsum, lane, A.status);
   } else {
     const int L = A.tr.cnt[recv];
     const int* keys = A.tr.keys + (size_t)recv * A.tr.cap;
@@ -273,9 +276,11 @@ __global__ __launch_bounds__(F_BLOCK) void gather_kernel(const real* __restrict_
     const int* mine = tr.full + ((size_t)b * N + a) * (nr + 1);
     int cnt = mine[0];
     if (cnt > nr) cnt = nr;
+    unsigned hsum = 0;
     for (int t = lane; t < nr; t += WAVE) {
       const int i = mine[1 + t];
       if (t >= cnt) break;
+      hsum += row_hash(i, t);
       const int p = i - tr.key_shift;
       if (p < 0 || p >= Nl) continue;
       const int s = slot_of(tr.full, b, N, nr, i, a);
@@ -285,6 +290,7 @@ __global__ __launch_bounds__(F_BLOCK) void gather_kernel(const real* __restrict_
       f[1] += g[1];
       f[2] += g[2];
     }
+    row_check(tr, (size_t)b * N + a, cnt, hsum, lane, status);
   } else {
     const int L = tr.cnt[recv];
     const int* keys = tr.keys + (size_t)recv * tr.cap;
@@ -326,6 +332,7 @@ struct TotalArgs {
   const int* full;             // intmap2b [nf, N, nr+1]
   real* total;                 // [nf, 3N]
   int* status;
+  const unsigned* rowsum;   // checksums of the map's rows as written (TransposeRef::rowsum), or null
   int nf, N, nr, nt;
 };
 
@@ -342,9 +349,11 @@ __global__ __launch_bounds__(F_BLOCK) void force_total_kernel(TotalArgs<real> A)
   const int* mine = A.full + ((size_t)b * N + a) * (nr + 1);
   int cnt = mine[0];
   if (cnt > nr) cnt = nr;
+  unsigned hsum = 0;
   for (int t = lane; t < nr; t += WAVE) {
     const int i = mine[1 + t];
     if (t >= cnt) break;
+    hsum += row_hash(i, t);
     int k = 0;
 #pragma unroll
     for (int q = 1; q < NT; q++) k += (q < nt && i >= A.first[q]) ? 1 : 0;
@@ -363,6 +372,10 @@ __global__ __launch_bounds__(F_BLOCK) void force_total_kernel(TotalArgs<real> A)
     for (int q = 0; q < NT; q++) {
       if (q == k) { acc[q][0] += g0; acc[q][1] += g1; acc[q][2] += g2; }
     }
+  }
+  {
+    const unsigned h = wave_sum_to_last(hsum) + (unsigned)cnt;
+    if (lane == WAVE - 1 && A.rowsum && h != A.rowsum[(size_t)b * N + a]) atomicOr(A.status, 4);
   }
   real tot = 0;
   bool have = false;
@@ -822,7 +835,7 @@ int force_total(const int* im2_full, int nr, int N, int nf, int nt, const int* n
   // wrote, and remembers, is known to be symmetric
   TransposeRef tr;
   if (!transpose_find(st, im2_full, nf, N, N, N, nr, &tr) || !tr.symmetric || tr.key_shift != 0) return STAF_E_BAD_ARG;
-  A.full = im2_full; A.total = total; A.status = status_word(st, stream);
+  A.full = im2_full; A.total = total; A.status = status_word(st, stream); A.rowsum = tr.rowsum;
   A.nf = nf; A.N = N; A.nr = nr; A.nt = nt;
   {
     KernelTimer kt_("force_total_kernel", stream);

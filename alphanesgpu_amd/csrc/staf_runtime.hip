@@ -142,7 +142,8 @@ bool bucket_reserve(DeviceState* st, size_t n_recv, int cap, hipStream_t stream,
 bool transpose_for_descriptor(DeviceState* st, const int* im2, int nf, int N, int Nrecv, int nr, int cap,
                               bool symmetric, hipStream_t stream, TransposeRef* out) {
   std::lock_guard<std::mutex> lock(g_mu);
-  const size_t want_recv = symmetric ? 0 : (size_t)nf * Nrecv, want_keys = want_recv * cap;
+  // a symmetric map needs no transpose, only one word per row for the rows' checksums (the counter part of a block)
+  const size_t want_recv = (size_t)nf * Nrecv, want_keys = symmetric ? 0 : want_recv * cap;
   Transpose* t = nullptr;
   for (auto& e : st->transposes)
     if (e.im2 == im2) { t = &e; break; }
@@ -152,17 +153,23 @@ bool transpose_for_descriptor(DeviceState* st, const int* im2, int nf, int N, in
     // such a place rebuilds the transpose in it on every replay, before it reads it).
     const bool capturing = stream_is_capturing(stream);
     for (auto& e : st->transposes) {
-      if (capturing && (e.cap_recv < want_recv || e.cap_keys < want_keys)) continue;
+      if (capturing && !symmetric && (e.cap_recv < want_recv || e.cap_keys < want_keys)) continue;
       if (!t || e.stamp < t->stamp) t = &e;
     }
     if (!t) return false;
   }
-  if (!symmetric && !transpose_block(st, &t->buf, &t->cap_recv, &t->cap_keys, want_recv, want_keys, stream))
+  // (a symmetric map whose place has no block for the checksums and cannot get one now -- a tensor first seen while
+  // its stream is captured -- goes without them)
+  bool have_block = true;
+  if (symmetric && stream_is_capturing(stream) && (t->cap_recv < want_recv))
+    have_block = false;
+  else if (!transpose_block(st, &t->buf, &t->cap_recv, &t->cap_keys, want_recv, want_keys, stream))
     return false;
   t->im2 = im2; t->nf = nf; t->N = N; t->Nrecv = Nrecv; t->nr = nr;
   t->ref = TransposeRef();
   t->ref.symmetric = symmetric ? 1 : 0;
   t->ref.full = im2;
+  if (symmetric && have_block) t->ref.rowsum = (const unsigned*)t->buf.buf;
   if (!symmetric) {
     t->ref.build_cnt = (int*)t->buf.buf;
     t->ref.cnt = t->ref.build_cnt + t->cap_recv;

@@ -35,6 +35,20 @@ __device__ inline void transpose_push(int* build_cnt, int* keys, int cap, size_t
   else atomicOr(status, 2);
 }
 
+// Checksum of a row of a map, order-free: the sum over its slots of row_hash(neighbour, slot), plus the count.  The
+// descriptor op stores it for every row of a map it writes; a kernel that takes an atom's own row as the list of
+// centres that list the atom recomputes it, so that other content at a remembered address (a caller's list copied
+// there, a tensor of another call at a recycled address) is reported instead of read as symmetric.
+__device__ inline unsigned row_hash(int neighbour, int slot) {
+  return ((unsigned)neighbour + 1u) * (2u * (unsigned)slot + 1u) * 0x9E3779B1u;
+}
+// `partial`: the lane's share of the sum over the row's slots below `cnt`; the last lane holds the sum and reports.
+__device__ inline void row_check(const TransposeRef& tr, size_t row, int cnt, unsigned partial, int lane, int* status) {
+  if (!tr.rowsum) return;
+  const unsigned h = wave_sum_to_last(partial) + (unsigned)cnt;
+  if (lane == WAVE - 1 && h != tr.rowsum[row]) atomicOr(status, 4);
+}
+
 // Slot of atom `a` in the row of centre `i` of frame b of the symmetric map `full` [nf, N, nr+1], or -1 (the map is
 // not symmetric after all: reported by the caller).  The whole row is requested at once, sixteen entries per round
 // in four 16-byte reads (rows are only 4-byte aligned), and compared without an early exit: one round trip to

@@ -1184,3 +1184,58 @@ def test_triplet_counts_out_of_range_are_clamped(dtype):
             assert torch.equal(x, y), k
     ops.descriptor_options(False, False)
     ops.poll_status()
+
+
+@pytest.mark.gpu
+def test_changed_row_of_a_remembered_map_is_reported_by_its_checksum():
+    """A remembered (symmetric) map whose content changes in a way the reciprocity check cannot see: two slots of a
+    row of an atom OUTSIDE the op's species swapped (every listed pair is still listed both ways, only the slot
+    order no longer matches the descriptor rows).  The atom that collects through that row recomputes the row's
+    checksum, which differs from the one the descriptor op stored: stale map, for the per-op force kernels and for
+    the collecting launch of the step-level path."""
+    import torch
+    from alphanesgpu_amd import ops, _lib
+    b = _synth("water96")
+    dev = torch.device("cuda:0")
+    dtype = np.dtype(np.float64)
+    params = _params(dtype)
+    N = b["N"]
+    T = lambda a: torch.as_tensor(np.ascontiguousarray(a)).to(dev)
+    tm, tp = T(b["type_map"]), T(b["tipos"])
+    at = torch.tensor([0], dtype=torch.int32, device=dev)
+    n0 = int(b["tipos"][0])
+    p0 = params[0]
+    G2 = torch.ones(1, n0, p0["alpha2b"].shape[1], dtype=torch.float64, device=dev)
+    G3 = torch.ones(1, n0, p0["alpha3b"].shape[1] // 3, dtype=torch.float64, device=dev)
+
+    def fresh():
+        ops.construct_descriptors_light(4.5, NR, NA, N, None, 2.25, 4.5, 1, dtype=torch.float64)
+        out = ops.compute_descriptors_light(T(b["pos"]), T(b["box"]))
+        im2 = out[3]
+        victim = N - 1                      # an atom of the other species
+        assert int(im2[0, victim, 0]) >= 2
+        a, c = int(im2[0, victim, 1]), int(im2[0, victim, 2])
+        im2[0, victim, 1], im2[0, victim, 2] = c, a
+        return out
+
+    rad, ang, sup, im2, im3, d2, d3, d3s, ntr = fresh()
+    with pytest.raises(_lib.StafError) as e:
+        ops.compute_force_radial(G2, d2[:, :n0], im2[:, :n0], rad[:, :n0], T(p0["alpha2b"]), T(p0["emb2b"]), tm, tp, at)
+    assert e.value.code == -14
+    rad, ang, sup, im2, im3, d2, d3, d3s, ntr = fresh()
+    with pytest.raises(_lib.StafError) as e:
+        ops.compute_force_tripl(G3, sup[:, :n0], ang[:, :n0], d3s[:, :n0], d3[:, :n0], im2[:, :n0], im3[:, :n0],
+                                T(p0["alpha3b"]), T(p0["emb3b"]), tm, tp, at, ntr[:, :n0])
+    assert e.value.code == -14
+    rad, ang, sup, im2, im3, d2, d3, d3s, ntr = fresh()
+    slots, selfs = ops.compute_force_tripl_slots(G3, sup[:, :n0], ang[:, :n0], d3s[:, :n0], d3[:, :n0], im2[:, :n0],
+                                                 im3[:, :n0], T(p0["alpha3b"]), T(p0["emb3b"]), tm, tp, at,
+                                                 ntr[:, :n0])
+    with pytest.raises(_lib.StafError) as e:
+        ops.force_total(im2, [int(x) for x in b["tipos"]], [slots, None], [selfs, None])
+    assert e.value.code == -14
+    # an untouched map of a new descriptor call is remembered afresh and collects without complaint
+    ops.construct_descriptors_light(4.5, NR, NA, N, None, 2.25, 4.5, 1, dtype=torch.float64)
+    rad, ang, sup, im2, im3, d2, d3, d3s, ntr = ops.compute_descriptors_light(T(b["pos"]), T(b["box"]))
+    ops.compute_force_radial(G2, d2[:, :n0], im2[:, :n0], rad[:, :n0], T(p0["alpha2b"]), T(p0["emb2b"]), tm, tp, at)
+    ops.poll_status()
