@@ -1,8 +1,10 @@
 // 3-body force, pass A: one workgroup of four or eight waves per centre atom, four barriers per centre.
 // Replaces computeforce_tripl_kernel (STAF/src/force/ang/reforce.cu.cc:96-214).
 //
-// The kernel is bound by vector-ALU issue and by latency, so the layout keeps the per-(triplet, channel) work
-// minimal, keeps everything else out of the inner loop and avoids workgroup barriers:
+// The kernel is bound by vector-ALU issue and LDS bandwidth in its channel loop (an item reads its parameter entry
+// and two table entries: 32 bytes per lane in single, 64 in double precision, which keeps a CU's LDS as busy as the
+// item's 13 / 30 instructions keep its vector units) and by latency around it, so the layout keeps the
+// per-(triplet, channel) work minimal, keeps everything else out of the inner loop and avoids workgroup barriers:
 //   * lane <-> triplet in storage order (nn = 64*pass + lane, passes dealt round-robin to the waves):
 //     angdescr and der3b are read coalesced, once; the triplets of a wave's NP passes (T, the three channel
 //     sums, packed indices) stay in registers from the first read to the slot sums.
@@ -23,8 +25,9 @@
 //     accumulators row by row (inside a row the k are distinct).  One accumulator per wave and slot takes both;
 //     the waves' accumulators are added in a fixed order: results are bit-reproducible.
 //     F_s = sum_p Sd(s,p) dT/dd_s(s,p) + (sum_p SB_s(s,p)) grad fc_s
-// The slot forces go to scratch (gslot, and the centre's own force to self); the atoms that receive them collect
-// them in gather_kernel through the transposed neighbour map.
+// The slot forces go to scratch or to the caller's arrays (gslot, and the centre's own force to self); the atoms
+// that receive them collect them in gather_kernel (per op) or force_total_kernel (all species at once) through the
+// neighbour map.
 #pragma once
 #include <type_traits>
 

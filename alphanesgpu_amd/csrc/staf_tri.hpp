@@ -3,10 +3,11 @@
 // force op (MODE 2), and both gradients in one pass (MODE 3: a training step
 // needs both, and everything but the last few accumulations per item -- set-up,
 // tables, staging, the exponential, the pair factors -- is shared).  One
-// 256-thread workgroup per centre atom (persistent over atoms for the gradient
-// modes).  These kernels are bound by vector-ALU
-// issue, so the layout below is chosen to keep the instruction count per
-// (triplet, channel) item low.
+// 256-thread workgroup per centre atom at a time; a launch has as many
+// workgroups as the device holds at once (or a whole number of such rounds,
+// tri_grid) and a workgroup walks over its centres.  These kernels are bound
+// by vector-ALU issue, so the layout below is chosen to keep the instruction
+// count per (triplet, channel) item low.
 //
 // Work decomposition inside a species class (ta,tb) of the centre's triplets
 // (see staf_tile.hpp for the class enumeration):
