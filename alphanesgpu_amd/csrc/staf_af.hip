@@ -11,6 +11,7 @@
 #include "staf_tile.hpp"
 #include "staf_reduce.hpp"
 #include "staf_tri.hpp"
+#include "staf_af2.hpp"
 
 #include <stdio.h>
 #include <mutex>
@@ -31,44 +32,25 @@ __global__ __launch_bounds__(AF_BLOCK) void af2_kernel(const real* __restrict__ 
                                                        const real* __restrict__ emb2b,
                                                        const int* __restrict__ type_map, real* __restrict__ out,
                                                        int nf, int Nl, int ld, int nr, int Ar, int nt) {
-  using HE = HotExp<real>;
   extern __shared__ __align__(16) unsigned char smem[];
   real* p_al = (real*)smem;          // [nt*Ar] alpha in the units of the hot exponential
   real* p_c2 = p_al + nt * Ar;       // [nt*Ar]
   real* w_D = p_c2 + nt * Ar;        // [AF_WAVES][nr]
   int* w_t = (int*)(w_D + AF_WAVES * nr);  // [AF_WAVES][nr]
-  for (int q = threadIdx.x; q < nt * Ar; q += blockDim.x) { p_al[q] = HE::scale(alpha2b[q]); p_c2[q] = emb2b[q]; }
+  af2_tables(alpha2b, emb2b, nt * Ar, p_al, p_c2);
   const int wave = threadIdx.x / WAVE, lane = lane_id();
   real* myD = w_D + wave * nr;
   int* myT = w_t + wave * nr;
   const int atom = blockIdx.x * AF_WAVES + wave;
   int cnt = 0;
-  size_t rowAtom = 0;
   if (atom < nf * Nl) {
     const int b = atom / Nl, p = atom - b * Nl;
-    rowAtom = (size_t)b * ld + p;
-    const int* im = im2 + rowAtom * (nr + 1);
-    cnt = im[0];
-    if (cnt > nr) cnt = nr;
-    for (int s = lane; s < cnt; s += WAVE) { myD[s] = D[rowAtom * nr + s]; myT[s] = type_map[im[1 + s]] * Ar; }
+    const size_t rowAtom = (size_t)b * ld + p;
+    cnt = af2_wave_load(D + rowAtom * nr, im2 + rowAtom * (nr + 1), type_map, nr, Ar, myD, myT, lane);
   }
   __syncthreads();
   if (atom >= nf * Nl) return;
-  const ChanSub cs(lane, Ar);
-  for (int a0 = 0; a0 < Ar; a0 += cs.chunk) {
-    const int a = a0 + cs.a;
-    const bool on = cs.sub < cs.nsub && a < Ar;
-    real acc = 0;
-    if (on) {
-      for (int s = cs.sub; s < cnt; s += cs.nsub) {
-        const real d = myD[s];
-        const int ta = myT[s] + a;
-        acc += d * (HE::eval(p_al[ta] * d) * p_c2[ta]);
-      }
-    }
-    acc = cs.combine(acc, lane);
-    if (on && cs.sub == 0) out[(size_t)atom * Ar + a] = acc;
-  }
+  af2_wave_sum(p_al, p_c2, myD, myT, cnt, Ar, out + (size_t)atom * Ar, lane);
 }
 
 // ---------------------------------------------------------------------------

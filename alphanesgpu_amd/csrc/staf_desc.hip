@@ -24,6 +24,8 @@
 #include "staf_common.hpp"
 #include "staf_reduce.hpp"
 #include "staf_transpose.hpp"
+#include "staf_tri.hpp"
+#include "staf_af2.hpp"
 
 #include <math.h>
 #include <stdio.h>
@@ -275,8 +277,11 @@ __device__ inline void zero_fill(char* p, unsigned nbytes, int tid) {
 // Waves per SIMD the allocation is held to: without a bound the single-precision kernel takes 112 scalar registers
 // (seven waves: 1792 resident workgroups for the 3072 centres of four 768-atom frames) and the double-precision
 // one 104 vector registers (four waves); at eight and five the launch needs fewer rounds of workgroups.
+constexpr int DESC_MIN_WAVES_F32 = 8, DESC_MIN_WAVES_F64 = 5;
+// The kernel's body for the 256-thread workgroup of centre `centre` (frame-major over all N atoms): desc_kernel
+// below, and the launch that goes on to the centre's fingerprints in the same workgroup.
 template <typename real>
-__global__ __launch_bounds__(256, sizeof(real) == 4 ? 8 : 5) void desc_kernel(DescArgs<real> A) {
+__device__ __forceinline__ void desc_body(const DescArgs<real> A, const int centre) {
   using real2 = typename Vec2<real>::type;
   extern __shared__ __align__(16) unsigned char smem[];
   const int nr = A.nr, na = A.na, N = A.N;
@@ -298,8 +303,8 @@ __global__ __launch_bounds__(256, sizeof(real) == 4 ? 8 : 5) void desc_kernel(De
   __shared__ real sinv[6];
 
   const int tid = threadIdx.x;
-  const int b = blockIdx.x / N;
-  const int i = blockIdx.x - b * N;
+  const int b = centre / N;
+  const int i = centre - b * N;
   if (tid == 0) { cnt_all = 0; cnt_ang = 0; row_sum = 0; }
   for (int e = tid; e < nr; e += blockDim.x) s_rank[e] = 0;
   // Box and centre position are the same for the whole workgroup: every thread reads them itself (reads of
@@ -617,8 +622,84 @@ __global__ __launch_bounds__(256, sizeof(real) == 4 ? 8 : 5) void desc_kernel(De
 }
 
 template <typename real>
+__global__ __launch_bounds__(256, sizeof(real) == 4 ? DESC_MIN_WAVES_F32 : DESC_MIN_WAVES_F64) void
+desc_kernel(DescArgs<real> A) {
+  desc_body<real>(A, (int)blockIdx.x);
+}
+
+template <typename real>
 size_t desc_lds_bytes(int nr) {
   return (size_t)nr * (12 * sizeof(real) + 3 * sizeof(int));
+}
+
+// ---------------------------------------------------------------------------
+// Descriptors and fingerprints of a centre in one workgroup.  A centre's fingerprints need nothing but the rows its
+// own descriptor workgroup writes, so the three launches of a step's first stage (descriptors, 2-body and 3-body
+// fingerprints of every species) can be one: a workgroup runs the descriptor body, then -- behind a barrier, reading
+// back through the cache of its own CU what it has just written -- the 3-body fingerprint body of tri_reduce_kernel
+// and, in its first wave, the 2-body fingerprints as af2_kernel computes them (same code, same bits).  No launch
+// of the stage then waits for another one's last workgroup, and the species' centres share one grid: entry e of
+// the launch is a species, the species with the most centres first.
+// ---------------------------------------------------------------------------
+template <typename real>
+struct Af2Args {
+  const real* alpha2b;   // [nt, Ar] of the centre species
+  const real* emb2b;     // [nt, Ar]
+  real* out;             // [nf, Nl, Ar]
+};
+template <typename real>
+struct FingerprintArgs {
+  TriArgs<real> tri[NT_MAX];   // 3-body fingerprint arguments of the entry's species (views of the descriptor outputs)
+  Af2Args<real> rad[NT_MAX];
+  int first[NT_MAX + 1];       // first workgroup of the entry
+  int shift[NT_MAX];           // first atom of the entry's species within a frame
+  int entries;
+  int Ar;                      // 0: no 2-body fingerprints
+  const real* raddescr;        // what the descriptor body writes, for the 2-body part
+  const int* intmap2b;
+};
+
+template <typename real>
+__global__ __launch_bounds__(256, sizeof(real) == 4 ? DESC_MIN_WAVES_F32 : DESC_MIN_WAVES_F64) void
+desc_fingerprints_kernel(DescArgs<real> D, FingerprintArgs<real> M) {
+  static_assert(TRI_BLOCK == 256 && TriCfg<float, 0>::MIN_WAVES == DESC_MIN_WAVES_F32 &&
+                    TriCfg<double, 0>::MIN_WAVES == DESC_MIN_WAVES_F64,
+                "both bodies are written for this workgroup size and register budget");
+  int e = 0;
+  while (e + 1 < M.entries && (int)blockIdx.x >= M.first[e + 1]) e++;
+  const TriArgs<real>& T = M.tri[e];
+  const int c = (int)blockIdx.x - M.first[e];   // centre within the species, frame-major
+  const int b = c / T.Nl, p = c - b * T.Nl;
+  const int centre = b * D.N + M.shift[e] + p;
+  desc_body<real>(D, centre);
+  __syncthreads();   // the rows written above are read below by other threads of this workgroup
+  tri_reduce_body<real, 0, false>(T, c, 0x3fffffff, 0);
+  if (M.Ar) {
+    // (the 3-body body ends behind a barrier: its LDS is free)
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int Ar = M.Ar, nr = D.nr, npar = T.nt * Ar;
+    real* p_al = (real*)smem;
+    real* p_c2 = p_al + npar;
+    real* myD = p_c2 + npar;
+    int* myT = (int*)(myD + nr);
+    const Af2Args<real>& R = M.rad[e];
+    af2_tables(R.alpha2b, R.emb2b, npar, p_al, p_c2);
+    int cnt = 0;
+    if (threadIdx.x < WAVE)
+      cnt = af2_wave_load(M.raddescr + (size_t)centre * nr, M.intmap2b + (size_t)centre * (nr + 1), T.type_map, nr, Ar,
+                          myD, myT, (int)threadIdx.x);
+    __syncthreads();
+    if (threadIdx.x < WAVE) af2_wave_sum(p_al, p_c2, myD, myT, cnt, Ar, R.out + (size_t)c * Ar, (int)threadIdx.x);
+  }
+}
+
+template <typename real>
+size_t desc_fingerprints_lds_bytes(int nr, int Aa, int Ar, int nt) {
+  size_t b = desc_lds_bytes<real>(nr);
+  const size_t t = TriLds<real, 0>::bytes(nr, Aa, nt, false);
+  const size_t r = (size_t)2 * nt * Ar * sizeof(real) + (size_t)nr * (sizeof(real) + sizeof(int));
+  b = b > t ? b : t;
+  return b > r ? b : r;
 }
 
 // ---- host side -------------------------------------------------------------
@@ -709,11 +790,30 @@ static int construct(real Rc, int nr, int na, int numpar, real Rs, real Ra, int 
   return STAF_OK;
 }
 
+// What a descriptor launch goes on to compute for every centre (desc_fingerprints_kernel): host arrays of nt
+// device pointers, one per centre species.
 template <typename real>
-int desc_launch(const DescConfig<real>& c, const real* pos, const real* box, int nf, int N, int Npos,
-                const int* inj_howmany, const int* inj_with, int skip_pbc, real* raddescr, real* angdescr,
-                real* des3bsupp, int* intmap2b, int* intmap3b, real* der2b, real* der3b, real* der3bsupp,
-                int* numtriplet, real* unit, hipStream_t stream) {
+struct FingerprintStep {
+  int nt;
+  int first_species, n_species;  // the centres of these species only
+  const int* n_local;            // host [nt] atoms per species (species-sorted atoms, summing to N)
+  const int* type_map;           // device [N]
+  int Aa;
+  const real* const* alpha3b;    // [ntc, 3*Aa] each
+  const real* const* emb3b;      // [ntc, Aa] each
+  real* const* af3;              // [nf, n_local[k], Aa] each
+  int Ar;                        // 0: no 2-body fingerprints
+  const real* const* alpha2b;    // [nt, Ar] each
+  const real* const* emb2b;
+  real* const* af2;              // [nf, n_local[k], Ar] each
+};
+
+template <typename real>
+static int desc_launch_impl(const DescConfig<real>& c, const real* pos, const real* box, int nf, int N, int Npos,
+                            const int* inj_howmany, const int* inj_with, int skip_pbc, real* raddescr,
+                            real* angdescr, real* des3bsupp, int* intmap2b, int* intmap3b, real* der2b, real* der3b,
+                            real* der3bsupp, int* numtriplet, real* unit, hipStream_t stream,
+                            const FingerprintStep<real>* fp) {
   if (!c.ready) return STAF_E_NOT_CONSTRUCTED;
   const bool angular = unit == nullptr;   // with `unit` the call is radial-only
   if (!pos || !box || !raddescr || !des3bsupp || !intmap2b || !der2b || !der3bsupp || !numtriplet || nf <= 0 ||
@@ -759,7 +859,37 @@ int desc_launch(const DescConfig<real>& c, const real* pos, const real* box, int
   }
   size_t lds = desc_lds_bytes<real>(c.nr);
   if (lds > 60 * 1024) return STAF_E_LIMIT;
-  {
+  if (fp) {
+    FingerprintArgs<real> M = {};
+    const int nt = fp->nt;
+    int order[NT_MAX], shift[NT_MAX], sum = 0;
+    for (int k = 0; k < nt; k++) { order[k] = k; shift[k] = sum; sum += fp->n_local[k]; }
+    // the species with the most centres first (stable): its workgroups are the first to be dispatched
+    for (int a = 1; a < nt; a++)
+      for (int q = a; q > 0 && fp->n_local[order[q]] > fp->n_local[order[q - 1]]; q--) std::swap(order[q], order[q - 1]);
+    int e = 0, wg = 0;
+    for (int o = 0; o < nt; o++) {
+      const int k = order[o], Nl = fp->n_local[k];
+      if (Nl == 0 || k < fp->first_species || k >= fp->first_species + fp->n_species) continue;
+      TriArgs<real>& T = M.tri[e];
+      T.Dsup = des3bsupp + (size_t)shift[k] * c.nr;
+      T.Tang = angdescr + (size_t)shift[k] * c.na;
+      T.im2 = intmap2b + (size_t)shift[k] * (c.nr + 1);
+      T.numtriplet = numtriplet + shift[k];
+      T.alpha3b = fp->alpha3b[k]; T.emb3b = fp->emb3b[k]; T.type_map = fp->type_map; T.out = fp->af3[k];
+      T.nf = nf; T.N = N; T.Nl = Nl; T.ld = N; T.nr = c.nr; T.na = c.na; T.Aa = fp->Aa; T.nt = nt;
+      if (fp->Ar) { M.rad[e].alpha2b = fp->alpha2b[k]; M.rad[e].emb2b = fp->emb2b[k]; M.rad[e].out = fp->af2[k]; }
+      M.first[e] = wg; M.shift[e] = shift[k];
+      wg += nf * Nl;
+      e++;
+    }
+    M.first[e] = wg; M.entries = e; M.Ar = fp->Ar; M.raddescr = raddescr; M.intmap2b = intmap2b;
+    if (wg == 0) return finish_op(st, stream);   // no centre of these species in the frames
+    lds = desc_fingerprints_lds_bytes<real>(c.nr, fp->Aa, fp->Ar, nt);
+    if (!lds_request(desc_fingerprints_kernel<real>, lds)) return STAF_E_LIMIT;
+    KernelTimer kt_("desc_fp_kernel", stream);
+    hipLaunchKernelGGL(desc_fingerprints_kernel<real>, dim3((unsigned)wg), dim3(256), lds, stream, A, M);
+  } else {
     KernelTimer kt_("desc_kernel", stream);
     hipLaunchKernelGGL(desc_kernel<real>, dim3((unsigned)(nf * N)), dim3(256), lds, stream, A);
   }
@@ -768,6 +898,16 @@ int desc_launch(const DescConfig<real>& c, const real* pos, const real* box, int
     launch_transpose_sort(A.tr, nf * Npos, stream);
   }
   return finish_op(st, stream);
+}
+
+template <typename real>
+int desc_launch(const DescConfig<real>& c, const real* pos, const real* box, int nf, int N, int Npos,
+                const int* inj_howmany, const int* inj_with, int skip_pbc, real* raddescr, real* angdescr,
+                real* des3bsupp, int* intmap2b, int* intmap3b, real* der2b, real* der3b, real* der3bsupp,
+                int* numtriplet, real* unit, hipStream_t stream) {
+  return desc_launch_impl<real>(c, pos, box, nf, N, Npos, inj_howmany, inj_with, skip_pbc, raddescr, angdescr,
+                                des3bsupp, intmap2b, intmap3b, der2b, der3b, der3bsupp, numtriplet, unit, stream,
+                                (const FingerprintStep<real>*)nullptr);
 }
 template int desc_launch<float>(const DescConfig<float>&, const float*, const float*, int, int, int, const int*,
                                 const int*, int, float*, float*, float*, int*, int*, float*, float*, float*, int*,
@@ -801,9 +941,70 @@ static int compute(const real* pos, const real* box, int nf, int N, real* raddes
                            intmap3b, der2b, der3b, der3bsupp, numtriplet, (real*)nullptr, (hipStream_t)stream_);
 }
 
+// Descriptors and fingerprints of every species in one launch (the library's own neighbour search, all N atoms
+// local).
+template <typename real>
+static int compute_with_fingerprints(const real* pos, const real* box, int nf, int N, real* raddescr, real* angdescr,
+                                     real* des3bsupp, int* intmap2b, int* intmap3b, real* der2b, real* der3b,
+                                     real* der3bsupp, int* numtriplet, int nt, const int* n_local,
+                                     int first_species, int n_species, const int* type_map, int Aa, const real* const* alpha3b,
+                                     const real* const* emb3b, real* const* af3, int Ar, const real* const* alpha2b,
+                                     const real* const* emb2b, real* const* af2, void* stream_) {
+  if (nt <= 0 || !n_local || first_species < 0 || n_species <= 0 || first_species + n_species > nt || !type_map ||
+      Aa <= 0 || !alpha3b || !emb3b || !af3 || Ar < 0 ||
+      (Ar > 0 && (!alpha2b || !emb2b || !af2)) || !angdescr)
+    return STAF_E_BAD_ARG;
+  if (nt > NT_MAX) return STAF_E_LIMIT;
+  long sum = 0;
+  for (int k = 0; k < nt; k++) {
+    if (n_local[k] < 0) return STAF_E_BAD_ARG;
+    sum += n_local[k];
+    const bool mine = k >= first_species && k < first_species + n_species;
+    if (mine && n_local[k] > 0 && (!alpha3b[k] || !emb3b[k] || !af3[k] || (Ar > 0 && (!alpha2b[k] || !emb2b[k] || !af2[k]))))
+      return STAF_E_BAD_ARG;
+  }
+  if (sum != N) return STAF_E_BAD_ARG;
+  DescConfig<real> c;
+  {
+    std::lock_guard<std::mutex> lock(g_cfg_mu);
+    c = cfg<real>().current();
+  }
+  FingerprintStep<real> fp = {nt, first_species, n_species, n_local, type_map, Aa, alpha3b, emb3b, af3, Ar, alpha2b, emb2b, af2};
+  return desc_launch_impl<real>(c, pos, box, nf, N, N, nullptr, nullptr, 0, raddescr, angdescr, des3bsupp, intmap2b,
+                                intmap3b, der2b, der3b, der3bsupp, numtriplet, (real*)nullptr,
+                                (hipStream_t)stream_, &fp);
+}
+
 }  // namespace staf
 
 extern "C" {
+
+int staf_op_descriptors_fingerprints_f32(const float* positions, const float* boxer, int nf, int N, float* raddescr,
+                                         float* angdescr, float* des3bsupp, int* intmap2b, int* intmap3b,
+                                         float* der2b, float* der3b, float* der3bsupp, int* numtriplet, int nt,
+                                         const int* n_local, int first_species, int n_species, const int* type_map,
+                                         int nsmooth_a, const float* const* alpha3b, const float* const* type_emb3b,
+                                         float* const* three_body_AFs, int nalpha_r, const float* const* alpha2b,
+                                         const float* const* type_emb2b, float* const* radial_AFs, void* stream) {
+  return staf::compute_with_fingerprints<float>(positions, boxer, nf, N, raddescr, angdescr, des3bsupp, intmap2b,
+                                                intmap3b, der2b, der3b, der3bsupp, numtriplet, nt, n_local,
+                                                first_species, n_species, type_map, nsmooth_a, alpha3b, type_emb3b, three_body_AFs, nalpha_r, alpha2b,
+                                                type_emb2b, radial_AFs, stream);
+}
+int staf_op_descriptors_fingerprints_f64(const double* positions, const double* boxer, int nf, int N,
+                                         double* raddescr, double* angdescr, double* des3bsupp, int* intmap2b,
+                                         int* intmap3b, double* der2b, double* der3b, double* der3bsupp,
+                                         int* numtriplet, int nt, const int* n_local, int first_species,
+                                         int n_species, const int* type_map, int nsmooth_a,
+                                         const double* const* alpha3b,
+                                         const double* const* type_emb3b, double* const* three_body_AFs,
+                                         int nalpha_r, const double* const* alpha2b,
+                                         const double* const* type_emb2b, double* const* radial_AFs, void* stream) {
+  return staf::compute_with_fingerprints<double>(positions, boxer, nf, N, raddescr, angdescr, des3bsupp, intmap2b,
+                                                 intmap3b, der2b, der3b, der3bsupp, numtriplet, nt, n_local,
+                                                 first_species, n_species, type_map, nsmooth_a, alpha3b, type_emb3b, three_body_AFs, nalpha_r,
+                                                 alpha2b, type_emb2b, radial_AFs, stream);
+}
 
 int staf_op_construct_descriptors_light_f32(float rc, int nr, int na, int numpar, float rs, float ra, int max_batch,
                                             const char* path) {

@@ -641,10 +641,14 @@ int force_tripl(const real* G, const real* Dsup, const real* Tang, const real* d
   real* self = deferred ? self_out : gslot + ng;
   real* vpart = self + ns;
   const bool fused = unit != nullptr;   // the MD entry: T and its Jacobian rebuilt from the unit vectors
-  // Single precision: eight waves per workgroup (a wave's registers then admit eight waves per SIMD, and a centre's
-  // critical path is half as long: measured 20.5 against 22.4 us for 1024 centres, 32.0 against 34.0 for 2048);
-  // double precision: four (eight measured no faster, its registers admit no more resident waves).
-  constexpr int NWV = sizeof(real) == 4 ? 8 : 4;
+  // Four waves per workgroup in both precisions.  Eight (Force3Cfg<real, 8>) are faster in single precision when
+  // the launch has the GPU to itself (a wave's registers then admit eight waves per SIMD and a centre's critical path
+  // is half as long: 32.0 against 34.0 us for 2048 centres) but slower inside a step, where its workgroups share the
+  // CUs with those of other launches: an eight-wave workgroup needs two free wave slots on every SIMD of a CU at
+  // once and waits while four-wave workgroups around it end one by one (the 3-body force launches of a step held
+  // 0.7-0.8 of the wave slots, 0.9 when alone; 4 frames of 768 atoms: 104.1 against 105.8 us per step, 8 frames
+  // with the gradient ops: 330 against 345).  In double precision eight measured no faster even alone.
+  constexpr int NWV = 4;
   auto launch = [&](auto fused_c, auto w2b_c) -> int {
     constexpr bool FUSED = decltype(fused_c)::value, W2B = decltype(w2b_c)::value;
     using L = Force3Cfg<real, NWV>;

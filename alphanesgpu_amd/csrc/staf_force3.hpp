@@ -1,4 +1,4 @@
-// 3-body force, pass A: one workgroup of four or eight waves per centre atom, four barriers per centre.
+// 3-body force, pass A: one workgroup of four waves per centre atom, four barriers per centre.
 // Replaces computeforce_tripl_kernel (STAF/src/force/ang/reforce.cu.cc:96-214).
 //
 // The kernel is bound by vector-ALU issue and LDS bandwidth in its channel loop (an item reads its parameter entry
@@ -56,8 +56,9 @@ __device__ inline void wave_scan4(T (&v)[4]) {
   for (int c = 0; c < 4; c++) v[c] = s[c];
 }
 
-// NW_: waves per workgroup, 4 or 8.  A sweep takes 16 passes of 64 triplets either way; with eight waves a wave holds
-// two of them, so that a centre's critical path and a wave's registers are about half of what they are with four.
+// NW_: waves per workgroup, 4 or 8 (the launches use 4, see force_tripl).  A sweep takes 16 passes of 64 triplets
+// either way; with eight waves a wave holds two of them, so that a centre's critical path and a wave's registers
+// are about half of what they are with four.
 template <typename real, int NW_ = 4>
 struct Force3Cfg {
   static_assert(NW_ == 4 || NW_ == 8, "four or eight waves per workgroup");

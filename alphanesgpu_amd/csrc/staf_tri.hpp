@@ -316,9 +316,12 @@ struct TriLds {
 // FUSED (MODE 0 only, the MD entry): the angular descriptor of a triplet is not read from angdescr but rebuilt from
 // the slots' unit vectors and cutoff values, T = 1/2 (u_j . u_k + 1) fc_j fc_k
 // (DescriptorsAngular_kernel, STAF/src/descriptor_builder/reforce.cu.cc:195-212), so no na-wide tensor exists.
+// The kernel's body, for a workgroup that takes centres first, first + stride, ... (row-major over frames and the
+// species' atoms) and leaves its parameter-gradient sums in row part_row of A.partial: tri_reduce_kernel below,
+// and the launch that computes descriptors and fingerprints of a centre in one workgroup.
 template <typename real, int MODE, bool FUSED = false>
-__global__ __launch_bounds__(TRI_BLOCK, (TriCfg<real, MODE, FUSED>::MIN_WAVES)) void
-tri_reduce_kernel(TriArgs<real> A) {
+__device__ __forceinline__ void tri_reduce_body(const TriArgs<real> A, const int first_centre, const int stride,
+                                                const int part_row) {
   static_assert(!FUSED || MODE == 0, "only the fingerprint mode rebuilds T");
   using real2 = typename Vec2<real>::type;
   using HE = HotExp<real>;
@@ -361,7 +364,7 @@ tri_reduce_kernel(TriArgs<real> A) {
   int m0, nj0 = 0;
   real d0 = 0, gr0[3] = {0, 0, 0}, un0[3] = {0, 0, 0};
   {
-    const int b0 = blockIdx.x / A.Nl, p0 = blockIdx.x - b0 * A.Nl;
+    const int b0 = first_centre / A.Nl, p0 = first_centre - b0 * A.Nl;
     const size_t row0 = (size_t)b0 * A.ld + p0;
     m0 = A.numtriplet[row0];
     if (tid < nr) {
@@ -463,7 +466,7 @@ tri_reduce_kernel(TriArgs<real> A) {
     }
     for (int q = tid; q < TRI_WAVES * Aa; q += TRI_BLOCK) outw[q] = 0;
   };
-  int atom = blockIdx.x;
+  int atom = first_centre;
   centre_setup(atom, std::true_type{});
   while (true) {
     if (m <= WAVE) {
@@ -672,13 +675,19 @@ tri_reduce_kernel(TriArgs<real> A) {
         A.out[(size_t)atom * Aa + a] = s;
       }
     __syncthreads();
-    atom += gridDim.x;
-    if (atom >= total) break;
+    if (stride > total - 1 - atom) break;   // (no overflow of atom + stride)
+    atom += stride;
     centre_setup(atom, std::false_type{});
   }
   if (MODE != 0) {
-    for (int q = tid; q < NG * nacc; q += TRI_BLOCK) A.partial[(size_t)blockIdx.x * NG * nacc + q] = accw[q];
+    for (int q = tid; q < NG * nacc; q += TRI_BLOCK) A.partial[(size_t)part_row * NG * nacc + q] = accw[q];
   }
+}
+
+template <typename real, int MODE, bool FUSED = false>
+__global__ __launch_bounds__(TRI_BLOCK, (TriCfg<real, MODE, FUSED>::MIN_WAVES)) void
+tri_reduce_kernel(TriArgs<real> A) {
+  tri_reduce_body<real, MODE, FUSED>(A, (int)blockIdx.x, (int)gridDim.x, (int)blockIdx.x);
 }
 
 }  // namespace staf

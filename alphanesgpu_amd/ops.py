@@ -192,6 +192,53 @@ def compute_descriptors_light(positions, boxer, out=None):
     return out
 
 
+def compute_descriptors_fingerprints(positions, boxer, type_map, n_local, alpha3b_parameters, type_emb3b_parameters,
+                                     alpha2b_parameters=None, type_emb2b_parameters=None, out=None, species=None):
+    """Descriptors and the fingerprints of every centre species in one launch (no counterpart as one op in the
+    reference): what compute_descriptors_light(positions, boxer) returns, then, per species k (n_local[k] atoms,
+    species-sorted, summing to N), three_body_afs[k] [nf,n_local[k],Aa] as compute_sort_proj3body gives it for the
+    species' rows with alpha3b_parameters[k], type_emb3b_parameters[k] and -- if the 2-body parameter lists are
+    given -- radial_afs[k] [nf,n_local[k],Ar] as compute_sort_proj gives it, same bits.
+    species = (first, count): only the centres of these species (the descriptor rows and fingerprint arrays of the
+    others are not touched): one call per species, each on a stream of its own, lets the ops that follow a species'
+    fingerprints start when that species is through.
+    -> (descriptor tuple, [three_body_afs[k]], [radial_afs[k]] or None)."""
+    dtype = positions.dtype
+    s, _ = sfx(dtype)
+    if dtype not in _constructed:
+        raise _lib.StafError(-1, "compute_descriptors_fingerprints")
+    nr, na = _constructed[dtype]
+    positions = _dense(positions)
+    boxer = _dense(boxer)
+    nf = boxer.shape[0]
+    N = positions.shape[1] // 3
+    dev = positions.device
+    nt = len(n_local)
+    e = lambda *sh: torch.empty(sh, dtype=dtype, device=dev)
+    ei = lambda *sh: torch.empty(sh, dtype=torch.int32, device=dev)
+    if out is None:
+        out = (e(nf, N, nr), e(nf, N, na), e(nf, N, nr), ei(nf, N, nr + 1), ei(nf, N, 2 * na), e(nf, N, 3, nr),
+               e(nf, N, 3, 2 * na), e(nf, N, 3, nr), ei(nf, N))
+    raddescr, angdescr, des3bsupp, intmap2b, intmap3b, der2b, der3b, der3bsupp, numtriplet = out
+    a3 = [_dense(t) for t in alpha3b_parameters]
+    e3 = [_dense(t) for t in type_emb3b_parameters]
+    Aa = e3[0].shape[1]
+    af3 = [e(nf, int(n), Aa) for n in n_local]
+    with2 = alpha2b_parameters is not None
+    a2 = [_dense(t) for t in alpha2b_parameters] if with2 else []
+    e2 = [_dense(t) for t in type_emb2b_parameters] if with2 else []
+    Ar = e2[0].shape[1] if with2 else 0
+    af2 = [e(nf, int(n), Ar) for n in n_local] if with2 else None
+    arr = lambda ts: (C.c_void_p * nt)(*[t.data_ptr() for t in ts]) if ts else None
+    tm = _i32(type_map)
+    first, count = (0, nt) if species is None else species
+    call(f"staf_op_descriptors_fingerprints_{s}", ptr(positions), ptr(boxer), _I(nf), _I(N), ptr(raddescr),
+         ptr(angdescr), ptr(des3bsupp), ptr(intmap2b), ptr(intmap3b), ptr(der2b), ptr(der3b), ptr(der3bsupp),
+         ptr(numtriplet), _I(nt), (C.c_int * nt)(*[int(n) for n in n_local]), _I(first), _I(count), ptr(tm), _I(Aa), arr(a3), arr(e3),
+         arr(af3), _I(Ar), arr(a2), arr(e2), arr(af2 or []), _stream())
+    return out, af3, af2
+
+
 # --------------------------------------------------------------------------- fingerprints
 
 

@@ -31,7 +31,7 @@ VALU_PEAK_WAVE_INST = 256 * 4 * 2.4e9 / 4
 # the op's accumulations; fp64 carries the written-out exponential instead of the hardware exp2: 15 instructions and a
 # table read in the reduce kernels, 18 in the force kernel).
 # Set-up, triplet decoding, table building, staging and reductions are overhead and not counted.
-ALGORITHMIC_INST = {"af3_kernel": (7, 21), "force3_kernel": (13, 30), "grad3_kernel": (14, 28),
+ALGORITHMIC_INST = {"af3_kernel": (7, 21), "desc_fp_kernel": (7, 21), "force3_kernel": (13, 30), "grad3_kernel": (14, 28),
                     "gradforce3_kernel": (36, 50), "grads3_kernel": (40, 54)}
 
 SETTLE_STEPS = 300   # untimed graph replays of the set-up, see run_workload()
@@ -40,9 +40,9 @@ REPEATS = 5          # timed blocks of --steps steps each; the median block is r
 PROFILES = os.path.join(ROOT, "profiles")
 # bench.py's kernel names (the library's timing names) -> the names the profiler prints
 PROFILED_NAME = {
-    ("force3_kernel", "f32"): "staf::force3_kernel<float, false, 8, true>",      # 2-body + 3-body slot forces
+    ("force3_kernel", "f32"): "staf::force3_kernel<float, false, 4, true>",      # 2-body + 3-body slot forces
     ("force3_kernel", "f64"): "staf::force3_kernel<double, false, 4, true>",
-    ("force3_kernel_3b_only", "f32"): "staf::force3_kernel<float, false, 8, false>",   # the reference's op sequence
+    ("force3_kernel_3b_only", "f32"): "staf::force3_kernel<float, false, 4, false>",   # the reference's op sequence
     ("force3_kernel_3b_only", "f64"): "staf::force3_kernel<double, false, 4, false>",
     ("gradforce3_kernel", "f32"): "staf::tri_reduce_kernel<float, 2, false>",
     ("gradforce3_kernel", "f64"): "staf::tri_reduce_kernel<double, 2, false>",
@@ -52,6 +52,8 @@ PROFILED_NAME = {
     ("grad3_kernel", "f64"): "staf::tri_reduce_kernel<double, 1, false>",
     ("grads3_kernel", "f32"): "staf::tri_reduce_kernel<float, 3, false>",
     ("grads3_kernel", "f64"): "staf::tri_reduce_kernel<double, 3, false>",
+    ("desc_fp_kernel", "f32"): "staf::desc_fingerprints_kernel<float>",     # descriptors + fingerprints, one launch
+    ("desc_fp_kernel", "f64"): "staf::desc_fingerprints_kernel<double>",
     ("desc_kernel", "f32"): "staf::desc_kernel<float>",
     ("desc_kernel", "f64"): "staf::desc_kernel<double>",
     ("af3_fused", "f64"): "staf::tri_reduce_kernel<double, 0, true>",
@@ -80,7 +82,7 @@ def profile_traffic(kernel, workload, prec):
         if not m:
             continue
         name, grid, ctr, v, n = m.group(1), int(m.group(2)), m.group(3), float(m.group(4)), int(m.group(5))
-        inst = re.search(r"staf::(force3_kernel|tri_reduce_kernel|desc_kernel)<[^>]*>", name)
+        inst = re.search(r"staf::(force3_kernel|tri_reduce_kernel|desc_kernel|desc_fingerprints_kernel)<[^>]*>", name)
         if inst and inst.group(0) not in PROFILED_NAME.values():
             # a row of an instantiation this library no longer builds: the file mixes runs of several builds
             raise ProfileMissing(f"{path} holds rows of {inst.group(0)}, which the current library does not build: "
@@ -510,6 +512,10 @@ def main():
                          "and added to the 2-body forces in one launch (staf_op_force_tripl_slots + "
                          "staf_op_force_total), both 3-body parameter gradients in one pass "
                          "(staf_op_grads_tripl_fused); same results")
+    ap.add_argument("--first-stage", choices=["auto", "fused", "separate"], default="auto",
+                    help="descriptors and fingerprints of a species in one launch (staf_op_descriptors_fingerprints) "
+                         "or as the descriptor op and the fingerprint ops; auto: fused for single-precision "
+                         "forward+force steps of at most 4096 atoms")
     ap.add_argument("--dense-embedding", action="store_true",
                     help="type embeddings without zeros: every 3-body channel is active for every species pair "
                          "(default: the 0/1 block embeddings the reference trains with, a third of them active)")
@@ -622,6 +628,8 @@ def run_workload(args, workload, mode):
     def body_op(k, v, body, phase, record):
         radk, angk, supk, im2k, im3k, d2k, d3k, d3sk, ntrk = v
         p = P[k]
+        if phase == 0 and one_launch:
+            return None    # the fingerprints come out of the step's first launch
         if body == 2:
             if phase == 0:
                 return timed("af2", lambda: ops.compute_sort_proj(radk, im2k, p["alpha2b"], p["emb2b"], tm), record)
@@ -675,8 +683,31 @@ def run_workload(args, workload, mode):
 
     big = int(np.argmax(tipos))   # the species with the most centres: its 3-body chain is the longest in the step
 
+    # The library's step-level entry points: descriptors and the fingerprints of every species in one launch
+    # (a workgroup per centre goes from the neighbour search to the centre's fingerprints), then per species the
+    # slot forces (and the fused gradient pass), then the collecting launch.
+    # It pays where the centres of a step number about what the GPU holds at once (2048 workgroups of the
+    # single-precision kernels: the three launches it replaces each leave the GPU half empty while their last
+    # workgroups run); with several rounds of workgroups per launch the separate launches, which walk over the
+    # centres with persistent workgroups and run the species' fingerprint launches side by side, are faster.
+    one_launch = (not args.reference_op_sequence and
+                  (args.first_stage == "fused" or
+                   (args.first_stage == "auto" and dtype == np.float32 and nf * N <= 4096 and mode == "fwd_force")))
+    par_a3, par_e3 = [p["alpha3b"] for p in P], [p["emb3b"] for p in P]
+    par_a2, par_e2 = [p["alpha2b"] for p in P], [p["emb2b"] for p in P]
+
+    def first_stage(record, species=None):
+        return timed("descriptor+fingerprints",
+                     lambda: ops.compute_descriptors_fingerprints(pos, box, tm, tipos, par_a3, par_e3, par_a2, par_e2,
+                                                                  out=dbuf, species=species)[0], record)
+
     def step(record=False, streams=side):
-        d = timed("descriptor", lambda: ops.compute_descriptors_light(pos, box, out=dbuf), record)
+        if one_launch and streams is not None:
+            d = dbuf   # written species by species below
+        elif one_launch:
+            d = first_stage(record)
+        else:
+            d = timed("descriptor", lambda: ops.compute_descriptors_light(pos, box, out=dbuf), record)
         forces = {}
         if streams is None:
             for k in range(nt):
@@ -686,71 +717,92 @@ def run_workload(args, workload, mode):
             ready = main_stream.record_event()
             done = []
             forces_done = []   # events behind the force op of a side chain: all the total force waits for
-
-            def small_species():
-                for k in sorted(range(nt), key=lambda k: -tipos[k]):
-                    if k == big and args.streams == 3:
-                        continue
-                    if args.streams == 3:
-                        # Fingerprints and 3-body ops on the species' stream; its 2-body force (and the 2-body ops
-                        # after it) on the step's stream, behind the largest species' 2-body ops and after both
-                        # fingerprint ops of the species: that stream is idle by then, and the species' own chain,
-                        # the last one to end otherwise, is shorter by those ops (126.0 -> 122.8 us per fp32 step).
-                        vk = species_views(k, d)
-                        with torch.cuda.stream(streams[k]):
-                            streams[k].wait_event(ready)
-                            body_op(k, vk, 2, 0, record)
-                            body_op(k, vk, 3, 0, record)
-                            fingerprints = streams[k].record_event()
-                            forces[(k, 3)] = body_op(k, vk, 3, 1, record)
-                            forces_done.append(streams[k].record_event())
-                            for phase in range(2, n_phase):
-                                body_op(k, vk, 3, phase, record)
-                            if n_phase > 2:
-                                done.append(streams[k].record_event())
-                        main_stream.wait_event(fingerprints)
-                        forces[(k, 2)] = body_op(k, vk, 2, 1, record)
-                        for phase in range(2, n_phase):
-                            body_op(k, vk, 2, phase, record)
-                        continue
+            if one_launch:
+                # Nothing of a species depends on another species before the total force: each species' chain on
+                # its own stream, from its first launch (descriptors and fingerprints of its centres) on, the species
+                # with the most centres first; the small 2-body gradient ops of all on the step's stream.
+                order = sorted(range(nt), key=lambda k: -tipos[k])
+                views = {k: species_views(k, d) for k in order}
+                fingerprints = {}
+                for k in order:
                     with torch.cuda.stream(streams[k]):
                         streams[k].wait_event(ready)
-                        species_chain(k, d, record, forces)
+                        first_stage(record, (k, 1))
+                        fingerprints[k] = streams[k].record_event()
+                        forces[(k, 3)] = body_op(k, views[k], 3, 1, record)
                         forces_done.append(streams[k].record_event())
+                        for phase in range(2, n_phase):
+                            body_op(k, views[k], 3, phase, record)
+                        for phase in range(2, n_phase):
+                            body_op(k, views[k], 2, phase, record)
+                        if n_phase > 2:
+                            done.append(streams[k].record_event())
+            else:
 
-            if args.streams == 3:
-                # The largest species in two chains: its 3-body ops on its own stream, its 2-body ops on the
-                # step's stream (idle otherwise until the forces are summed).  Each chain's force op waits for the
-                # other's fingerprint op, the dependency the network creates in a real step.  (The gradient ops take
-                # their upstream gradients as given, here as in the per-species chains: no wait between them.)
-                # Issue order = the order in which a graph replay submits the chains: the longest one (the 3-body ops
-                # of the largest species) goes first, so that it starts right behind the descriptors, the other
-                # species' chains last (issued between the two, they held back the large species' 2-body ops
-                # until they were through).
-                sb = streams[big]
-                v = species_views(big, d)
-                for phase in range(2):
-                    with torch.cuda.stream(sb):
+                def small_species():
+                    for k in sorted(range(nt), key=lambda k: -tipos[k]):
+                        if k == big and args.streams == 3:
+                            continue
+                        if args.streams == 3:
+                            # Fingerprints and 3-body ops on the species' stream; its 2-body force (and the 2-body ops
+                            # after it) on the step's stream, behind the largest species' 2-body ops and after both
+                            # fingerprint ops of the species: that stream is idle by then, and the species' own chain,
+                            # the last one to end otherwise, is shorter by those ops (126.0 -> 122.8 us per fp32 step).
+                            vk = species_views(k, d)
+                            with torch.cuda.stream(streams[k]):
+                                streams[k].wait_event(ready)
+                                body_op(k, vk, 2, 0, record)
+                                body_op(k, vk, 3, 0, record)
+                                fingerprints = streams[k].record_event()
+                                forces[(k, 3)] = body_op(k, vk, 3, 1, record)
+                                forces_done.append(streams[k].record_event())
+                                for phase in range(2, n_phase):
+                                    body_op(k, vk, 3, phase, record)
+                                if n_phase > 2:
+                                    done.append(streams[k].record_event())
+                            main_stream.wait_event(fingerprints)
+                            forces[(k, 2)] = body_op(k, vk, 2, 1, record)
+                            for phase in range(2, n_phase):
+                                body_op(k, vk, 2, phase, record)
+                            continue
+                        with torch.cuda.stream(streams[k]):
+                            streams[k].wait_event(ready)
+                            species_chain(k, d, record, forces)
+                            forces_done.append(streams[k].record_event())
+
+                if args.streams == 3:
+                    # The largest species in two chains: its 3-body ops on its own stream, its 2-body ops on the
+                    # step's stream (idle otherwise until the forces are summed).  Each chain's force op waits for the
+                    # other's fingerprint op, the dependency the network creates in a real step.  (The gradient ops take
+                    # their upstream gradients as given, here as in the per-species chains: no wait between them.)
+                    # Issue order = the order in which a graph replay submits the chains: the longest one (the 3-body ops
+                    # of the largest species) goes first, so that it starts right behind the descriptors, the other
+                    # species' chains last (issued between the two, they held back the large species' 2-body ops
+                    # until they were through).
+                    sb = streams[big]
+                    v = species_views(big, d)
+                    for phase in range(2):
+                        with torch.cuda.stream(sb):
+                            if phase == 0:
+                                sb.wait_event(ready)
+                            out3 = body_op(big, v, 3, phase, record)
+                            e3 = sb.record_event()
+                        out2 = body_op(big, v, 2, phase, record)
+                        e2 = main_stream.record_event()
                         if phase == 0:
-                            sb.wait_event(ready)
-                        out3 = body_op(big, v, 3, phase, record)
-                        e3 = sb.record_event()
-                    out2 = body_op(big, v, 2, phase, record)
-                    e2 = main_stream.record_event()
-                    if phase == 0:
-                        main_stream.wait_event(e3)
-                        sb.wait_event(e2)
-                    else:
-                        forces[(big, 2)], forces[(big, 3)] = out2, out3
-                with torch.cuda.stream(sb):
-                    forces_done.append(e3)
+                            main_stream.wait_event(e3)
+                            sb.wait_event(e2)
+                        else:
+                            forces[(big, 2)], forces[(big, 3)] = out2, out3
+                    with torch.cuda.stream(sb):
+                        forces_done.append(e3)
+                        for phase in range(2, n_phase):
+                            body_op(big, v, 3, phase, record)
+                        if n_phase > 2:
+                            done.append(sb.record_event())
                     for phase in range(2, n_phase):
-                        body_op(big, v, 3, phase, record)
-                    if n_phase > 2:
-                        done.append(sb.record_event())
-                for phase in range(2, n_phase):
-                    body_op(big, v, 2, phase, record)
-            small_species()
+                        body_op(big, v, 2, phase, record)
+                small_species()
             for ev in forces_done:
                 main_stream.wait_event(ev)
             # eager steps: the force arrays were allocated on the side streams and are consumed on this one.  Under
@@ -874,6 +926,11 @@ def run_workload(args, workload, mode):
         # the 3-body force launch also does the 2-body force op's work: it is priced on the bytes of both signatures
         # less the force arrays neither op writes here, plus the slot forces it writes instead
         ab["force3_kernel"] += ab["force2_kernel"] - 2 * nt * 3 * N * s + N * (nr + 1) * 3 * s
+        # the step's first launch does the work of the descriptor op and of both fingerprint ops of every species:
+        # it is priced on what the three signatures hold less the descriptor tensors the fingerprint ops would
+        # read back (here they come out of the cache of the CU that wrote them)
+        ab["desc_fp_kernel"] = (ab["desc_kernel"] + N * (Ar + Aa) * s
+                                + nt * ((2 * nt * Ar) + (nt * (nt + 1) // 2) * 4 * Aa) * s + N * 4)
     kern = {}
     for name in list(ab) + ["gather_kernel", "force_total_kernel", "transpose_sort_kernel", "cell_build_kernel"]:
         ms, n = ops.kernel_time(name)
@@ -958,12 +1015,16 @@ def run_workload(args, workload, mode):
                                          "numtriplet zero beyond the active slots; der3b padding left untouched",
                    "species_tensors": "contiguous copies" if args.contiguous_splits else "views",
                    "species_streams": args.streams,
-                   "schedule": {1: "one stream", 2: "one stream per species",
-                                3: "one stream per species; on the step's stream the 2-body ops of the largest "
-                                   "species and the 2-body force ops of the others"}[args.streams],
+                   "schedule": ({1: "one stream", 2: "one stream per species",
+                                 3: "one stream per species; on the step's stream the 2-body ops of the largest "
+                                    "species and the 2-body force ops of the others"}[args.streams]
+                                if args.reference_op_sequence or args.streams == 1 else
+                                "first launch on the step's stream, then one stream per species for its 3-body ops; "
+                                "the 2-body gradient ops on the step's stream"),
                    "op_sequence": ("the reference's: one force array per force op and one launch that adds them; "
                                    "one op per parameter gradient" if args.reference_op_sequence else
-                                   "the library's step-level entry points: per species one launch for the 2-body and "
+                                   "the library's step-level entry points: descriptors and the fingerprints of all "
+                                   "species in one launch (staf_op_descriptors_fingerprints), per species one launch for the 2-body and "
                                    "3-body slot forces (staf_op_forces_slots), collected by the receiving atoms of all "
                                    "species in one launch (staf_op_force_total)" + ("; both 3-body parameter gradients in one pass "
                                                              "(staf_op_grads_tripl_fused)" if mode == "full_step"
@@ -987,8 +1048,9 @@ def run_workload(args, workload, mode):
         "kernel_hbm_frac": {k: ab[k] * nf / (kern[k]["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS
                             for k in kern if k in ab},
         # desc_kernel against the bytes it writes (its signature's bytes include der3b padding it leaves alone)
-        "desc_kernel_hbm_frac_of_written_bytes": desc_written * nf / (kern["desc_kernel"]["ms_per_step"] * 1e-3) / 1e9
-                                                 / HBM_PEAK_GBS,
+        "desc_kernel_hbm_frac_of_written_bytes": (
+            desc_written * nf / (kern["desc_kernel"]["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS
+            if "desc_kernel" in kern else None),
         "kernel_valu_frac_algorithmic": valu_frac,
         "whole_step_valu_frac_algorithmic": step_alg_inst / (el / args.steps) / VALU_PEAK_WAVE_INST,
         "triplet_channel_items_per_step": total_items,

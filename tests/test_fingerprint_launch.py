@@ -1,0 +1,134 @@
+"""Descriptors and fingerprints of all species in one launch (staf_op_descriptors_fingerprints) against the ops it
+stands for, on a real MI355X: every descriptor tensor and every fingerprint array bit for bit (the launch runs the
+same code per centre as staf_op_compute_descriptors_light, staf_op_angular_afs and staf_op_radial_afs; those are
+held to the oracle in test_gpu_parity.py), and one case directly against the oracle."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _separate(ops, torch, pos, box, tm, tipos, P, with2):
+    d = ops.compute_descriptors_light(pos, box)
+    rad, ang, sup, im2, im3, d2, d3, d3s, ntr = d
+    af3, af2, o = [], [], 0
+    nt = len(tipos)
+    for k, n in enumerate(tipos):
+        s = slice(o, o + n)
+        o += n
+        af3.append(ops.compute_sort_proj3body(ang[:, s], sup[:, s], im3[:, s], im2[:, s], P[k]["alpha3b"],
+                                              P[k]["emb3b"], tm, ntr[:, s], nt=nt))
+        if with2:
+            af2.append(ops.compute_sort_proj(rad[:, s], im2[:, s], P[k]["alpha2b"], P[k]["emb2b"], tm))
+    return d, af3, af2
+
+
+def _check(ops, torch, pos, box, tm, tipos, P, with2=True):
+    want_d, want3, want2 = _separate(ops, torch, pos, box, tm, tipos, P, with2)
+    got_d, got3, got2 = ops.compute_descriptors_fingerprints(
+        pos, box, tm, tipos, [p["alpha3b"] for p in P], [p["emb3b"] for p in P],
+        [p["alpha2b"] for p in P] if with2 else None, [p["emb2b"] for p in P] if with2 else None)
+    ops.poll_status()
+    names = ("raddescr", "angdescr", "des3bsupp", "intmap2b", "intmap3b", "der2b", "der3b", "der3bsupp", "numtriplet")
+    for name, a, b in zip(names, want_d, got_d):
+        if name == "der3b":   # beyond an atom's triplets der3b is left as it was: compare what is written
+            ntr = want_d[8].to(torch.int64)
+            m = torch.clamp(ntr * (ntr - 1) // 2, max=a.shape[-1] // 2)
+            idx = torch.arange(a.shape[-1] // 2, device=a.device)
+            live = (idx[None, None, :] < m[:, :, None])[:, :, None, :, None].expand(a.shape[0], a.shape[1], 3, -1, 2)
+            a = torch.where(live, a.view(a.shape[0], a.shape[1], 3, -1, 2), torch.zeros((), dtype=a.dtype, device=a.device))
+            b = torch.where(live, b.view(b.shape[0], b.shape[1], 3, -1, 2), torch.zeros((), dtype=b.dtype, device=b.device))
+        assert torch.equal(a, b), name
+    for k in range(len(tipos)):
+        assert got3[k].shape == want3[k].shape and torch.equal(got3[k], want3[k]), f"three_body_afs[{k}]"
+        if with2:
+            assert got2[k].shape == want2[k].shape and torch.equal(got2[k], want2[k]), f"radial_afs[{k}]"
+    if not with2:
+        assert got2 is None
+    return got_d, got3, got2
+
+
+def _water(name, dtype, nf=None, dense=False):
+    import torch
+    from alphanesgpu_amd import ops, synth
+    b = synth.water_batch(name)
+    nf = b["nf"] if nf is None else nf
+    tdt = torch.float32 if np.dtype(dtype) == np.float32 else torch.float64
+    dev = torch.device("cuda:0")
+    T = lambda a: torch.as_tensor(np.ascontiguousarray(a)).to(dev)
+    pos, box = T(b["pos"][:nf].astype(dtype)), T(b["box"][:nf].astype(dtype))
+    params = synth.fingerprint_params(dtype=np.dtype(dtype), dense_embedding=dense)
+    P = [{k: T(v) for k, v in m.items()} for m in params]
+    ops.construct_descriptors_light(synth.RC, synth.NR, synth.NA, b["N"], box, synth.RS, synth.RA, nf, dtype=tdt)
+    return ops, torch, pos, box, T(b["type_map"]), [int(x) for x in b["tipos"]], P, b, params
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_one_launch_gives_the_bits_of_the_three_ops(dtype):
+    ops, torch, pos, box, tm, tipos, P, _, _ = _water("water768_f64", dtype, nf=2)
+    _check(ops, torch, pos, box, tm, tipos, P)
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_dense_embeddings_and_no_two_body_part(dtype):
+    ops, torch, pos, box, tm, tipos, P, _, _ = _water("water96", dtype, dense=True)
+    _check(ops, torch, pos, box, tm, tipos, P, with2=False)
+    _check(ops, torch, pos, box, tm, tipos, P, with2=True)
+
+
+def test_cell_list_frames():
+    """6144 atoms: the neighbour search of the launch goes through the cell list."""
+    ops, torch, pos, box, tm, tipos, P, _, _ = _water("water6144", np.float64)
+    _check(ops, torch, pos, box, tm, tipos, P)
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_three_species_one_of_them_empty(dtype):
+    import torch
+    from alphanesgpu_amd import ops, synth
+    rng = np.random.default_rng(8)
+    tip = [6, 0, 7]
+    n = sum(tip)
+    pts = []
+    while len(pts) < n:
+        c = rng.uniform(-3.0, 3.0, 3)
+        if all(np.linalg.norm(c - q) > 0.9 for q in pts):
+            pts.append(c)
+    dev = torch.device("cuda:0")
+    tdt = torch.float32 if np.dtype(dtype) == np.float32 else torch.float64
+    T = lambda a: torch.as_tensor(np.ascontiguousarray(a)).to(dev)
+    pos = T(np.array(pts).reshape(1, -1).astype(dtype))
+    box = T(np.array([[13.0, 0, 0, 14.0, 0, 15.0]]).astype(dtype))
+    params = synth.fingerprint_params(nt=3, ar_map=(3, 2, 4), aa_map=(2, 3, 2, 2, 3, 2), dtype=np.dtype(dtype),
+                                      dense_embedding=True)
+    P = [{k: T(v) for k, v in m.items()} for m in params]
+    tm = T(np.repeat(np.arange(3), tip).astype(np.int32))
+    ops.construct_descriptors_light(4.5, 16, 60, n, box, 1.5, 3.5, 1, dtype=tdt)
+    _, af3, af2 = _check(ops, torch, pos, box, tm, tip, P)
+    assert af3[1].shape == (1, 0, 14) and af2[1].shape == (1, 0, 9)
+
+
+def test_against_the_oracle(oracle):
+    """fp64, two 768-atom frames: fingerprints of the launch within 1e-12 of the oracle's."""
+    import pipeline
+    from util import nerr
+    ops, torch, pos, box, tm, tipos, P, b, params = _water("water768_f64", np.float64, nf=2)
+    _, af3, af2 = ops.compute_descriptors_fingerprints(pos, box, tm, tipos, [p["alpha3b"] for p in P],
+                                                       [p["emb3b"] for p in P], [p["alpha2b"] for p in P],
+                                                       [p["emb2b"] for p in P])
+    ops.poll_status()
+    from alphanesgpu_amd import synth
+    up = synth.synthetic_upstream(2, b["tipos"], params, 11, np.float64)
+    ref = pipeline.run_oracle(oracle, b["pos"][:2], b["box"][:2], b["tipos"], b["type_map"], params, up, synth.NR,
+                              synth.NA, np.float64)
+    for k in range(2):
+        assert nerr(af3[k].cpu().numpy(), ref["af3"][k]) < 1e-12
+        assert nerr(af2[k].cpu().numpy(), ref["af2"][k]) < 1e-12
+
+
+def test_bad_arguments_are_refused():
+    from alphanesgpu_amd import _lib
+    ops, torch, pos, box, tm, tipos, P, _, _ = _water("water96", np.float64)
+    with pytest.raises(_lib.StafError):   # species counts that do not sum to the number of atoms
+        ops.compute_descriptors_fingerprints(pos, box, tm, [tipos[0], tipos[1] - 1], [p["alpha3b"] for p in P],
+                                             [p["emb3b"] for p in P])
