@@ -160,6 +160,8 @@ int main(int argc, char** argv) {
   const double* Q = up_d("Q");
   // per species: the force ops' outputs and the slot forces, kept for the collecting launch after the loop
   std::vector<const double*> f2_of(nt), f3_of(nt), slots_of(nt), selfs_of(nt), both_slots_of(nt), both_selfs_of(nt);
+  std::vector<const double*> a2_of(nt), e2_of(nt), a3_of(nt), e3_of(nt);
+  int Ar_all = 0, Aa_all = 0;
   int first = 0;   // first atom of the centre species: its rows are views into the descriptor outputs (ld_atoms = N)
   for (int k = 0; k < nt; first += tipos_h[k], k++) {
     const int Nl = tipos_h[k];
@@ -237,6 +239,7 @@ int main(int argc, char** argv) {
     STAF_CALL(staf_op_forces_slots_f64(G3, G2, supk, angk, d3sk, d3k, radk, d2k, im2k, im3k, nr, na, N, nf, Aa, Ar, e3,
                                        a3, a2, e2, nt, tipos, actual, both_slots, both_selfs, ntrk, type_map, Nl, N,
                                        stream));
+    a2_of[k] = a2, e2_of[k] = e2, a3_of[k] = a3, e3_of[k] = e3, Ar_all = Ar, Aa_all = Aa;
     f2_of[k] = f2, f3_of[k] = f3, slots_of[k] = slots, selfs_of[k] = selfs;
     both_slots_of[k] = both_slots, both_selfs_of[k] = both_selfs;
     HIP_OK(hipStreamSynchronize(stream));
@@ -258,6 +261,41 @@ int main(int argc, char** argv) {
     check_d("gf3n_" + s, gf3n, L * Aa);
     check_d("gf3a_" + s, gf3a, ntc * 3 * Aa);
     check_d("gf3e_" + s, gf3e, ntc * Aa);
+  }
+  // ---- descriptors and fingerprints of every species in one launch, into fresh tensors
+  {
+    double* rad1 = dev_alloc<double>(A * nr);
+    double* ang1 = dev_alloc<double>(A * na);
+    double* sup1 = dev_alloc<double>(A * nr);
+    int* im21 = dev_alloc<int>(A * (nr + 1));
+    int* im31 = dev_alloc<int>(A * 2 * na);
+    double* d21 = dev_alloc<double>(A * 3 * nr);
+    double* d31 = dev_alloc<double>(A * 6 * na);
+    double* d3s1 = dev_alloc<double>(A * 3 * nr);
+    int* ntr1 = dev_alloc<int>(A);
+    std::vector<double*> af3_of(nt), af2_of(nt);
+    for (int k = 0; k < nt; k++) {
+      af3_of[k] = dev_alloc<double>((size_t)nf * tipos_h[k] * Aa_all);
+      af2_of[k] = dev_alloc<double>((size_t)nf * tipos_h[k] * Ar_all);
+    }
+    STAF_CALL(staf_op_descriptors_fingerprints_f64(pos, box, nf, N, rad1, ang1, sup1, im21, im31, d21, d31, d3s1, ntr1,
+                                                   nt, tipos_h.data(), 0, nt, type_map, Aa_all, a3_of.data(),
+                                                   e3_of.data(), af3_of.data(), Ar_all, a2_of.data(), e2_of.data(),
+                                                   af2_of.data(), stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    check_d("raddescr", rad1, A * nr);
+    check_d("angdescr", ang1, A * na);
+    check_d("des3bsupp", sup1, A * nr);
+    check_i("intmap2b", im21, A * (nr + 1));
+    check_i("intmap3b", im31, A * 2 * na);
+    check_d("der2b", d21, A * 3 * nr);
+    check_d("der3b", d31, A * 6 * na);
+    check_d("der3bsupp", d3s1, A * 3 * nr);
+    check_i("numtriplet", ntr1, A);
+    for (int k = 0; k < nt; k++) {
+      check_d("af3_" + std::to_string(k), af3_of[k], (size_t)nf * tipos_h[k] * Aa_all);
+      check_d("af2_" + std::to_string(k), af2_of[k], (size_t)nf * tipos_h[k] * Ar_all);
+    }
   }
   // ---- the collecting launch: total force of the step from the slot forces of every centre species
   const size_t F = (size_t)nf * 3 * N;
