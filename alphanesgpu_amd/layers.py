@@ -12,7 +12,8 @@ here have the same names, constructor arguments and call signatures on top of `a
     ComputeForceTripl        ComputeForceTriplGrad             netderiv, alpha3b, emb3b   register_force_3bAFs_grad.py:14-24
     ...Virial forms          ...VirialGrad                     the same                   register_force_*_virial_grad.py
 
-Descriptors, maps and positions receive no gradient (the reference returns None for them): the descriptor op is not
+`descriptor_physics_layer` runs the descriptor op and the two fingerprint ops of all species as one launch and routes
+the same gradient ops.  Descriptors, maps and positions receive no gradient (the reference returns None for them): the descriptor op is not
 differentiated, forces come from the stored Jacobians.  Every tensor lives on the GPU; the ops run on torch's current
 stream.
 """
@@ -117,6 +118,50 @@ class _ForceTripl(torch.autograd.Function):
         return gn, None, None, None, None, None, None, ga, ge, None, None, None, None, None, None
 
 
+class _DescriptorsFingerprints(torch.autograd.Function):
+    """ComputeDescriptorsLight, then ComputeSortProj3body and ComputeSortProj for every centre species, as one launch
+    (ops.compute_descriptors_fingerprints).  Outputs: the nine descriptor tensors (no gradient), then per species
+    the 3-body fingerprints, then per species the 2-body fingerprints; gradients go to the parameter tensors through
+    the gradient ops of the two fingerprint ops, species by species, exactly as from _SortProj3body / _SortProj."""
+
+    @staticmethod
+    def forward(ctx, pos, box, type_map, n_local, *params):
+        nt = len(n_local)
+        a3, e3, a2, e2 = (list(params[i * nt:(i + 1) * nt]) for i in range(4))
+        desc, af3, af2 = ops.compute_descriptors_fingerprints(pos, box, type_map, n_local, a3, e3, a2, e2)
+        ctx.n_local = [int(n) for n in n_local]
+        ctx.save_for_backward(type_map, *desc, *params)
+        ctx.mark_non_differentiable(*desc)
+        return (*desc, *af3, *af2)
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, *grads):
+        nt = len(ctx.n_local)
+        type_map = ctx.saved_tensors[0]
+        rad, ang, sup, im2, im3, _, _, _, ntr = ctx.saved_tensors[1:10]
+        params = ctx.saved_tensors[10:]
+        a3, e3, a2, e2 = (params[i * nt:(i + 1) * nt] for i in range(4))
+        g3, g2 = grads[9:9 + nt], grads[9 + nt:9 + 2 * nt]
+        ga3, ge3, ga2, ge2 = [], [], [], []
+        first = 0
+        for k, n in enumerate(ctx.n_local):
+            s = slice(first, first + n)
+            first += n
+            if g3[k] is None or n == 0:
+                ga3.append(None), ge3.append(None)
+            else:
+                a, e = ops.compute_sort_proj3body_grad(g3[k].contiguous(), ang[:, s], sup[:, s], im3[:, s], im2[:, s],
+                                                       a3[k], e3[k], type_map, ntr[:, s], nt=nt)
+                ga3.append(a), ge3.append(e)
+            if g2[k] is None or n == 0:
+                ga2.append(None), ge2.append(None)
+            else:
+                a, e = ops.compute_two_body_par_grad(g2[k].contiguous(), rad[:, s], im2[:, s], a2[k], e2[k], type_map)
+                ga2.append(a), ge2.append(e)
+        return (None, None, None, None, *ga3, *ge3, *ga2, *ge2)
+
+
 def _type_now(x, device):
     return x if torch.is_tensor(x) else torch.tensor([int(x)], dtype=torch.int32, device=device)
 
@@ -170,6 +215,28 @@ class physics_layer(torch.nn.Module):
         np.savetxt(f"{folder_ou}/{prefix}type_emb_3b.dat", g(self.type_emb_3b))
         np.savetxt(f"{folder_ou}/{prefix}type_emb_2b_sq.dat", g(self.type_emb_2b) ** 2)
         np.savetxt(f"{folder_ou}/{prefix}type_emb_3b_sq.dat", g(self.type_emb_3b) ** 2)
+
+
+class descriptor_physics_layer(torch.nn.Module):
+    """descriptor_layer followed by the physics_layer of every centre species, as one launch (no counterpart as one
+    layer in the reference): `descriptors` is a descriptor_layer (it has configured the descriptor op), `physics` the
+    physics_layer modules of the species in species order, `n_local` the atoms per species (species-sorted atoms).
+    The call returns what descriptors(pos, box) returns and, per species, what its physics_layer returns for the
+    species' rows, with the same bits and the same gradients."""
+
+    def __init__(self, descriptors, physics, n_local):
+        super().__init__()
+        self.descriptors = descriptors
+        self.physics = torch.nn.ModuleList(physics)
+        self.n_local = [int(n) for n in n_local]
+
+    def forward(self, pos, box, type_map):
+        nt = len(self.n_local)
+        params = ([p.alpha3b for p in self.physics] + [torch.square(p.type_emb_3b) for p in self.physics] +
+                  [p.alpha2b for p in self.physics] + [torch.square(p.type_emb_2b) for p in self.physics])
+        out = _DescriptorsFingerprints.apply(pos, box, type_map, self.n_local, *params)
+        desc, af3, af2 = list(out[:9]), out[9:9 + nt], out[9 + nt:9 + 2 * nt]
+        return desc, [torch.cat([af2[k], af3[k]], dim=2) for k in range(nt)]
 
 
 class lognorm_layer(torch.nn.Module):

@@ -132,3 +132,46 @@ def test_bad_arguments_are_refused():
     with pytest.raises(_lib.StafError):   # species counts that do not sum to the number of atoms
         ops.compute_descriptors_fingerprints(pos, box, tm, [tipos[0], tipos[1] - 1], [p["alpha3b"] for p in P],
                                              [p["emb3b"] for p in P])
+
+
+def test_layer_gives_the_outputs_and_gradients_of_the_separate_layers():
+    """layers.descriptor_physics_layer against descriptor_layer + one physics_layer per species: same descriptor
+    tensors, same fingerprints, and the same parameter gradients of a loss that is linear in the fingerprints."""
+    import torch
+    from alphanesgpu_amd import layers, synth
+    dev = torch.device("cuda:0")
+    b = synth.water_batch("water96")
+    T = lambda a: torch.as_tensor(np.ascontiguousarray(a)).to(dev)
+    pos, box, tm = T(b["pos"]), T(b["box"]), T(b["type_map"])
+    tipos = [int(x) for x in b["tipos"]]
+    params = synth.fingerprint_params(dtype=np.float64, dense_embedding=True)
+    desc = layers.descriptor_layer(synth.RC, synth.NR, synth.RA, synth.NA, b["N"], box, synth.RS, b["nf"])
+
+    def physics():
+        return [layers.physics_layer(T(m["alpha2b"]), T(m["alpha3b"]), [T(np.sqrt(m["emb2b"])), T(np.sqrt(m["emb3b"]))])
+                for m in params]
+
+    rng = np.random.default_rng(3)
+    weights = [T(rng.standard_normal((b["nf"], n, params[0]["alpha2b"].shape[1] + params[0]["alpha3b"].shape[1] // 3)))
+               for n in tipos]
+    # the separate layers
+    ph = physics()
+    rad, ang, sup, im2, im3, d2, d3, d3s, ntr = desc(pos, box)
+    want, first = [], 0
+    for k, n in enumerate(tipos):
+        s = slice(first, first + n)
+        first += n
+        want.append(ph[k](rad[:, s], sup[:, s], im2[:, s], ang[:, s], im3[:, s], ntr[:, s], tm))
+    sum((w * a).sum() for w, a in zip(weights, want)).backward()
+    # one launch
+    ph1 = physics()
+    both = layers.descriptor_physics_layer(desc, ph1, tipos)
+    d1, got = both(pos, box, tm)
+    sum((w * a).sum() for w, a in zip(weights, got)).backward()
+    for a, c in zip((rad, ang, sup, im2, im3, d2, d3s, ntr), (d1[0], d1[1], d1[2], d1[3], d1[4], d1[5], d1[7], d1[8])):
+        assert torch.equal(a, c)
+    for k in range(len(tipos)):
+        assert torch.equal(want[k], got[k])
+        for name in ("alpha2b", "alpha3b", "type_emb_2b", "type_emb_3b"):
+            g0, g1 = getattr(ph[k], name).grad, getattr(ph1[k], name).grad
+            assert g0 is not None and g1 is not None and torch.equal(g0, g1), (k, name)
