@@ -47,15 +47,17 @@ constexpr int TRI_CAPP = TRI_CAP + 1;   // table row pitch: the entry after a ro
 constexpr int TRI_SUBS = TRI_BLOCK / TRI_CAP;
 template <typename real, int MODE, bool FUSED = false>
 struct TriCfg {
-  // triplets staged per block.  The double-precision pass that gives both gradients stages fewer: with 512 (or with
-  // 256 beside the table of the exponential) its LDS footprint would admit three workgroups per CU instead of four.
+  // triplets staged per block.  The double-precision pass that gives both gradients stages 256: with 512 its LDS
+  // footprint would admit three workgroups per CU instead of four; with 256 it is 40496 bytes, 32 of the 128
+  // pieces of 1280 bytes a CU hands out, which is exactly a fourth (192, counted on 40 KB per workgroup, was the
+  // earlier choice: 336.7 -> 333.3 us per fp64 training step; 272, not a power of two, is slower again).
   // The fused double-precision fingerprint kernel (the MD entry: thousands of centres per launch, several per
   // workgroup) stages 160: five workgroups per CU instead of four.  The plain double-precision fingerprint kernel
   // stages 448: a CU hands out its 160 KB of LDS in pieces of 1280 bytes, so the 32496 bytes that 512 staged triplets
   // make count as 33280 and four workgroups fit, not the five that the occupancy query of the runtime reports
   // (measured with a kernel that counts its resident workgroups per CU); with 448 it is 31472 bytes and five
   // (6144-atom step 360.6 -> 356.8 us).
-  static constexpr int QB = sizeof(real) == 8 ? (MODE == 3 ? 192 : MODE == 2 ? 448 : FUSED ? 160 : MODE == 0 ? 448 : 512) : 512;
+  static constexpr int QB = sizeof(real) == 8 ? (MODE == 3 ? 256 : MODE == 2 ? 448 : FUSED ? 160 : MODE == 0 ? 448 : 512) : 512;
   // waves per SIMD the register allocation is held to: without a bound the allocation comes out a few registers
   // above the next occupancy step.  The
   // single-precision pass for both gradients is held to six (80 registers, 56 bytes of spill per lane outside the
