@@ -175,3 +175,65 @@ def test_layer_gives_the_outputs_and_gradients_of_the_separate_layers():
         for name in ("alpha2b", "alpha3b", "type_emb_2b", "type_emb_3b"):
             g0, g1 = getattr(ph[k], name).grad, getattr(ph1[k], name).grad
             assert g0 is not None and g1 is not None and torch.equal(g0, g1), (k, name)
+
+
+def test_random_configurations():
+    """Twelve seeded random configurations through the one-launch entry and the three ops: 1-3 species with 1-13
+    atoms each, 1-3 frames, orthorhombic and triclinic boxes with the cluster shifted far outside the cell, random
+    cutoffs Rs < Ra <= Rc, 1-6 channels per block, an angular buffer anywhere between the atom count and the full
+    triangle (truncated triplet lists included), either precision, block or dense embeddings; once per case the
+    species are also computed by one call each."""
+    import torch
+    from alphanesgpu_amd import ops, synth
+    dev = torch.device("cuda:0")
+    T = lambda a: torch.as_tensor(np.ascontiguousarray(a)).to(dev)
+    rng = np.random.default_rng(20250307)
+    for case in range(12):
+        nt = int(rng.integers(1, 4))
+        tip = [int(x) for x in rng.integers(1, 14, nt)]
+        n = sum(tip)
+        nf = int(rng.integers(1, 4))
+        L = float(rng.uniform(9.5, 16.0))
+        spread = float(rng.uniform(2.2, 4.5))
+        tric = float(rng.random() < 0.5)
+        pos, box = np.zeros((nf, 3 * n)), np.zeros((nf, 6))
+        for b in range(nf):
+            pts = []
+            while len(pts) < n:
+                c = rng.uniform(-spread, spread, 3)
+                if all(np.linalg.norm(c - q) > 0.85 for q in pts):
+                    pts.append(c)
+            pos[b] = (np.array(pts) + rng.uniform(-30, 30, 3)).reshape(-1)
+            box[b] = [L, 0.6 * tric, -0.3 * tric, L + 0.7, 0.4 * tric, L + 1.3]
+        rc = float(rng.uniform(3.0, 4.6))
+        ra = float(rng.uniform(2.0, rc))
+        rs = float(rng.uniform(0.9, 0.5 * rc))
+        nr = n + 2
+        na = int(rng.integers(max(3, n), nr * (nr - 1) // 2 + 1))
+        ar = tuple(int(x) for x in rng.integers(1, 7, nt))
+        aa = tuple(int(x) for x in rng.integers(1, 7, nt * (nt + 1) // 2))
+        dtype = np.float64 if rng.random() < 0.6 else np.float32
+        dense = bool(rng.random() < 0.5)
+        tdt = torch.float32 if dtype == np.float32 else torch.float64
+        params = synth.fingerprint_params(nt=nt, ar_map=ar, aa_map=aa, seed=case + 1, dtype=np.dtype(dtype),
+                                          dense_embedding=dense)
+        P = [{k: T(v) for k, v in m.items()} for m in params]
+        tpos, tbox = T(pos.astype(dtype)), T(box.astype(dtype))
+        tm = T(np.repeat(np.arange(nt), tip).astype(np.int32))
+        ops.construct_descriptors_light(rc, nr, na, n, tbox, rs, ra, nf, dtype=tdt)
+        try:
+            _check(ops, torch, tpos, tbox, tm, tip, P)
+            # species by species into one set of tensors
+            want_d, want3, want2 = _separate(ops, torch, tpos, tbox, tm, tip, P, True)
+            out = None
+            for k in range(nt):
+                out, af3, af2 = ops.compute_descriptors_fingerprints(
+                    tpos, tbox, tm, tip, [p["alpha3b"] for p in P], [p["emb3b"] for p in P],
+                    [p["alpha2b"] for p in P], [p["emb2b"] for p in P], out=out, species=(k, 1))
+                assert torch.equal(af3[k], want3[k]) and torch.equal(af2[k], want2[k])
+            ops.poll_status()
+            for idx in (0, 1, 2, 3, 4, 5, 7, 8):
+                assert torch.equal(out[idx], want_d[idx]), idx
+        except AssertionError as e:
+            raise AssertionError(f"case {case}: nt={nt} tipos={tip} nf={nf} rc={rc:.2f} ra={ra:.2f} rs={rs:.2f} "
+                                 f"nr={nr} na={na} ar={ar} aa={aa} {np.dtype(dtype).name} dense={dense}: {e}") from e
