@@ -199,8 +199,8 @@ def compute_descriptors_fingerprints(positions, boxer, type_map, n_local, alpha3
     species-sorted, summing to N), three_body_afs[k] [nf,n_local[k],Aa] as compute_sort_proj3body gives it for the
     species' rows with alpha3b_parameters[k], type_emb3b_parameters[k] and -- if the 2-body parameter lists are
     given -- radial_afs[k] [nf,n_local[k],Ar] as compute_sort_proj gives it, same bits.
-    species = (first, count): only the centres of these species (the descriptor rows and fingerprint arrays of the
-    others are not touched): one call per species, each on a stream of its own, lets the ops that follow a species'
+    species = (first, count): only the centres of these species (the descriptor rows of the others are not touched
+    and their entries of the returned lists are None): one call per species, each on a stream of its own, lets the ops that follow a species'
     fingerprints start when that species is through.
     -> (descriptor tuple, [three_body_afs[k]], [radial_afs[k]] or None)."""
     dtype = positions.dtype
@@ -223,15 +223,16 @@ def compute_descriptors_fingerprints(positions, boxer, type_map, n_local, alpha3
     a3 = [_dense(t) for t in alpha3b_parameters]
     e3 = [_dense(t) for t in type_emb3b_parameters]
     Aa = e3[0].shape[1]
-    af3 = [e(nf, int(n), Aa) for n in n_local]
+    first, count = (0, nt) if species is None else species
+    mine = lambda k: first <= k < first + count
+    af3 = [e(nf, int(n), Aa) if mine(k) else None for k, n in enumerate(n_local)]   # (None: not one of `species`)
     with2 = alpha2b_parameters is not None
     a2 = [_dense(t) for t in alpha2b_parameters] if with2 else []
     e2 = [_dense(t) for t in type_emb2b_parameters] if with2 else []
     Ar = e2[0].shape[1] if with2 else 0
-    af2 = [e(nf, int(n), Ar) for n in n_local] if with2 else None
-    arr = lambda ts: (C.c_void_p * nt)(*[t.data_ptr() for t in ts]) if ts else None
+    af2 = [e(nf, int(n), Ar) if mine(k) else None for k, n in enumerate(n_local)] if with2 else None
+    arr = lambda ts: (C.c_void_p * nt)(*[None if t is None else t.data_ptr() for t in ts]) if ts else None
     tm = _i32(type_map)
-    first, count = (0, nt) if species is None else species
     call(f"staf_op_descriptors_fingerprints_{s}", ptr(positions), ptr(boxer), _I(nf), _I(N), ptr(raddescr),
          ptr(angdescr), ptr(des3bsupp), ptr(intmap2b), ptr(intmap3b), ptr(der2b), ptr(der3b), ptr(der3bsupp),
          ptr(numtriplet), _I(nt), (C.c_int * nt)(*[int(n) for n in n_local]), _I(first), _I(count), ptr(tm), _I(Aa), arr(a3), arr(e3),
