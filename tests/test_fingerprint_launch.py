@@ -237,3 +237,24 @@ def test_random_configurations():
         except AssertionError as e:
             raise AssertionError(f"case {case}: nt={nt} tipos={tip} nf={nf} rc={rc:.2f} ra={ra:.2f} rs={rs:.2f} "
                                  f"nr={nr} na={na} ar={ar} aa={aa} {np.dtype(dtype).name} dense={dense}: {e}") from e
+
+
+def test_radial_overflow_is_reported_by_the_launch_too():
+    """More neighbours than radial_buffer: STAF_E_RADIAL_OVERFLOW as from the descriptor op, every kernel exits
+    normally, and a call with a large enough buffer right afterwards gives the bits of the three ops."""
+    import torch
+    from alphanesgpu_amd import ops, synth, _lib
+    b = synth.water_batch("water96")
+    dev = torch.device("cuda:0")
+    T = lambda a: torch.as_tensor(np.ascontiguousarray(a)).to(dev)
+    pos, box, tm = T(b["pos"]), T(b["box"]), T(b["type_map"])
+    tipos = [int(x) for x in b["tipos"]]
+    params = synth.fingerprint_params(dtype=np.float64)
+    P = [{k: T(v) for k, v in m.items()} for m in params]
+    ops.construct_descriptors_light(4.5, 20, 190, b["N"], None, 2.25, 4.5, 1, dtype=torch.float64)
+    with pytest.raises(_lib.StafError) as e:
+        ops.compute_descriptors_fingerprints(pos, box, tm, tipos, [p["alpha3b"] for p in P], [p["emb3b"] for p in P],
+                                             [p["alpha2b"] for p in P], [p["emb2b"] for p in P])
+    assert e.value.code == -10
+    ops.construct_descriptors_light(synth.RC, synth.NR, synth.NA, b["N"], box, synth.RS, synth.RA, 1, dtype=torch.float64)
+    _check(ops, torch, pos, box, tm, tipos, P)
