@@ -258,3 +258,30 @@ def test_radial_overflow_is_reported_by_the_launch_too():
     assert e.value.code == -10
     ops.construct_descriptors_light(synth.RC, synth.NR, synth.NA, b["N"], box, synth.RS, synth.RA, 1, dtype=torch.float64)
     _check(ops, torch, pos, box, tm, tipos, P)
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_wide_channel_sets(dtype):
+    """Three species with 141 three-body and 57 two-body channels (classes of up to 42 active channels: three table
+    chunks, and in double precision an LDS request beyond what a launch gets without asking)."""
+    import torch
+    from alphanesgpu_amd import ops, synth
+    dev = torch.device("cuda:0")
+    T = lambda a: torch.as_tensor(np.ascontiguousarray(a)).to(dev)
+    rng = np.random.default_rng(21)
+    tip = [18, 15, 13]
+    n = sum(tip)
+    pts = []
+    while len(pts) < n:
+        c = rng.uniform(-3.2, 3.2, 3)
+        if all(np.linalg.norm(c - q) > 0.75 for q in pts):
+            pts.append(c)
+    pos = T((np.array(pts) + rng.uniform(-5, 5, 3)).reshape(1, -1).astype(dtype))
+    box = T(np.array([[16.0, 0.5, -0.3, 16.7, 0.4, 17.3]]).astype(dtype))
+    params = synth.fingerprint_params(nt=3, ar_map=(11, 16, 30), aa_map=(12, 5, 40, 4, 42, 38), seed=2,
+                                      dtype=np.dtype(dtype))
+    P = [{k: T(v) for k, v in m.items()} for m in params]
+    tm = T(np.repeat(np.arange(3), tip).astype(np.int32))
+    tdt = torch.float32 if np.dtype(dtype) == np.float32 else torch.float64
+    ops.construct_descriptors_light(5.4, n + 2, 938, n, box, 1.5, 4.9, 1, dtype=tdt)
+    _check(ops, torch, pos, box, tm, tip, P)
