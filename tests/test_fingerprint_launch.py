@@ -285,3 +285,80 @@ def test_wide_channel_sets(dtype):
     tdt = torch.float32 if np.dtype(dtype) == np.float32 else torch.float64
     ops.construct_descriptors_light(5.4, n + 2, 938, n, box, 1.5, 4.9, 1, dtype=tdt)
     _check(ops, torch, pos, box, tm, tip, P)
+
+
+def test_hip_graph_replay_of_the_species_launches_matches_eager():
+    """One launch per species, each followed by the species' slot forces, on the species' own stream, the collecting
+    launch on the step's stream; captured once into a HIP graph: every replay, with eager steps and
+    synchronisations in between, gives the eager single-stream result bit for bit."""
+    import torch
+    from alphanesgpu_amd import ops, synth
+    dev = torch.device("cuda:0")
+    b = synth.water_batch("water96")
+    T = lambda a: torch.as_tensor(np.ascontiguousarray(a)).to(dev)
+    pos, box, tm, tp = T(b["pos"]), T(b["box"]), T(b["type_map"]), T(b["tipos"])
+    tipos = [int(x) for x in b["tipos"]]
+    nt, nf, N = len(tipos), b["nf"], b["N"]
+    params = synth.fingerprint_params(dtype=np.float64)
+    P = [{k: T(v) for k, v in m.items()} for m in params]
+    up = synth.synthetic_upstream(nf, b["tipos"], params, 3, np.float64)
+    G2, G3 = [T(x) for x in up["G2"]], [T(x) for x in up["G3"]]
+    at = [torch.tensor([k], dtype=torch.int32, device=dev) for k in range(nt)]
+    nr, na = synth.NR, synth.NA
+    ops.construct_descriptors_light(synth.RC, nr, na, N, box, synth.RS, synth.RA, nf, dtype=torch.float64)
+    e = lambda *sh: torch.empty(sh, dtype=torch.float64, device=dev)
+    ei = lambda *sh: torch.empty(sh, dtype=torch.int32, device=dev)
+    dbuf = (e(nf, N, nr), e(nf, N, na), e(nf, N, nr), ei(nf, N, nr + 1), ei(nf, N, 2 * na), e(nf, N, 3, nr),
+            e(nf, N, 3, 2 * na), e(nf, N, 3, nr), ei(nf, N))
+    side = [torch.cuda.Stream() for _ in range(nt)]
+    lists = ([p["alpha3b"] for p in P], [p["emb3b"] for p in P], [p["alpha2b"] for p in P], [p["emb2b"] for p in P])
+    first = [sum(tipos[:k]) for k in range(nt)]
+
+    def species(k):
+        d, af3, af2 = ops.compute_descriptors_fingerprints(pos, box, tm, tipos, *lists, out=dbuf, species=(k, 1))
+        rad, ang, sup, im2, im3, d2, d3, d3s, ntr = [x[:, first[k]:first[k] + tipos[k]] for x in d]
+        p = P[k]
+        slots = ops.compute_forces_slots(G3[k], G2[k], sup, ang, d3s, d3, rad, d2, im2, im3, p["alpha3b"], p["emb3b"],
+                                         p["alpha2b"], p["emb2b"], tm, tp, at[k], ntr)
+        return af3[k], af2[k], slots
+
+    def step(streams):
+        outs = [None] * nt
+        if streams is None:
+            for k in range(nt):
+                outs[k] = species(k)
+        else:
+            main = torch.cuda.current_stream()
+            ready = main.record_event()
+            done = []
+            for k in sorted(range(nt), key=lambda k: -tipos[k]):
+                with torch.cuda.stream(streams[k]):
+                    streams[k].wait_event(ready)
+                    outs[k] = species(k)
+                    done.append(streams[k].record_event())
+            for ev in done:
+                main.wait_event(ev)
+        total = ops.force_total(dbuf[3], tipos, [o[2][0] for o in outs], [o[2][1] for o in outs])
+        return [o[0] for o in outs] + [o[1] for o in outs] + [total]
+
+    ops.set_sync_errors(False)
+    try:
+        want = [t.clone() for t in step(None)]
+        step(side)                      # sizes the per-stream work areas before the capture
+        ops.poll_status()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            held = step(side)
+        for rep in range(3):
+            g.replay()
+            torch.cuda.synchronize()
+            for x, y in zip(held, want):
+                assert torch.equal(x, y), f"replay {rep}"
+            again = step(None)          # eager work between the replays
+            ops.poll_status()
+            torch.cuda.synchronize()
+            for x, y in zip(again, want):
+                assert torch.equal(x, y)
+    finally:
+        ops.set_sync_errors(True)
