@@ -989,7 +989,10 @@ def run_workload(args, workload, mode):
                 "note": "algorithmic = the instructions the op's formulas need per (triplet, active channel) item; "
                         "executed_issue_share = all vector instructions the kernel issues (SQ_INSTS_VALU x 4 cycles "
                         "over the launch's SIMD-cycles, rocprofv3): the difference is set-up, decoding, tables, "
-                        "staging and reductions"}
+                        "staging and reductions"
+                        + ("; this launch also holds the descriptor op's work (neighbour search, descriptor rows and "
+                           "their Jacobians), for which no per-item count is defined: the algorithmic figure counts the "
+                           "3-body fingerprint items only" if dom == "desc_fp_kernel" else "")}
     # bytes desc_kernel really writes: the nr-wide tensors, angdescr and intmap3b over their whole rows (padding is
     # written as 0 like the reference's memsets), der3b over the triplets that exist only
     desc_written = N * (8 * nr + na) * s + N * (nr + 1 + 2 * na + 1) * 4 + N * 6 * na_act * s + (3 * N + 6) * s
