@@ -259,6 +259,18 @@ struct StreamWork {
   Workspace buckets;         // transpose a force op builds for itself: build counters, counts, keys
   size_t bucket_counters = 0;    // capacity, in ints, of each of the two counter parts
   size_t bucket_entries = 0;     // capacity, in ints, of the key part
+  Workspace cells;           // cell list of the descriptor op: set toggle, two sets of cell counters, tables, records
+  size_t cell_counters = 0;      // capacity, in ints, of each of the two counter sets
+};
+
+// The cell-list block of a stream (see cell_build_kernel).  The toggle and the counters live as long as the block:
+// the counter set the toggle names reads zero whenever a descriptor call starts, whatever the shapes of the calls
+// before it (a fresh block is cleared on the caller's stream).
+struct CellBlock {
+  int* toggle = nullptr;     // [1]
+  int* counts = nullptr;     // [2][set_ints]
+  size_t set_ints = 0;
+  char* rest = nullptr;      // rest_bytes, 256-byte aligned: tables and records of this call
 };
 
 // What a force kernel needs to find the slots that list an atom (see staf_transpose.hpp).  Two forms:
@@ -328,6 +340,7 @@ int* status_word(DeviceState* st, hipStream_t stream);
 // Both grow on demand and never shrink; under capture a request that does not fit what the stream already holds
 // returns null (the caller reports STAF_E_CAPTURE) instead of freeing and allocating.
 void* scratch_reserve(DeviceState* st, hipStream_t stream, size_t bytes);
+bool cells_reserve(DeviceState* st, hipStream_t stream, size_t counters, size_t rest_bytes, CellBlock* out);
 // Transpose a force op builds for itself (n_recv receiving atoms, cap keys each), in the stream's own work area.
 bool bucket_reserve(DeviceState* st, size_t n_recv, int cap, hipStream_t stream, TransposeRef* out);
 // What the library keeps beside the intmap2b tensor `im2` the descriptor op is about to write (nf frames, N centres,

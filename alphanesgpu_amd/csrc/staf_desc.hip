@@ -43,11 +43,14 @@ struct DescArgs {
   int skip_pbc;            // no minimum-image wrap (neighbours carry their periodic image)
   real Rc, Ra, Rs, cA, cB, cC, pa, pb;
   int dist2_fma, zero_padding;
-  // cell list of the frame (null: every atom is a candidate): atoms grouped by cell, see cell_build_kernel
-  const int* cell_dims;    // [nf, 4] cells along a, b, c (1: the axis is not divided), number of cells
-  const int* cell_start;   // [nf, CELL_MAX + 1]
-  const void* cell_recs;   // [nf, N] CellRec<real>: position and index of every atom, in cell order
-  const int* cell_of;      // [nf, N] cell of every atom
+  // cell list of the frames (cell_dims null: every atom is a candidate), see cell_build_kernel
+  const int* cell_dims;    // [nf, 8] cells along a, b, c (1: the axis is not divided), number of cells, counter set
+  const int* cell_counts;  // [2 sets][cell_set_ints]; of a set: [nf, cell_max] atoms per cell (may exceed cell_cap)
+  const void* cell_recs;   // [nf, cell_max, cell_cap] CellRec<real>: position and index of the atoms of every cell
+  const int* cell_of;      // [nf, N] cell of every atom: its three coordinates in the grid, 10 bits each
+  int* cell_toggle;        // the counter set the next build uses (flipped by this launch)
+  size_t cell_set_ints;    // ints between the two counter sets
+  int cell_max, cell_cap;  // cells a frame may have, atoms a cell holds
   real* raddescr;
   real* angdescr;
   real* des3bsupp;
@@ -117,56 +120,48 @@ __device__ inline real norm_plain(const real* d) {
 // library's own).  The box is cut into nx x ny x nz cells in fractional coordinates with every cell at least Rc
 // wide measured perpendicular to its faces, so that all atoms within Rc of a centre (minimum image by rounding the
 // fractional difference, as the scan does) lie in the centre's cell or one of its 26 neighbours.  An axis with
-// fewer than three such cells is not divided (its two neighbours would coincide).  One workgroup per frame.
-// The order of the atoms inside a cell is arbitrary: the neighbour search sorts what it finds.
+// fewer than three such cells is not divided (its two neighbours would coincide).
+// A cell holds up to `cap` atoms as packed position+index records; a thread per atom takes the atom's place in
+// its cell with one atomic add on the cell's counter, so a frame is binned by as many workgroups as it has
+// 256-atom pieces (one workgroup per frame, with a prefix sum over the cells between a counting and a fill pass,
+// took 13-16 us for 6144 atoms: a single CU's memory pipeline).  The order of the atoms inside a cell is
+// arbitrary: the neighbour search sorts what it finds.  A cell that counts more atoms than it holds lacks some of
+// them: the search of a centre in or beside such a cell tests every atom of the frame instead.
+// The counters must read zero when a build starts.  There are two sets of them: a build takes the set the
+// device-side toggle names, clears the whole other set, and the descriptor launch that follows flips the toggle --
+// no launch of its own for the clearing, and nothing a replayed graph would have to be told.
 // ---------------------------------------------------------------------------
-constexpr int CELL_MAX = 4096;
-constexpr int CELL_THREADS = 1024;   // one workgroup bins a whole frame: as wide as a workgroup gets
-constexpr int CELL_APT = 8;          // atoms a thread holds in registers from the counting pass to the fill pass
+constexpr int CELL_MAX = 4096;       // most cells of a frame
+constexpr int CELL_THREADS = 256;
 
 // An atom as the neighbour search reads it: Cartesian position and index in one 16-byte (float) or 32-byte (double)
-// record, stored in cell order, so that the atoms of a cell -- and of the cells next to it along the last axis --
-// are one contiguous run of records.
+// record.
 template <typename real> struct CellRec;
 template <> struct __align__(16) CellRec<float> { float x, y, z; int j; };
 template <> struct __align__(16) CellRec<double> { double x, y, z; int j, pad; };
 
-// inclusive prefix sum over the 1024 threads of the workgroup (two barriers); sc: 16 ints of LDS
-__device__ inline int block_scan_1024(int v, int* sc) {
-  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
-#pragma unroll
-  for (int o = 1; o < WAVE; o <<= 1) {
-    const int t = __shfl_up(v, o, WAVE);
-    if (lane >= o) v += t;
-  }
-  if (lane == WAVE - 1) sc[wave] = v;
-  __syncthreads();
-  int before = 0;
-  for (int w = 0; w < wave; w++) before += sc[w];
-  __syncthreads();
-  return v + before;
-}
-
 template <typename real>
 __global__ __launch_bounds__(CELL_THREADS) void cell_build_kernel(const real* __restrict__ pos, const real* __restrict__ boxes,
-                                                         int N, real Rc, int* __restrict__ cell_dims,
-                                                         int* __restrict__ cell_start, CellRec<real>* __restrict__ cell_recs,
+                                                         int N, real Rc, const int* __restrict__ toggle,
+                                                         size_t set_ints, int cell_max, int cap,
+                                                         int* __restrict__ cell_dims, int* __restrict__ counts,
+                                                         CellRec<real>* __restrict__ cell_recs,
                                                          int* __restrict__ cell_of) {
-  __shared__ int cnt[CELL_MAX];
   __shared__ int dims[4];
-  __shared__ int sc[CELL_THREADS / WAVE];
-  const int tid = threadIdx.x, b = blockIdx.x;
+  const int tid = threadIdx.x, b = blockIdx.y;
+  const int a = blockIdx.x * CELL_THREADS + tid;
   real box[6], inv[6];
 #pragma unroll
   for (int c = 0; c < 6; c++) box[c] = boxes[b * 6 + c];
   const real* pf = pos + (size_t)b * N * 3;
-  // the positions of the first CELL_APT x 1024 atoms are requested before anything is computed, and kept
-  real px[CELL_APT], py[CELL_APT], pz[CELL_APT];
-  int cl[CELL_APT];
-#pragma unroll
-  for (int u = 0; u < CELL_APT; u++) {
-    const int a = tid + u * CELL_THREADS < N ? tid + u * CELL_THREADS : N - 1;
-    px[u] = pf[3 * a]; py[u] = pf[3 * a + 1]; pz[u] = pf[3 * a + 2];
+  real px = 0, py = 0, pz = 0;
+  if (a < N) { px = pf[3 * a]; py = pf[3 * a + 1]; pz = pf[3 * a + 2]; }
+  const int set = toggle[0] & 1;
+  // the other set is cleared, all of it (what earlier calls of other shapes counted included)
+  {
+    int* other = counts + (size_t)(1 - set) * set_ints;
+    const size_t step = (size_t)gridDim.x * gridDim.y * CELL_THREADS;
+    for (size_t e = ((size_t)b * gridDim.x + blockIdx.x) * CELL_THREADS + tid; e < set_ints; e += step) other[e] = 0;
   }
   inverse_box(box, inv);
   if (tid == 0) {
@@ -179,85 +174,38 @@ __global__ __launch_bounds__(CELL_THREADS) void cell_build_kernel(const real* __
     const double hb = vol / sqrt(cax * cax + cay * cay + caz * caz);
     const double hc = vol / fabs(ax * by);
     int n[3] = {(int)(ha / (double)Rc), (int)(hb / (double)Rc), (int)(hc / (double)Rc)};
-    for (int c = 0; c < 3; c++) n[c] = n[c] < 3 ? 1 : n[c];
-    while ((long long)n[0] * n[1] * n[2] > CELL_MAX) {   // coarser cells only widen the search
+    for (int c = 0; c < 3; c++) n[c] = n[c] < 3 ? 1 : (n[c] > 1023 ? 1023 : n[c]);   // (10 bits each in cell_of)
+    while ((long long)n[0] * n[1] * n[2] > cell_max) {   // coarser cells only widen the search
       int big = n[0] >= n[1] && n[0] >= n[2] ? 0 : (n[1] >= n[2] ? 1 : 2);
       n[big] = n[big] - 1 < 3 ? 1 : n[big] - 1;
     }
     dims[0] = n[0]; dims[1] = n[1]; dims[2] = n[2]; dims[3] = n[0] * n[1] * n[2];
-    for (int c = 0; c < 4; c++) cell_dims[b * 4 + c] = dims[c];
-  }
-  for (int c = tid; c < CELL_MAX; c += CELL_THREADS) cnt[c] = 0;
-  __syncthreads();
-  const int nx = dims[0], ny = dims[1], nz = dims[2], ncell = dims[3];
-  int* of = cell_of + (size_t)b * N;
-  auto cell_index = [&](real x, real y, real z) -> int {
-    real s[3];
-    to_frac(inv, x, y, z, s);
-    int c3[3];
-    const int nn[3] = {nx, ny, nz};
-#pragma unroll
-    for (int c = 0; c < 3; c++) {
-      const real f = s[c] - r_floor(s[c]);   // [0, 1]
-      int q = (int)(f * (real)nn[c]);
-      c3[c] = q < 0 ? 0 : (q >= nn[c] ? nn[c] - 1 : q);
+    if (blockIdx.x == 0) {
+      for (int c = 0; c < 4; c++) cell_dims[b * 8 + c] = dims[c];
+      cell_dims[b * 8 + 4] = set;
     }
-    return (c3[0] * ny + c3[1]) * nz + c3[2];
-  };
-  // ---- counting pass
-#pragma unroll
-  for (int u = 0; u < CELL_APT; u++) {
-    const int a = tid + u * CELL_THREADS;
-    cl[u] = 0;
-    if (a < N) {
-      cl[u] = cell_index(px[u], py[u], pz[u]);
-      of[a] = cl[u];
-      atomicAdd(&cnt[cl[u]], 1);
-    }
-  }
-  for (int a = tid + CELL_APT * CELL_THREADS; a < N; a += CELL_THREADS) {   // frames beyond 8192 atoms
-    const int c = cell_index(pf[3 * a], pf[3 * a + 1], pf[3 * a + 2]);
-    of[a] = c;
-    atomicAdd(&cnt[c], 1);
   }
   __syncthreads();
-  // ---- exclusive prefix over the cells: a thread takes CPT consecutive cells
-  int* start = cell_start + (size_t)b * (CELL_MAX + 1);
-  constexpr int CPT = CELL_MAX / CELL_THREADS;
-  int mine[CPT], tot = 0;
+  if (a >= N) return;
+  const int nx = dims[0], ny = dims[1], nz = dims[2];
+  real s3[3];
+  to_frac(inv, px, py, pz, s3);
+  int c3[3];
+  const int nn[3] = {nx, ny, nz};
 #pragma unroll
-  for (int u = 0; u < CPT; u++) {
-    const int c = tid * CPT + u;
-    mine[u] = c < ncell ? cnt[c] : 0;
-    tot += mine[u];
+  for (int c = 0; c < 3; c++) {
+    const real f = s3[c] - r_floor(s3[c]);   // [0, 1]
+    int q = (int)(f * (real)nn[c]);
+    c3[c] = q < 0 ? 0 : (q >= nn[c] ? nn[c] - 1 : q);
   }
-  int run = block_scan_1024(tot, sc) - tot;   // atoms in the cells before this thread's
-#pragma unroll
-  for (int u = 0; u < CPT; u++) {
-    const int c = tid * CPT + u;
-    if (c < ncell) {
-      start[c] = run;
-      cnt[c] = run;   // becomes the fill cursor
-    }
-    run += mine[u];
-  }
-  if (tid == CELL_THREADS - 1) start[ncell] = run;
-  __syncthreads();
-  // ---- fill pass: records in cell order (the order inside a cell is arbitrary: the search sorts what it finds)
-  CellRec<real>* recs = cell_recs + (size_t)b * N;
-#pragma unroll
-  for (int u = 0; u < CELL_APT; u++) {
-    const int a = tid + u * CELL_THREADS;
-    if (a < N) {
-      CellRec<real> r;
-      r.x = px[u]; r.y = py[u]; r.z = pz[u]; r.j = a;
-      recs[atomicAdd(&cnt[cl[u]], 1)] = r;
-    }
-  }
-  for (int a = tid + CELL_APT * CELL_THREADS; a < N; a += CELL_THREADS) {
+  const int cell = (c3[0] * ny + c3[1]) * nz + c3[2];
+  cell_of[(size_t)b * N + a] = c3[0] | c3[1] << 10 | c3[2] << 20;
+  int* cnt = counts + (size_t)set * set_ints + (size_t)b * cell_max;
+  const int slot = atomicAdd(&cnt[cell], 1);
+  if (slot < cap) {   // (the centres around a cell whose count has passed its places test every atom of the frame)
     CellRec<real> r;
-    r.x = pf[3 * a]; r.y = pf[3 * a + 1]; r.z = pf[3 * a + 2]; r.j = a;
-    recs[atomicAdd(&cnt[of[a]], 1)] = r;
+    r.x = px; r.y = py; r.z = pz; r.j = a;
+    cell_recs[((size_t)b * cell_max + cell) * cap + slot] = r;
   }
 }
 
@@ -299,6 +247,7 @@ __device__ __forceinline__ void desc_body(const DescArgs<real> A, const int cent
   int* s_j = c_j + nr;                 // [nr] sorted neighbour index
   int* s_rank = s_j + nr;              // [nr] rank of every candidate
   __shared__ int cnt_all, cnt_ang;
+  __shared__ int nb_groups;      // cell search: groups of records to test; -1: a cell holds more atoms than it has places
   __shared__ unsigned row_sum;   // checksum of the row being written (row_hash over its slots)
   __shared__ real sinv[6];
 
@@ -329,49 +278,56 @@ __device__ __forceinline__ void desc_body(const DescArgs<real> A, const int cent
 
   // 1. candidate scan -- or the caller's list (already cut off and sorted by distance)
   const bool injected = A.inj_howmany != nullptr;
-  if (!injected && A.cell_start) {
+  // (the launch that reads a build's counters is the one that hands the next build the other set)
+  if (A.cell_dims && blockIdx.x == 0 && tid == 0) A.cell_toggle[0] ^= 1;
+  bool by_cells = false;
+  if (!injected && A.cell_dims) {
     // Candidates = the atoms of the centre's cell and its neighbours (every atom appears once: an axis has one cell or
-    // at least three).  Cells that follow each other along the last axis are contiguous in the record array, so the
-    // 27 cells are at most 18 runs of records: one per (dx, dy), two where the last axis wraps.  Each wave takes
-    // every fourth run, lane <-> record: one coalesced read per run, all of a wave's runs requested before the first
-    // is used.
-    constexpr int RUNS = 18, RPW = (RUNS + 3) / 4;
-    __shared__ int run_start[RUNS], run_len[RUNS];
-    const int* dm = A.cell_dims + b * 4;
+    // at least three).  The records of the up to 27 cells are taken in groups of 16 consecutive ones (a cell's last
+    // group may be short), listed in a table that lies where the sorted neighbours' records will go: thread <-> place
+    // in a group, one table read per candidate, and four candidates per thread are requested before the first is used.
+    constexpr int CELLS = 27, BATCH = 4, GROUP = 16;
+    int* group = (int*)s_rec;   // [groups] (first record / GROUP) << 5 | records
+    const int* dm = A.cell_dims + b * 8;
     const int nx = dm[0], ny = dm[1], nz = dm[2];
-    const int* cstart = A.cell_start + (size_t)b * (CELL_MAX + 1);
-    const CellRec<real>* recs = (const CellRec<real>*)A.cell_recs + (size_t)b * N;
-    if (tid < 9) {
-      const int ci = A.cell_of[(size_t)b * N + i];
-      const int cz = ci % nz, cy = (ci / nz) % ny, cx = ci / (nz * ny);
-      const int dx = tid / 3 - 1, dy = tid % 3 - 1;
-      int s0 = 0, l0 = 0, s1 = 0, l1 = 0;
-      if ((nx > 1 || dx == 0) && (ny > 1 || dy == 0)) {
-        const int x = (cx + dx + nx) % nx, y = (cy + dy + ny) % ny;
-        const int base = (x * ny + y) * nz;
-        // cells z0 .. z1 of this column without wrapping; a wrapped end is a second run
-        int z0 = nz > 1 ? cz - 1 : cz, z1 = nz > 1 ? cz + 1 : cz;
-        int w = -1;                      // the wrapped cell, if any
-        if (z0 < 0) { z0 = 0; w = nz - 1; }
-        if (z1 >= nz) { z1 = nz - 1; w = 0; }
-        s0 = cstart[base + z0];
-        l0 = cstart[base + z1 + 1] - s0;
-        if (w >= 0) { s1 = cstart[base + w]; l1 = cstart[base + w + 1] - s1; }
+    const int* cell_cnt = A.cell_counts + (size_t)dm[4] * A.cell_set_ints + (size_t)b * A.cell_max;
+    const int cap = A.cell_cap;   // a multiple of 2 * GROUP
+    const CellRec<real>* recs = (const CellRec<real>*)A.cell_recs + (size_t)b * A.cell_max * cap;
+    if (tid < WAVE) {   // lane <-> cell
+      int c = 0, l = 0;
+      if (tid < CELLS) {
+        const int ci = A.cell_of[(size_t)b * N + i];
+        const int cx = ci & 1023, cy = ci >> 10 & 1023, cz = ci >> 20;
+        const int dx = tid / 9 - 1, dy = (tid / 3) % 3 - 1, dz = tid % 3 - 1;
+        if ((nx > 1 || dx == 0) && (ny > 1 || dy == 0) && (nz > 1 || dz == 0)) {
+          int x = cx + dx, y = cy + dy, z = cz + dz;
+          x = x < 0 ? x + nx : (x >= nx ? x - nx : x);
+          y = y < 0 ? y + ny : (y >= ny ? y - ny : y);
+          z = z < 0 ? z + nz : (z >= nz ? z - nz : z);
+          c = (x * ny + y) * nz + z;
+          l = cell_cnt[c];
+        }
       }
-      run_start[2 * tid] = s0; run_len[2 * tid] = l0;
-      run_start[2 * tid + 1] = s1; run_len[2 * tid + 1] = l1;
+      // groups before a lane's own: a prefix sum over the lanes, register to register (same tree as wave_scan4)
+      const unsigned g = (unsigned)(l + GROUP - 1) / GROUP;
+      unsigned incl = g + dpp_get<0x111, 0xf>(g);
+      incl += dpp_get<0x112, 0xf>(g);
+      incl += dpp_get<0x113, 0xf>(g);
+      incl += dpp_get<0x114, 0xf>(incl);
+      incl += dpp_get<0x118, 0xf>(incl);
+      dpp_rows_carry(incl);
+      const bool over = __any(l > cap);
+      if (tid == CELLS) nb_groups = over ? -1 : (int)incl;   // (this lane has no cell: the sum of all before it)
+      if (!over) {
+        const int first = (int)(incl - g), base = c * (cap / GROUP);
+        for (int k = 0; k < (int)g; k++)
+          group[first + k] = (base + k) << 5 | (l - k * GROUP < GROUP ? l - k * GROUP : GROUP);
+      }
     }
     __syncthreads();
-    const int lane = tid & (WAVE - 1), wave = tid / WAVE;
-    CellRec<real> rc_[RPW];
-    int rl[RPW], rs[RPW];
-#pragma unroll
-    for (int u = 0; u < RPW; u++) {
-      const int r = wave + 4 * u;
-      rl[u] = r < RUNS ? run_len[r] : 0;
-      rs[u] = r < RUNS ? run_start[r] : 0;
-      if (lane < rl[u]) rc_[u] = recs[rs[u] + lane];
-    }
+    // (an overfull cell lacks the records of some of its atoms: this centre then tests every atom of the frame)
+    by_cells = nb_groups >= 0;
+    const int total = by_cells ? nb_groups * GROUP : 0;
     auto candidate = [&](const CellRec<real>& c) {
       const int j = c.j;
       if (j == i) return;
@@ -389,11 +345,25 @@ __device__ __forceinline__ void desc_body(const DescArgs<real> A, const int cent
         }
       }
     };
+    for (int t0 = 0; t0 < total; t0 += BATCH * 256) {
+      CellRec<real> rc_[BATCH];
+      bool have[BATCH];
 #pragma unroll
-    for (int u = 0; u < RPW; u++) {
-      if (lane < rl[u]) candidate(rc_[u]);
-      for (int q = lane + WAVE; q < rl[u]; q += WAVE) candidate(recs[rs[u] + q]);   // runs of more than 64 atoms
+      for (int u = 0; u < BATCH; u++) {
+        const int t = t0 + u * 256 + tid;
+        have[u] = false;
+        if (t < total) {
+          const int w = group[t / GROUP], e = t % GROUP;
+          have[u] = e < (w & 31);
+          if (have[u]) rc_[u] = recs[(size_t)(w >> 5) * GROUP + e];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < BATCH; u++)
+        if (have[u]) candidate(rc_[u]);
     }
+  }
+  if (by_cells) {
   } else if (!injected) {
     // the position reads of four candidates per thread are issued together
     for (int j0 = tid; j0 < A.Npos; j0 += 4 * 256) {
@@ -837,26 +807,34 @@ static int desc_launch_impl(const DescConfig<real>& c, const real* pos, const re
   const bool symmetric = inj_howmany == nullptr;
   if (!transpose_for_descriptor(st, intmap2b, nf, N, Npos, c.nr, 4 * c.nr, symmetric, stream, &A.tr))
     return reserve_failure(stream);
-  A.cell_dims = A.cell_start = A.cell_of = nullptr;
+  A.cell_dims = A.cell_counts = A.cell_of = nullptr;
   A.cell_recs = nullptr;
   const int cell_from = g_cell_threshold;
-  if (!inj_howmany && cell_from > 0 && N >= cell_from) {
-    // records first (16-byte aligned), then the integer tables
-    const size_t rec_bytes = (size_t)nf * N * sizeof(CellRec<real>);
-    const size_t ints = (size_t)nf * (4 + (CELL_MAX + 1) + (size_t)N);
-    char* w = (char*)scratch_reserve(st, stream, rec_bytes + ints * sizeof(int));
-    if (!w) return reserve_failure(stream);
-    CellRec<real>* recs = (CellRec<real>*)w;
-    int* dims = (int*)(w + rec_bytes);
-    int* start = dims + (size_t)nf * 4;
-    int* of = start + (size_t)nf * (CELL_MAX + 1);
-    {
-      KernelTimer kt_("cell_build_kernel", stream);
-      hipLaunchKernelGGL(cell_build_kernel<real>, dim3(nf), dim3(CELL_THREADS), 0, stream, pos, box, N, c.Rc, dims, start,
-                         recs, of);
-    }
-    A.cell_dims = dims; A.cell_start = start; A.cell_recs = recs; A.cell_of = of;
-  }
+  // The cell list is built by the launch below, just before the kernel that reads it (and that hands the next
+  // build its counters: the two go together).
+  auto build_cells = [&]() -> bool {
+    if (inj_howmany || cell_from <= 0 || N < cell_from || c.nr < 8) return true;   // (the search keeps a table of
+                                                                                   // nr * 27 / 16 + 54 ints in 8 * nr words)
+    // A cell is at least Rc wide and at most 4/3 of that per axis, a sphere of radius Rc holds at most nr atoms: a
+    // cell of nr places overflows only in frames far denser in one spot than on average (and those are searched
+    // atom by atom).  More cells than an eighth of the atoms would be mostly empty.
+    const int cap = std::min(256, (c.nr + 31) / 32 * 32);
+    const int cell_max = std::min(CELL_MAX, std::max(27, N / 8));
+    const size_t counters = (size_t)nf * cell_max;
+    const size_t rec_bytes = (size_t)nf * cell_max * cap * sizeof(CellRec<real>);
+    const size_t ints = (size_t)nf * (8 + (size_t)N);
+    CellBlock blk;
+    if (!cells_reserve(st, stream, counters, rec_bytes + ints * sizeof(int), &blk)) return false;
+    CellRec<real>* recs = (CellRec<real>*)blk.rest;   // records first (aligned), then the integer tables
+    int* dims = (int*)(blk.rest + rec_bytes);
+    int* of = dims + (size_t)nf * 8;
+    KernelTimer kt_("cell_build_kernel", stream);
+    hipLaunchKernelGGL(cell_build_kernel<real>, dim3((N + CELL_THREADS - 1) / CELL_THREADS, nf), dim3(CELL_THREADS), 0,
+                       stream, pos, box, N, c.Rc, blk.toggle, blk.set_ints, cell_max, cap, dims, blk.counts, recs, of);
+    A.cell_dims = dims; A.cell_counts = blk.counts; A.cell_recs = recs; A.cell_of = of;
+    A.cell_toggle = blk.toggle; A.cell_set_ints = blk.set_ints; A.cell_max = cell_max; A.cell_cap = cap;
+    return true;
+  };
   size_t lds = desc_lds_bytes<real>(c.nr);
   if (lds > 60 * 1024) return STAF_E_LIMIT;
   if (fp) {
@@ -887,9 +865,11 @@ static int desc_launch_impl(const DescConfig<real>& c, const real* pos, const re
     if (wg == 0) return finish_op(st, stream);   // no centre of these species in the frames
     lds = desc_fingerprints_lds_bytes<real>(c.nr, fp->Aa, fp->Ar, nt);
     if (!lds_request(desc_fingerprints_kernel<real>, lds)) return STAF_E_LIMIT;
+    if (!build_cells()) return reserve_failure(stream);
     KernelTimer kt_("desc_fp_kernel", stream);
     hipLaunchKernelGGL(desc_fingerprints_kernel<real>, dim3((unsigned)wg), dim3(256), lds, stream, A, M);
   } else {
+    if (!build_cells()) return reserve_failure(stream);
     KernelTimer kt_("desc_kernel", stream);
     hipLaunchKernelGGL(desc_kernel<real>, dim3((unsigned)(nf * N)), dim3(256), lds, stream, A);
   }

@@ -106,6 +106,28 @@ void* scratch_reserve(DeviceState* st, hipStream_t stream, size_t bytes) {
   return grow(st, &w->scratch, bytes, stream) ? w->scratch.buf : nullptr;
 }
 
+// Layout of a cell-list block: [toggle, padded to 256 bytes | two counter sets | this call's tables and records].
+bool cells_reserve(DeviceState* st, hipStream_t stream, size_t counters, size_t rest_bytes, CellBlock* out) {
+  constexpr size_t HEAD = 64;   // ints
+  StreamWork* w = stream_work(st, stream);
+  std::lock_guard<std::mutex> lock(g_mu);
+  counters = (counters + 63) / 64 * 64;
+  const size_t have = w->cell_counters;
+  const size_t cnt = counters > have ? counters : have;
+  const size_t bytes = (HEAD + 2 * cnt) * sizeof(int) + rest_bytes;
+  if (cnt > have || bytes > w->cells.bytes) {
+    if (!grow(st, &w->cells, bytes, stream)) return false;
+    w->cell_counters = cnt;
+    launch_fill_zero<int>((int*)w->cells.buf, (int)(HEAD + 2 * cnt), stream);
+    if (hipGetLastError() != hipSuccess) return false;
+  }
+  out->toggle = (int*)w->cells.buf;
+  out->counts = out->toggle + HEAD;
+  out->set_ints = w->cell_counters;
+  out->rest = (char*)(out->counts + 2 * w->cell_counters);
+  return true;
+}
+
 // Layout of a transpose block: [build counters | counts | keys].  The build counters must read zero when a build
 // starts: a fresh block is cleared once, on the caller's stream (a clear on the default stream is not ordered
 // before work on a non-blocking stream), and every build's sort pass leaves them at zero again.
@@ -313,6 +335,7 @@ void staf_ops_release(void) {
   for (auto& kv : st->work) {
     if (kv.second.scratch.buf) (void)hipFree(kv.second.scratch.buf);
     if (kv.second.buckets.buf) (void)hipFree(kv.second.buckets.buf);
+    if (kv.second.cells.buf) (void)hipFree(kv.second.cells.buf);
   }
   for (auto& t : st->transposes)
     if (t.buf.buf) (void)hipFree(t.buf.buf);

@@ -404,7 +404,8 @@ def test_angular_buffer_smaller_than_triplet_count(oracle, dtype):
 def test_cell_list_gives_the_same_descriptors(dtype):
     """Large frames find their neighbours through a cell list, small ones test every atom: every output of the
     descriptor op must have the same bits either way.  768 atoms (4 x 4 x 4 cells at Rc = 4.5), an orthorhombic and
-    a sheared box, some atoms moved by whole lattice vectors (positions outside the box)."""
+    a sheared box, some atoms moved by whole lattice vectors (positions outside the box); boxes divided along no or
+    one axis only; a frame with a cell that holds more atoms than the list has places for."""
     import torch
     from alphanesgpu_amd import ops, synth
     b = _synth("water768_f32")
@@ -448,6 +449,31 @@ def test_cell_list_gives_the_same_descriptors(dtype):
             every = [x.clone() for x in ops.compute_descriptors_light(tp, tb)]
             ops.descriptor_cell_threshold(1)
             cells = ops.compute_descriptors_light(tp, tb)
+            for x, y in zip(every, cells):
+                assert torch.equal(x, y)
+        # a cell with more atoms than it has places (nr = 80: 96 places): two clumps of 49 atoms in opposite corners of
+        # one cell, out of each other's reach, in a thin gas.  The centres in and around that cell test every atom.
+        Lg, ncell = 19.72, 4
+        side = Lg / ncell
+        lo = np.array([1.0, 2.0, 1.0]) * side
+        ca, cb = lo + 0.45, lo + side - 0.45
+        clump = lambda centre: centre + (rng.random((49, 3)) - 0.5) * 0.6
+        gas = rng.random((160, 3)) * Lg
+        far = lambda c: np.linalg.norm(gas - c - Lg * np.round((gas - c) / Lg), axis=1) > synth.RC + 0.6
+        gas = gas[far(ca) & far(cb)]   # (an atom between the clumps would have both for neighbours)
+        pos = np.concatenate([clump(ca), clump(cb), gas])
+        pos = pos[rng.permutation(len(pos))]
+        ng = len(pos)
+        tp = torch.as_tensor(pos.reshape(1, -1).astype(dtype)).cuda()
+        tb = torch.as_tensor(np.array([[Lg, 0, 0, Lg, 0, Lg]], dtype)).cuda()
+        ops.construct_descriptors_light(synth.RC, 80, NA, ng, tb, synth.RS, synth.RA, 1, dtype=tdt)
+        ops.descriptor_options(dist2_fma=False, zero_padding=True)
+        ops.descriptor_cell_threshold(0)
+        every = [x.clone() for x in ops.compute_descriptors_light(tp, tb)]
+        ops.descriptor_cell_threshold(1)
+        for _ in range(3):   # (the counters of the cells alternate between two sets from call to call)
+            cells = ops.compute_descriptors_light(tp, tb)
+            assert 48 <= int(every[3][..., 0].max()) < 80
             for x, y in zip(every, cells):
                 assert torch.equal(x, y)
     finally:
