@@ -280,6 +280,27 @@ __device__ __forceinline__ void desc_body(const DescArgs<real> A, const int cent
   const bool injected = A.inj_howmany != nullptr;
   // (the launch that reads a build's counters is the one that hands the next build the other set)
   if (A.cell_dims && blockIdx.x == 0 && tid == 0) A.cell_toggle[0] ^= 1;
+  // A candidate within reach takes the next place of the candidate arrays.  The lanes of a wave that have found one
+  // take their places together: one add on the counter per wave instead of one per lane (adds of several lanes on one
+  // LDS word are done one after the other).
+  auto keep = [&](const bool hit, const int j, const real d2, const real (&d)[3]) {
+    const unsigned long long m = __ballot(hit);
+    if (m == 0) return;
+    const int leader = __ffsll((long long)m) - 1;
+    int first = 0;
+    if ((tid & (WAVE - 1)) == leader) first = atomicAdd(&cnt_all, __popcll(m));
+    first = __builtin_amdgcn_readlane(first, leader);
+    if (hit) {
+      const int slot = first + (int)__builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
+      if (slot < nr) {
+        c_j[slot] = j;
+        c_d2[slot] = d2;
+        c_d[3 * slot] = d[0];
+        c_d[3 * slot + 1] = d[1];
+        c_d[3 * slot + 2] = d[2];
+      }
+    }
+  };
   bool by_cells = false;
   if (!injected && A.cell_dims) {
     // Candidates = the atoms of the centre's cell and its neighbours (every atom appears once: an axis has one cell or
@@ -328,23 +349,6 @@ __device__ __forceinline__ void desc_body(const DescArgs<real> A, const int cent
     // (an overfull cell lacks the records of some of its atoms: this centre then tests every atom of the frame)
     by_cells = nb_groups >= 0;
     const int total = by_cells ? nb_groups * GROUP : 0;
-    auto candidate = [&](const CellRec<real>& c) {
-      const int j = c.j;
-      if (j == i) return;
-      real sj[3], d[3];
-      to_frac(inv, c.x, c.y, c.z, sj);
-      const real d2 = mic_delta(box, sj, si, A.dist2_fma, A.skip_pbc, d);
-      if (d2 < rc2) {
-        const int slot = atomicAdd(&cnt_all, 1);
-        if (slot < nr) {
-          c_j[slot] = j;
-          c_d2[slot] = d2;
-          c_d[3 * slot] = d[0];
-          c_d[3 * slot + 1] = d[1];
-          c_d[3 * slot + 2] = d[2];
-        }
-      }
-    };
     for (int t0 = 0; t0 < total; t0 += BATCH * 256) {
       CellRec<real> rc_[BATCH];
       bool have[BATCH];
@@ -359,8 +363,17 @@ __device__ __forceinline__ void desc_body(const DescArgs<real> A, const int cent
         }
       }
 #pragma unroll
-      for (int u = 0; u < BATCH; u++)
-        if (have[u]) candidate(rc_[u]);
+      for (int u = 0; u < BATCH; u++) {
+        real sj[3], d[3] = {0, 0, 0};
+        real d2 = rc2;
+        int j = i;
+        if (have[u]) {
+          j = rc_[u].j;
+          to_frac(inv, rc_[u].x, rc_[u].y, rc_[u].z, sj);
+          d2 = mic_delta(box, sj, si, A.dist2_fma, A.skip_pbc, d);
+        }
+        keep(d2 < rc2 && j != i, j, d2, d);
+      }
     }
   }
   if (by_cells) {
@@ -381,16 +394,7 @@ __device__ __forceinline__ void desc_body(const DescArgs<real> A, const int cent
         real sj[3], d[3];
         to_frac(inv, px[u], py[u], pz[u], sj);
         real d2 = mic_delta(box, sj, si, A.dist2_fma, A.skip_pbc, d);
-        if (d2 < rc2 && j != i) {
-          int slot = atomicAdd(&cnt_all, 1);
-          if (slot < nr) {
-            c_j[slot] = j;
-            c_d2[slot] = d2;
-            c_d[3 * slot] = d[0];
-            c_d[3 * slot + 1] = d[1];
-            c_d[3 * slot + 2] = d[2];
-          }
-        }
+        keep(d2 < rc2 && j != i, j, d2, d);
       }
     }
   } else {
