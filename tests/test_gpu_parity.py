@@ -480,6 +480,50 @@ def test_cell_list_gives_the_same_descriptors(dtype):
         ops.descriptor_cell_threshold(2048)
 
 
+def test_cell_list_in_a_replayed_graph():
+    """The descriptor op with the cell list, captured once in a HIP graph: the cells' counters alternate between two
+    sets from call to call, also from replay to replay and across eager calls on the same stream in between.  Every
+    replay, on new positions each time, gives what the search over all atoms gives for them, bit for bit."""
+    import torch
+    from alphanesgpu_amd import ops, synth
+    b = _synth("water768_f32")
+    N, nf = b["N"], 2
+    pos0 = b["pos"][:nf].astype(np.float64).reshape(nf, -1)
+    tb = torch.as_tensor(np.ascontiguousarray(b["box"][:nf]).astype(np.float64)).cuda()
+    rng = np.random.default_rng(11)
+    frames = [torch.as_tensor(pos0 + rng.normal(0, 0.05, pos0.shape)).cuda() for _ in range(5)]
+    ops.construct_descriptors_light(synth.RC, 80, NA, N, tb, synth.RS, synth.RA, nf, dtype=torch.float64)
+    ops.descriptor_options(dist2_fma=False, zero_padding=True)
+    try:
+        ops.descriptor_cell_threshold(0)
+        want = [[x.clone() for x in ops.compute_descriptors_light(f, tb)] for f in frames]
+        ops.descriptor_cell_threshold(1)
+        tp = frames[0].clone()
+        side = torch.cuda.Stream()                       # the library keeps its work areas, cells included, per stream
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            held = ops.compute_descriptors_light(tp, tb)     # sizes the work areas before the capture
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            held = ops.compute_descriptors_light(tp, tb, out=held)
+        for rep, (f, w) in enumerate(zip(frames, want)):
+            tp.copy_(f)
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            for x, y in zip(held, w):
+                assert torch.equal(x, y), f"replay {rep}"
+            with torch.cuda.stream(side):
+                for _ in range(rep % 2 + 1):             # one or two eager calls: the next replay starts on either set
+                    eager = ops.compute_descriptors_light(f, tb)
+            torch.cuda.synchronize()
+            for x, y in zip(eager, w):
+                assert torch.equal(x, y)
+    finally:
+        ops.descriptor_cell_threshold(2048)
+
+
 def test_hip_graph_replay_with_two_streams_matches_eager():
     """The whole op sequence captured once in a HIP graph, the two per-species chains forked onto their own streams
     (per-stream scratch inside the library): every replay, with eager calls and synchronisations in between, gives
