@@ -131,7 +131,6 @@ __device__ inline real norm_plain(const real* d) {
 // device-side toggle names, clears the whole other set, and the descriptor launch that follows flips the toggle --
 // no launch of its own for the clearing, and nothing a replayed graph would have to be told.
 // ---------------------------------------------------------------------------
-constexpr int CELL_MAX = 4096;       // most cells of a frame
 constexpr int CELL_THREADS = 256;
 
 // An atom as the neighbour search reads it: Cartesian position and index in one 16-byte (float) or 32-byte (double)
@@ -175,7 +174,17 @@ __global__ __launch_bounds__(CELL_THREADS) void cell_build_kernel(const real* __
     const double hc = vol / fabs(ax * by);
     int n[3] = {(int)(ha / (double)Rc), (int)(hb / (double)Rc), (int)(hc / (double)Rc)};
     for (int c = 0; c < 3; c++) n[c] = n[c] < 3 ? 1 : (n[c] > 1023 ? 1023 : n[c]);   // (10 bits each in cell_of)
-    while ((long long)n[0] * n[1] * n[2] > cell_max) {   // coarser cells only widen the search
+    // coarser cells only widen the search: all axes by the same factor first, then the longest one step at a time
+    if ((long long)n[0] * n[1] * n[2] > cell_max) {
+      const double f = cbrt((double)cell_max / ((double)n[0] * n[1] * n[2]));
+      for (int c = 0; c < 3; c++)
+        if (n[c] > 1) {
+          int m = (int)(n[c] * f) + 1;
+          m = m < 3 ? 3 : m;
+          n[c] = m < n[c] ? m : n[c];   // never finer than the cut-off allows
+        }
+    }
+    while ((long long)n[0] * n[1] * n[2] > cell_max) {
       int big = n[0] >= n[1] && n[0] >= n[2] ? 0 : (n[1] >= n[2] ? 1 : 2);
       n[big] = n[big] - 1 < 3 ? 1 : n[big] - 1;
     }
@@ -823,7 +832,8 @@ static int desc_launch_impl(const DescConfig<real>& c, const real* pos, const re
     // cell of nr places overflows only in frames far denser in one spot than on average (and those are searched
     // atom by atom).  More cells than an eighth of the atoms would be mostly empty.
     const int cap = std::min(256, (c.nr + 31) / 32 * 32);
-    const int cell_max = std::min(CELL_MAX, std::max(27, N / 8));
+    // (the search numbers a cell's groups of 16 records in 26 bits)
+    const int cell_max = (int)std::min<long long>((1ll << 26) / (cap / 16) - 1, std::max(27, N / 8));
     const size_t counters = (size_t)nf * cell_max;
     const size_t rec_bytes = (size_t)nf * cell_max * cap * sizeof(CellRec<real>);
     const size_t ints = (size_t)nf * (8 + (size_t)N);

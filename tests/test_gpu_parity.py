@@ -476,6 +476,22 @@ def test_cell_list_gives_the_same_descriptors(dtype):
             assert 48 <= int(every[3][..., 0].max()) < 80
             for x, y in zip(every, cells):
                 assert torch.equal(x, y)
+        # a thin frame: the 96-atom box 3 x 3 x 3 times, stretched by 1.3 -- 8 cells of width Rc fit along an axis, but
+        # the grid has at most N / 8 = 324 cells: a coarser one (6 x 7 x 7) serves
+        t = np.array([[x, y, z] for x in range(3) for y in range(3) for z in range(3)], dtype)
+        pos = (1.3 * (p96.reshape(1, -1, 3) + L9 * t[:, None, :])).reshape(1, -1)
+        nthin = pos.shape[1] // 3
+        tp = torch.as_tensor(np.ascontiguousarray(pos.astype(dtype))).cuda()
+        tb = torch.as_tensor(np.array([[3.9 * L9, 0, 0, 3.9 * L9, 0, 3.9 * L9]], dtype)).cuda()
+        ops.construct_descriptors_light(synth.RC, 80, NA, nthin, tb, synth.RS, synth.RA, 1, dtype=tdt)
+        ops.descriptor_options(dist2_fma=False, zero_padding=True)
+        ops.descriptor_cell_threshold(0)
+        every = [x.clone() for x in ops.compute_descriptors_light(tp, tb)]
+        ops.descriptor_cell_threshold(1)
+        cells = ops.compute_descriptors_light(tp, tb)
+        assert nthin == 2592 and int(every[3][..., 0].min()) > 5
+        for x, y in zip(every, cells):
+            assert torch.equal(x, y)
     finally:
         ops.descriptor_cell_threshold(2048)
 
