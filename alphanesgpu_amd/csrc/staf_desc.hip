@@ -688,7 +688,10 @@ size_t desc_fingerprints_lds_bytes(int nr, int Aa, int Ar, int nt) {
 // ---- host side -------------------------------------------------------------
 
 static std::mutex g_cfg_mu;
-static int g_cell_threshold = 2048;   // frames of at least this many atoms search through a cell list
+// Frames of at least this many atoms search through a cell list.  Testing every atom of a 4096-atom frame costs a
+// centre's workgroup about what the launch that builds the cells costs the call (measured: the search over all
+// atoms is 3-8 us per call faster up to 3456 atoms, level at 4608-6144, twice as slow at 20736).
+static int g_cell_threshold = 4096;
 // Geometry set by construct: one configuration per device and precision.  construct() stores it for the device
 // that is current and as the process default, which serves devices construct() was never called on (the
 // reference keeps one process-wide configuration, STAF/src/descriptor_builder/reforce.cc:97-158).

@@ -136,7 +136,7 @@ def descriptor_options(dist2_fma=False, zero_padding=False):
     call("staf_op_descriptor_options", _I(int(bool(dist2_fma))), _I(int(bool(zero_padding))))
 
 
-def descriptor_cell_threshold(n_atoms=2048):
+def descriptor_cell_threshold(n_atoms=4096):
     """Frames of at least n_atoms atoms search their neighbours through a cell list (same outputs)."""
     call("staf_op_descriptor_cell_threshold", _I(int(n_atoms)))
 

@@ -383,7 +383,7 @@ def run_md(args, workload):
         "config": {"workload": workload, "entry": "staf_compute (MD entry, include/staf.h)", "mode": "energy + forces + virial",
                    "atoms": N, "frames_per_step": 1, "Rc": synth.RC, "radial_buffer": nr, "angular_buffer": na,
                    "Ar": Ar, "Aa": Aa, "mlp": "60-140-140-1 tanh per species, float64, random init, on the GPU",
-                   "neighbour_list": "the library's own, rebuilt on every call (cell list from 2048 atoms on)",
+                   "neighbour_list": "the library's own, rebuilt on every call (cell list from 4096 atoms on)",
                    "boundary": "host arrays in (positions, box, species) and out (energy, forces, virial): the PCIe "
                                "copies and the call's one synchronisation are inside the timed region",
                    "launch": "the call's kernel sequence recorded once as a HIP graph and replayed",

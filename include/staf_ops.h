@@ -137,7 +137,7 @@ int staf_op_construct_descriptors_light_f64(double radial_cutoff, int radial_buf
 int staf_op_descriptor_options(int dist2_fma, int zero_padding);
 
 /* Frames of at least n_atoms atoms find their neighbours through a cell list (the role of the binning kernels of
- * celle_gpu.cu.cc:11-101), smaller ones test every atom of the frame; default 2048, n_atoms <= 0: never.  The
+ * celle_gpu.cu.cc:11-101), smaller ones test every atom of the frame; default 4096, n_atoms <= 0: never.  The
  * outputs are the same either way. */
 int staf_op_descriptor_cell_threshold(int n_atoms);
 

@@ -493,7 +493,7 @@ def test_cell_list_gives_the_same_descriptors(dtype):
         for x, y in zip(every, cells):
             assert torch.equal(x, y)
     finally:
-        ops.descriptor_cell_threshold(2048)
+        ops.descriptor_cell_threshold(4096)
 
 
 def test_cell_list_in_a_replayed_graph():
@@ -537,7 +537,7 @@ def test_cell_list_in_a_replayed_graph():
             for x, y in zip(eager, w):
                 assert torch.equal(x, y)
     finally:
-        ops.descriptor_cell_threshold(2048)
+        ops.descriptor_cell_threshold(4096)
 
 
 def test_hip_graph_replay_with_two_streams_matches_eager():
@@ -891,9 +891,9 @@ def test_config5_water6144_fp64(oracle):
     """The large-box configuration: 6144 atoms, one frame, fp64; above the library's default threshold, so the neighbours are
     found through the cell list (8 x 8 x 8 cells) while the oracle tests all pairs."""
     from alphanesgpu_amd import ops
-    ops.descriptor_cell_threshold(2048)
+    ops.descriptor_cell_threshold(4096)
     b = _synth("water6144")
-    assert b["N"] == 6144 and b["N"] >= 2048
+    assert b["N"] == 6144 and b["N"] >= 4096
     print(_run_case(oracle, b, np.float64))
 
 

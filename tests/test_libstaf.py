@@ -164,7 +164,7 @@ def test_compute_matches_oracle_pipeline_fp64_model(oracle):
 @pytest.mark.gpu
 def test_compute_6144_atom_box_matches_oracle_pipeline(oracle):
     """The large-box configuration through the MD entry: 2048 water molecules, one call, neighbour list rebuilt by the library
-    (cell list: 6144 >= 2048 atoms), no tensor of the angular buffer's width on the device; energy and forces against
+    (cell list: 6144 >= 4096 atoms), no tensor of the angular buffer's width on the device; energy and forces against
     the oracle ops wired in the reference's order (all-pairs neighbour search there), 1e-10."""
     from alphanesgpu_amd import libstaf, synth
     from test_oracle_pins import energy_and_forces
