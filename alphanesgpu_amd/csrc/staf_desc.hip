@@ -234,10 +234,10 @@ __device__ inline void zero_fill(char* p, unsigned nbytes, int tid) {
 // Waves per SIMD the allocation is held to: without a bound the single-precision kernel takes 112 scalar registers
 // (seven waves: 1792 resident workgroups for the 3072 centres of four 768-atom frames) and the double-precision
 // one 104 vector registers (four waves); at eight and five the launch needs fewer rounds of workgroups.
-constexpr int DESC_MIN_WAVES_F32 = 8, DESC_MIN_WAVES_F64 = 5;
+constexpr int DESC_MIN_WAVES_F32 = 8, DESC_MIN_WAVES_F64 = 5, DESC_RADIAL_MIN_WAVES_F64 = 7;
 // The kernel's body for the 256-thread workgroup of centre `centre` (frame-major over all N atoms): desc_kernel
 // below, and the launch that goes on to the centre's fingerprints in the same workgroup.
-template <typename real>
+template <typename real, bool ANGULAR = true>
 __device__ __forceinline__ void desc_body(const DescArgs<real> A, const int centre) {
   using real2 = typename Vec2<real>::type;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -544,7 +544,7 @@ __device__ __forceinline__ void desc_body(const DescArgs<real> A, const int cent
     if (A.tr.rowsum) const_cast<unsigned*>(A.tr.rowsum)[atom] = row_sum + (unsigned)n;
   }
 
-  if (!A.angular) return;
+  if (!ANGULAR || !A.angular) return;
   // 4. angular fill: triplet nn <-> (j<k) over the first m sorted neighbours
   int ntr = (m * (m - 1)) / 2;
   if (ntr > na) ntr = na;
@@ -608,6 +608,13 @@ template <typename real>
 __global__ __launch_bounds__(256, sizeof(real) == 4 ? DESC_MIN_WAVES_F32 : DESC_MIN_WAVES_F64) void
 desc_kernel(DescArgs<real> A) {
   desc_body<real>(A, (int)blockIdx.x);
+}
+
+// The radial-only launch (MD entry) without the code of the triplet fill: fewer registers, more workgroups per CU
+// to hide the chain of dependent reads and barriers the search and the sort are.
+template <typename real>
+__global__ __launch_bounds__(256, sizeof(real) == 4 ? DESC_MIN_WAVES_F32 : DESC_RADIAL_MIN_WAVES_F64) void desc_radial_kernel(DescArgs<real> A) {
+  desc_body<real, false>(A, (int)blockIdx.x);
 }
 
 template <typename real>
@@ -888,7 +895,8 @@ static int desc_launch_impl(const DescConfig<real>& c, const real* pos, const re
   } else {
     if (!build_cells()) return reserve_failure(stream);
     KernelTimer kt_("desc_kernel", stream);
-    hipLaunchKernelGGL(desc_kernel<real>, dim3((unsigned)(nf * N)), dim3(256), lds, stream, A);
+    if (angular) hipLaunchKernelGGL(desc_kernel<real>, dim3((unsigned)(nf * N)), dim3(256), lds, stream, A);
+    else hipLaunchKernelGGL(desc_radial_kernel<real>, dim3((unsigned)(nf * N)), dim3(256), lds, stream, A);
   }
   if (!symmetric) {
     KernelTimer kt_("transpose_sort_kernel", stream);
